@@ -1,0 +1,84 @@
+"""Run single quantized operators on any art-ABI workspace (reference `quant`, or the repo's `hip`)
+from numpy inputs.  Signatures mirror oracle/orc.py so that tests can compare the two directly."""
+import numpy as np
+
+from nart_amd import art
+
+
+def _zero_ref_conv_scratch(op):
+    """Give the reference conv the zeroed column buffer it silently assumes.
+
+    The reference's im2col leaves the padding taps of its column buffer unwritten and relies on the
+    buffer being zero (im2col.cpp:568-600; the buffer comes from realloc(NULL, n), art/src/mem.c:45-55).
+    That holds for first-touch pages of a freshly started runner, not for a recycled heap chunk inside
+    a long test process.  `temp_data` is the mem_t* that follows op_t (64 bytes), eight uint32, nine
+    data pointers and three function pointers in op_conv_2d_t (conv_2d.h:40-72), i.e. offset 192."""
+    import ctypes as C
+    mem = C.cast(C.c_void_p.from_address(C.addressof(op.ptr.contents) + 192).value, C.POINTER(art.mem_t))
+    tp = mem.contents.tp.contents
+    C.memset(tp.cpu_data_func(mem), 0, tp.size_func(mem))
+
+
+def _q(**kw):
+    return kw
+
+
+def _run(op):
+    op.prepare().run()
+    out = op.output(0).numpy()
+    op.delete()
+    return out
+
+
+def conv2d_u8(ws, x, w, bias, pad, stride, group, ialpha, izp, walpha, wzp, oalpha, ozp,
+              per_image=True, relu=None):
+    """per_image: the reference CPU conv aborts for batch > 1 (conv_2d_uint8_impl.c:104), so feed it
+    one image at a time; other workspaces may take the whole batch."""
+    q = _q(ialpha=ialpha, izp=izp, walpha=walpha, wzp=wzp, oalpha=oalpha, ozp=ozp)
+    tw = ws.tensor(w)
+    tb = ws.tensor(np.asarray(bias, np.int32)) if bias is not None else None
+    outs = []
+    chunks = [x[i:i + 1] for i in range(x.shape[0])] if per_image else [x]
+    for xc in chunks:
+        tx = ws.tensor(xc)
+        op = ws.conv2d(tx, tw, tb, pad, stride, group, q, relu=relu).prepare()
+        if ws.name.startswith("quant"):  # the reference names its workspaces quant<i>
+            _zero_ref_conv_scratch(op)
+        outs.append(op.run().output(0).numpy())
+        op.delete()
+    return np.concatenate(outs, 0)
+
+
+def ip_u8(ws, x, w, bias, ialpha, izp, walpha, wzp, oalpha, ozp):
+    q = _q(ialpha=ialpha, izp=izp, walpha=walpha, wzp=wzp, oalpha=oalpha, ozp=ozp)
+    if x.ndim == 2:  # the reference sizes its scratch from dim[1..3] (ip.cpp:305-308)
+        x = x.reshape(x.shape[0], x.shape[1], 1, 1)
+    tb = ws.tensor(np.asarray(bias, np.int32)) if bias is not None else None
+    return _run(ws.ip(ws.tensor(x), ws.tensor(w), tb, q))
+
+
+def add_u8(ws, a, b, ialpha0, izp0, ialpha1, izp1, oalpha, ozp):
+    q = _q(ialpha=[ialpha0, ialpha1], izp=[izp0, izp1], oalpha=oalpha, ozp=ozp)
+    return _run(ws.add(ws.tensor(a), ws.tensor(b), q))
+
+
+def eltwise_u8(ws, ins, ialpha, izp, oalpha, ozp, operation=1, coeff=None):
+    q = _q(ialpha=list(ialpha), izp=list(izp), oalpha=oalpha, ozp=ozp)
+    return _run(ws.eltwise([ws.tensor(a) for a in ins], q, operation, coeff))
+
+
+def relu_u8(ws, x, ialpha, izp, oalpha, ozp):
+    return _run(ws.relu(ws.tensor(x), _q(ialpha=ialpha, izp=izp, oalpha=oalpha, ozp=ozp)))
+
+
+def pool_u8(ws, x, kernel, pad, stride, method, ceil_mode, ialpha, izp, oalpha, ozp):
+    q = _q(ialpha=ialpha, izp=izp, oalpha=oalpha, ozp=ozp)
+    return _run(ws.pool(ws.tensor(x), kernel, pad, stride, method, ceil_mode, q))
+
+
+def quantize_u8(ws, x, oalpha, ozp):
+    return _run(ws.quantize(ws.tensor(np.asarray(x, np.float32)), oalpha, ozp))
+
+
+def dequantize_u8(ws, x, ialpha, izp):
+    return _run(ws.dequantize(ws.tensor(x), ialpha, izp))
