@@ -1,0 +1,138 @@
+/*
+ * hipq — C ABI of the MI355X (gfx950) quantized-inference kernels.
+ *
+ * This is the boundary between host code (the `hip` case module for NART's art runtime, the Python
+ * runner, tests, benchmarks) and the hand-written HIP kernels.  Only plain C types cross it: device
+ * and host pointers, sizes, scalars, one POD descriptor per operator and opaque plan handles.
+ *
+ * Each entry point names the function of the reference CPU `quant` module (paths relative to
+ * art/modules/quant/) whose results it reproduces BIT-EXACTLY on the same inputs:
+ *   - integer operators (conv, ip, add, eltwise, relu, pool): identical int32 accumulators and
+ *     identical uint8 outputs, no tolerance;
+ *   - quantize: IEEE fp32 subtract and divide followed by the reference's "+0.5 in double, truncate"
+ *     rounding, identical bytes; dequantize: one fp32 multiply, identical bits.
+ *
+ * Device tensor layout.  The reference works on dense NCHW.  On the device, 4-D uint8 activations
+ * are kept channels-last ("NHWC") with the channel count padded to a stride `cs`:
+ *       element (n, c, h, w) lives at byte ((n*H + h)*W + w)*cs + c,          cs = hipq_channel_stride(C)
+ * cs is 4 for C <= 4 (network inputs), otherwise C rounded up to a multiple of 16.  Bytes in the pad
+ * channels are unspecified and never influence valid outputs.  2-D activations [M, K] are NHWC with
+ * H = W = 1.  hipq_nchw_to_nhwc_u8 / hipq_nhwc_to_nchw_u8 convert at the host boundary.
+ *
+ * Conventions: every function returns 0 on success and a non-zero code on failure, with a
+ * human-readable reason available from hipq_last_error().  `stream` is a hipStream_t passed as
+ * void* (NULL = the default stream); all launches are asynchronous on it.  No function falls back to
+ * host computation: without a usable GPU every compute entry point fails with an error.
+ */
+#ifndef HIPQ_H
+#define HIPQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define HIPQ_ABI_VERSION 1
+
+#define HIPQ_ELTWISE_SUM 1 /* SETTING_ELTWISE_OP_SUM */
+#define HIPQ_ELTWISE_MAX 2 /* SETTING_ELTWISE_OP_MAX */
+#define HIPQ_POOL_MAX 0    /* SETTING_POOL_MAX */
+#define HIPQ_POOL_AVE 1    /* SETTING_POOL_AVE */
+#define HIPQ_MAX_ELTWISE_INPUTS 8
+
+int hipq_abi_version(void);
+const char *hipq_last_error(void);
+
+/* Fixed-point scale decomposition, get_quant_scale* — include/art/quant/quant_helper.h:60-118. */
+void hipq_quant_scale(float scale, int bits, uint32_t *mult, int *shift);
+
+/* Channel stride of the device layout for a tensor with C channels. */
+int hipq_channel_stride(int C);
+
+/* ---- layout conversion at the host boundary (no counterpart in the reference, which is NCHW only) */
+int hipq_nchw_to_nhwc_u8(const void *src_nchw, void *dst_nhwc, int N, int C, int H, int W, int cs,
+                         void *stream);
+int hipq_nhwc_to_nchw_u8(const void *src_nhwc, void *dst_nchw, int N, int C, int H, int W, int cs,
+                         void *stream);
+
+/* ---- convolution ---------------------------------------------------------------------------- */
+typedef struct hipq_conv2d_desc {
+    int32_t N, C, H, W;       /* input, logical dims */
+    int32_t K, R, S;          /* output channels, kernel height / width */
+    int32_t pad_h, pad_w, stride_h, stride_w, group;
+    int32_t in_cs, out_cs;    /* channel strides of x and y on the device */
+    float ialpha, walpha, oalpha;
+    int32_t izp, wzp, ozp;    /* zero points, 0..255 */
+    int32_t obits;            /* output saturates to [0, 2^obits - 1] */
+    int32_t relu;             /* 1: y = max(y, ozp) after requantisation (== a following quant relu
+                                 op with equal in/out scale and zero point, src/op/relu.c:76-115) */
+} hipq_conv2d_desc;
+
+typedef struct hipq_conv2d_plan hipq_conv2d_plan;
+
+/*
+ * Setup: derives (mult, shift) from ialpha*walpha/oalpha, re-packs the weights for the kernel chosen
+ * for this shape (int8 MFMA fragments for dense convolutions; tap-major vectors for depthwise) and
+ * folds bias and the zero-point terms into one int32 per output channel; uploads both.
+ * w: host, uint8 [K, C/group, R, S]; bias: host, int32 [K] or NULL (NULL == zeros).
+ * Replaces op_quant_conv_2d_tp_prepare + the per-run widening in op_conv_2d_u8xu8_run
+ * (src/op/conv_2d.c:95-147, src/op/conv_2d_uint8_impl.c:107-124).
+ */
+int hipq_conv2d_plan_create(const hipq_conv2d_desc *desc, const uint8_t *w, const int32_t *bias,
+                            hipq_conv2d_plan **plan_out);
+void hipq_conv2d_plan_destroy(hipq_conv2d_plan *plan);
+/* Name of the kernel variant the plan dispatches to (for logs and tests). */
+const char *hipq_conv2d_plan_kernel(const hipq_conv2d_plan *plan);
+
+/*
+ * Run: op_conv_2d_u8xu8_run — src/op/conv_2d_uint8_impl.c:39-165 (im2col src/utils/im2col.cpp:487,
+ * GEMM src/gemm/default/gemm.c:306).  x, y: device NHWC.  acc_out: optional device int32
+ * [N*OH*OW, out_cs] that receives the raw accumulators (bias included), NULL to skip.
+ * Unlike the reference (which aborts for N > 1, conv_2d_uint8_impl.c:104) any batch size runs.
+ */
+int hipq_conv2d_run(const hipq_conv2d_plan *plan, const void *x, void *y, int32_t *acc_out,
+                    void *stream);
+
+/* ---- inner product: op_quant_ip_u8xu8_run — src/op/ip.cpp:133-209.
+ * Expressed as a 1x1 convolution over M "pixels": desc {N=M, C=Kdim, H=W=1, K=Nout, R=S=1}.
+ * When the reference's input is [M, C, H, W] with H*W > 1, pass the weights re-ordered from
+ * (c, h, w) to (h, w, c-with-stride) — hipq_ip_reorder_weights does that on the host. */
+int hipq_ip_reorder_weights(const uint8_t *w, uint8_t *w_out, int Nout, int C, int H, int W, int cs,
+                            int wzp);
+
+/* ---- element-wise --------------------------------------------------------------------------- */
+/* op_quant_add_run — src/op/add.c:83-148.  count = number of bytes (pad channels included). */
+int hipq_add_u8(const void *a, const void *b, void *y, size_t count, float ialpha0, int izp0,
+                float ialpha1, int izp1, float oalpha, int ozp, int obits, void *stream);
+/* op_quant_eltwise_accumulate_output_sum / _max — src/op/eltwise.c:137-271. */
+int hipq_eltwise_u8(const void *const *in, int n_in, const float *coeff, const float *ialpha,
+                    const uint8_t *izp, void *y, size_t count, int operation, float oalpha, int ozp,
+                    int obits, void *stream);
+/* op_quant_relu_run — src/op/relu.c:76-115. */
+int hipq_relu_u8(const void *x, void *y, size_t count, float ialpha, int izp, float oalpha, int ozp,
+                 int obits, void *stream);
+
+/* ---- pooling: op_quant_pool_max_run / op_quant_pool_average_run — src/op/pool.c:96-249.
+ * x: NHWC [N,H,W,cs], y: NHWC [N,OH,OW,cs]; OH, OW as inferred by art/src/op.c:903-967. */
+int hipq_pool_u8(const void *x, void *y, int N, int C, int H, int W, int OH, int OW, int cs, int kh,
+                 int kw, int pad_h, int pad_w, int stride_h, int stride_w, int method, float ialpha,
+                 int izp, float oalpha, int ozp, int obits, void *stream);
+
+/* ---- quantize / dequantize -------------------------------------------------------------------
+ * op_quantize_run_u8 — src/op/quantize.c:145-157: x fp32 dense NCHW (as the host wrote it), y uint8
+ * NHWC with stride cs (pass H = W = 1, cs = C for a flat tensor). */
+int hipq_quantize_u8(const float *x_nchw, void *y_nhwc, int N, int C, int H, int W, int cs,
+                     float oalpha, int ozp, int obits, void *stream);
+/* op_dequantize_run_u8 — src/op/dequantize.c:111-123: x uint8 NHWC, y fp32 dense NCHW. */
+int hipq_dequantize_u8(const void *x_nhwc, float *y_nchw, int N, int C, int H, int W, int cs,
+                       float ialpha, int izp, void *stream);
+
+/* A plain device-to-device copy kernel of known size; the calibration reference for HBM counters. */
+int hipq_copy_bytes(const void *src, void *dst, size_t count, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HIPQ_H */

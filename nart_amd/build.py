@@ -1,0 +1,88 @@
+"""Builds the native libraries of the package in-tree (no GPU needed: hipcc cross-compiles gfx950).
+
+  nart_amd/lib/libhipq.so             HIP kernels + their C ABI (include/hipq.h)
+  nart_amd/lib/libart.so              the minimal host core implementing the art C API (include/art/)
+  nart_amd/lib/libart_module_hip.so   the `hip` case module (exports hip_module_tp)
+
+Usage: python -m nart_amd.build [--force]
+"""
+import os
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+CSRC = os.path.join(HERE, "csrc")
+LIB = os.path.join(HERE, "lib")
+INC = os.path.join(ROOT, "include")
+
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+# packed-fp32 instructions are switched off on purpose (they have produced wrong results on this pool)
+HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function"]
+
+
+def _run(cmd):
+    print(" ".join(cmd), flush=True)
+    subprocess.check_call(cmd)
+
+
+def _newer(target, sources):
+    if not os.path.exists(target):
+        return False
+    t = os.path.getmtime(target)
+    return all(os.path.getmtime(s) <= t for s in sources)
+
+
+def _glob(sub, exts):
+    d = os.path.join(CSRC, sub)
+    if not os.path.isdir(d):
+        return []
+    return sorted(os.path.join(d, f) for f in os.listdir(d) if f.endswith(exts))
+
+
+def build_hipq(force=False):
+    srcs = _glob("hipq", (".hip", ".cpp"))
+    deps = srcs + _glob("hipq", (".h",)) + [os.path.join(INC, "hipq.h")]
+    out = os.path.join(LIB, "libhipq.so")
+    if not force and _newer(out, deps):
+        return out
+    os.makedirs(LIB, exist_ok=True)
+    objs = []
+    for s in srcs:
+        o = os.path.join(LIB, "obj_hipq_" + os.path.basename(s) + ".o")
+        lang = ["-x", "hip"] if s.endswith(".hip") else []
+        _run([HIPCC] + HIP_FLAGS + ["-I" + INC, "-I" + os.path.join(CSRC, "hipq"), "-c"] + lang + [s, "-o", o])
+        objs.append(o)
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + objs)
+    return out
+
+
+def build_art(force=False):
+    outs = []
+    core_src = _glob("core", (".c", ".cpp"))
+    if core_src:
+        out = os.path.join(LIB, "libart.so")
+        deps = core_src + _glob("core", (".h",)) + [os.path.join(INC, "art", f) for f in os.listdir(os.path.join(INC, "art"))]
+        if force or not _newer(out, deps):
+            _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-DART_CONSTRAINT_WITH_NAME", "-I" + INC,
+                  "-o", out] + core_src + ["-lm", "-ldl"])
+        outs.append(out)
+    mod_src = _glob("module", (".cpp",))
+    if mod_src:
+        out = os.path.join(LIB, "libart_module_hip.so")
+        deps = mod_src + _glob("module", (".h",)) + [os.path.join(INC, "hipq.h")]
+        if force or not _newer(out, deps):
+            _run([HIPCC, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-DART_CONSTRAINT_WITH_NAME", "-I" + INC,
+                  "-I" + os.path.join(CSRC, "module"), "-o", out] + mod_src
+                 + ["-L" + LIB, "-lhipq", "-Wl,-rpath,$ORIGIN"])
+        outs.append(out)
+    return outs
+
+
+def build_all(force=False):
+    return [build_hipq(force)] + build_art(force)
+
+
+if __name__ == "__main__":
+    print("\n".join(build_all("--force" in sys.argv)))

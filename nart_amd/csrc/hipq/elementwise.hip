@@ -1,0 +1,502 @@
+// Memory-bound uint8 operators for gfx950: add, n-ary eltwise, relu, pooling, quantize, dequantize,
+// layout conversion.  Each is a grid-stride wavefront kernel moving 128 bits per lane per access so that
+// a wave touches 1 KiB of contiguous HBM per instruction; the integer arithmetic is the reference's
+// fixed-point arithmetic, statement for statement (files under art/modules/quant/src/op/).
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+
+#include "common.h"
+
+namespace hipq {
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+static inline unsigned grid_for(size_t work_items, int per_block = 256)
+{
+    const size_t b = (work_items + per_block - 1) / per_block;
+    return (unsigned)std::min<size_t>(std::max<size_t>(b, 1), 256 * 16);
+}
+
+// ---- add (add.c:83-148) -----------------------------------------------------------------------
+struct AddArgs {
+    const uint8_t *a, *b; // already ordered so that alpha(a) <= alpha(b)
+    uint8_t *y;
+    size_t count;
+    uint32_t m0, m1;
+    int s0, s1, sh; // s0 - sh, s1 - sh, sh
+    int z0, z1, oz, hi;
+};
+
+__device__ static inline uint32_t add_one(uint32_t x0, uint32_t x1, const AddArgs &p)
+{
+    const int32_t i0 = (int32_t)x0 - p.z0, i1 = (int32_t)x1 - p.z1;
+    const int32_t p0 = (int32_t)(p.m0 * (uint32_t)i0), p1 = (int32_t)(p.m1 * (uint32_t)i1);
+    const int32_t t = (int32_t)(rshift_rn(p0, p.s0) + rshift_rn(p1, p.s1));
+    return (uint32_t)sat_hi((int32_t)(rshift_rn(t, p.sh) + p.oz), p.hi);
+}
+
+__global__ __launch_bounds__(256) void add_u8_kernel(const AddArgs p)
+{
+    const size_t nvec = p.count / 16;
+    const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nthr = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = tid; i < nvec; i += nthr) {
+        const u32x4 va = reinterpret_cast<const u32x4 *>(p.a)[i], vb = reinterpret_cast<const u32x4 *>(p.b)[i];
+        u32x4 vy;
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            uint32_t o = 0;
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                o |= add_one((va[d] >> (8 * e)) & 255, (vb[d] >> (8 * e)) & 255, p) << (8 * e);
+            vy[d] = o;
+        }
+        reinterpret_cast<u32x4 *>(p.y)[i] = vy;
+    }
+    for (size_t i = nvec * 16 + tid; i < p.count; i += nthr)
+        p.y[i] = (uint8_t)add_one(p.a[i], p.b[i], p);
+}
+
+// ---- n-ary eltwise (eltwise.c:137-271) ---------------------------------------------------------
+struct EltArgs {
+    const uint8_t *in[HIPQ_MAX_ELTWISE_INPUTS];
+    uint32_t mult[HIPQ_MAX_ELTWISE_INPUTS];
+    int shift[HIPQ_MAX_ELTWISE_INPUTS]; // shift[n] - s0
+    int zp[HIPQ_MAX_ELTWISE_INPUTS];
+    int n_in, s0, oz, hi, is_max;
+    uint8_t *y;
+    size_t count;
+};
+
+__global__ __launch_bounds__(256) void eltwise_u8_kernel(const EltArgs p)
+{
+    const size_t nvec = p.count / 4;
+    const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nthr = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = tid; i < nvec + (p.count & 3); i += nthr) {
+        const bool tail = i >= nvec;
+        const size_t base = tail ? nvec * 4 + (i - nvec) : i * 4;
+        const int ne = tail ? 1 : 4;
+        int32_t t[4];
+        for (int e = 0; e < 4; e++)
+            t[e] = p.is_max ? -1 : 0; // the reference's running maximum starts at 0xffffffff (eltwise.c:198)
+        for (int n = 0; n < p.n_in; n++) {
+            uint32_t v = tail ? p.in[n][base] : reinterpret_cast<const uint32_t *>(p.in[n])[i];
+            for (int e = 0; e < ne; e++) {
+                const int32_t pr = (int32_t)((uint32_t)((int32_t)((v >> (8 * e)) & 255) - p.zp[n]) * p.mult[n]);
+                const int64_t r = rshift_rn(pr, p.shift[n]);
+                if (p.is_max)
+                    t[e] = t[e] < (int32_t)r ? (int32_t)r : t[e];
+                else
+                    t[e] = (int32_t)(t[e] + r);
+            }
+        }
+        uint32_t o = 0;
+        for (int e = 0; e < ne; e++)
+            o |= (uint32_t)sat_hi((int32_t)(rshift_rn(t[e], p.s0) + p.oz), p.hi) << (8 * e);
+        if (tail)
+            p.y[base] = (uint8_t)o;
+        else
+            reinterpret_cast<uint32_t *>(p.y)[i] = o;
+    }
+}
+
+// ---- relu (relu.c:76-115) ----------------------------------------------------------------------
+struct ReluArgs {
+    const uint8_t *x;
+    uint8_t *y;
+    size_t count;
+    uint32_t mult;
+    int shift, iz, oz, hi;
+};
+
+__device__ static inline uint32_t relu_one(uint32_t x, const ReluArgs &p)
+{
+    const int32_t v = (int32_t)x >= p.iz ? (int32_t)x : p.iz;
+    const uint32_t pr = (uint32_t)(v - p.iz) * p.mult; // evaluated unsigned, widened without sign
+    return (uint32_t)sat_hi((int32_t)(rshift_rn((int64_t)pr, p.shift) + p.oz), p.hi);
+}
+
+__global__ __launch_bounds__(256) void relu_u8_kernel(const ReluArgs p)
+{
+    const size_t nvec = p.count / 16;
+    const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nthr = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = tid; i < nvec; i += nthr) {
+        const u32x4 v = reinterpret_cast<const u32x4 *>(p.x)[i];
+        u32x4 o;
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                w |= relu_one((v[d] >> (8 * e)) & 255, p) << (8 * e);
+            o[d] = w;
+        }
+        reinterpret_cast<u32x4 *>(p.y)[i] = o;
+    }
+    for (size_t i = nvec * 16 + tid; i < p.count; i += nthr)
+        p.y[i] = (uint8_t)relu_one(p.x[i], p);
+}
+
+// ---- pooling (pool.c:96-249), NHWC: one thread = 4 channels of one output pixel ------------------
+struct PoolArgs {
+    const uint8_t *x;
+    uint8_t *y;
+    int N, H, W, OH, OW, cs, kh, kw, ph, pw, sh, sw;
+    int is_avg, iz, oz, hi;
+    float ia_over_oa; // fp32 ialpha / oalpha, as the reference forms it before dividing by the pool size
+    uint32_t mult;    // max pooling: uint16 multiplier
+    int shift;
+};
+
+// get_quant_scale(x, 16) evaluated on the device with the same fp32 operations (quant_helper.h:98-118)
+__device__ static inline void quant_scale16(float x, uint32_t &mult, int &shift)
+{
+    int s = 0;
+    mult = 0;
+    shift = 0;
+    if (fabs((double)x) < 1e-10)
+        return;
+    while (x >= 1.0f) {
+        x /= 2;
+        s -= 1;
+    }
+    while (x < 0.5f) {
+        x *= 2;
+        s += 1;
+    }
+    mult = (uint32_t)(x * 32768.0f);
+    shift = s + 15;
+}
+
+__global__ __launch_bounds__(256) void pool_u8_kernel(const PoolArgs p)
+{
+    const int cq = p.cs >> 2;
+    const size_t total = (size_t)p.N * p.OH * p.OW * cq;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (size_t)gridDim.x * blockDim.x) {
+        const size_t m = idx / cq;
+        const int c0 = (int)(idx - m * cq) * 4;
+        const int n = (int)(m / ((size_t)p.OH * p.OW)), rem = (int)(m - (size_t)n * p.OH * p.OW);
+        const int oh = rem / p.OW, ow = rem - oh * p.OW;
+        int hs = oh * p.sh - p.ph, ws = ow * p.sw - p.pw;
+        uint32_t o = 0;
+        if (!p.is_avg) {
+            const int he = min(hs + p.kh, p.H), we = min(ws + p.kw, p.W);
+            hs = max(hs, 0), ws = max(ws, 0);
+            uint32_t mx[4] = {0, 0, 0, 0};
+            for (int i = hs; i < he; i++)
+                for (int j = ws; j < we; j++) {
+                    const uint32_t v = *reinterpret_cast<const uint32_t *>(
+                        p.x + ((size_t)(n * p.H + i) * p.W + j) * p.cs + c0);
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        mx[e] = max(mx[e], (v >> (8 * e)) & 255);
+                }
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int32_t pr = (int32_t)p.mult * ((int32_t)mx[e] - p.iz);
+                o |= (uint32_t)sat_hi((int32_t)(rshift_rn(pr, p.shift) + p.oz), p.hi) << (8 * e);
+            }
+        } else {
+            int he = min(hs + p.kh, p.H + p.ph), we = min(ws + p.kw, p.W + p.pw);
+            const uint32_t pool_size = (uint32_t)((he - hs) * (we - ws)); // padding counts (pool.c:211-213)
+            uint32_t mult;
+            int shift;
+            quant_scale16(p.ia_over_oa / (float)pool_size, mult, shift);
+            hs = max(hs, 0), ws = max(ws, 0), he = min(he, p.H), we = min(we, p.W);
+            int32_t sum[4] = {0, 0, 0, 0};
+            for (int i = hs; i < he; i++)
+                for (int j = ws; j < we; j++) {
+                    const uint32_t v = *reinterpret_cast<const uint32_t *>(
+                        p.x + ((size_t)(n * p.H + i) * p.W + j) * p.cs + c0);
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        sum[e] += (int32_t)((v >> (8 * e)) & 255) - p.iz;
+                }
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int32_t pr = (int32_t)(mult * (uint32_t)sum[e]);
+                o |= (uint32_t)sat_hi((int32_t)(rshift_rn(pr, shift) + p.oz), p.hi) << (8 * e);
+            }
+        }
+        *reinterpret_cast<uint32_t *>(p.y + m * p.cs + c0) = o;
+    }
+}
+
+// ---- quantize (quantize.c:145-157): fp32 NCHW -> uint8 NHWC --------------------------------------
+// One thread produces the 4 channels of one dword of the output; reads are coalesced along W per
+// channel plane, writes along the pixel index.
+struct QuantArgs {
+    const float *x;
+    uint8_t *y;
+    int N, C, H, W, cs;
+    float alpha, beta, hi;
+};
+
+__device__ static inline uint32_t quantize_one(float x, const QuantArgs &p)
+{
+    const float q = __fdiv_rn(__fsub_rn(x, p.beta), p.alpha); // IEEE fp32 subtract and divide, no contraction
+    if (q > p.hi)
+        return (uint32_t)p.hi;
+    if (q < 0)
+        return 0;
+    return (uint32_t)(uint8_t)((double)q + 0.5); // saturate_float_by_bits: +0.5 in double, truncate
+}
+
+__global__ __launch_bounds__(256) void quantize_u8_kernel(const QuantArgs p)
+{
+    const int cq = p.cs >> 2;
+    const size_t hw = (size_t)p.H * p.W, total = (size_t)p.N * hw * cq;
+    // pixel index fastest across threads: each channel plane is read with unit stride
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (size_t)gridDim.x * blockDim.x) {
+        const size_t pix = idx % hw, rest = idx / hw;
+        const int q4 = (int)(rest % cq), n = (int)(rest / cq);
+        uint32_t o = 0;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int c = q4 * 4 + e;
+            if (c < p.C)
+                o |= quantize_one(p.x[((size_t)n * p.C + c) * hw + pix], p) << (8 * e);
+        }
+        *reinterpret_cast<uint32_t *>(p.y + ((size_t)n * hw + pix) * p.cs + q4 * 4) = o;
+    }
+}
+
+// ---- dequantize (dequantize.c:111-123): uint8 NHWC -> fp32 NCHW ----------------------------------
+struct DequantArgs {
+    const uint8_t *x;
+    float *y;
+    int N, C, H, W, cs;
+    float alpha;
+    int zp;
+};
+
+__global__ __launch_bounds__(256) void dequantize_u8_kernel(const DequantArgs p)
+{
+    const size_t hw = (size_t)p.H * p.W, total = (size_t)p.N * p.C * hw;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (size_t)gridDim.x * blockDim.x) {
+        const size_t pix = idx % hw, rest = idx / hw;
+        const int c = (int)(rest % p.C), n = (int)(rest / p.C);
+        const int v = (int)p.x[((size_t)n * hw + pix) * p.cs + c] - p.zp;
+        p.y[idx] = __fmul_rn((float)v, p.alpha);
+    }
+}
+
+// ---- layout conversion ---------------------------------------------------------------------------
+struct LayoutArgs {
+    const uint8_t *src;
+    uint8_t *dst;
+    int N, C, H, W, cs;
+};
+
+__global__ __launch_bounds__(256) void nchw_to_nhwc_kernel(const LayoutArgs p)
+{
+    const int cq = p.cs >> 2;
+    const size_t hw = (size_t)p.H * p.W, total = (size_t)p.N * hw * cq;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (size_t)gridDim.x * blockDim.x) {
+        const size_t pix = idx % hw, rest = idx / hw;
+        const int q4 = (int)(rest % cq), n = (int)(rest / cq);
+        uint32_t o = 0;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int c = q4 * 4 + e;
+            if (c < p.C)
+                o |= (uint32_t)p.src[((size_t)n * p.C + c) * hw + pix] << (8 * e);
+        }
+        *reinterpret_cast<uint32_t *>(p.dst + ((size_t)n * hw + pix) * p.cs + q4 * 4) = o;
+    }
+}
+
+__global__ __launch_bounds__(256) void nhwc_to_nchw_kernel(const LayoutArgs p)
+{
+    const size_t hw = (size_t)p.H * p.W, total = (size_t)p.N * p.C * hw;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (size_t)gridDim.x * blockDim.x) {
+        const size_t pix = idx % hw, rest = idx / hw;
+        const int c = (int)(rest % p.C), n = (int)(rest / p.C);
+        p.dst[idx] = p.src[((size_t)n * hw + pix) * p.cs + c];
+    }
+}
+
+__global__ __launch_bounds__(256) void copy_bytes_kernel(const u32x4 *src, u32x4 *dst, size_t nvec)
+{
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += (size_t)gridDim.x * blockDim.x)
+        dst[i] = src[i];
+}
+
+} // namespace hipq
+
+// =================================================================================================
+using namespace hipq;
+
+static bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+extern "C" int hipq_add_u8(const void *a, const void *b, void *y, size_t count, float ia0, int iz0, float ia1,
+                           int iz1, float oa, int oz, int obits, void *stream)
+{
+    clear_error();
+    HIPQ_REQUIRE(a && b && y, "hipq_add_u8: null pointer");
+    HIPQ_REQUIRE(aligned16(a) && aligned16(b) && aligned16(y), "hipq_add_u8: buffers must be 16-byte aligned");
+    if (count == 0)
+        return 0;
+    if (ia0 > ia1) { // add.c:105-118
+        std::swap(ia0, ia1);
+        std::swap(iz0, iz1);
+        std::swap(a, b);
+    }
+    AddArgs p;
+    int s0, s1;
+    hipq_quant_scale(ia0 / oa, 23, &p.m0, &s0);
+    hipq_quant_scale(ia1 / oa, 23, &p.m1, &s1);
+    p.sh = std::min(s0, s1) - 1;
+    p.s0 = s0 - p.sh, p.s1 = s1 - p.sh;
+    HIPQ_REQUIRE(valid_shift(p.sh) && valid_shift(p.s0) && valid_shift(p.s1),
+                 "hipq_add_u8: scales out of the fixed-point range (shifts %d, %d)", s0, s1);
+    p.a = static_cast<const uint8_t *>(a), p.b = static_cast<const uint8_t *>(b), p.y = static_cast<uint8_t *>(y);
+    p.count = count, p.z0 = iz0, p.z1 = iz1, p.oz = oz, p.hi = (1 << obits) - 1;
+    hipLaunchKernelGGL(add_u8_kernel, dim3(grid_for(count / 16)), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+    return launch_status("add_u8_kernel");
+}
+
+extern "C" int hipq_eltwise_u8(const void *const *in, int n_in, const float *coeff, const float *ialpha,
+                               const uint8_t *izp, void *y, size_t count, int operation, float oa, int oz,
+                               int obits, void *stream)
+{
+    clear_error();
+    HIPQ_REQUIRE(in && ialpha && izp && y, "hipq_eltwise_u8: null pointer");
+    HIPQ_REQUIRE(n_in >= 2 && n_in <= HIPQ_MAX_ELTWISE_INPUTS, "hipq_eltwise_u8: %d inputs (2..%d supported)", n_in,
+                 HIPQ_MAX_ELTWISE_INPUTS);
+    HIPQ_REQUIRE(operation == HIPQ_ELTWISE_SUM || operation == HIPQ_ELTWISE_MAX,
+                 "hipq_eltwise_u8: operation %d is not implemented (PROD is rejected by the reference too)", operation);
+    if (count == 0)
+        return 0;
+    EltArgs p;
+    memset(&p, 0, sizeof p);
+    int smin = 127, sh[HIPQ_MAX_ELTWISE_INPUTS];
+    for (int n = 0; n < n_in; n++) {
+        HIPQ_REQUIRE(in[n] && (reinterpret_cast<uintptr_t>(in[n]) & 3) == 0, "hipq_eltwise_u8: input %d unaligned", n);
+        hipq_quant_scale((coeff ? coeff[n] : 1.0f) * ialpha[n] / oa, 23, &p.mult[n], &sh[n]);
+        smin = std::min(smin, sh[n]);
+        p.in[n] = static_cast<const uint8_t *>(in[n]);
+        p.zp[n] = izp[n];
+    }
+    p.s0 = smin - 1;
+    HIPQ_REQUIRE(valid_shift(p.s0), "hipq_eltwise_u8: scales out of the fixed-point range");
+    for (int n = 0; n < n_in; n++) {
+        p.shift[n] = sh[n] - p.s0;
+        HIPQ_REQUIRE(valid_shift(p.shift[n]), "hipq_eltwise_u8: scales out of the fixed-point range");
+    }
+    p.n_in = n_in, p.oz = oz, p.hi = (1 << obits) - 1, p.is_max = operation == HIPQ_ELTWISE_MAX;
+    p.y = static_cast<uint8_t *>(y), p.count = count;
+    hipLaunchKernelGGL(eltwise_u8_kernel, dim3(grid_for(count / 4 + 4)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), p);
+    return launch_status("eltwise_u8_kernel");
+}
+
+extern "C" int hipq_relu_u8(const void *x, void *y, size_t count, float ia, int iz, float oa, int oz, int obits,
+                            void *stream)
+{
+    clear_error();
+    HIPQ_REQUIRE(x && y && aligned16(x) && aligned16(y), "hipq_relu_u8: null or unaligned pointer");
+    if (count == 0)
+        return 0;
+    ReluArgs p;
+    hipq_quant_scale(ia / oa, 24, &p.mult, &p.shift);
+    HIPQ_REQUIRE(valid_shift(p.shift), "hipq_relu_u8: scale out of the fixed-point range");
+    p.x = static_cast<const uint8_t *>(x), p.y = static_cast<uint8_t *>(y), p.count = count;
+    p.iz = iz, p.oz = oz, p.hi = (1 << obits) - 1;
+    hipLaunchKernelGGL(relu_u8_kernel, dim3(grid_for(count / 16)), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+    return launch_status("relu_u8_kernel");
+}
+
+extern "C" int hipq_pool_u8(const void *x, void *y, int N, int C, int H, int W, int OH, int OW, int cs, int kh, int kw,
+                            int ph, int pw, int sh, int sw, int method, float ia, int iz, float oa, int oz, int obits,
+                            void *stream)
+{
+    clear_error();
+    HIPQ_REQUIRE(x && y, "hipq_pool_u8: null pointer");
+    HIPQ_REQUIRE(N > 0 && C > 0 && H > 0 && W > 0 && OH > 0 && OW > 0 && cs >= C && cs % 4 == 0, "hipq_pool_u8: bad shape");
+    HIPQ_REQUIRE(kh > 0 && kw > 0 && sh > 0 && sw > 0 && ph >= 0 && pw >= 0, "hipq_pool_u8: bad window");
+    // every window must overlap the padded image, otherwise the reference divides by a pool size <= 0
+    HIPQ_REQUIRE((OH - 1) * sh - ph < H + ph && (OW - 1) * sw - pw < W + pw, "hipq_pool_u8: a window lies outside the image");
+    PoolArgs p;
+    p.x = static_cast<const uint8_t *>(x), p.y = static_cast<uint8_t *>(y);
+    p.N = N, p.H = H, p.W = W, p.OH = OH, p.OW = OW, p.cs = cs, p.kh = kh, p.kw = kw, p.ph = ph, p.pw = pw, p.sh = sh, p.sw = sw;
+    p.is_avg = method != HIPQ_POOL_MAX, p.iz = iz, p.oz = oz, p.hi = (1 << obits) - 1;
+    p.ia_over_oa = ia / oa;
+    hipq_quant_scale(ia / oa, 16, &p.mult, &p.shift);
+    p.mult &= 0xffff; // get_quant_scale_int16 stores the multiplier in a uint16_t
+    HIPQ_REQUIRE(valid_shift(p.shift), "hipq_pool_u8: scale out of the fixed-point range");
+    const size_t total = (size_t)N * OH * OW * (cs / 4);
+    hipLaunchKernelGGL(pool_u8_kernel, dim3(grid_for(total)), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+    return launch_status("pool_u8_kernel");
+}
+
+extern "C" int hipq_quantize_u8(const float *x, void *y, int N, int C, int H, int W, int cs, float oa, int oz, int obits,
+                                void *stream)
+{
+    clear_error();
+    HIPQ_REQUIRE(x && y && N > 0 && C > 0 && H > 0 && W > 0 && cs >= C && cs % 4 == 0, "hipq_quantize_u8: bad argument");
+    QuantArgs p;
+    p.x = x, p.y = static_cast<uint8_t *>(y), p.N = N, p.C = C, p.H = H, p.W = W, p.cs = cs;
+    p.alpha = oa;
+    p.beta = -(oa * (float)oz); // quantize.c:152
+    p.hi = (float)((1 << obits) - 1);
+    const size_t total = (size_t)N * H * W * (cs / 4);
+    hipLaunchKernelGGL(quantize_u8_kernel, dim3(grid_for(total)), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+    return launch_status("quantize_u8_kernel");
+}
+
+extern "C" int hipq_dequantize_u8(const void *x, float *y, int N, int C, int H, int W, int cs, float ia, int iz,
+                                  void *stream)
+{
+    clear_error();
+    HIPQ_REQUIRE(x && y && N > 0 && C > 0 && H > 0 && W > 0 && cs >= C, "hipq_dequantize_u8: bad argument");
+    DequantArgs p;
+    p.x = static_cast<const uint8_t *>(x), p.y = y, p.N = N, p.C = C, p.H = H, p.W = W, p.cs = cs, p.alpha = ia, p.zp = iz;
+    hipLaunchKernelGGL(dequantize_u8_kernel, dim3(grid_for((size_t)N * C * H * W)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), p);
+    return launch_status("dequantize_u8_kernel");
+}
+
+static int layout_args(LayoutArgs &p, const void *src, void *dst, int N, int C, int H, int W, int cs)
+{
+    HIPQ_REQUIRE(src && dst && N > 0 && C > 0 && H > 0 && W > 0 && cs >= C && cs % 4 == 0, "layout conversion: bad argument");
+    p.src = static_cast<const uint8_t *>(src), p.dst = static_cast<uint8_t *>(dst);
+    p.N = N, p.C = C, p.H = H, p.W = W, p.cs = cs;
+    return 0;
+}
+
+extern "C" int hipq_nchw_to_nhwc_u8(const void *src, void *dst, int N, int C, int H, int W, int cs, void *stream)
+{
+    clear_error();
+    LayoutArgs p;
+    if (int rc = layout_args(p, src, dst, N, C, H, W, cs))
+        return rc;
+    hipLaunchKernelGGL(nchw_to_nhwc_kernel, dim3(grid_for((size_t)N * H * W * (cs / 4))), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), p);
+    return launch_status("nchw_to_nhwc_kernel");
+}
+
+extern "C" int hipq_nhwc_to_nchw_u8(const void *src, void *dst, int N, int C, int H, int W, int cs, void *stream)
+{
+    clear_error();
+    LayoutArgs p;
+    if (int rc = layout_args(p, src, dst, N, C, H, W, cs))
+        return rc;
+    hipLaunchKernelGGL(nhwc_to_nchw_kernel, dim3(grid_for((size_t)N * C * H * W)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), p);
+    return launch_status("nhwc_to_nchw_kernel");
+}
+
+extern "C" int hipq_copy_bytes(const void *src, void *dst, size_t count, void *stream)
+{
+    clear_error();
+    HIPQ_REQUIRE(src && dst && aligned16(src) && aligned16(dst) && count % 16 == 0, "hipq_copy_bytes: need 16-byte granularity");
+    hipLaunchKernelGGL(copy_bytes_kernel, dim3(grid_for(count / 16)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const u32x4 *>(src), static_cast<u32x4 *>(dst), count / 16);
+    return launch_status("copy_bytes_kernel");
+}

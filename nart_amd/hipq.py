@@ -1,0 +1,209 @@
+"""ctypes binding of the hipq C ABI (include/hipq.h) for Python callers.
+
+PyTorch is used for one thing only: owning device memory and streams (torch.uint8 / float32 CUDA
+tensors whose data_ptr() is handed to the library).  All arithmetic happens in the HIP kernels; there
+is no host fallback — loading fails loudly if the library has not been built.
+"""
+import ctypes as C
+import os
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "lib", "libhipq.so")
+_LIB = None
+
+
+class HipqError(RuntimeError):
+    pass
+
+
+class ConvDesc(C.Structure):  # hipq_conv2d_desc
+    _fields_ = [(n, C.c_int32) for n in ("N", "C", "H", "W", "K", "R", "S", "pad_h", "pad_w", "stride_h",
+                                         "stride_w", "group", "in_cs", "out_cs")] \
+        + [(n, C.c_float) for n in ("ialpha", "walpha", "oalpha")] \
+        + [(n, C.c_int32) for n in ("izp", "wzp", "ozp", "obits", "relu")]
+
+
+# every symbol include/hipq.h declares, with its signature
+_SIGS = {
+    "hipq_abi_version": (C.c_int, []),
+    "hipq_last_error": (C.c_char_p, []),
+    "hipq_quant_scale": (None, [C.c_float, C.c_int, C.POINTER(C.c_uint32), C.POINTER(C.c_int)]),
+    "hipq_channel_stride": (C.c_int, [C.c_int]),
+    "hipq_nchw_to_nhwc_u8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_void_p]),
+    "hipq_nhwc_to_nchw_u8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_void_p]),
+    "hipq_conv2d_plan_create": (C.c_int, [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p)]),
+    "hipq_conv2d_plan_destroy": (None, [C.c_void_p]),
+    "hipq_conv2d_plan_kernel": (C.c_char_p, [C.c_void_p]),
+    "hipq_conv2d_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "hipq_ip_reorder_weights": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 6),
+    "hipq_add_u8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_float, C.c_int, C.c_float,
+                              C.c_int, C.c_float, C.c_int, C.c_int, C.c_void_p]),
+    "hipq_eltwise_u8": (C.c_int, [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p,
+                                  C.c_size_t, C.c_int, C.c_float, C.c_int, C.c_int, C.c_void_p]),
+    "hipq_relu_u8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_float, C.c_int, C.c_float, C.c_int,
+                               C.c_int, C.c_void_p]),
+    "hipq_pool_u8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 14 + [C.c_float, C.c_int, C.c_float, C.c_int,
+                                                                          C.c_int, C.c_void_p]),
+    "hipq_quantize_u8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_float, C.c_int, C.c_int, C.c_void_p]),
+    "hipq_dequantize_u8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_float, C.c_int, C.c_void_p]),
+    "hipq_copy_bytes": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+}
+EXPORTS = tuple(_SIGS)
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        if not os.path.exists(LIB_PATH):
+            raise HipqError("%s is missing: build it with `python -m nart_amd.build`" % LIB_PATH)
+        L = C.CDLL(LIB_PATH)
+        for name, (res, args) in _SIGS.items():
+            f = getattr(L, name)  # AttributeError here = the library does not export a declared symbol
+            f.restype, f.argtypes = res, args
+        _LIB = L
+    return _LIB
+
+
+def check(rc):
+    if rc != 0:
+        raise HipqError(lib().hipq_last_error().decode() or "hipq call failed (%d)" % rc)
+
+
+def channel_stride(c):
+    return lib().hipq_channel_stride(int(c))
+
+
+def quant_scale(x, bits):
+    m, s = C.c_uint32(), C.c_int()
+    lib().hipq_quant_scale(C.c_float(np.float32(x)), bits, C.byref(m), C.byref(s))
+    return m.value, s.value
+
+
+def _stream():
+    import torch
+    return C.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else C.c_void_p(0)
+
+
+def conv_out_dim(i, pad, k, stride):
+    return (i + 2 * pad - k) // stride + 1
+
+
+# ---- device tensors in the library's layout -------------------------------------------------------
+def to_device_nhwc(x_nchw):
+    """numpy uint8 [N,C,H,W] -> CUDA uint8 [N,H,W,cs] (channels-last, padded channel stride)."""
+    import torch
+    x = np.ascontiguousarray(x_nchw, np.uint8)
+    N, Cc, H, W = x.shape
+    cs = channel_stride(Cc)
+    src = torch.from_numpy(x).cuda()
+    dst = torch.empty((N, H, W, cs), dtype=torch.uint8, device="cuda")
+    check(lib().hipq_nchw_to_nhwc_u8(_ptr(src), _ptr(dst), N, Cc, H, W, cs, _stream()))
+    return dst
+
+
+def from_device_nhwc(t, Cc):
+    """CUDA uint8 [N,H,W,cs] -> numpy uint8 [N,C,H,W]."""
+    import torch
+    N, H, W, cs = t.shape
+    dst = torch.empty((N, Cc, H, W), dtype=torch.uint8, device="cuda")
+    check(lib().hipq_nhwc_to_nchw_u8(_ptr(t), _ptr(dst), N, Cc, H, W, cs, _stream()))
+    return dst.cpu().numpy()
+
+
+class Conv2d:
+    """A convolution plan (weights packed and resident on the device) plus its launch."""
+
+    def __init__(self, x_shape, w, bias, pad, stride, group, ialpha, izp, walpha, wzp, oalpha, ozp, obits=8,
+                 relu=False, in_cs=None, out_cs=None):
+        N, Cc, H, W = x_shape
+        w = np.ascontiguousarray(w, np.uint8)
+        K, _, R, S = w.shape
+        ph, pw = (pad, pad) if np.isscalar(pad) else pad
+        sh, sw = (stride, stride) if np.isscalar(stride) else stride
+        d = ConvDesc(N=N, C=Cc, H=H, W=W, K=K, R=R, S=S, pad_h=ph, pad_w=pw, stride_h=sh, stride_w=sw, group=group,
+                     in_cs=in_cs or channel_stride(Cc), out_cs=out_cs or channel_stride(K),
+                     ialpha=ialpha, walpha=walpha, oalpha=oalpha, izp=izp, wzp=wzp, ozp=ozp, obits=obits,
+                     relu=int(relu))
+        self.desc = d
+        self.OH, self.OW = conv_out_dim(H, ph, R, sh), conv_out_dim(W, pw, S, sw)
+        b = None if bias is None else np.ascontiguousarray(bias, np.int32)
+        h = C.c_void_p()
+        check(lib().hipq_conv2d_plan_create(C.byref(d), C.c_void_p(w.ctypes.data),
+                                            C.c_void_p(b.ctypes.data) if b is not None else None, C.byref(h)))
+        self.handle = h
+        self.kernel = lib().hipq_conv2d_plan_kernel(h).decode()
+        self.ops = 2 * N * K * self.OH * self.OW * (Cc // group) * R * S
+
+    def empty_output(self):
+        import torch
+        d = self.desc
+        return torch.empty((d.N, self.OH, self.OW, d.out_cs), dtype=torch.uint8, device="cuda")
+
+    def __call__(self, x, y=None, acc=None):
+        if y is None:
+            y = self.empty_output()
+        check(lib().hipq_conv2d_run(self.handle, _ptr(x), _ptr(y), _ptr(acc), _stream()))
+        return y
+
+    def close(self):
+        if self.handle:
+            lib().hipq_conv2d_plan_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+
+def add_u8(a, b, y, ialpha0, izp0, ialpha1, izp1, oalpha, ozp, obits=8):
+    check(lib().hipq_add_u8(_ptr(a), _ptr(b), _ptr(y), a.numel(), ialpha0, izp0, ialpha1, izp1, oalpha, ozp, obits,
+                            _stream()))
+    return y
+
+
+def eltwise_u8(ins, y, ialpha, izp, oalpha, ozp, operation=1, coeff=None, obits=8):
+    n = len(ins)
+    ptrs = (C.c_void_p * n)(*[t.data_ptr() for t in ins])
+    ia = np.ascontiguousarray(ialpha, np.float32)
+    iz = np.ascontiguousarray(izp, np.uint8)
+    cf = None if coeff is None else np.ascontiguousarray(coeff, np.float32)
+    check(lib().hipq_eltwise_u8(ptrs, n, C.c_void_p(cf.ctypes.data) if cf is not None else None,
+                                C.c_void_p(ia.ctypes.data), C.c_void_p(iz.ctypes.data), _ptr(y), y.numel(),
+                                operation, oalpha, ozp, obits, _stream()))
+    return y
+
+
+def relu_u8(x, y, ialpha, izp, oalpha, ozp, obits=8):
+    check(lib().hipq_relu_u8(_ptr(x), _ptr(y), x.numel(), ialpha, izp, oalpha, ozp, obits, _stream()))
+    return y
+
+
+def pool_u8(x, y, Cc, kernel, pad, stride, method, ialpha, izp, oalpha, ozp, obits=8):
+    N, H, W, cs = x.shape
+    _, OH, OW, _ = y.shape
+    (kh, kw) = (kernel, kernel) if np.isscalar(kernel) else kernel
+    (ph, pw) = (pad, pad) if np.isscalar(pad) else pad
+    (sh, sw) = (stride, stride) if np.isscalar(stride) else stride
+    check(lib().hipq_pool_u8(_ptr(x), _ptr(y), N, Cc, H, W, OH, OW, cs, kh, kw, ph, pw, sh, sw, method, ialpha, izp,
+                             oalpha, ozp, obits, _stream()))
+    return y
+
+
+def quantize_u8(x_nchw, y, oalpha, ozp, obits=8):
+    N, Cc, H, W = x_nchw.shape
+    check(lib().hipq_quantize_u8(_ptr(x_nchw), _ptr(y), N, Cc, H, W, y.shape[-1], oalpha, ozp, obits, _stream()))
+    return y
+
+
+def dequantize_u8(x, y_nchw, ialpha, izp):
+    N, Cc, H, W = y_nchw.shape
+    check(lib().hipq_dequantize_u8(_ptr(x), _ptr(y_nchw), N, Cc, H, W, x.shape[-1], ialpha, izp, _stream()))
+    return y_nchw

@@ -1,0 +1,60 @@
+"""CPU-side checks of the C-ABI libraries: they load without a GPU, export every symbol their headers
+declare, and their host-only entry points agree with the oracle.  No kernel is launched here."""
+import os
+import re
+
+import numpy as np
+import pytest
+
+from nart_amd import hipq
+from oracle import orc
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_functions(header):
+    text = open(os.path.join(ROOT, "include", header)).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return set(re.findall(r"\b(hipq_[a-z0-9_]+)\s*\(", text))
+
+
+def test_hipq_exports_every_declared_symbol():
+    L = hipq.lib()  # raises if the library is missing or lacks a symbol of hipq.EXPORTS
+    declared = declared_functions("hipq.h")
+    assert declared == set(hipq.EXPORTS), declared ^ set(hipq.EXPORTS)
+    for name in declared:
+        assert getattr(L, name) is not None
+    assert L.hipq_abi_version() == 1
+
+
+def test_quant_scale_matches_oracle():
+    rng = np.random.default_rng(0)
+    for bits in (16, 23, 24, 32):
+        for _ in range(500):
+            f = np.float32(np.exp(rng.uniform(np.log(1e-7), np.log(100.0))))
+            assert hipq.quant_scale(f, bits) == orc.quant_scale(f, bits)
+    assert hipq.quant_scale(0.0, 32) == (0, 0)
+
+
+def test_channel_stride_rule():
+    assert [hipq.channel_stride(c) for c in (1, 3, 4, 5, 16, 17, 24, 64, 1000)] == [4, 4, 4, 16, 16, 32, 32, 64, 1008]
+
+
+def test_ip_weight_reorder_host():
+    rng = np.random.default_rng(1)
+    No, C, H, W, cs = 5, 6, 2, 3, 16
+    w = rng.integers(0, 256, (No, C, H, W), dtype=np.uint8)
+    out = np.empty((No, H, W, cs), np.uint8)
+    hipq.check(hipq.lib().hipq_ip_reorder_weights(w.ctypes.data, out.ctypes.data, No, C, H, W, cs, 77))
+    assert np.array_equal(out[..., :C], w.transpose(0, 2, 3, 1)) and (out[..., C:] == 77).all()
+
+
+def test_compute_entry_points_fail_loudly_without_gpu():
+    try:
+        import torch
+        if torch.cuda.is_available():
+            pytest.skip("a GPU is present")
+    except ImportError:
+        pass
+    with pytest.raises(hipq.HipqError):
+        hipq.Conv2d((1, 16, 4, 4), np.zeros((16, 16, 1, 1), np.uint8), None, 0, 1, 1, 0.1, 0, 0.1, 0, 0.1, 0)

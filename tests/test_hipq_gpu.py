@@ -1,0 +1,225 @@
+"""GPU parity of the hipq kernels against the CPU oracle, through the C ABI (ctypes -> libhipq.so).
+
+Bar: bit-exact uint8 outputs AND bit-exact int32 accumulators for conv / ip; bit-exact bytes for add,
+eltwise, relu, pool and quantize (the kernel uses IEEE fp32 divide, so the 1-LSB allowance is not
+needed); bit-exact fp32 for dequantize.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+from oracle import orc  # noqa: E402  (checker only)
+from nart_amd import hipq  # noqa: E402
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+
+
+def rand_q(rng, lo=1e-3, hi=1e-1):
+    return float(np.float32(np.exp(rng.uniform(np.log(lo), np.log(hi)))))
+
+
+def run_conv(x, w, b, pad, stride, group, q, relu=False, want_acc=True):
+    plan = hipq.Conv2d(x.shape, w, b, pad, stride, group, *q, relu=relu)
+    xd = hipq.to_device_nhwc(x)
+    acc = torch.zeros((x.shape[0], plan.OH, plan.OW, plan.desc.out_cs), dtype=torch.int32, device="cuda") if want_acc else None
+    yd = plan(xd, acc=acc)
+    torch.cuda.synchronize()
+    y = hipq.from_device_nhwc(yd, w.shape[0])
+    a = acc.cpu().numpy()[..., :w.shape[0]].transpose(0, 3, 1, 2) if want_acc else None
+    return y, a, plan.kernel
+
+
+def check_conv(x, w, b, pad, stride, group, q, tag=""):
+    print("conv case", tag, x.shape, w.shape, pad, stride, group, q, flush=True)
+    want_y, want_acc = orc.conv2d_u8(x, w, b, pad, stride, group, *q, return_acc=True)
+    y, acc, kern = run_conv(x, w, b, pad, stride, group, q)
+    assert np.array_equal(acc, want_acc), (tag, kern, "accumulators differ", int((acc != want_acc).sum()))
+    assert np.array_equal(y, want_y), (tag, kern, "outputs differ", int((y != want_y).sum()))
+    return kern
+
+
+with open(os.path.join(HERE, "golden", "conv_kat.json")) as f:
+    KATS = json.load(f)["cases"]
+
+
+@pytest.mark.parametrize("c", KATS, ids=lambda c: c["id"])
+def test_conv_known_answers_on_gpu(c):
+    """The reference's recorded checksums, reproduced by the HIP kernels (config 1 is the first)."""
+    from test_oracle import kat_case
+    x, w, b = kat_case(c)
+    y, _, kern = run_conv(x, w, b, c["pad"], c["stride"], c["group"], (0.02, c["izp"], 0.005, 128, 0.05, c["ozp"]),
+                          want_acc=False)
+    assert "%016x" % orc.fnv1a64(y) == c["fnv"], kern
+
+
+def test_conv_mfma_shapes():
+    rng = np.random.default_rng(11)
+    kerns = set()
+    cases = [  # N, C, H, W, K, R, S, pad, stride
+        (2, 64, 14, 14, 64, 3, 3, 1, 1), (1, 64, 9, 11, 128, 1, 1, 0, 1), (3, 32, 10, 7, 48, 3, 3, 1, 2),
+        (1, 16, 12, 12, 24, 5, 3, 1, 1), (2, 128, 7, 7, 256, 1, 1, 0, 2), (1, 48, 8, 8, 200, 3, 3, 0, 1),
+        (1, 3, 33, 29, 64, 7, 7, 3, 2), (2, 3, 16, 16, 16, 3, 3, 1, 1), (1, 1, 9, 9, 8, 5, 5, 2, 1),
+        (1, 20, 6, 6, 10, 3, 3, 1, 1), (1, 256, 4, 4, 64, 3, 3, 1, 1), (5, 24, 5, 5, 40, 1, 1, 0, 1),
+    ]
+    for i, (N, C, H, W, K, R, S, pad, st) in enumerate(cases):
+        x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+        w = rng.integers(0, 256, (K, C, R, S), dtype=np.uint8)
+        b = rng.integers(-30000, 30000, K).astype(np.int32)
+        for wzp in (128, int(rng.integers(0, 256))):
+            q = (rand_q(rng), int(rng.integers(0, 256)), rand_q(rng), wzp, rand_q(rng, 1e-2, 1.0), int(rng.integers(0, 256)))
+            kerns.add(check_conv(x, w, b, pad, st, 1, q, tag="mfma%d" % i))
+    assert any("mfma" in k and "_wzp" in k for k in kerns) and any("_c4" in k for k in kerns), kerns
+
+
+def test_conv_edge_cases():
+    rng = np.random.default_rng(12)
+    # extreme values: all-255 activations against all-0 / all-255 weights, zero points at both ends
+    for xv, wv, izp, wzp in ((255, 255, 0, 0), (255, 0, 0, 255), (0, 255, 255, 0), (0, 0, 255, 255)):
+        x = np.full((1, 64, 6, 6), xv, np.uint8)
+        w = np.full((64, 64, 3, 3), wv, np.uint8)
+        check_conv(x, w, None, 1, 1, 1, (0.01, izp, 0.01, wzp, 0.9, 3), tag="extreme")
+    # no bias, asymmetric padding and stride, ragged pixel count (not a multiple of any tile)
+    x = rng.integers(0, 256, (1, 32, 13, 5), dtype=np.uint8)
+    w = rng.integers(0, 256, (33, 32, 3, 2), dtype=np.uint8)
+    check_conv(x, w, None, (2, 0), (2, 1), 1, (0.02, 7, 0.005, 128, 0.05, 0), tag="ragged")
+    # accumulator wrap-around: 4608 taps of (255-0)*(255-0) stay below 2^31, so force it with a huge bias
+    x = np.full((1, 512, 3, 3), 255, np.uint8)
+    w = np.full((16, 512, 3, 3), 255, np.uint8)
+    b = np.full(16, 2**31 - 1000, np.int32)
+    check_conv(x, w, b, 1, 1, 1, (0.01, 0, 0.01, 0, 0.5, 0), tag="wrap")
+    # fused ReLU == conv followed by the reference relu with identical scales / zero point
+    x = rng.integers(0, 256, (1, 16, 8, 8), dtype=np.uint8)
+    w = rng.integers(0, 256, (16, 16, 3, 3), dtype=np.uint8)
+    q = (0.02, 100, 0.005, 128, 0.05, 90)
+    y, _, _ = run_conv(x, w, None, 1, 1, 1, q, relu=True, want_acc=False)
+    want = orc.relu_u8(orc.conv2d_u8(x, w, None, 1, 1, 1, *q), 0.05, 90, 0.05, 90)
+    assert np.array_equal(y, want)
+
+
+def test_conv_grouped_and_depthwise():
+    rng = np.random.default_rng(13)
+    kerns = set()
+    for (N, C, H, W, K, R, S, pad, st, grp) in [(2, 32, 14, 14, 32, 3, 3, 1, 1, 32), (1, 96, 9, 9, 96, 3, 3, 1, 2, 96),
+                                                 (1, 24, 7, 7, 24, 5, 5, 2, 1, 24), (1, 16, 8, 8, 32, 3, 3, 1, 1, 4),
+                                                 (2, 12, 6, 6, 6, 1, 1, 0, 1, 3)]:
+        x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+        w = rng.integers(0, 256, (K, C // grp, R, S), dtype=np.uint8)
+        b = rng.integers(-3000, 3000, K).astype(np.int32)
+        q = (rand_q(rng), int(rng.integers(0, 256)), rand_q(rng), int(rng.integers(0, 256)), rand_q(rng, 1e-2, 1.0),
+             int(rng.integers(0, 256)))
+        kerns.add(check_conv(x, w, b, pad, st, grp, q, tag="grouped"))
+    assert "conv_depthwise_u8" in kerns and "conv_direct_u8" in kerns
+
+
+def test_ip_as_1x1():
+    rng = np.random.default_rng(14)
+    for M, Kd, No in ((128, 512, 256), (5, 300, 37), (1, 2048, 1000)):
+        x = rng.integers(0, 256, (M, Kd), dtype=np.uint8)
+        w = rng.integers(0, 256, (No, Kd), dtype=np.uint8)
+        b = rng.integers(-50000, 50000, No).astype(np.int32)
+        q = (rand_q(rng), 128, rand_q(rng), int(rng.choice([128, 90])), rand_q(rng, 1e-1, 2.0), int(rng.integers(0, 256)))
+        want_y, want_acc = orc.ip_u8(x, w, b, *q, return_acc=True)
+        y, acc, _ = run_conv(x.reshape(M, Kd, 1, 1), w.reshape(No, Kd, 1, 1), b, 0, 1, 1, q)
+        assert np.array_equal(acc.reshape(M, No), want_acc) and np.array_equal(y.reshape(M, No), want_y)
+    # FC fed by a [M, C, H, W] tensor: weights re-ordered from (c,h,w) to the device's (h,w,c)
+    M, Cc, H, W, No = 3, 20, 2, 3, 11
+    x = rng.integers(0, 256, (M, Cc, H, W), dtype=np.uint8)
+    w = rng.integers(0, 256, (No, Cc * H * W), dtype=np.uint8)
+    q = (0.02, 128, 0.004, 131, 0.3, 5)
+    want = orc.ip_u8(x.reshape(M, -1), w, None, *q)
+    cs = hipq.channel_stride(Cc)
+    w2 = np.empty((No, H * W * cs), np.uint8)
+    hipq.check(hipq.lib().hipq_ip_reorder_weights(w.ctypes.data, w2.ctypes.data, No, Cc, H, W, cs, 131))
+    plan = hipq.Conv2d((M, H * W * cs, 1, 1), w2.reshape(No, -1, 1, 1), None, 0, 1, 1, *q, in_cs=H * W * cs)
+    yd = plan(hipq.to_device_nhwc(x))  # [M,H,W,cs] bytes == [M,1,1,H*W*cs]
+    torch.cuda.synchronize()
+    assert np.array_equal(yd.cpu().numpy().reshape(M, -1)[:, :No], want)
+
+
+def test_elementwise():
+    rng = np.random.default_rng(15)
+    for n in (1, 15, 16, 4099, 64 * 56 * 56 * 16 + 3):
+        a = rng.integers(0, 256, n, dtype=np.uint8)
+        b = rng.integers(0, 256, n, dtype=np.uint8)
+        c = rng.integers(0, 256, n, dtype=np.uint8)
+        ia = [rand_q(rng) for _ in range(3)]
+        iz = [int(rng.integers(0, 256)) for _ in range(3)]
+        oa, oz = rand_q(rng, 3e-3, 0.3), int(rng.integers(0, 256))
+        ta, tb, tc = (torch.from_numpy(v).cuda() for v in (a, b, c))
+        ty = torch.empty_like(ta)
+        got = hipq.add_u8(ta, tb, ty, ia[0], iz[0], ia[1], iz[1], oa, oz).cpu().numpy()
+        assert np.array_equal(got, orc.add_u8(a, b, ia[0], iz[0], ia[1], iz[1], oa, oz)), ("add", n)
+        for operation in (1, 2):
+            got = hipq.eltwise_u8([ta, tb, tc], ty, ia, iz, oa, oz, operation).cpu().numpy()
+            assert np.array_equal(got, orc.eltwise_u8([a, b, c], ia, iz, oa, oz, operation)), ("eltwise", n, operation)
+        got = hipq.eltwise_u8([ta, tb], ty, ia[:2], iz[:2], oa, oz, 1, coeff=[0.5, 1.75]).cpu().numpy()
+        assert np.array_equal(got, orc.eltwise_u8([a, b], ia[:2], iz[:2], oa, oz, 1, coeff=[0.5, 1.75]))
+        got = hipq.relu_u8(ta, ty, ia[0], iz[0], oa, oz).cpu().numpy()
+        assert np.array_equal(got, orc.relu_u8(a, ia[0], iz[0], oa, oz)), ("relu", n)
+
+
+def test_pool():
+    rng = np.random.default_rng(16)
+    cases = [(2, 64, 112, 112, 3, 1, 2, 0, False), (2, 64, 13, 13, 3, 1, 2, 0, True), (3, 40, 7, 7, 7, 0, 1, 1, True),
+             (1, 20, 9, 11, 3, 1, 2, 1, True), (1, 3, 8, 8, 2, 0, 2, 1, False), (2, 17, 10, 10, (3, 2), (1, 0), (2, 1), 1, True)]
+    for N, C, H, W, k, pad, st, method, ceil_mode in cases:
+        x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+        q = (rand_q(rng), int(rng.integers(0, 256)), rand_q(rng), int(rng.integers(0, 256)))
+        want = orc.pool_u8(x, k, pad, st, method, ceil_mode, *q)
+        xd = hipq.to_device_nhwc(x)
+        yd = torch.empty((N, want.shape[2], want.shape[3], xd.shape[3]), dtype=torch.uint8, device="cuda")
+        hipq.pool_u8(xd, yd, C, k, pad, st, method, *q)
+        assert np.array_equal(hipq.from_device_nhwc(yd, C), want), (N, C, H, W, k, pad, st, method)
+
+
+def test_quantize_dequantize():
+    rng = np.random.default_rng(17)
+    for shape in ((2, 3, 224, 224), (1, 16, 9, 9), (4, 1000, 1, 1)):
+        oa, oz = rand_q(rng, 5e-3, 0.1), int(rng.integers(0, 256))
+        x = (rng.standard_normal(shape) * 60 * oa).astype(np.float32)
+        x.flat[:512] = (np.arange(512, dtype=np.float32) * 0.5 - oz) * np.float32(oa)  # exact ties, both clamps
+        xd = torch.from_numpy(x).cuda()
+        cs = hipq.channel_stride(shape[1])
+        yd = torch.empty((shape[0], shape[2], shape[3], cs), dtype=torch.uint8, device="cuda")
+        hipq.quantize_u8(xd, yd, oa, oz)
+        want = orc.quantize_u8(x, oa, oz)
+        got = hipq.from_device_nhwc(yd, shape[1])
+        assert np.array_equal(got, want), (shape, int((got != want).sum()))
+        fd = torch.empty(shape, dtype=torch.float32, device="cuda")
+        hipq.dequantize_u8(yd, fd, oa, oz)
+        assert np.array_equal(fd.cpu().numpy().view(np.uint32), orc.dequantize_u8(want, oa, oz).view(np.uint32))
+
+
+def test_layout_round_trip_and_errors():
+    rng = np.random.default_rng(18)
+    x = rng.integers(0, 256, (2, 19, 5, 7), dtype=np.uint8)
+    assert np.array_equal(hipq.from_device_nhwc(hipq.to_device_nhwc(x), 19), x)
+    # error behaviour: a bad descriptor is refused with a message, nothing is launched
+    with pytest.raises(hipq.HipqError, match="group"):
+        hipq.Conv2d((1, 6, 4, 4), np.zeros((4, 2, 1, 1), np.uint8), None, 0, 1, 4, 0.1, 0, 0.1, 0, 0.1, 0)
+    with pytest.raises(hipq.HipqError, match="shift"):
+        hipq.Conv2d((1, 16, 4, 4), np.zeros((16, 16, 1, 1), np.uint8), None, 0, 1, 1, 1e4, 0, 1e4, 0, 1e-4, 0)
+
+
+def test_full_size_properties():
+    """BASELINE-size checks that do not need the slow CPU oracle on the full tensor: linearity in the
+    bias (a per-channel constant shift of the accumulators) and batch independence at N = 64."""
+    rng = np.random.default_rng(19)
+    N, C, H, K = 64, 64, 56, 64
+    x = rng.integers(0, 256, (N, C, H, H), dtype=np.uint8)
+    w = rng.integers(1, 256, (K, C, 3, 3), dtype=np.uint8)
+    b = rng.integers(-1000, 1000, K).astype(np.int32)
+    q = (0.02, 128, 0.005, 128, 0.05, 0)
+    y, acc, _ = run_conv(x, w, b, 1, 1, 1, q)
+    y0, acc0, _ = run_conv(x, w, None, 1, 1, 1, q)
+    assert np.array_equal(acc - acc0, np.broadcast_to(b[None, :, None, None], acc.shape))
+    # images 0 and 63 alone give the same bytes as inside the batch, and match the oracle
+    for i in (0, 63):
+        want = orc.conv2d_u8(x[i:i + 1], w, b, 1, 1, 1, *q)
+        assert np.array_equal(y[i:i + 1], want)
