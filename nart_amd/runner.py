@@ -1,0 +1,120 @@
+"""Runs a Case (nart_amd/cases.py) on the GPU through the hipq C ABI.
+
+This is the Python-side counterpart of the reference's parade: a flat list of prepared operators that
+`run()` launches in order on the current HIP stream (art/src/parade.c:184-197).  `capture()` records one
+pass into a HIP graph so that a launch-bound step replays without per-kernel host overhead.
+All device tensors are channels-last with padded channel stride (see include/hipq.h).
+"""
+import numpy as np
+import torch
+
+from . import hipq
+
+
+class HipqExecutor:
+    def __init__(self, case):
+        self.case = case
+        self.buf = {}        # tensor name -> device tensor
+        self.steps = []      # (label, kernel name, callable, algorithmic ops, compulsory bytes)
+        self.plans = []
+        self.graph = None
+        T = case.tensors
+        inp = case.input
+        if inp.dtype == "f32":
+            self.buf[inp.name] = torch.zeros(inp.shape, dtype=torch.float32, device="cuda")
+        else:
+            N, C, H, W = inp.shape
+            self.buf[inp.name] = torch.zeros((N, H, W, hipq.channel_stride(C)), dtype=torch.uint8, device="cuda")
+        for node in case.nodes:
+            y = T[node.output]
+            xs = [T[i] for i in node.inputs]
+            N, C, H, W = y.shape
+            if y.dtype == "f32":
+                out = torch.zeros(y.shape, dtype=torch.float32, device="cuda")
+            else:
+                out = torch.zeros((N, H, W, hipq.channel_stride(C)), dtype=torch.uint8, device="cuda")
+            self.buf[y.name] = out
+            ins = [self.buf[i] for i in node.inputs]
+            a = node.attrs
+            if node.kind == "quantize":
+                fn = (lambda i=ins[0], o=out, y=y: hipq.quantize_u8(i, o, y.alpha, y.zp))
+                self._add(node, "quantize_u8_kernel", fn, 0, 5 * int(np.prod(y.shape)))
+            elif node.kind == "dequantize":
+                x = xs[0]
+                fn = (lambda i=ins[0], o=out, x=x: hipq.dequantize_u8(i, o, x.alpha, x.zp))
+                self._add(node, "dequantize_u8_kernel", fn, 0, 5 * int(np.prod(y.shape)))
+            elif node.kind == "conv":
+                x = xs[0]
+                plan = hipq.Conv2d(x.shape, case.weights[a["w"]], case.weights[a["b"]], a["pad"], a["stride"],
+                                   a["group"], x.alpha, x.zp, a["walpha"], a["wzp"], y.alpha, y.zp, relu=a["relu"])
+                self.plans.append(plan)
+                fn = (lambda p=plan, i=ins[0], o=out: p(i, o))
+                nbytes = int(np.prod(x.shape)) + int(np.prod(y.shape)) + case.weights[a["w"]].size + 4 * a["K"]
+                self._add(node, plan.kernel, fn, plan.ops, nbytes)
+            elif node.kind == "ip":
+                x = xs[0]
+                Nn, Cc, Hh, Ww = x.shape
+                w = np.ascontiguousarray(case.weights[a["w"]])
+                cs = hipq.channel_stride(Cc)
+                if Hh * Ww > 1 or cs != Cc:
+                    w2 = np.empty((a["K"], Hh * Ww * cs), np.uint8)
+                    hipq.check(hipq.lib().hipq_ip_reorder_weights(w.ctypes.data, w2.ctypes.data, a["K"], Cc, Hh, Ww, cs,
+                                                                  a["wzp"]))
+                    w = w2
+                kd = Hh * Ww * cs
+                plan = hipq.Conv2d((Nn, kd, 1, 1), w.reshape(a["K"], kd, 1, 1), case.weights[a["b"]], 0, 1, 1, x.alpha,
+                                   x.zp, a["walpha"], a["wzp"], y.alpha, y.zp, in_cs=kd)
+                self.plans.append(plan)
+                fn = (lambda p=plan, i=ins[0], o=out: p(i, o))
+                self._add(node, plan.kernel, fn, 2 * Nn * a["K"] * Cc * Hh * Ww,
+                          Nn * Cc * Hh * Ww + Nn * a["K"] + a["K"] * Cc * Hh * Ww + 4 * a["K"])
+            elif node.kind == "pool":
+                x = xs[0]
+                fn = (lambda i=ins[0], o=out, x=x, y=y, a=a: hipq.pool_u8(i, o, x.shape[1], a["k"], a["pad"], a["stride"],
+                                                                         a["method"], x.alpha, x.zp, y.alpha, y.zp))
+                self._add(node, "pool_u8_kernel", fn, 0, int(np.prod(x.shape)) + int(np.prod(y.shape)))
+            elif node.kind == "add":
+                fn = (lambda i=ins, o=out, xs=xs, y=y: hipq.add_u8(i[0], i[1], o, xs[0].alpha, xs[0].zp, xs[1].alpha,
+                                                                 xs[1].zp, y.alpha, y.zp))
+                self._add(node, "add_u8_kernel", fn, 0, 3 * int(np.prod(y.shape)))
+            else:
+                raise ValueError("unknown node kind " + node.kind)
+
+    def _add(self, node, kernel, fn, ops, nbytes):
+        self.steps.append({"label": node.output, "kind": node.kind, "kernel": kernel, "fn": fn, "ops": ops,
+                           "bytes": nbytes})
+
+    # ---- data in / out ---------------------------------------------------------------------------
+    def set_input(self, x):
+        inp = self.case.input
+        if inp.dtype == "f32":
+            self.buf[inp.name].copy_(torch.from_numpy(np.ascontiguousarray(x, np.float32)))
+        else:
+            self.buf[inp.name].copy_(hipq.to_device_nhwc(x))
+
+    def fetch(self, name):
+        t = self.case.tensors[name]
+        if t.dtype == "f32":
+            return self.buf[name].cpu().numpy()
+        return hipq.from_device_nhwc(self.buf[name], t.shape[1])
+
+    def output(self):
+        return self.fetch(self.case.output.name)
+
+    # ---- execution -------------------------------------------------------------------------------
+    def run(self):
+        for s in self.steps:
+            s["fn"]()
+
+    def capture(self):
+        """Record one pass into a HIP graph (kernel nodes only: no memsets, no allocations)."""
+        self.run()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            self.run()
+        self.graph = g
+        return g
+
+    def replay(self):
+        self.graph.replay()

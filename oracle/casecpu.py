@@ -1,0 +1,126 @@
+"""Evaluates a Case (nart_amd/cases.py) on the CPU with the oracle, operator by operator, in NCHW.
+Returns every intermediate tensor so that a GPU mismatch can be pinned to the first diverging layer."""
+import numpy as np
+
+from oracle import orc
+
+
+def run_case(case, x):
+    T = case.tensors
+    vals = {case.input.name: x}
+    for node in case.nodes:
+        y = T[node.output]
+        xs = [T[i] for i in node.inputs]
+        ins = [vals[i] for i in node.inputs]
+        a = node.attrs
+        if node.kind == "quantize":
+            out = orc.quantize_u8(ins[0], y.alpha, y.zp)
+        elif node.kind == "dequantize":
+            out = orc.dequantize_u8(ins[0], xs[0].alpha, xs[0].zp)
+        elif node.kind == "conv":
+            out = orc.conv2d_u8(ins[0], case.weights[a["w"]], case.weights[a["b"]], a["pad"], a["stride"], a["group"],
+                                xs[0].alpha, xs[0].zp, a["walpha"], a["wzp"], y.alpha, y.zp)
+            if a["relu"]:  # "followed by a quant relu op with equal scales and zero point"
+                out = orc.relu_u8(out, y.alpha, y.zp, y.alpha, y.zp)
+        elif node.kind == "ip":
+            out = orc.ip_u8(ins[0].reshape(ins[0].shape[0], -1), case.weights[a["w"]], case.weights[a["b"]],
+                            xs[0].alpha, xs[0].zp, a["walpha"], a["wzp"], y.alpha, y.zp)
+            out = out.reshape(y.shape)
+        elif node.kind == "pool":
+            out = orc.pool_u8(ins[0], a["k"], a["pad"], a["stride"], a["method"], a["ceil_mode"], xs[0].alpha, xs[0].zp,
+                              y.alpha, y.zp)
+        elif node.kind == "add":
+            out = orc.add_u8(ins[0], ins[1], xs[0].alpha, xs[0].zp, xs[1].alpha, xs[1].zp, y.alpha, y.zp)
+        else:
+            raise ValueError(node.kind)
+        assert out.shape == y.shape, (node.kind, out.shape, y.shape)
+        vals[y.name] = out
+    return vals
+
+
+def random_input(case, seed=0):
+    rng = np.random.default_rng(seed)
+    t = case.input
+    if t.dtype == "f32":
+        return (rng.standard_normal(t.shape) * 1.2).astype(np.float32)
+    return rng.integers(0, 256, t.shape, dtype=np.uint8)
+
+
+# ---- the same evaluation on the REAL reference (oracle/_ref), one image at a time --------------------
+REF_SO = __import__("os").path.join(__import__("os").path.dirname(__import__("os").path.abspath(__file__)), "_ref",
+                                    "libnart_ref.so")
+
+
+def reference_available():
+    import os
+    return os.path.exists(REF_SO)
+
+
+class ReferenceCase:
+    """A Case instantiated on the reference CPU `quant` module through its C API (ops created once,
+    weights resident, batch 1 — the reference's conv aborts for larger batches,
+    conv_2d_uint8_impl.c:104).  run(x) feeds one image and returns the output tensor."""
+
+    def __init__(self, case):
+        import ctypes as C
+        from nart_amd import art
+        assert case.input.shape[0] == 1
+        self.case, self.art = case, art
+        rt = art.Runtime(REF_SO)
+        ws = self.ws = rt.workspace("quant")
+        T = case.tensors
+        inp = case.input
+        self.t = {inp.name: ws.tensor(dtype=np.float32 if inp.dtype == "f32" else np.uint8, shape=inp.shape)}
+        self.t[inp.name].alloc()
+        self.ops = []
+        for node in case.nodes:
+            y, xs, a = T[node.output], [T[i] for i in node.inputs], node.attrs
+            ins = [self.t[i] for i in node.inputs]
+            if node.kind == "quantize":
+                op = ws.quantize(ins[0], y.alpha, y.zp)
+            elif node.kind == "dequantize":
+                op = ws.dequantize(ins[0], xs[0].alpha, xs[0].zp)
+            elif node.kind in ("conv", "ip"):
+                q = dict(ialpha=xs[0].alpha, izp=xs[0].zp, walpha=a["walpha"], wzp=a["wzp"], oalpha=y.alpha, ozp=y.zp)
+                w, b = ws.tensor(case.weights[a["w"]]), ws.tensor(case.weights[a["b"]])
+                if node.kind == "conv":
+                    op = ws.conv2d(ins[0], w, b, a["pad"], a["stride"], a["group"], q)
+                    if a["relu"]:  # the reference CPU conv has no fused ReLU: a relu op follows
+                        op.prepare()
+                        self._zero_conv_scratch(op)
+                        self.ops.append(op)
+                        op = ws.relu(op.output(0), dict(ialpha=y.alpha, izp=y.zp, oalpha=y.alpha, ozp=y.zp))
+                else:
+                    op = ws.ip(ins[0], w, b, q)
+            elif node.kind == "pool":
+                q = dict(ialpha=xs[0].alpha, izp=xs[0].zp, oalpha=y.alpha, ozp=y.zp)
+                op = ws.pool(ins[0], a["k"], a["pad"], a["stride"], a["method"], a["ceil_mode"], q)
+            elif node.kind == "add":
+                q = dict(ialpha=[xs[0].alpha, xs[1].alpha], izp=[xs[0].zp, xs[1].zp], oalpha=y.alpha, ozp=y.zp)
+                op = ws.add(ins[0], ins[1], q)
+            else:
+                raise ValueError(node.kind)
+            op.prepare()
+            if node.kind == "conv" and not a["relu"]:
+                self._zero_conv_scratch(op)
+            self.ops.append(op)
+            self.t[y.name] = op.output(0)
+
+    def _zero_conv_scratch(self, op):
+        # the column buffer must start zeroed: the reference's im2col never writes padding taps
+        # (im2col.cpp:568-600); `temp_data` sits at offset 192 of op_conv_2d_t (conv_2d.h:40-72)
+        import ctypes as C
+        art = self.art
+        mem = C.cast(C.c_void_p.from_address(C.addressof(op.ptr.contents) + 192).value, C.POINTER(art.mem_t))
+        tp = mem.contents.tp.contents
+        C.memset(tp.cpu_data_func(mem), 0, tp.size_func(mem))
+
+    def run(self, x):
+        self.t[self.case.input.name].write(x)
+        for op in self.ops:
+            op.run()
+        return self.fetch(self.case.output.name)
+
+    def fetch(self, name):
+        # the reference's ip output is 2-D [M, Nout] (op.c:862-869); cases carry it as [M, Nout, 1, 1]
+        return self.t[name].numpy().reshape(self.case.tensors[name].shape)

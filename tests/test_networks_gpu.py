@@ -1,0 +1,81 @@
+"""Whole-network parity on the GPU: every intermediate tensor of the synthetic ResNet-18 / ResNet-50 /
+MobileNetV2 cases must equal the CPU oracle's, byte for byte (fp32 bit patterns for dequantize)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+from nart_amd import cases  # noqa: E402
+from nart_amd.runner import HipqExecutor  # noqa: E402
+
+from oracle import casecpu as case_oracle  # noqa: E402
+
+
+def compare_all(case, ex, vals):
+    for node in case.nodes:
+        got, want = ex.fetch(node.output), vals[node.output]
+        if want.dtype == np.float32:
+            ok = np.array_equal(got.view(np.uint32), want.view(np.uint32))
+        else:
+            ok = np.array_equal(got, want)
+        assert ok, "first mismatch at %s %s (%d elements differ)" % (node.kind, node.output, int((got != want).sum()))
+
+
+@pytest.mark.parametrize("build", [lambda: cases.resnet18(N=1), lambda: cases.resnet18(N=3, hw=96),
+                                   lambda: cases.mobilenet_v2(N=2, hw=96), lambda: cases.resnet50(N=2, hw=64),
+                                   lambda: cases.single_conv(N=2), lambda: cases.single_fc(M=16, K=1024, Nout=512)],
+                         ids=["resnet18_n1_224", "resnet18_n3_96", "mobilenetv2_n2_96", "resnet50_n2_64", "conv_cfg1", "fc"])
+def test_network_parity(build):
+    case = build()
+    print("case", case.name, flush=True)
+    x = case_oracle.random_input(case, seed=3)
+    vals = case_oracle.run_case(case, x)
+    ex = HipqExecutor(case)
+    ex.set_input(x)
+    ex.run()
+    torch.cuda.synchronize()
+    compare_all(case, ex, vals)
+
+
+def test_graph_replay_matches_eager():
+    """A captured HIP graph of the whole pass must reproduce the eager result on every replay, with
+    eager work and synchronisation in between (new inputs each time)."""
+    case = cases.resnet50(N=2, hw=64)
+    ex = HipqExecutor(case)
+    ex.set_input(case_oracle.random_input(case, seed=0))
+    ex.capture()
+    for seed in (1, 2, 3):
+        x = case_oracle.random_input(case, seed=seed)
+        ex.set_input(x)
+        ex.run()
+        torch.cuda.synchronize()
+        eager = {n.output: ex.fetch(n.output) for n in case.nodes}
+        for n in case.nodes:  # scribble over every buffer so that a replay has to recompute it
+            ex.buf[n.output].zero_()
+        torch.cuda.synchronize()
+        ex.replay()
+        torch.cuda.synchronize()
+        for n in case.nodes:
+            got = ex.fetch(n.output)
+            assert np.array_equal(got.view(np.uint8), eager[n.output].view(np.uint8)), (seed, n.output)
+
+
+def test_batch64_properties_resnet50_stage():
+    """Full batch size without the CPU oracle on the whole tensor: images are independent, so image i of
+    a batch-64 run equals the same image run alone (whose layers are oracle-checked above)."""
+    case64 = cases.resnet50(N=64, hw=64)
+    case1 = cases.resnet50(N=1, hw=64)
+    x = case_oracle.random_input(case64, seed=5)
+    ex64, ex1 = HipqExecutor(case64), HipqExecutor(case1)
+    ex64.set_input(x)
+    ex64.run()
+    out64 = ex64.output()
+    for i in (0, 31, 63):
+        ex1.set_input(x[i:i + 1])
+        ex1.run()
+        torch.cuda.synchronize()
+        assert np.array_equal(ex1.output().view(np.uint32), out64[i:i + 1].view(np.uint32)), i
+        want = case_oracle.run_case(case1, x[i:i + 1])[case1.output.name]
+        assert np.array_equal(out64[i:i + 1].view(np.uint32), want.view(np.uint32)), i
