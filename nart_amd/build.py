@@ -16,7 +16,8 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "lib")
 INC = os.path.join(ROOT, "include")
 
-HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
+HIPCC = os.environ.get("HIPCC", os.path.join(ROCM, "bin", "hipcc"))
 # packed-fp32 instructions are switched off on purpose (they have produced wrong results on this pool)
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function"]
@@ -65,19 +66,41 @@ def build_art(force=False):
         out = os.path.join(LIB, "libart.so")
         deps = core_src + _glob("core", (".h",)) + [os.path.join(INC, "art", f) for f in os.listdir(os.path.join(INC, "art"))]
         if force or not _newer(out, deps):
-            _run(["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-DART_CONSTRAINT_WITH_NAME", "-I" + INC,
-                  "-o", out] + core_src + ["-lm", "-ldl"])
+            _run(["gcc", "-O2", "-std=gnu11", "-fPIC", "-shared", "-Wall", "-fvisibility=hidden", "-I" + INC,
+                  "-I" + os.path.join(CSRC, "core"), "-o", out] + core_src + ["-lm"])
         outs.append(out)
-    mod_src = _glob("module", (".cpp",))
-    if mod_src:
-        out = os.path.join(LIB, "libart_module_hip.so")
-        deps = mod_src + _glob("module", (".h",)) + [os.path.join(INC, "hipq.h")]
-        if force or not _newer(out, deps):
-            _run([HIPCC, "-O2", "-std=c++17", "-fPIC", "-shared", "-Wall", "-DART_CONSTRAINT_WITH_NAME", "-I" + INC,
-                  "-I" + os.path.join(CSRC, "module"), "-o", out] + mod_src
-                 + ["-L" + LIB, "-lhipq", "-Wl,-rpath,$ORIGIN"])
-        outs.append(out)
+    outs += build_module(force)
     return outs
+
+
+def build_module(force=False, nart_tree=None, out_name="libart_module_hip.so"):
+    """The `hip` case module.  nart_tree: path of a NART checkout — then the module is compiled against the
+    runtime's own headers instead of include/art/art.h (how a NART maintainer would build it)."""
+    mod_src = _glob("module", (".cpp", ".c"))
+    if not mod_src:
+        return []
+    out = os.path.join(LIB, out_name)
+    deps = mod_src + _glob("module", (".h",)) + [os.path.join(INC, "hipq.h"), os.path.join(INC, "art", "art.h")]
+    if not force and _newer(out, deps):
+        return [out]
+    inc = ["-I" + INC, "-I" + os.path.join(CSRC, "module")]
+    if nart_tree:
+        art = os.path.join(nart_tree, "art")
+        inc += ["-DNART_HIP_USE_NART_HEADERS", "-DART_CONSTRAINT_WITH_NAME", "-DNART_LOG_LEVEL=1",
+                "-I" + os.path.join(art, "include"), "-I" + os.path.join(art, "modules", "quant", "include")]
+    objs = []
+    for s in mod_src:
+        o = os.path.join(LIB, "obj_%s_%s.o" % (out_name.split(".")[0], os.path.basename(s)))
+        if s.endswith(".c"):
+            _run(["gcc", "-O2", "-std=gnu11", "-fPIC", "-Wall"] + inc + ["-c", s, "-o", o])
+        else:
+            # host-only C++ (no device code in the module): the HIP runtime API through its AMD platform headers
+            _run(["g++", "-O2", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function", "-D__HIP_PLATFORM_AMD__",
+                  "-I" + os.path.join(ROCM, "include")] + inc + ["-c", s, "-o", o])
+        objs.append(o)
+    _run(["g++", "-shared", "-fPIC", "-o", out] + objs + ["-L" + LIB, "-lhipq", "-L" + os.path.join(ROCM, "lib"),
+                                                          "-lamdhip64", "-Wl,-rpath,$ORIGIN"])
+    return [out]
 
 
 def build_all(force=False):

@@ -1,0 +1,524 @@
+// The `hip` case module: workspace, op table and the operators' alloc/config/destroy/dealloc/prepare/run.
+//
+// Each operator mirrors its counterpart in the reference CPU quant module (art/modules/quant/src/op/*.c):
+// the same settings are read in `config` (missing required ones abort, as there), `prepare` allocates the
+// tensors, derives everything that does not depend on the activations (for conv/ip: the packed weights and
+// folded per-channel constants, which the reference recomputes on every run) and selects the run function;
+// `run` only launches kernels on the workspace stream.
+#include <cstring>
+#include <new>
+#include <vector>
+
+#include "hip_module.h"
+
+namespace {
+
+// ---- the quantisation settings every op reads (e.g. conv_2d.c:42-69) ----------------------------------------
+struct QSet {
+    float *alpha = nullptr;
+    uint8_t *zp = nullptr;
+    uint8_t *bits = nullptr;
+    size_t n = 0;
+};
+
+void read_qset(op_t *op, uint32_t ia, uint32_t iz, uint32_t ib, QSet *q)
+{
+    size_t n1 = 0, n2 = 0, n3 = 0;
+    HIPM_CHECK(op_setting_array_get(op, ia, dtFLOAT32, &n1, &q->alpha));
+    HIPM_CHECK(op_setting_array_get(op, iz, dtUINT8, &n2, &q->zp));
+    HIPM_CHECK(op_setting_array_get(op, ib, dtUINT8, &n3, &q->bits));
+    HIPM_CHECK(q->alpha && q->zp && q->bits && n1 >= 1 && n2 >= 1 && n3 >= 1);
+    q->n = n1 < n2 ? n1 : n2;
+}
+#define READ_I(op, q) read_qset(op, SETTING_QUANT_IALPHA, SETTING_QUANT_IZERO_POINT, SETTING_QUANT_IBITS, q)
+#define READ_W(op, q) read_qset(op, SETTING_QUANT_WALPHA, SETTING_QUANT_WZERO_POINT, SETTING_QUANT_WBITS, q)
+#define READ_O(op, q) read_qset(op, SETTING_QUANT_OALPHA, SETTING_QUANT_OZERO_POINT, SETTING_QUANT_OBITS, q)
+
+void alloc_and_tag(op_t *op)
+{
+    for (size_t i = 0; i < op->input_size; ++i) {
+        tensor_alloc(op->input_tensors[i]);
+    }
+    for (size_t i = 0; i < op->output_size; ++i) {
+        tensor_alloc(&op->output_tensors[i]);
+        hip_mem_tag(&op->output_tensors[i]);
+    }
+}
+
+template <class T>
+op_t *alloc_op(workspace_t *)
+{
+    T *p = static_cast<T *>(calloc(1, sizeof(T)));
+    return reinterpret_cast<op_t *>(p);
+}
+
+void dealloc_op(op_t *op) { free(op); }
+void destroy_nothing(op_t *) {}
+
+const void *in_ptr(op_t *op, int i) { return hip_mem_dev_in(op->input_tensors[i]->mem, op_stream(op)); }
+void *out_ptr(op_t *op) { return hip_mem_dev_out(op->output_tensors[0].mem, op_stream(op)); }
+
+void require_hip_u8(op_t *op, size_t n_act)
+{
+    for (size_t i = 0; i < n_act; ++i) {
+        if (op->input_tensors[i]->dtype != dtUINT8) {
+            fprintf(stderr, "[hip module] %s: input %zu has dtype %u; only uint8 activations are implemented\n",
+                    op->entry->tp->name, i, op->input_tensors[i]->dtype);
+            abort(); // the reference aborts on unsupported dtypes as well (conv_2d.c:143-145)
+        }
+        HIPM_CHECK(is_hip_mem(op->input_tensors[i]->mem));
+        hip_mem_tag(op->input_tensors[i]);
+    }
+}
+
+// ---- conv_2d and ip share one structure: both run a hipq convolution plan -------------------------------------
+struct conv_op_t {
+    op_t o;
+    uint32_t num_output, pad_h, pad_w, kernel_h, kernel_w, stride_h, stride_w, group;
+    QSet qi, qw, qo;
+    hipq_conv2d_plan *plan;
+    hipq_conv2d_desc desc; // what the plan was built for (re-used when prepare is called again unchanged)
+    const void *w_seen;    // identity of the weights the plan was packed from
+};
+
+void conv_config(op_t *op)
+{
+    conv_op_t *c = reinterpret_cast<conv_op_t *>(op);
+    HIPM_CHECK(op_setting_single_get(op, SETTING_CONV_2D_NUM_OUTPUT, dtUINT32, &c->num_output));
+    HIPM_CHECK(op_setting_single_get(op, SETTING_CONV_2D_KERNEL_H, dtUINT32, &c->kernel_h));
+    HIPM_CHECK(op_setting_single_get(op, SETTING_CONV_2D_KERNEL_W, dtUINT32, &c->kernel_w));
+    HIPM_CHECK(op_setting_single_get(op, SETTING_CONV_2D_PAD_H, dtUINT32, &c->pad_h));
+    HIPM_CHECK(op_setting_single_get(op, SETTING_CONV_2D_PAD_W, dtUINT32, &c->pad_w));
+    HIPM_CHECK(op_setting_single_get(op, SETTING_CONV_2D_STRIDE_H, dtUINT32, &c->stride_h));
+    HIPM_CHECK(op_setting_single_get(op, SETTING_CONV_2D_STRIDE_W, dtUINT32, &c->stride_w));
+    HIPM_CHECK(op_setting_single_get(op, SETTING_CONV_2D_GROUP, dtUINT32, &c->group));
+    READ_I(op, &c->qi);
+    READ_W(op, &c->qw);
+    READ_O(op, &c->qo);
+}
+
+void ip_config(op_t *op)
+{
+    conv_op_t *c = reinterpret_cast<conv_op_t *>(op);
+    HIPM_CHECK(op_setting_single_get(op, SETTING_IP_NUM_OUTPUT, dtUINT32, &c->num_output));
+    READ_I(op, &c->qi);
+    READ_W(op, &c->qw);
+    READ_O(op, &c->qo);
+}
+
+void conv_destroy(op_t *op)
+{
+    conv_op_t *c = reinterpret_cast<conv_op_t *>(op);
+    hipq_conv2d_plan_destroy(c->plan);
+    c->plan = nullptr;
+}
+
+void conv_run(op_t *op)
+{
+    conv_op_t *c = reinterpret_cast<conv_op_t *>(op);
+    HIPM_HIPQ(hipq_conv2d_run(c->plan, in_ptr(op, 0), out_ptr(op), nullptr, op_stream(op)));
+}
+
+void build_plan(op_t *op, const hipq_conv2d_desc &d, const uint8_t *w, const void *w_id)
+{
+    conv_op_t *c = reinterpret_cast<conv_op_t *>(op);
+    if (c->plan && memcmp(&c->desc, &d, sizeof d) == 0 && c->w_seen == w_id)
+        return; // prepare is called again after a reshape (art/src/parade.c:199-215): nothing changed
+    hipq_conv2d_plan_destroy(c->plan);
+    c->plan = nullptr;
+    const int32_t *bias = nullptr;
+    if (op->input_size == 3) {
+        HIPM_CHECK(op->input_tensors[2]->dtype == dtINT32);
+        bias = static_cast<const int32_t *>(is_hip_mem(op->input_tensors[2]->mem)
+                                                ? hip_mem_host_in(op->input_tensors[2]->mem)
+                                                : mem_cpu_data(op->input_tensors[2]->mem));
+    } // without a bias the accumulator starts at zero (the reference reads an unset buffer there)
+    HIPM_HIPQ(hipq_conv2d_plan_create(&d, w, bias, &c->plan));
+    c->desc = d;
+    c->w_seen = w_id;
+    op->run_func = conv_run;
+}
+
+const uint8_t *host_weights(op_t *op)
+{
+    tensor_t *w = op->input_tensors[1];
+    HIPM_CHECK(w->dtype == dtUINT8);
+    return static_cast<const uint8_t *>(is_hip_mem(w->mem) ? hip_mem_host_in(w->mem) : mem_cpu_data(w->mem));
+}
+
+void conv_prepare(op_t *op)
+{
+    conv_op_t *c = reinterpret_cast<conv_op_t *>(op);
+    require_hip_u8(op, 1);
+    alloc_and_tag(op);
+    const shape_t &xs = op->input_tensors[0]->shape;
+    const hip_mem_t *xm = as_hip(op->input_tensors[0]->mem), *ym = as_hip(op->output_tensors[0].mem);
+    HIPM_CHECK(xs.dim_size == 4 && xm->layout == HIP_LAYOUT_NHWC_U8 && ym->layout == HIP_LAYOUT_NHWC_U8);
+    hipq_conv2d_desc d;
+    memset(&d, 0, sizeof d);
+    d.N = (int)xs.dim[0], d.C = (int)xs.dim[1], d.H = (int)xs.dim[2], d.W = (int)xs.dim[3];
+    d.K = (int)c->num_output, d.R = (int)c->kernel_h, d.S = (int)c->kernel_w;
+    d.pad_h = (int)c->pad_h, d.pad_w = (int)c->pad_w, d.stride_h = (int)c->stride_h, d.stride_w = (int)c->stride_w;
+    d.group = (int)c->group;
+    d.in_cs = xm->cs, d.out_cs = ym->cs;
+    // per-tensor parameters: element [0] of each array, like the reference (conv_2d_uint8_impl.c:57-66)
+    d.ialpha = c->qi.alpha[0], d.walpha = c->qw.alpha[0], d.oalpha = c->qo.alpha[0];
+    d.izp = c->qi.zp[0], d.wzp = c->qw.zp[0], d.ozp = c->qo.zp[0];
+    d.obits = c->qo.bits[0];
+    d.relu = 0; // the reference CPU module ignores SETTING_CONV_2D_RELU_FLAG (conv_2d.c:27-70); so does this one
+    build_plan(op, d, host_weights(op), op->input_tensors[1]->mem);
+}
+
+void ip_prepare(op_t *op)
+{
+    conv_op_t *c = reinterpret_cast<conv_op_t *>(op);
+    require_hip_u8(op, 1);
+    alloc_and_tag(op);
+    const hip_mem_t *xm = as_hip(op->input_tensors[0]->mem), *ym = as_hip(op->output_tensors[0].mem);
+    HIPM_CHECK(xm->layout == HIP_LAYOUT_NHWC_U8 && ym->layout == HIP_LAYOUT_NHWC_U8);
+    // the input's true geometry is the producer's (a flatten/reshape in between does not move bytes)
+    const int M = xm->N, kd = xm->H * xm->W * xm->cs;
+    const size_t kin = (size_t)xm->C * xm->H * xm->W;
+    HIPM_CHECK(shape_count(&op->input_tensors[1]->shape) == (size_t)c->num_output * kin);
+    HIPM_CHECK(ym->N == M && ym->C == (int)c->num_output && ym->H == 1 && ym->W == 1);
+    const uint8_t *w = host_weights(op);
+    std::vector<uint8_t> reordered;
+    if (xm->H * xm->W > 1 || xm->cs != xm->C) { // (c,h,w) order of the reference -> (h,w,c) with channel stride
+        reordered.resize((size_t)c->num_output * kd);
+        HIPM_HIPQ(hipq_ip_reorder_weights(w, reordered.data(), (int)c->num_output, xm->C, xm->H, xm->W, xm->cs,
+                                          c->qw.zp[0]));
+        w = reordered.data();
+    }
+    hipq_conv2d_desc d;
+    memset(&d, 0, sizeof d);
+    d.N = M, d.C = kd, d.H = 1, d.W = 1, d.K = (int)c->num_output, d.R = 1, d.S = 1;
+    d.stride_h = d.stride_w = 1, d.group = 1;
+    d.in_cs = kd, d.out_cs = ym->cs;
+    d.ialpha = c->qi.alpha[0], d.walpha = c->qw.alpha[0], d.oalpha = c->qo.alpha[0];
+    d.izp = c->qi.zp[0], d.wzp = c->qw.zp[0], d.ozp = c->qo.zp[0];
+    d.obits = c->qo.bits[0];
+    build_plan(op, d, w, op->input_tensors[1]->mem);
+}
+
+// ---- element-wise ops ------------------------------------------------------------------------------------------
+struct ew_op_t {
+    op_t o;
+    QSet qi, qo;
+    uint32_t operation;
+    float *coeff;
+    size_t bytes; // device bytes to process (pad channels included)
+};
+
+size_t device_bytes_of(const tensor_t *t)
+{
+    const hip_mem_t *m = as_hip(t->mem);
+    return m->layout == HIP_LAYOUT_NHWC_U8 ? (size_t)m->N * m->H * m->W * m->cs : m->size;
+}
+
+void same_geometry(op_t *op)
+{
+    const hip_mem_t *a = as_hip(op->input_tensors[0]->mem);
+    for (size_t i = 1; i < op->input_size; ++i) {
+        const hip_mem_t *b = as_hip(op->input_tensors[i]->mem);
+        HIPM_CHECK(shape_count(&op->input_tensors[i]->shape) == shape_count(&op->input_tensors[0]->shape));
+        HIPM_CHECK(a->layout == b->layout && a->N == b->N && a->C == b->C && a->H == b->H && a->W == b->W);
+    }
+    const hip_mem_t *y = as_hip(op->output_tensors[0].mem);
+    HIPM_CHECK(a->layout == y->layout && a->N == y->N && a->C == y->C && a->H == y->H && a->W == y->W);
+}
+
+void add_config(op_t *op)
+{
+    ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    READ_I(op, &e->qi);
+    READ_O(op, &e->qo);
+    HIPM_CHECK(e->qi.n >= 2);
+}
+
+void add_run(op_t *op)
+{
+    ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    HIPM_HIPQ(hipq_add_u8(in_ptr(op, 0), in_ptr(op, 1), out_ptr(op), e->bytes, e->qi.alpha[0], e->qi.zp[0], e->qi.alpha[1],
+                          e->qi.zp[1], e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0], op_stream(op)));
+}
+
+void add_prepare(op_t *op)
+{
+    ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    require_hip_u8(op, 2);
+    alloc_and_tag(op);
+    same_geometry(op); // broadcasting adds are not implemented (the reference's loop has none either, add.c:135)
+    e->bytes = device_bytes_of(&op->output_tensors[0]);
+    op->run_func = add_run;
+}
+
+void eltwise_config(op_t *op)
+{
+    ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    HIPM_CHECK(op_setting_single_get(op, SETTING_ELTWISE_OPERATION, dtUINT32, &e->operation));
+    if (!op_setting_if_set(op, SETTING_ELTWISE_COEFF)) { // default coefficients: all ones (eltwise.c:60-68)
+        std::vector<float> ones(op->input_size, 1.0f);
+        HIPM_CHECK(op_setting_array_set(op, SETTING_ELTWISE_COEFF, dtFLOAT32, op->input_size, ones.data()));
+    }
+    size_t n = 0;
+    HIPM_CHECK(op_setting_array_get(op, SETTING_ELTWISE_COEFF, dtFLOAT32, &n, &e->coeff));
+    HIPM_CHECK(n == op->input_size);
+    READ_I(op, &e->qi);
+    READ_O(op, &e->qo);
+    HIPM_CHECK(e->qi.n >= op->input_size);
+}
+
+void eltwise_run(op_t *op)
+{
+    ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    const void *ins[HIPQ_MAX_ELTWISE_INPUTS];
+    for (size_t i = 0; i < op->input_size; ++i)
+        ins[i] = in_ptr(op, (int)i);
+    HIPM_HIPQ(hipq_eltwise_u8(ins, (int)op->input_size, e->coeff, e->qi.alpha, e->qi.zp, out_ptr(op), e->bytes,
+                              (int)e->operation, e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0], op_stream(op)));
+}
+
+void eltwise_prepare(op_t *op)
+{
+    ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    HIPM_CHECK(e->operation == SETTING_ELTWISE_OP_SUM || e->operation == SETTING_ELTWISE_OP_MAX); // PROD: eltwise.c:237
+    HIPM_CHECK(op->input_size <= HIPQ_MAX_ELTWISE_INPUTS);
+    require_hip_u8(op, op->input_size);
+    alloc_and_tag(op);
+    same_geometry(op);
+    e->bytes = device_bytes_of(&op->output_tensors[0]);
+    op->run_func = eltwise_run;
+}
+
+void relu_config(op_t *op)
+{
+    ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    READ_I(op, &e->qi);
+    READ_O(op, &e->qo);
+}
+
+void relu_run(op_t *op)
+{
+    ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    HIPM_HIPQ(hipq_relu_u8(in_ptr(op, 0), out_ptr(op), e->bytes, e->qi.alpha[0], e->qi.zp[0], e->qo.alpha[0], e->qo.zp[0],
+                           e->qo.bits[0], op_stream(op)));
+}
+
+void relu_prepare(op_t *op)
+{
+    ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    require_hip_u8(op, 1);
+    alloc_and_tag(op);
+    same_geometry(op);
+    e->bytes = device_bytes_of(&op->output_tensors[0]);
+    op->run_func = relu_run;
+}
+
+// ---- pool ----------------------------------------------------------------------------------------------------------
+struct pool_op_t {
+    op_t o;
+    uint32_t method, pad_h, pad_w, kernel_h, kernel_w, stride_h, stride_w;
+    bool ceil_mode;
+    QSet qi, qo;
+};
+
+void pool_config(op_t *op)
+{
+    pool_op_t *p = reinterpret_cast<pool_op_t *>(op);
+    HIPM_CHECK(op_setting_single_get(op, SETTING_POOL_KERNEL_H, dtUINT32, &p->kernel_h));
+    HIPM_CHECK(op_setting_single_get(op, SETTING_POOL_KERNEL_W, dtUINT32, &p->kernel_w));
+    HIPM_CHECK(op_setting_single_get(op, SETTING_POOL_METHOD, dtUINT32, &p->method));
+    HIPM_CHECK(op_setting_single_get(op, SETTING_POOL_PAD_H, dtUINT32, &p->pad_h));
+    HIPM_CHECK(op_setting_single_get(op, SETTING_POOL_PAD_W, dtUINT32, &p->pad_w));
+    HIPM_CHECK(op_setting_single_get(op, SETTING_POOL_STRIDE_H, dtUINT32, &p->stride_h));
+    HIPM_CHECK(op_setting_single_get(op, SETTING_POOL_STRIDE_W, dtUINT32, &p->stride_w));
+    HIPM_CHECK(op_setting_single_get(op, SETTING_POOL_CEIL_MODE, dtBOOL, &p->ceil_mode));
+    READ_I(op, &p->qi);
+    READ_O(op, &p->qo);
+}
+
+void pool_run(op_t *op)
+{
+    pool_op_t *p = reinterpret_cast<pool_op_t *>(op);
+    const hip_mem_t *x = as_hip(op->input_tensors[0]->mem), *y = as_hip(op->output_tensors[0].mem);
+    HIPM_HIPQ(hipq_pool_u8(in_ptr(op, 0), out_ptr(op), x->N, x->C, x->H, x->W, y->H, y->W, x->cs, (int)p->kernel_h,
+                           (int)p->kernel_w, (int)p->pad_h, (int)p->pad_w, (int)p->stride_h, (int)p->stride_w,
+                           p->method == SETTING_POOL_MAX ? HIPQ_POOL_MAX : HIPQ_POOL_AVE, p->qi.alpha[0], p->qi.zp[0],
+                           p->qo.alpha[0], p->qo.zp[0], p->qo.bits[0], op_stream(op)));
+}
+
+void pool_prepare(op_t *op)
+{
+    require_hip_u8(op, 1);
+    alloc_and_tag(op);
+    HIPM_CHECK(op->input_tensors[0]->shape.dim_size == 4);
+    op->run_func = pool_run;
+}
+
+// ---- reshape: zero-copy view (the output shares the input's memory, art/src/op.c:1115) -----------------------
+void reshape_config(op_t *) {}
+void reshape_run(op_t *) {}
+void reshape_prepare(op_t *op)
+{
+    for (size_t i = 0; i < op->input_size; ++i)
+        tensor_alloc(op->input_tensors[i]);
+    op->run_func = reshape_run;
+}
+
+// ---- quantize / dequantize -------------------------------------------------------------------------------------------
+struct qdq_op_t {
+    op_t o;
+    QSet q;
+    int32_t qtype;
+};
+
+void dims4(const tensor_t *t, int d[4])
+{
+    const int nd = t->shape.dim_size;
+    d[0] = (int)t->shape.dim[0];
+    d[1] = nd > 1 ? (int)t->shape.dim[1] : 1;
+    d[2] = nd > 2 ? (int)t->shape.dim[2] : 1;
+    d[3] = nd > 3 ? (int)t->shape.dim[3] : 1;
+}
+
+void quantize_config(op_t *op)
+{
+    qdq_op_t *q = reinterpret_cast<qdq_op_t *>(op);
+    READ_O(op, &q->q);
+    HIPM_CHECK(op_setting_single_get(op, SETTING_QUANT_QTYPE, dtINT32, &q->qtype));
+}
+
+void quantize_run(op_t *op)
+{
+    qdq_op_t *q = reinterpret_cast<qdq_op_t *>(op);
+    int d[4];
+    dims4(op->input_tensors[0], d);
+    const hip_mem_t *y = as_hip(op->output_tensors[0].mem);
+    HIPM_HIPQ(hipq_quantize_u8(static_cast<const float *>(in_ptr(op, 0)), out_ptr(op), d[0], d[1], d[2], d[3], y->cs,
+                               q->q.alpha[0], q->q.zp[0], q->q.bits[0], op_stream(op)));
+}
+
+void quantize_prepare(op_t *op)
+{
+    qdq_op_t *q = reinterpret_cast<qdq_op_t *>(op);
+    HIPM_CHECK(op->input_tensors[0]->dtype == dtFLOAT32 && is_hip_mem(op->input_tensors[0]->mem));
+    const int32_t key = q->qtype << 8 | q->q.bits[0];
+    if (key != 0x0008 && key != 0x0108) { // quantize.c:233-262: this module implements the uint8 rows
+        fprintf(stderr, "[hip module] quantization for %d bits with type %d is not implemented\n", q->q.bits[0], q->qtype);
+        abort();
+    }
+    const int nd = op->input_tensors[0]->shape.dim_size;
+    HIPM_CHECK(nd == 4 || nd == 2);
+    hip_mem_tag(op->input_tensors[0]);
+    alloc_and_tag(op);
+    op->run_func = quantize_run;
+}
+
+void dequantize_config(op_t *op)
+{
+    qdq_op_t *q = reinterpret_cast<qdq_op_t *>(op);
+    READ_I(op, &q->q);
+    HIPM_CHECK(op_setting_single_get(op, SETTING_QUANT_QTYPE, dtINT32, &q->qtype));
+}
+
+void dequantize_run(op_t *op)
+{
+    qdq_op_t *q = reinterpret_cast<qdq_op_t *>(op);
+    const hip_mem_t *x = as_hip(op->input_tensors[0]->mem);
+    HIPM_HIPQ(hipq_dequantize_u8(in_ptr(op, 0), static_cast<float *>(out_ptr(op)), x->N, x->C, x->H, x->W, x->cs,
+                                 q->q.alpha[0], q->q.zp[0], op_stream(op)));
+}
+
+void dequantize_prepare(op_t *op)
+{
+    qdq_op_t *q = reinterpret_cast<qdq_op_t *>(op);
+    const int32_t key = q->qtype << 8 | q->q.bits[0];
+    if (key != 0x0008 && key != 0x0108) { // dequantize.c:150-167
+        fprintf(stderr, "[hip module] dequantization for %d bits with type %d is not implemented\n", q->q.bits[0], q->qtype);
+        abort();
+    }
+    require_hip_u8(op, 1);
+    alloc_and_tag(op);
+    HIPM_CHECK(as_hip(op->input_tensors[0]->mem)->layout == HIP_LAYOUT_NHWC_U8);
+    op->run_func = dequantize_run;
+}
+
+// ---- workspace ------------------------------------------------------------------------------------------------------------
+int g_ws_count = 0;
+
+const char *ws_name(const workspace_t *ws) { return reinterpret_cast<const hip_workspace_t *>(ws)->name; }
+const mem_tp *ws_memtype(const workspace_t *) { return &hip_mem_tp_st; }
+
+void ws_delete(workspace_t *w)
+{
+    hip_workspace_t *ws = reinterpret_cast<hip_workspace_t *>(w);
+    if (ws->own_stream && ws->stream)
+        (void)hipStreamDestroy(ws->stream);
+    free(ws);
+}
+
+} // namespace
+
+extern "C" {
+
+extern const module_t hip_module_tp;
+
+#define SETTING_HIP_WORKSPACE_DEVID 1 /* same id as SETTING_CUDA_QUANT_WORKSPACE_DEVID (cuda_quant_module.c:98-114) */
+
+static workspace_t *ws_new(const setting_entry_t *settings)
+{
+    hip_workspace_t *ws = static_cast<hip_workspace_t *>(calloc(1, sizeof(hip_workspace_t)));
+    ws->ws.module_type = &hip_module_tp;
+    snprintf(ws->name, sizeof ws->name, "hip:%d", g_ws_count++);
+    for (const setting_entry_t *s = settings; s != nullptr && s->item != 0; ++s)
+        if (s->item == SETTING_HIP_WORKSPACE_DEVID)
+            ws->dev_id = (int)s->v.single.value.u32;
+    // the device is touched here, once; without a usable GPU the workspace cannot exist
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= ws->dev_id) {
+        fprintf(stderr, "[hip module] no usable GPU for device id %d (%s)\n", ws->dev_id,
+                e == hipSuccess ? "device count too small" : hipGetErrorString(e));
+        free(ws);
+        return nullptr;
+    }
+    HIPM_HIP(hipSetDevice(ws->dev_id));
+    HIPM_HIP(hipStreamCreateWithFlags(&ws->stream, hipStreamNonBlocking)); // default priority
+    ws->own_stream = true;
+    return &ws->ws;
+}
+
+// Extra entry points for runners that own a stream already (graph capture, event timing).
+ART_PUBLIC void *hip_workspace_stream(workspace_t *w) { return reinterpret_cast<hip_workspace_t *>(w)->stream; }
+
+ART_PUBLIC void hip_workspace_set_stream(workspace_t *w, void *stream)
+{
+    hip_workspace_t *ws = reinterpret_cast<hip_workspace_t *>(w);
+    if (ws->own_stream && ws->stream)
+        (void)hipStreamDestroy(ws->stream);
+    ws->stream = static_cast<hipStream_t>(stream);
+    ws->own_stream = false;
+}
+
+#define HIP_ENTRY(TP, T, CONFIG, DESTROY, PREPARE) {&TP, alloc_op<T>, CONFIG, DESTROY, dealloc_op, PREPARE}
+
+ART_PUBLIC op_tp_entry_t hip_op_table[] = {
+    HIP_ENTRY(op_hip_quantize_tp, qdq_op_t, quantize_config, destroy_nothing, quantize_prepare),
+    HIP_ENTRY(op_hip_dequantize_tp, qdq_op_t, dequantize_config, destroy_nothing, dequantize_prepare),
+    HIP_ENTRY(op_conv_2d_tp, conv_op_t, conv_config, conv_destroy, conv_prepare),
+    HIP_ENTRY(op_ip_tp, conv_op_t, ip_config, conv_destroy, ip_prepare),
+    HIP_ENTRY(op_relu_tp, ew_op_t, relu_config, destroy_nothing, relu_prepare),
+    HIP_ENTRY(op_add_tp, ew_op_t, add_config, destroy_nothing, add_prepare),
+    HIP_ENTRY(op_eltwise_tp, ew_op_t, eltwise_config, destroy_nothing, eltwise_prepare),
+    HIP_ENTRY(op_pool_tp, pool_op_t, pool_config, destroy_nothing, pool_prepare),
+    HIP_ENTRY(op_reshape_tp, ew_op_t, reshape_config, destroy_nothing, reshape_prepare),
+    {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr},
+};
+
+// op_group 6 = OP_GROUP_CODE_QUANT: an engine file written by the quant converter stamps every op with it,
+// so the strict pass of the loader's workspace choice picks this module (art/src/serialize_v1.c:103-120).
+ART_PUBLIC const module_t hip_module_tp = {
+    6, ws_name, ws_memtype, ws_new, ws_delete, hip_op_table,
+};
+
+} // extern "C"

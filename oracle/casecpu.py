@@ -124,3 +124,22 @@ class ReferenceCase:
     def fetch(self, name):
         # the reference's ip output is 2-D [M, Nout] (op.c:862-869); cases carry it as [M, Nout, 1, 1]
         return self.t[name].numpy().reshape(self.case.tensors[name].shape)
+
+
+def zero_reference_conv_scratch(parade):
+    """For a parade loaded on the REFERENCE runtime: zero every conv's column buffer once after prepare, which
+    is the state a freshly started reference runner finds it in (see ReferenceCase._zero_conv_scratch).
+    parade_t starts with {size_t op_count; op_t **ops} (art/src/parade_impl.h:23-32); an op's type name is
+    op->entry->tp->name."""
+    import ctypes as C
+    from nart_amd import art
+    n = C.c_size_t.from_address(parade.ptr).value
+    ops = C.cast(C.c_void_p.from_address(parade.ptr + 8).value, C.POINTER(C.POINTER(art.op_t)))
+    for i in range(n):
+        op = ops[i]
+        entry = C.cast(op.contents.entry, C.POINTER(C.c_void_p))       # op_tp_entry_t: first member is tp
+        name = C.cast(C.c_void_p.from_address(entry[0] + 8).value, C.c_char_p).value  # op_tp_t: code, then name
+        if name == b"conv_2d":
+            mem = C.cast(C.c_void_p.from_address(C.addressof(op.contents) + 192).value, C.POINTER(art.mem_t))
+            tp = mem.contents.tp.contents
+            C.memset(tp.cpu_data_func(mem), 0, tp.size_func(mem))
