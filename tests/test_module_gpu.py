@@ -1,0 +1,120 @@
+"""The drop-in boundary on a real GPU: an engine.bin written by nart_amd.engine (the file the unchanged quant
+converter would hand over) is loaded by an art runtime with the `hip` workspace selected, run, and its
+output compared with the CPU oracle, bit for bit.
+
+Two runtimes are driven through the same C ABI:
+  * the repo's own host core (nart_amd/lib/libart.so) + libart_module_hip.so;
+  * where it was built (oracle/_ref, from the reference's own sources): the REFERENCE libart with the module
+    compiled against the reference's own headers — the module is then a true plug-in of the unmodified
+    runtime, and the reference's CPU quant module runs the same file in the same process as a second checker.
+"""
+import os
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+torch = pytest.importorskip("torch")
+
+from nart_amd import art, cases, engine  # noqa: E402
+
+from oracle import casecpu  # noqa: E402
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB = os.path.join(ROOT, "nart_amd", "lib")
+REF_SO = os.path.join(ROOT, "oracle", "_ref", "libnart_ref.so")
+HIP_FOR_REF = os.path.join(LIB, "libart_module_hip_narttree.so")
+
+
+def small_cases():
+    return [cases.single_conv(N=1), cases.single_fc(M=5, K=256, Nout=64), cases.resnet18(N=2, hw=96),
+            cases.mobilenet_v2(N=1, hw=96), cases.resnet50(N=2, hw=64)]
+
+
+def same_bits(a, b):
+    return a.shape == b.shape and np.array_equal(np.ascontiguousarray(a).view(np.uint8), np.ascontiguousarray(b).view(np.uint8))
+
+
+@pytest.fixture(scope="module")
+def own_rt():
+    return art.Runtime(os.path.join(LIB, "libart.so"), [os.path.join(LIB, "libart_module_hip.so")])
+
+
+def test_engine_file_runs_on_hip_workspace(own_rt):
+    ws = own_rt.workspace("hip")
+    assert ws.name.startswith("hip")
+    for case in small_cases():
+        print("case", case.name, flush=True)
+        p = engine.Parade(own_rt, engine.write_engine(case), [ws])
+        for seed in (7, 8):  # the second pass re-uses every prepared plan and buffer
+            x = casecpu.random_input(case, seed)
+            got = p.forward(x).reshape(case.output.shape)
+            want = casecpu.run_case(case, x)[case.output.name]
+            assert same_bits(got, want), (case.name, seed)
+        p.delete()
+    ws.delete()
+
+
+def test_prepare_twice_and_batch_reshape(own_rt):
+    """parade_apply_reshape re-infers every shape and calls prepare again (art/src/parade.c:199-215): plans and
+    device buffers must follow the new batch size."""
+    ws = own_rt.workspace("hip")
+    case1, case3 = cases.resnet18(N=1, hw=64), cases.resnet18(N=3, hw=64)
+    p = engine.Parade(own_rt, engine.write_engine(case1), [ws])
+    x1 = casecpu.random_input(case1, 1)
+    assert same_bits(p.forward(x1).reshape(case1.output.shape), casecpu.run_case(case1, x1)[case1.output.name])
+    own_rt.core.parade_prepare(p.ptr)  # idempotent
+    assert same_bits(p.forward(x1).reshape(case1.output.shape), casecpu.run_case(case1, x1)[case1.output.name])
+    inp = p.inputs()[0]
+    inp.set_shape(case3.input.shape)
+    assert own_rt.core.parade_apply_reshape(p.ptr)
+    x3 = casecpu.random_input(case3, 2)
+    got = p.forward(x3).reshape(case3.output.shape)
+    assert same_bits(got, casecpu.run_case(case3, x3)[case3.output.name])
+    p.delete()
+    ws.delete()
+
+
+def test_single_ops_through_the_op_api(own_rt):
+    """workspace_new_op / op_config / op_prepare / op_run on device tensors, the way the reference's tests drive a
+    module without a file."""
+    from oracle import orc
+    ws = own_rt.workspace("hip")
+    rng = np.random.default_rng(11)
+    x = rng.integers(0, 256, (2, 24, 9, 11), dtype=np.uint8)
+    w = rng.integers(0, 256, (40, 24, 3, 3), dtype=np.uint8)
+    b = rng.integers(-5000, 5000, 40).astype(np.int32)
+    q = dict(ialpha=0.031, izp=77, walpha=0.0042, wzp=131, oalpha=0.09, ozp=13)
+    tx, tw, tb = ws.tensor(x), ws.tensor(w), ws.tensor(b)
+    conv = ws.conv2d(tx, tw, tb, 1, 2, 1, q).prepare().run()
+    want = orc.conv2d_u8(x, w, b, 1, 2, 1, 0.031, 77, 0.0042, 131, 0.09, 13)
+    assert same_bits(conv.output(0).numpy(), want)
+    relu = ws.relu(conv.output(0), dict(ialpha=0.09, izp=13, oalpha=0.05, ozp=3)).prepare().run()
+    want_r = orc.relu_u8(want, 0.09, 13, 0.05, 3)
+    assert same_bits(relu.output(0).numpy(), want_r)
+    elt = ws.eltwise([conv.output(0), relu.output(0)], dict(ialpha=[0.09, 0.05], izp=[13, 3], oalpha=0.11, ozp=9),
+                     coeff=[1.0, 0.5]).prepare().run()
+    want_e = orc.eltwise_u8([want, want_r], [0.09, 0.05], [13, 3], 0.11, 9, operation=1, coeff=[1.0, 0.5])
+    assert same_bits(elt.output(0).numpy(), want_e)
+    # overwrite the input through the host mirror: the next run must see it
+    x2 = rng.integers(0, 256, x.shape, dtype=np.uint8)
+    tx.write(x2)
+    conv.run()
+    assert same_bits(conv.output(0).numpy(), orc.conv2d_u8(x2, w, b, 1, 2, 1, 0.031, 77, 0.0042, 131, 0.09, 13))
+    for o in (elt, relu, conv):
+        o.delete()
+    ws.delete()
+
+
+@pytest.mark.skipif(not (os.path.exists(REF_SO) and os.path.exists(HIP_FOR_REF)),
+                    reason="reference runtime / module built against its headers not present")
+def test_module_plugs_into_the_reference_runtime():
+    """Runs in a process of its own: two art cores in one process would resolve each other's global symbols."""
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, "-u", os.path.join(ROOT, "tests", "refruntime_hip.py")], cwd=ROOT,
+                       stdout=subprocess.PIPE, stderr=subprocess.STDOUT, timeout=170)
+    out = r.stdout.decode()
+    print(out, flush=True)
+    assert r.returncode == 0 and "refruntime_hip ok" in out, out[-2000:]
