@@ -20,7 +20,9 @@ ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 HIPCC = os.environ.get("HIPCC", os.path.join(ROCM, "bin", "hipcc"))
 # packed-fp32 instructions are switched off on purpose (they have produced wrong results on this pool)
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",
-             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function"]
+             "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wno-unused-function",
+             # MFMA accumulators live in ordinary VGPRs: the epilogue reads them without v_accvgpr_read round trips
+             "-mllvm", "-amdgpu-mfma-vgpr-form"]
 
 
 def _run(cmd):

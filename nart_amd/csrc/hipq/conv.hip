@@ -12,22 +12,30 @@
 //     points, so both are re-centred: xs = x - 128 (a byte-wise XOR with 0x80), ws = w - 128, and with
 //     a = 128 - izp, b = 128 - wzp
 //         sum (x - izp)(w - wzp) = sum xs*ws + b * sum xs + a * sum ws + Kp*a*b.
-//     The last two terms are per-output-channel constants folded, with the bias, into `bias2` at setup.
-//     The second term is per pixel and non-zero only for wzp != 128; it is accumulated with v_dot4 from
-//     the very bytes that feed the MFMA (template flag HAS_WZP).  Taps that fall outside the image read
-//     the byte izp (xs = -a), which makes their (x - izp) exactly zero; k slots that exist only because
-//     of padding (pad channels, tail of the last 64-byte slab) carry the weight wzp (ws = -b), which
-//     makes their contribution zero whatever activation byte happens to sit there.
-//   * A (weights) is pre-packed at setup in MFMA fragment order, so a wave fetches a 32x32 fragment with
-//     one fully coalesced 1 KiB global load (L2/L1 resident; it never touches LDS).
-//     B (activations) is gathered from global memory 16 bytes per thread, XOR-ed, staged in LDS
-//     (row stride 80 bytes: conflict-free 128-bit reads) and double buffered.
-//   * A work-group of 4 waves computes a (WM*64 pixels) x (WN*64 channels) tile; each wave owns a
-//     64x64 sub-tile = 2x2 MFMA tiles = 64 int32 accumulators per lane.
-//   * Epilogue: each lane holds 4 consecutive output channels of one pixel per accumulator quad, so the
-//     requantised bytes are packed into one dword and stored straight into the NHWC output.
+//     The last two terms are per-output-channel constants folded, with the bias, into `bias2` at setup;
+//     the accumulators START at bias2, so the epilogue adds nothing.  The second term is per pixel and
+//     non-zero only for wzp != 128; it is accumulated with v_dot4 from the very bytes that feed the MFMA
+//     (template flag HAS_WZP).  Taps that fall outside the image read the byte izp (xs = -a), which makes
+//     their (x - izp) exactly zero; k slots that exist only because of padding (pad channels, tail of the
+//     last 64-byte slab) carry the weight wzp (ws = -b), which makes their contribution zero whatever
+//     activation byte happens to sit there.
+//   * A work-group of 4 waves computes a BM pixels x BN channels tile, 64 bytes of k ("slab") at a time.
+//     Both operands go through LDS: the weight slab [BN][64] is a straight copy of the pre-packed weights
+//     (coalesced, L2 resident), the activation slab [BM][64] is gathered 16 bytes per lane.  Rows are 64
+//     bytes without padding; the four 16-byte chunks of a row are stored at chunk ^ ((row >> 2) & 3), which
+//     makes both the 128-bit stores and the MFMA fragment reads bank-conflict free.  The weights are
+//     packed in that order on the host, so the copy is linear.  Two LDS stages; the global loads of slab
+//     i+1 are in flight while slab i is multiplied.
+//   * Epilogue.  mult = m * 2^7 with m < 2^24, and for 33 <= shift <= 52 (every realistic scale)
+//         floor((acc*mult + 2^(shift-1)) / 2^shift) + zp == (mulhi(acc, mult) + 2^(t-1) + zp*2^t) >> t,  t = shift-32
+//     because the low 32 bits of the product cannot carry across the floor.  That is one v_mul_hi_i32, one
+//     add, one shift and one clamp per output instead of a 64-bit multiply-add-shift.  Other shifts take
+//     the 64-bit path.  Each lane then holds 4 consecutive channels of one pixel per accumulator quad;
+//     the packed dwords are transposed through LDS so that every pixel's channels leave as 128-bit stores.
 //   * Work-groups are renumbered so that each of the 8 XCDs (round-robin dispatch) gets a contiguous
-//     range of pixel tiles: neighbouring tiles share input halos and weight fragments in that XCD's L2.
+//     range of pixel tiles: neighbouring tiles share input halos and weight slabs in that XCD's L2.
+#include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <string>
 #include <vector>
@@ -38,38 +46,161 @@ namespace hipq {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
+struct __attribute__((packed, aligned(4))) v4i_a4 { v4i v; }; // a 16-byte load that is only 4-byte aligned
 
 struct ConvArgs {
     const uint8_t *x;
     uint8_t *y;
     int32_t *acc_out;
-    const uint8_t *wpack; // MFMA: A fragments; depthwise: [tap][cs] int8 (w - wzp may not fit: stored as int16)
-    const int32_t *bias2; // per output channel, padded
+    const uint8_t *wpack; // MFMA: [slab][kout_pad][64] swizzled int8; depthwise: [tap][cs] int16
+    const int32_t *bias2; // per output channel, padded to kout_pad
+    const uint8_t *padbuf; // 64 bytes of the byte izp (source of out-of-image taps)
     int N, C, H, W, K, OH, OW;
     int in_cs, out_cs;
     int R, S, pad_h, pad_w, stride_h, stride_w, group;
-    int P;     // N*OH*OW output pixels
-    int rowb;  // bytes of one k "row": in_cs (generic) or 4*round_up(S,4) (small-C mode)
-    int Ktot;  // generic: R*S*in_cs; small-C: R*rowb
-    int nslab; // ceil(Ktot / 64)
+    int P;        // N*OH*OW output pixels
+    int rowb;     // bytes of one k "row": in_cs (generic) or 4*round_up(S,4) (small-C mode)
+    int Ktot;     // generic: R*S*in_cs; small-C: R*rowb
+    int nslab;    // ceil(Ktot / 64)
+    int kout_pad; // K rounded up to a multiple of 128
     int nbm, nbn;
     int bwz;          // b = 128 - wzp
     int izp, wzp;     // for the non-MFMA kernels
     uint32_t padword; // byte izp in all four lanes
     Requant q;
-    int lo; // lower clamp: ozp when ReLU is fused, else 0
+    int lo;    // lower clamp: ozp when ReLU is fused, else 0
+    int fastq; // 1: the one-multiply requantisation is valid for q.shift
+    int qt;    // shift - 32
+    int qadd;  // 2^(qt-1) + zp * 2^qt
+    double inv_ohw, inv_ow; // 1 / (OH*OW), 1 / OW
 };
+
+// x / d for 0 <= x < 2^31, d >= 1, inv = 1.0 / d: the double product is within one of the quotient, one
+// compare settles it (a handful of full-rate instructions instead of the generic 32-bit division sequence)
+__device__ static inline int fast_div(int x, int d, double inv)
+{
+    int q = (int)((double)x * inv);
+    q -= q * d > x;
+    q += (q + 1) * d <= x;
+    return q;
+}
 
 __device__ static inline v4i ldg128(const uint8_t *p) { return *reinterpret_cast<const v4i *>(p); }
 
 // ------------------------------------------------------------------------------------------------
+// Epilogue shared by the MFMA kernels: requantise the wave's accumulators and write the tile.
+// FAST selects the one-multiply requantisation (valid for 33 <= shift <= 52, see the file header).
+// The caller guarantees that no wave still reads the LDS stages and that no load into them is in flight.
+template <bool FAST>
+__device__ static inline int32_t conv_requant(const ConvArgs &a, int32_t v)
+{
+    int32_t r;
+    if (FAST)
+        r = (__mulhi(v, (int)a.q.mult) + a.qadd) >> a.qt;
+    else
+        r = (int32_t)(rshift_rn((int64_t)v * (int64_t)a.q.mult, a.q.shift) + a.q.zp);
+    int32_t out;
+    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(out) : "v"(r), "s"(a.lo), "v"(a.q.hi)); // lo <= hi: the median is the clamp
+    return out;
+}
+
+template <int BM, int BN, int WM, int WN, bool HAS_WZP, bool FAST, bool PLAIN_SAT, int TM, int TN>
+__device__ static inline void conv_epilogue(const ConvArgs &a, v16i (&acc)[TN][TM], int (&colsum)[TM], uint8_t *lds,
+                                            int bm, int bn, int wm, int wn)
+{
+    constexpr int OSTR = BN + 16; // row stride of the output staging tile
+    const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5;
+    const int ch0 = bn * BN + wn * (TN * 32);
+    const int m0 = bm * BM; // first pixel of the tile
+    if (a.acc_out != nullptr || (a.out_cs & 15)) {
+        // plain path: accumulator dump requested, or an output too narrow for 128-bit rows
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++) {
+            const int m = m0 + wm * (TM * 32) + tm * 32 + (lane & 31);
+            if (m >= a.P)
+                continue;
+#pragma unroll
+            for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+                for (int g = 0; g < 4; g++) {
+                    const int ko = ch0 + tn * 32 + g * 8 + half * 4;
+                    if (ko >= a.out_cs)
+                        continue;
+                    uint32_t packed = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int32_t v = (int32_t)((uint32_t)acc[tn][tm][g * 4 + e] + (HAS_WZP ? (uint32_t)colsum[tm] : 0u));
+                        if (a.acc_out)
+                            a.acc_out[(size_t)m * a.out_cs + ko + e] = v;
+                        packed |= (uint32_t)conv_requant<FAST>(a, v) << (8 * e);
+                    }
+                    *reinterpret_cast<uint32_t *>(a.y + (size_t)m * a.out_cs + ko) = packed;
+                }
+        }
+        return;
+    }
+    // each lane holds 4 consecutive channels of one pixel per accumulator quad: transpose the packed dwords
+    // through LDS so that every pixel's channels leave as 128-bit stores
+#pragma unroll
+    for (int tm = 0; tm < TM; tm++) {
+        const int pl = wm * (TM * 32) + tm * 32 + (lane & 31);
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                uint32_t packed = 0;
+                if (FAST && PLAIN_SAT) {
+                    // clamp range is exactly [0, 255]: two saturating packs replace four clamps and the shifts
+                    int32_t r[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int32_t v = (int32_t)((uint32_t)acc[tn][tm][g * 4 + e] + (HAS_WZP ? (uint32_t)colsum[tm] : 0u));
+                        r[e] = (__mulhi(v, (int)a.q.mult) + a.qadd) >> a.qt;
+                    }
+                    uint32_t p01, p23, b01, b23;
+                    asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p01) : "v"(r[0]), "v"(r[1]));
+                    asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(r[2]), "v"(r[3]));
+                    asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
+                    asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
+                    packed = (b01 & 0xffffu) | (b23 << 16);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const int32_t v = (int32_t)((uint32_t)acc[tn][tm][g * 4 + e] + (HAS_WZP ? (uint32_t)colsum[tm] : 0u));
+                        packed |= (uint32_t)conv_requant<FAST>(a, v) << (8 * e);
+                    }
+                }
+                *reinterpret_cast<uint32_t *>(lds + pl * OSTR + wn * (TN * 32) + tn * 32 + g * 8 + half * 4) = packed;
+            }
+    }
+    __syncthreads();
+    constexpr int LPR = BN / 16;   // lanes per pixel row
+    constexpr int RPP = 256 / LPR; // rows per pass
+    const int c16 = (tid % LPR) * 16;
+    if (bn * BN + c16 < a.out_cs) {
+#pragma unroll
+        for (int r = tid / LPR; r < BM; r += RPP) {
+            const int m = m0 + r;
+            if (m < a.P)
+                *reinterpret_cast<v4i *>(a.y + (size_t)m * a.out_cs + bn * BN + c16)
+                    = *reinterpret_cast<const v4i *>(lds + r * OSTR + c16);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // MFMA implicit-GEMM kernel.  SMALLC: input has channel stride 4 (C <= 4, e.g. the RGB stem); then one
 // 16-byte piece is 4 horizontally adjacent taps x 4 channels and k = (r, s padded to 4, c4).
-template <int WM, int WN, bool HAS_WZP, bool SMALLC>
+template <int BM, int BN, int WM, int WN, bool HAS_WZP, bool SMALLC>
 __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvArgs a)
 {
-    constexpr int BM = WM * 64, BN = WN * 64, NPT = BM / 64, LSTR = 80;
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * BM * LSTR];
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32; // MFMA tiles per wave: pixels x channels
+    constexpr int NPB = BM / 64, NPA = BN / 64;         // 16-byte pieces per thread and slab
+    constexpr int STAGE = (BM + BN) * 64;
+    constexpr int OSTR = BN + 16; // row stride of the output staging tile
+    constexpr int LDS_BYTES = 2 * STAGE > BM * OSTR ? 2 * STAGE : BM * OSTR;
+    static_assert(WM * WN == 4 && TM >= 1 && TN >= 1 && NPB >= 1 && NPA >= 1, "tile shape");
+    __shared__ __attribute__((aligned(16))) uint8_t lds[LDS_BYTES];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave % WM, wn = wave / WM;
@@ -81,12 +212,12 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvArgs a)
         return;
     const int bm = L / a.nbn, bn = L % a.nbn;
 
-    // ---- loader state: this thread fetches piece (tid & 3) of pixels (tid >> 2) + 64 * j ----------
-    int lp_pix[NPT], lp_ih0[NPT], lp_iw0[NPT];
-    bool lp_ok[NPT];
+    // ---- activation loader: this thread fetches piece (tid & 3) of pixels (tid >> 2) + 64 * j -------
+    int lp_pix[NPB], lp_ih0[NPB], lp_iw0[NPB];
+    bool lp_ok[NPB];
     const int ohw = a.OH * a.OW;
 #pragma unroll
-    for (int j = 0; j < NPT; j++) {
+    for (int j = 0; j < NPB; j++) {
         const int m = bm * BM + (tid >> 2) + 64 * j;
         lp_ok[j] = m < a.P;
         const int mm = lp_ok[j] ? m : 0;
@@ -112,10 +243,10 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvArgs a)
     };
     normalise();
 
-    v4i breg[NPT];
+    v4i breg[NPB], areg[NPA];
     auto load_b = [&]() {
 #pragma unroll
-        for (int j = 0; j < NPT; j++) {
+        for (int j = 0; j < NPB; j++) {
             const int ih = lp_ih0[j] + kr;
             const bool row_ok = lp_ok[j] && kr < a.R && (unsigned)ih < (unsigned)a.H;
             v4i v = {(int)a.padword, (int)a.padword, (int)a.padword, (int)a.padword};
@@ -124,124 +255,350 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvArgs a)
                 const int iw = lp_iw0[j] + s0;
                 if (row_ok) {
                     const uint32_t *p = reinterpret_cast<const uint32_t *>(a.x) + (lp_pix[j] + ih * a.W + iw);
+                    if (iw >= 0 && iw + 3 < a.W) { // weights of taps beyond S are "zero": any byte will do
+                        v = reinterpret_cast<const v4i_a4 *>(p)->v;
+                    } else {
 #pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        if (s0 + e < a.S && (unsigned)(iw + e) < (unsigned)a.W)
-                            v[e] = (int)p[e];
+                        for (int e = 0; e < 4; e++)
+                            if ((unsigned)(iw + e) < (unsigned)a.W)
+                                v[e] = (int)p[e];
+                    }
                 }
             } else {
                 const int iw = lp_iw0[j] + ks;
                 if (row_ok && (unsigned)iw < (unsigned)a.W)
                     v = ldg128(a.x + (size_t)(lp_pix[j] + ih * a.W + iw) * a.in_cs + kc);
             }
-            breg[j] = v ^ (int)0x80808080;
+            breg[j] = v;
         }
         kc += 64;
         normalise();
     };
-    auto store_b = [&](uint8_t *buf) {
+    const uint8_t *wsrc = a.wpack + (size_t)bn * BN * 64 + tid * 16;
+    auto load_a = [&](int slab) {
 #pragma unroll
-        for (int j = 0; j < NPT; j++)
-            *reinterpret_cast<v4i *>(buf + ((tid >> 2) + 64 * j) * LSTR + (tid & 3) * 16) = breg[j];
+        for (int j = 0; j < NPA; j++)
+            areg[j] = ldg128(wsrc + (size_t)slab * a.kout_pad * 64 + j * 4096);
+    };
+    // chunk (tid & 3) of row (tid >> 2) + 64 j lands at chunk ^ ((row >> 2) & 3)
+    const int bst = BN * 64 + (tid >> 2) * 64 + (((tid & 3) ^ ((tid >> 4) & 3)) << 4);
+    auto store_ab = [&](uint8_t *stage) {
+#pragma unroll
+        for (int j = 0; j < NPA; j++)
+            *reinterpret_cast<v4i *>(stage + tid * 16 + j * 4096) = areg[j];
+#pragma unroll
+        for (int j = 0; j < NPB; j++)
+            *reinterpret_cast<v4i *>(stage + bst + j * 4096) = breg[j];
     };
 
-    // ---- A fragments: [kout tile][slab][half][lane] x 16 bytes -------------------------------------
-    const int T0 = (bn * BN + wn * 64) >> 5;
-    const uint8_t *wbase = a.wpack + (size_t)lane * 16;
-    auto load_a = [&](v4i(&dst)[2][2], int slab) {
+    // ---- accumulators start at the folded per-channel constant ---------------------------------
+    const int ch0 = bn * BN + wn * (TN * 32); // first channel of this wave
+    v16i acc[TN][TM];
 #pragma unroll
-        for (int tn = 0; tn < 2; tn++)
+    for (int tn = 0; tn < TN; tn++)
 #pragma unroll
-            for (int kk = 0; kk < 2; kk++)
-                dst[kk][tn] = ldg128(wbase + ((((size_t)(T0 + tn) * a.nslab + slab) * 2 + kk) << 10));
-    };
+        for (int g = 0; g < 4; g++) {
+            const v4i bias = *reinterpret_cast<const v4i *>(a.bias2 + ch0 + tn * 32 + g * 8 + (lane >> 5) * 4);
+#pragma unroll
+            for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    acc[tn][tm][g * 4 + e] = bias[e];
+        }
+    int colsum[TM];
+#pragma unroll
+    for (int tm = 0; tm < TM; tm++)
+        colsum[tm] = 0;
 
-    v16i acc[2][2];
-#pragma unroll
-    for (int i = 0; i < 2; i++)
-#pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int e = 0; e < 16; e++)
-                acc[i][j][e] = 0;
-    int colsum[2] = {0, 0};
+    // fragment addresses: row (lane & 31) of a 32-row tile, k bytes [32 kk + 16 (lane >> 5), +16)
+    const int swz = (lane >> 2) & 3, half = lane >> 5;
+    const int foff0 = (lane & 31) * 64 + (((0 + half) ^ swz) << 4);
+    const int foff1 = (lane & 31) * 64 + (((2 + half) ^ swz) << 4);
+    const int arow = wn * (TN * 32) * 64, brow = BN * 64 + wm * (TM * 32) * 64;
 
-    v4i acur[2][2], anext[2][2];
+    load_a(0);
     load_b();
-    load_a(acur, 0);
-    store_b(lds);
+    store_ab(lds);
     __syncthreads();
 
-    const int brow = (wm * 64 + (lane & 31)) * LSTR + (lane >> 5) * 16;
-    int cur = 0;
     for (int i = 0; i < a.nslab; i++) {
         const bool more = i + 1 < a.nslab;
         if (more) {
+            load_a(i + 1);
             load_b();
-            load_a(anext, i + 1);
         }
-        const uint8_t *buf = lds + cur * (BM * LSTR);
+        const uint8_t *buf = lds + (i & 1) * STAGE;
 #pragma unroll
         for (int kk = 0; kk < 2; kk++) {
-            const v4i b0 = *reinterpret_cast<const v4i *>(buf + brow + kk * 32);
-            const v4i b1 = *reinterpret_cast<const v4i *>(buf + brow + 32 * LSTR + kk * 32);
-            acc[0][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(acur[kk][0], b0, acc[0][0], 0, 0, 0);
-            acc[0][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(acur[kk][0], b1, acc[0][1], 0, 0, 0);
-            acc[1][0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(acur[kk][1], b0, acc[1][0], 0, 0, 0);
-            acc[1][1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(acur[kk][1], b1, acc[1][1], 0, 0, 0);
+            const int fo = kk ? foff1 : foff0;
+            v4i af[TN], bf[TM];
+#pragma unroll
+            for (int tn = 0; tn < TN; tn++)
+                af[tn] = *reinterpret_cast<const v4i *>(buf + arow + tn * 2048 + fo);
+#pragma unroll
+            for (int tm = 0; tm < TM; tm++)
+                bf[tm] = *reinterpret_cast<const v4i *>(buf + brow + tm * 2048 + fo) ^ (int)0x80808080;
+#pragma unroll
+            for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+                for (int tm = 0; tm < TM; tm++)
+                    acc[tn][tm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[tn], bf[tm], acc[tn][tm], 0, 0, 0);
             if (HAS_WZP) {
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    colsum[0] = __builtin_amdgcn_sdot4(b0[e], 0x01010101, colsum[0], false);
-                    colsum[1] = __builtin_amdgcn_sdot4(b1[e], 0x01010101, colsum[1], false);
-                }
+                for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        colsum[tm] = __builtin_amdgcn_sdot4(bf[tm][e], 0x01010101, colsum[tm], false);
             }
         }
         if (more)
-            store_b(lds + (cur ^ 1) * (BM * LSTR));
+            store_ab(lds + ((i + 1) & 1) * STAGE);
         __syncthreads();
-#pragma unroll
-        for (int kk = 0; kk < 2; kk++)
-#pragma unroll
-            for (int tn = 0; tn < 2; tn++)
-                acur[kk][tn] = anext[kk][tn];
-        cur ^= 1;
     }
 
     // ---- epilogue ------------------------------------------------------------------------------
     if (HAS_WZP) {
         // a lane's B fragment covers half of the k range of its pixel; lanes l and l^32 share the pixel
-        colsum[0] += __shfl_xor(colsum[0], 32);
-        colsum[1] += __shfl_xor(colsum[1], 32);
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+            colsum[tm] = a.bwz * (colsum[tm] + __shfl_xor(colsum[tm], 32));
     }
+    // the last barrier of the main loop has retired every read of the stages
+    if (a.fastq && a.lo == 0 && a.q.hi == 255)
+        conv_epilogue<BM, BN, WM, WN, HAS_WZP, true, true, TM, TN>(a, acc, colsum, lds, bm, bn, wm, wn);
+    else if (a.fastq)
+        conv_epilogue<BM, BN, WM, WN, HAS_WZP, true, false, TM, TN>(a, acc, colsum, lds, bm, bn, wm, wn);
+    else
+        conv_epilogue<BM, BN, WM, WN, HAS_WZP, false, false, TM, TN>(a, acc, colsum, lds, bm, bn, wm, wn);
+}
+
+// ------------------------------------------------------------------------------------------------
+// The same tile computation with the operands streamed global -> LDS by the load unit itself
+// (global_load_lds_dwordx4: every lane names a 16-byte global source, the wave's 64 pieces land
+// contiguously at the LDS address in M0), NS stages deep.  HBM latency on this chip is of the order of a
+// microsecond, a slab of MFMA work a tenth of that: only several slabs in flight per work-group keep
+// the matrix cores fed.  No VGPR staging, no LDS store instructions.  Out-of-image taps read 16 bytes of
+// the byte izp from `padbuf`, so every lane always issues a load and the counts below are uniform.
+// Synchronisation: vmcnt counts this wave's loads in issue order; after waiting until at most the
+// younger slabs are outstanding, one barrier per slab makes the stage visible to all waves and at the
+// same time retires every read of the stage that is about to be refilled.
+template <int N>
+__device__ static inline void wait_vmcnt()
+{
+    // gfx9 encoding: vmcnt = {imm[15:14], imm[3:0]}, expcnt = imm[6:4], lgkmcnt = imm[11:8] (left at their maxima)
+    __builtin_amdgcn_s_waitcnt((N & 15) | (7 << 4) | (15 << 8) | ((N >> 4) << 14));
+}
+
+typedef const __attribute__((address_space(1))) void *gptr_t;
+typedef __attribute__((address_space(3))) void *lptr_t;
+
+// ALIGNED: in_cs is a multiple of 64, so a slab never straddles two taps; the source addresses then advance by
+// a wave-uniform offset and the bounds tests are redone only when the tap changes.
+template <int BM, int BN, int WM, int WN, int NS, bool HAS_WZP, bool ALIGNED>
+__global__ __launch_bounds__(256) void conv_mfma_dma_kernel(const ConvArgs a)
+{
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int NPB = BM / 64, NPA = BN / 64, LPS = NPA + NPB; // loads per thread and stage
+    constexpr int STAGE = (BM + BN) * 64;
+    constexpr int OSTR = BN + 16;
+    constexpr int LDS_BYTES = NS * STAGE > BM * OSTR ? NS * STAGE : BM * OSTR;
+    static_assert(WM * WN == 4 && TM >= 1 && TN >= 1 && NPB >= 1 && NPA >= 1 && NS >= 2, "tile shape");
+    static_assert((NS - 2) * LPS <= 63, "vmcnt range");
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[LDS_BYTES];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave % WM, wn = wave / WM;
+    const int nblk = a.nbm * a.nbn;
+    const int L = (int)(blockIdx.x % 8) * (int)(gridDim.x / 8) + (int)(blockIdx.x / 8);
+    if (L >= nblk)
+        return;
+    const int bm = L / a.nbn, bn = L % a.nbn;
+
+    // ---- activation source: LDS slot tid (+256 j) = phys chunk (tid & 3) of row (tid >> 2) + 64 j holds the
+    // logical chunk (tid & 3) ^ ((row >> 2) & 3) of that pixel's 64-byte k slab
+    int lp_pix[NPB], lp_ih0[NPB], lp_iw0[NPB];
+    bool lp_ok[NPB];
+    const int ohw = a.OH * a.OW;
 #pragma unroll
-    for (int tm = 0; tm < 2; tm++) {
-        const int m = bm * BM + wm * 64 + tm * 32 + (lane & 31);
-        if (m >= a.P)
-            continue;
-        const int corr = HAS_WZP ? a.bwz * colsum[tm] : 0;
-#pragma unroll
-        for (int tn = 0; tn < 2; tn++) {
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const int ko = bn * BN + wn * 64 + tn * 32 + g * 8 + (lane >> 5) * 4;
-                if (ko >= a.out_cs)
-                    continue;
-                const v4i bias = *reinterpret_cast<const v4i *>(a.bias2 + ko);
-                uint32_t packed = 0;
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const int32_t v = (int32_t)((uint32_t)acc[tn][tm][g * 4 + e] + (uint32_t)bias[e] + (uint32_t)corr);
-                    if (a.acc_out)
-                        a.acc_out[(size_t)m * a.out_cs + ko + e] = v;
-                    int32_t r = requant_acc(v, a.q);
-                    r = r < a.lo ? a.lo : r;
-                    packed |= (uint32_t)r << (8 * e);
-                }
-                *reinterpret_cast<uint32_t *>(a.y + (size_t)m * a.out_cs + ko) = packed;
+    for (int j = 0; j < NPB; j++) {
+        const int m = bm * BM + (tid >> 2) + 64 * j;
+        lp_ok[j] = m < a.P;
+        const int mm = lp_ok[j] ? m : 0;
+        const int n = fast_div(mm, ohw, a.inv_ohw), rem = mm - n * ohw;
+        const int oh = fast_div(rem, a.OW, a.inv_ow), ow = rem - oh * a.OW;
+        lp_ih0[j] = oh * a.stride_h - a.pad_h;
+        lp_iw0[j] = ow * a.stride_w - a.pad_w;
+        lp_pix[j] = n * a.H * a.W;
+    }
+    const int chunk16 = ((tid & 3) ^ ((tid >> 4) & 3)) * 16;
+    int kc = chunk16, kr = 0, ks = 0; // generic mode: this thread's position in k space
+    auto normalise = [&]() {
+        while (kc >= a.rowb) {
+            kc -= a.rowb;
+            if (++ks == a.S) {
+                ks = 0;
+                kr++;
             }
         }
+    };
+    // aligned mode: per-pixel base pointers (possibly outside the tensor for border pixels: never dereferenced
+    // unless the tap is inside the image) + a uniform byte offset of the current (tap, channel slab)
+    const uint8_t *lp_ptr[NPB];
+    bool lp_in[NPB];
+    int tap_r = 0, tap_s = 0, tap_c = 0, tap_off = 0;
+    auto set_tap = [&]() {
+#pragma unroll
+        for (int j = 0; j < NPB; j++)
+            lp_in[j] = lp_ok[j] && (unsigned)(lp_ih0[j] + tap_r) < (unsigned)a.H && (unsigned)(lp_iw0[j] + tap_s) < (unsigned)a.W;
+        tap_off = (tap_r * a.W + tap_s) * a.in_cs;
+    };
+    if (ALIGNED) {
+#pragma unroll
+        for (int j = 0; j < NPB; j++)
+            lp_ptr[j] = a.x + (ptrdiff_t)(lp_pix[j] + lp_ih0[j] * a.W + lp_iw0[j]) * a.in_cs + chunk16;
+        set_tap();
+    } else {
+        normalise();
     }
+    const uint8_t *wsrc = a.wpack + (size_t)bn * BN * 64 + tid * 16;
+    const int wave_off = __builtin_amdgcn_readfirstlane(wave) * 1024;
+    const size_t wslab = (size_t)a.kout_pad * 64;
+
+    int st_issue = 0; // stage the next issue() fills; stages are used round-robin
+    auto issue = [&](int slab) {
+        uint8_t *st = lds + st_issue * STAGE + wave_off;
+        st_issue = st_issue + 1 == NS ? 0 : st_issue + 1;
+        const uint8_t *ws = wsrc + slab * wslab;
+#pragma unroll
+        for (int j = 0; j < NPA; j++)
+            __builtin_amdgcn_global_load_lds((gptr_t)(ws + j * 4096), (lptr_t)(st + j * 4096), 16, 0, 0);
+        if (ALIGNED) {
+            const int off = tap_off + tap_c;
+#pragma unroll
+            for (int j = 0; j < NPB; j++) {
+                const uint8_t *src = lp_in[j] ? lp_ptr[j] + off : a.padbuf;
+                __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(st + BN * 64 + j * 4096), 16, 0, 0);
+            }
+            tap_c += 64;
+            if (tap_c == a.in_cs) {
+                tap_c = 0;
+                if (++tap_s == a.S) {
+                    tap_s = 0;
+                    ++tap_r;
+                }
+                set_tap();
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < NPB; j++) {
+                const int ih = lp_ih0[j] + kr, iw = lp_iw0[j] + ks;
+                const bool ok = lp_ok[j] && kr < a.R && (unsigned)ih < (unsigned)a.H && (unsigned)iw < (unsigned)a.W;
+                const uint8_t *src = ok ? a.x + (size_t)(lp_pix[j] + ih * a.W + iw) * a.in_cs + kc : a.padbuf;
+                __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(st + BN * 64 + j * 4096), 16, 0, 0);
+            }
+            kc += 64;
+            normalise();
+        }
+    };
+
+    const int swz = (lane >> 2) & 3, half = lane >> 5;
+    const int foff0 = (lane & 31) * 64 + (((0 + half) ^ swz) << 4);
+    const int foff1 = (lane & 31) * 64 + (((2 + half) ^ swz) << 4);
+    const int arow = wn * (TN * 32) * 64, brow = BN * 64 + wm * (TM * 32) * 64;
+
+    // first the stage loads, then the (ordinary) loads of the folded bias: the bias loads are YOUNGER than the
+    // first NS-1 slabs, which makes the very first wait below conservative (it also waits for slabs 1..NS-2) and
+    // every later one exact; in exchange the bias latency overlaps with the activations' on their way from HBM
+    for (int s = 0; s < NS - 1 && s < a.nslab; s++)
+        issue(s);
+
+    const int ch0 = bn * BN + wn * (TN * 32);
+    v16i acc[TN][TM];
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const v4i bias = *reinterpret_cast<const v4i *>(a.bias2 + ch0 + tn * 32 + g * 8 + (lane >> 5) * 4);
+#pragma unroll
+            for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    acc[tn][tm][g * 4 + e] = bias[e];
+        }
+    int colsum[TM];
+#pragma unroll
+    for (int tm = 0; tm < TM; tm++)
+        colsum[tm] = 0;
+
+
+    // Fragment reads run one k-step (32 bytes of k) ahead of the MFMAs that consume them, so the LDS latency
+    // hides behind the matrix pipe.  make_ready(i) = slab i has landed for every wave, and the stage that
+    // slab i+NS-1 will occupy has been read for the last time by every wave.
+    int st_comp = 0;
+    auto make_ready = [&](int i) {
+        if (i + NS - 2 <= a.nslab - 1)
+            wait_vmcnt<(NS - 2) * LPS>(); // slabs i+1 .. i+NS-2 may still be in flight
+        else
+            wait_vmcnt<0>();
+        __builtin_amdgcn_s_barrier();
+        if (i + NS - 1 < a.nslab)
+            issue(i + NS - 1);
+    };
+    auto read_frags = [&](v4i(&af)[TN], v4i(&bf)[TM], const uint8_t *buf, int fo) {
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++)
+            af[tn] = *reinterpret_cast<const v4i *>(buf + arow + tn * 2048 + fo);
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+            bf[tm] = *reinterpret_cast<const v4i *>(buf + brow + tm * 2048 + fo);
+    };
+    auto multiply = [&](v4i(&af)[TN], v4i(&bf)[TM]) {
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+            bf[tm] ^= (int)0x80808080;
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+            for (int tm = 0; tm < TM; tm++)
+                acc[tn][tm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[tn], bf[tm], acc[tn][tm], 0, 0, 0);
+        if (HAS_WZP) {
+#pragma unroll
+            for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    colsum[tm] = __builtin_amdgcn_sdot4(bf[tm][e], 0x01010101, colsum[tm], false);
+        }
+    };
+
+    v4i af0[TN], bf0[TM], af1[TN], bf1[TM];
+    make_ready(0);
+    read_frags(af0, bf0, lds, foff0);
+    for (int i = 0; i + 1 < a.nslab; i++) { // the last slab is peeled off: no conditional reads inside the loop
+        const uint8_t *buf = lds + st_comp * STAGE;
+        st_comp = st_comp + 1 == NS ? 0 : st_comp + 1;
+        read_frags(af1, bf1, buf, foff1);
+        multiply(af0, bf0);
+        make_ready(i + 1);
+        read_frags(af0, bf0, lds + st_comp * STAGE, foff0);
+        multiply(af1, bf1);
+    }
+    read_frags(af1, bf1, lds + st_comp * STAGE, foff1);
+    multiply(af0, bf0);
+    multiply(af1, bf1);
+
+    // ---- epilogue -----------------------------------------------------------------------------------------
+    if (HAS_WZP) {
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+            colsum[tm] = a.bwz * (colsum[tm] + __shfl_xor(colsum[tm], 32));
+    }
+    __syncthreads(); // every wave has finished reading the last stage; no load is in flight any more
+    if (a.fastq && a.lo == 0 && a.q.hi == 255)
+        conv_epilogue<BM, BN, WM, WN, HAS_WZP, true, true, TM, TN>(a, acc, colsum, lds, bm, bn, wm, wn);
+    else if (a.fastq)
+        conv_epilogue<BM, BN, WM, WN, HAS_WZP, true, false, TM, TN>(a, acc, colsum, lds, bm, bn, wm, wn);
+    else
+        conv_epilogue<BM, BN, WM, WN, HAS_WZP, false, false, TM, TN>(a, acc, colsum, lds, bm, bn, wm, wn);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -334,11 +691,18 @@ using namespace hipq;
 
 enum ConvVariant { kMfma, kMfmaSmallC, kDepthwise, kDirect };
 
+// Tile shapes of the MFMA kernel: BM pixels x BN channels per work-group, waves arranged WM x WN.
+struct TileShape {
+    int bm, bn;
+};
+static const TileShape kTiles[] = {{128, 128}, {256, 64}, {128, 64}, {64, 128}, {64, 64}};
+constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
+
 struct hipq_conv2d_plan {
     hipq_conv2d_desc d;
     ConvArgs args;
     ConvVariant variant;
-    int wm, wn;
+    int tile; // index into kTiles
     bool has_wzp;
     void *d_w = nullptr, *d_bias = nullptr;
     std::string name;
@@ -348,6 +712,21 @@ static int conv_out_dim(int in, int pad, int k, int stride)
 {
     // art/src/op.c:549-555 (unsigned arithmetic, hole == 1)
     return (int)(((uint32_t)in + 2u * (uint32_t)pad - (uint32_t)k) / (uint32_t)stride + 1u);
+}
+
+// Largest tile that still gives every CU a few work-groups to overlap (two waves per SIMD hide the
+// global-load latency of one another); HIPQ_CONV_TILE=<index into kTiles> overrides for tuning runs.
+static int choose_tile(long long P, int out_cs)
+{
+    if (const char *e = getenv("HIPQ_CONV_TILE")) {
+        const int t = atoi(e);
+        if (t >= 0 && t < kNumTiles)
+            return t;
+    }
+    auto count = [&](int t) { return ((P + kTiles[t].bm - 1) / kTiles[t].bm) * ((out_cs + kTiles[t].bn - 1) / kTiles[t].bn); };
+    if (out_cs <= 64)
+        return count(2) >= 1024 ? 2 : 4; // 128x64, or 64x64 for small images
+    return count(0) >= 200 ? 0 : 3;      // 128x128, or 64x128 when that leaves most CUs idle
 }
 
 extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t *w, const int32_t *bias,
@@ -391,6 +770,11 @@ extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t
         return fail("conv: requantisation shift %d outside 1..62 (scale %g)", a.q.shift,
                     (double)(d.ialpha * d.walpha / d.oalpha));
     }
+    a.fastq = a.q.shift >= 33 && a.q.shift <= 52;
+    a.qt = a.fastq ? a.q.shift - 32 : 1;
+    a.qadd = a.fastq ? (1 << (a.qt - 1)) + (d.ozp << a.qt) : 0;
+    a.inv_ohw = 1.0 / ((double)a.OH * a.OW);
+    a.inv_ow = 1.0 / (double)a.OW;
     a.padword = 0x01010101u * (uint32_t)d.izp;
     const int aoff = 128 - d.izp, boff = 128 - d.wzp;
     a.bwz = boff;
@@ -398,48 +782,49 @@ extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t
     const int cg = d.C / d.group;
     std::vector<uint8_t> wbuf;
     std::vector<int32_t> bbuf;
+    size_t pad_off = 0;
     if (d.group == 1 && (d.in_cs % 16 == 0 || d.in_cs == 4)) {
         const bool smallc = d.in_cs == 4;
         p->variant = smallc ? kMfmaSmallC : kMfma;
-        p->wn = d.K <= 64 ? 1 : 2;
-        p->wm = 4 / p->wn;
-        const int BM = p->wm * 64, BN = p->wn * 64;
+        p->tile = choose_tile(a.P, d.out_cs);
+        const int BM = kTiles[p->tile].bm, BN = kTiles[p->tile].bn;
         a.nbm = (a.P + BM - 1) / BM;
         a.nbn = (d.out_cs + BN - 1) / BN;
         a.rowb = smallc ? 4 * ((d.S + 3) / 4 * 4) : d.in_cs;
         a.Ktot = smallc ? d.R * a.rowb : d.R * d.S * d.in_cs;
         a.nslab = (a.Ktot + 63) / 64;
+        a.kout_pad = (d.K + 127) / 128 * 128;
         p->has_wzp = boff != 0;
-        const int NT = a.nbn * BN / 32;
-        wbuf.assign((size_t)NT * a.nslab * 2048, 0);
-        bbuf.assign((size_t)NT * 32, 0);
-        for (int T = 0; T < NT; T++)
-            for (int l = 0; l < 32; l++) {
-                const int ko = T * 32 + l;
-                if (ko >= d.K)
-                    continue; // rows of pad output channels stay zero; their outputs are don't-care
-                long long wsum = 0;
-                for (int kp = 0; kp < a.nslab * 64; kp++) {
-                    int ws = -boff; // a padding slot: (ws + b) == 0
-                    if (kp < a.Ktot) {
-                        int r, s, c;
-                        if (smallc) {
-                            r = kp / a.rowb, s = (kp % a.rowb) / 4, c = kp % 4;
-                        } else {
-                            const int tap = kp / d.in_cs;
-                            c = kp % d.in_cs, r = tap / d.S, s = tap % d.S;
-                        }
-                        if (s < d.S && c < d.C)
-                            ws = (int)w[(((size_t)ko * d.C + c) * d.R + r) * d.S + s] - 128;
+        // weights: [slab][kout_pad][64 bytes]; chunk c of row ko is stored at chunk c ^ ((ko >> 2) & 3),
+        // the order the kernel keeps in LDS.  Rows of pad output channels stay zero (their outputs are
+        // don't-care bytes in the pad channels of y).
+        wbuf.assign((size_t)a.nslab * a.kout_pad * 64, 0);
+        bbuf.assign((size_t)a.kout_pad, 0);
+        for (int ko = 0; ko < d.K; ko++) {
+            long long wsum = 0;
+            for (int kp = 0; kp < a.nslab * 64; kp++) {
+                int ws = -boff; // a padding slot: (ws + b) == 0
+                if (kp < a.Ktot) {
+                    int r, s, c;
+                    if (smallc) {
+                        r = kp / a.rowb, s = (kp % a.rowb) / 4, c = kp % 4;
+                    } else {
+                        const int tap = kp / d.in_cs;
+                        c = kp % d.in_cs, r = tap / d.S, s = tap % d.S;
                     }
-                    wsum += ws;
-                    const int slab = kp >> 6, kk = (kp >> 5) & 1, half = (kp >> 4) & 1, i = kp & 15;
-                    wbuf[((((size_t)T * a.nslab + slab) * 2 + kk) * 64 + half * 32 + l) * 16 + i] = (uint8_t)(int8_t)ws;
+                    if (s < d.S && c < d.C)
+                        ws = (int)w[(((size_t)ko * d.C + c) * d.R + r) * d.S + s] - 128;
                 }
-                const long long c0 = (bias ? (long long)bias[ko] : 0) + (long long)aoff * wsum
-                    + (long long)a.nslab * 64 * aoff * boff;
-                bbuf[ko] = (int32_t)(uint32_t)(unsigned long long)c0;
+                wsum += ws;
+                const int slab = kp >> 6, chunk = ((kp >> 4) & 3) ^ ((ko >> 2) & 3);
+                wbuf[((size_t)slab * a.kout_pad + ko) * 64 + chunk * 16 + (kp & 15)] = (uint8_t)(int8_t)ws;
             }
+            const long long c0 = (bias ? (long long)bias[ko] : 0) + (long long)aoff * wsum
+                + (long long)a.nslab * 64 * aoff * boff;
+            bbuf[ko] = (int32_t)(uint32_t)(unsigned long long)c0;
+        }
+        pad_off = wbuf.size();
+        wbuf.resize(pad_off + 64, (uint8_t)d.izp); // source of out-of-image taps
         char nm[96];
         snprintf(nm, sizeof nm, "conv_mfma_i8_%dx%d%s%s", BM, BN, smallc ? "_c4" : "", p->has_wzp ? "_wzp" : "");
         p->name = nm;
@@ -476,6 +861,7 @@ extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t
     }
     a.wpack = static_cast<const uint8_t *>(p->d_w);
     a.bias2 = static_cast<const int32_t *>(p->d_bias);
+    a.padbuf = a.wpack + pad_off;
     *plan_out = p;
     return 0;
 }
@@ -493,22 +879,41 @@ extern "C" void hipq_conv2d_plan_destroy(hipq_conv2d_plan *p)
 
 extern "C" const char *hipq_conv2d_plan_kernel(const hipq_conv2d_plan *p) { return p ? p->name.c_str() : ""; }
 
-template <int WM, int WN>
+template <int BM, int BN, int WM, int WN, int NS>
 static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_t st)
 {
     const int nblk = a.nbm * a.nbn;
     const dim3 grid((nblk + 7) / 8 * 8), block(256);
     if (p->variant == kMfmaSmallC) {
         if (p->has_wzp)
-            hipLaunchKernelGGL((conv_mfma_kernel<WM, WN, true, true>), grid, block, 0, st, a);
+            hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, true, true>), grid, block, 0, st, a);
         else
-            hipLaunchKernelGGL((conv_mfma_kernel<WM, WN, false, true>), grid, block, 0, st, a);
-    } else {
-        if (p->has_wzp)
-            hipLaunchKernelGGL((conv_mfma_kernel<WM, WN, true, false>), grid, block, 0, st, a);
-        else
-            hipLaunchKernelGGL((conv_mfma_kernel<WM, WN, false, false>), grid, block, 0, st, a);
+            hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, false, true>), grid, block, 0, st, a);
+        return;
     }
+    const bool aligned = a.in_cs % 64 == 0;
+    // few slabs: two stages are all the pipeline can use, and the smaller LDS footprint lets more work-groups
+    // share a CU, which is what hides the latency of such short kernels
+    const bool shallow = a.nslab <= 2;
+#define HIPQ_LAUNCH_DMA(NSV, WZ, AL) \
+    hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, NSV, WZ, AL>), grid, block, 0, st, a)
+    if (p->has_wzp) { // rare (asymmetric weights): generic addressing only
+        if (shallow)
+            HIPQ_LAUNCH_DMA(2, true, false);
+        else
+            HIPQ_LAUNCH_DMA(NS, true, false);
+    } else if (aligned) {
+        if (shallow)
+            HIPQ_LAUNCH_DMA(2, false, true);
+        else
+            HIPQ_LAUNCH_DMA(NS, false, true);
+    } else {
+        if (shallow)
+            HIPQ_LAUNCH_DMA(2, false, false);
+        else
+            HIPQ_LAUNCH_DMA(NS, false, false);
+    }
+#undef HIPQ_LAUNCH_DMA
 }
 
 extern "C" int hipq_conv2d_run(const hipq_conv2d_plan *p, const void *x, void *y, int32_t *acc_out, void *stream)
@@ -523,10 +928,13 @@ extern "C" int hipq_conv2d_run(const hipq_conv2d_plan *p, const void *x, void *y
     switch (p->variant) {
     case kMfma:
     case kMfmaSmallC:
-        if (p->wn == 1)
-            launch_mfma<4, 1>(p, a, st);
-        else
-            launch_mfma<2, 2>(p, a, st);
+        switch (p->tile) {
+        case 0: launch_mfma<128, 128, 2, 2, 4>(p, a, st); break; // 4 x 16 KiB
+        case 1: launch_mfma<256, 64, 4, 1, 3>(p, a, st); break;  // 3 x 20 KiB
+        case 2: launch_mfma<128, 64, 2, 2, 4>(p, a, st); break;  // 4 x 12 KiB
+        case 3: launch_mfma<64, 128, 1, 4, 4>(p, a, st); break;
+        default: launch_mfma<64, 64, 2, 2, 4>(p, a, st); break;  // 4 x 8 KiB
+        }
         break;
     case kDepthwise: {
         const size_t total = (size_t)a.P * (a.in_cs / 4);
