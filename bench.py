@@ -98,6 +98,7 @@ def main():
     ap.add_argument("--kernel-reps", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--no-fuse", action="store_true", help="run every residual add as its own kernel")
     ap.add_argument("--layers", action="store_true", help="print a per-layer table to stderr")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -116,7 +117,7 @@ def main():
                 "fc": lambda n: cases.single_fc(M=n)}
     build = builders[args.workload]
     case = build(args.batch)
-    ex = HipqExecutor(case)
+    ex = HipqExecutor(case, fuse_add=not args.no_fuse)
     rng = np.random.default_rng(0)
     if case.input.dtype == "f32":
         x = (rng.standard_normal(case.input.shape) * 1.2).astype(np.float32)
@@ -175,7 +176,7 @@ def main():
            "ms_per_step": round(ms, 4), "wall_ms_per_step": round(wall_ms, 4), "higher_is_better": True,
            "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
            "config": {"workload": case.name, "batch": args.batch, "input": list(case.input.shape),
-                      "operators": len(case.nodes), "graph_replay": not args.no_graph,
+                      "operators": len(case.nodes), "graph_replay": not args.no_graph, "fused_residual_adds": len(ex.fused),
                       "conv_fc_gop_per_step": round(case.conv_ops() / 1e9, 2)},
            "conv_tops_whole_step": round(case.conv_ops() / (ms * 1e-3) / 1e12, 2),
            "roofline": roof, "kernel_families": families}

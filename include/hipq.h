@@ -95,6 +95,18 @@ const char *hipq_conv2d_plan_kernel(const hipq_conv2d_plan *plan);
 int hipq_conv2d_run(const hipq_conv2d_plan *plan, const void *x, void *y, int32_t *acc_out,
                     void *stream);
 
+/*
+ * Convolution with the residual add fused into its epilogue: y = add(conv(x), residual), bit-identical to
+ * hipq_conv2d_run followed by hipq_add_u8 on the stored bytes (op_conv_2d_u8xu8_run, then op_quant_add_run —
+ * src/op/add.c:83-148), but the convolution's own uint8 result never travels to memory.  `residual` has the
+ * layout and geometry of y.  The add's inputs are (conv, residual), or (residual, conv) when
+ * residual_is_input0 != 0; the convolution's output scale and zero point are the plan's oalpha / ozp, the
+ * residual's are res_alpha / res_zp; oalpha / ozp / obits describe the sum.  Only plans that run an MFMA
+ * kernel support it (others fail with an error: run the two operators separately).
+ */
+int hipq_conv2d_run_add(const hipq_conv2d_plan *plan, const void *x, const void *residual, int residual_is_input0,
+                        float res_alpha, int res_zp, float oalpha, int ozp, int obits, void *y, void *stream);
+
 /* ---- inner product: op_quant_ip_u8xu8_run — src/op/ip.cpp:133-209.
  * Expressed as a 1x1 convolution over M "pixels": desc {N=M, C=Kdim, H=W=1, K=Nout, R=S=1}.
  * When the reference's input is [M, C, H, W] with H*W > 1, pass the weights re-ordered from

@@ -66,4 +66,63 @@ __host__ __device__ static inline int32_t requant_acc(int32_t acc, const Requant
 
 static inline int valid_shift(int s) { return s >= 1 && s <= 62; }
 
+// ---- quantized two-input add (op_quant_add_run, art/modules/quant/src/op/add.c:83-148) ------------------
+// Shared by the stand-alone add kernel and by the convolution epilogue that fuses a residual add.
+//   t = rrn((int32)(m0*(x0-z0)), s0) + rrn((int32)(m1*(x1-z1)), s1);   y = sat(rrn(t, sh) + oz)
+// The operation is symmetric in its inputs (the reference's swap by scale only orders them).
+// Fast form, valid when every shift is small enough for 32-bit arithmetic (`fast`): with
+// c = 2^(s-1) - z*m the two terms are (x*m + c) >> s (|m*(x-z)| < 2^30, so nothing wraps), and with
+// cadd = 2^(sh-1) + oz*2^sh the result is (t + cadd) >> sh before the clamp.
+struct AddParams {
+    uint32_t m0, m1;    // 22-bit multipliers (get_quant_scale(alpha_i / oalpha, 23))
+    int32_t s0, s1, sh; // s0 - sh, s1 - sh, sh
+    int32_t z0, z1, oz, hi;
+    int32_t c0, c1, cadd;
+    int32_t fast;
+};
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ static inline uint32_t add_one_generic(uint32_t x0, uint32_t x1, const AddParams &p)
+{
+    const int32_t i0 = (int32_t)x0 - p.z0, i1 = (int32_t)x1 - p.z1;
+    const int32_t p0 = (int32_t)(p.m0 * (uint32_t)i0), p1 = (int32_t)(p.m1 * (uint32_t)i1);
+    const int32_t t = (int32_t)(rshift_rn(p0, p.s0) + rshift_rn(p1, p.s1));
+    return (uint32_t)sat_hi((int32_t)(rshift_rn(t, p.sh) + p.oz), p.hi);
+}
+
+template <bool FAST>
+__device__ static inline uint32_t add_dword(uint32_t a, uint32_t b, const AddParams &p)
+{
+    uint32_t o = 0;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const uint32_t x0 = (a >> (8 * e)) & 255, x1 = (b >> (8 * e)) & 255;
+        uint32_t r;
+        if (FAST) {
+            // operands fit 24 bits: v_mad_i32_i24 is a full-rate instruction
+            const int32_t t0 = __mul24((int)x0, (int)p.m0) + p.c0, t1 = __mul24((int)x1, (int)p.m1) + p.c1;
+            const int32_t v = (((t0 >> p.s0) + (t1 >> p.s1)) + p.cadd) >> p.sh;
+            r = (uint32_t)(v > p.hi ? p.hi : (v < 0 ? 0 : v));
+        } else {
+            r = add_one_generic(x0, x1, p);
+        }
+        o |= r << (8 * e);
+    }
+    return o;
+}
+
+template <bool FAST>
+__device__ static inline u32x4 add_16(u32x4 a, u32x4 b, const AddParams &p)
+{
+    u32x4 y;
+#pragma unroll
+    for (int d = 0; d < 4; d++)
+        y[d] = add_dword<FAST>(a[d], b[d], p);
+    return y;
+}
+
+// Fills *p from the operator's settings; returns false if a scale is outside the fixed-point range.
+bool make_add_params(float ia0, int iz0, float ia1, int iz1, float oa, int oz, int obits, AddParams *p);
+
 } // namespace hipq

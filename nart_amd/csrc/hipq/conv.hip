@@ -38,6 +38,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <string>
+#include <type_traits>
 #include <vector>
 
 #include "common.h"
@@ -73,6 +74,9 @@ struct ConvArgs {
     int qt;    // shift - 32
     int qadd;  // 2^(qt-1) + zp * 2^qt
     double inv_ohw, inv_ow; // 1 / (OH*OW), 1 / OW
+    const uint8_t *res; // fused residual add: the other operand (same layout as y), or nullptr
+    int res_first;      // 1: the residual is input 0 of the add, the convolution's output input 1
+    AddParams addq;
 };
 
 // x / d for 0 <= x < 2^31, d >= 1, inv = 1.0 / d: the double product is within one of the quotient, one
@@ -134,6 +138,10 @@ __device__ static inline void conv_epilogue(const ConvArgs &a, v16i (&acc)[TN][T
                             a.acc_out[(size_t)m * a.out_cs + ko + e] = v;
                         packed |= (uint32_t)conv_requant<FAST>(a, v) << (8 * e);
                     }
+                    if (a.res) {
+                        const uint32_t rv = *reinterpret_cast<const uint32_t *>(a.res + (size_t)m * a.out_cs + ko);
+                        packed = a.res_first ? add_dword<false>(rv, packed, a.addq) : add_dword<false>(packed, rv, a.addq);
+                    }
                     *reinterpret_cast<uint32_t *>(a.y + (size_t)m * a.out_cs + ko) = packed;
                 }
         }
@@ -177,7 +185,9 @@ __device__ static inline void conv_epilogue(const ConvArgs &a, v16i (&acc)[TN][T
     constexpr int LPR = BN / 16;   // lanes per pixel row
     constexpr int RPP = 256 / LPR; // rows per pass
     const int c16 = (tid % LPR) * 16;
-    if (bn * BN + c16 < a.out_cs) {
+    if (bn * BN + c16 >= a.out_cs)
+        return;
+    if (a.res == nullptr) {
 #pragma unroll
         for (int r = tid / LPR; r < BM; r += RPP) {
             const int m = m0 + r;
@@ -185,7 +195,27 @@ __device__ static inline void conv_epilogue(const ConvArgs &a, v16i (&acc)[TN][T
                 *reinterpret_cast<v4i *>(a.y + (size_t)m * a.out_cs + bn * BN + c16)
                     = *reinterpret_cast<const v4i *>(lds + r * OSTR + c16);
         }
+        return;
     }
+    // fused residual add (the convolution's own uint8 result exists only in LDS): y = add(conv, residual),
+    // exactly what a separate add kernel would compute from the stored bytes
+    auto fused = [&](auto fast) {
+        constexpr bool AF = decltype(fast)::value;
+#pragma unroll
+        for (int r = tid / LPR; r < BM; r += RPP) {
+            const int m = m0 + r;
+            if (m >= a.P)
+                continue;
+            const size_t off = (size_t)m * a.out_cs + bn * BN + c16;
+            const u32x4 cv = *reinterpret_cast<const u32x4 *>(lds + r * OSTR + c16);
+            const u32x4 rv = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(a.res + off));
+            *reinterpret_cast<u32x4 *>(a.y + off) = a.res_first ? add_16<AF>(rv, cv, a.addq) : add_16<AF>(cv, rv, a.addq);
+        }
+    };
+    if (a.addq.fast)
+        fused(std::true_type{});
+    else
+        fused(std::false_type{});
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -916,6 +946,8 @@ static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_
 #undef HIPQ_LAUNCH_DMA
 }
 
+static int run_conv(const hipq_conv2d_plan *p, ConvArgs &a, hipStream_t st);
+
 extern "C" int hipq_conv2d_run(const hipq_conv2d_plan *p, const void *x, void *y, int32_t *acc_out, void *stream)
 {
     clear_error();
@@ -924,7 +956,32 @@ extern "C" int hipq_conv2d_run(const hipq_conv2d_plan *p, const void *x, void *y
     a.x = static_cast<const uint8_t *>(x);
     a.y = static_cast<uint8_t *>(y);
     a.acc_out = acc_out;
-    hipStream_t st = static_cast<hipStream_t>(stream);
+    return run_conv(p, a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int hipq_conv2d_run_add(const hipq_conv2d_plan *p, const void *x, const void *residual, int residual_is_input0,
+                                   float res_alpha, int res_zp, float oalpha, int ozp, int obits, void *y, void *stream)
+{
+    clear_error();
+    HIPQ_REQUIRE(p && x && y && residual, "hipq_conv2d_run_add: null argument");
+    HIPQ_REQUIRE(p->variant == kMfma || p->variant == kMfmaSmallC,
+                 "hipq_conv2d_run_add: only the MFMA convolution kernels fuse the add (this plan runs %s)", p->name.c_str());
+    HIPQ_REQUIRE(res_zp >= 0 && res_zp <= 255 && ozp >= 0 && ozp <= 255 && obits >= 1 && obits <= 8,
+                 "hipq_conv2d_run_add: zero points must be in 0..255, obits in 1..8");
+    ConvArgs a = p->args;
+    a.x = static_cast<const uint8_t *>(x);
+    a.y = static_cast<uint8_t *>(y);
+    a.res = static_cast<const uint8_t *>(residual);
+    a.res_first = residual_is_input0 ? 1 : 0;
+    const bool ok = residual_is_input0
+        ? make_add_params(res_alpha, res_zp, p->d.oalpha, p->d.ozp, oalpha, ozp, obits, &a.addq)
+        : make_add_params(p->d.oalpha, p->d.ozp, res_alpha, res_zp, oalpha, ozp, obits, &a.addq);
+    HIPQ_REQUIRE(ok, "hipq_conv2d_run_add: scales out of the fixed-point range");
+    return run_conv(p, a, static_cast<hipStream_t>(stream));
+}
+
+static int run_conv(const hipq_conv2d_plan *p, ConvArgs &a, hipStream_t st)
+{
     switch (p->variant) {
     case kMfma:
     case kMfmaSmallC:

@@ -10,51 +10,32 @@
 
 namespace hipq {
 
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
-
 static inline unsigned grid_for(size_t work_items, int per_block = 256)
 {
     const size_t b = (work_items + per_block - 1) / per_block;
     return (unsigned)std::min<size_t>(std::max<size_t>(b, 1), 256 * 16);
 }
 
-// ---- add (add.c:83-148) -----------------------------------------------------------------------
+// ---- add (add.c:83-148); arithmetic in common.h ------------------------------------------------
 struct AddArgs {
-    const uint8_t *a, *b; // already ordered so that alpha(a) <= alpha(b)
+    const uint8_t *a, *b;
     uint8_t *y;
     size_t count;
-    uint32_t m0, m1;
-    int s0, s1, sh; // s0 - sh, s1 - sh, sh
-    int z0, z1, oz, hi;
+    AddParams q;
 };
 
-__device__ static inline uint32_t add_one(uint32_t x0, uint32_t x1, const AddArgs &p)
-{
-    const int32_t i0 = (int32_t)x0 - p.z0, i1 = (int32_t)x1 - p.z1;
-    const int32_t p0 = (int32_t)(p.m0 * (uint32_t)i0), p1 = (int32_t)(p.m1 * (uint32_t)i1);
-    const int32_t t = (int32_t)(rshift_rn(p0, p.s0) + rshift_rn(p1, p.s1));
-    return (uint32_t)sat_hi((int32_t)(rshift_rn(t, p.sh) + p.oz), p.hi);
-}
-
+template <bool FAST>
 __global__ __launch_bounds__(256) void add_u8_kernel(const AddArgs p)
 {
     const size_t nvec = p.count / 16;
     const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nthr = (size_t)gridDim.x * blockDim.x;
     for (size_t i = tid; i < nvec; i += nthr) {
-        const u32x4 va = reinterpret_cast<const u32x4 *>(p.a)[i], vb = reinterpret_cast<const u32x4 *>(p.b)[i];
-        u32x4 vy;
-#pragma unroll
-        for (int d = 0; d < 4; d++) {
-            uint32_t o = 0;
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-                o |= add_one((va[d] >> (8 * e)) & 255, (vb[d] >> (8 * e)) & 255, p) << (8 * e);
-            vy[d] = o;
-        }
-        reinterpret_cast<u32x4 *>(p.y)[i] = vy;
+        const u32x4 va = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p.a) + i);
+        const u32x4 vb = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p.b) + i);
+        reinterpret_cast<u32x4 *>(p.y)[i] = add_16<FAST>(va, vb, p.q);
     }
     for (size_t i = nvec * 16 + tid; i < p.count; i += nthr)
-        p.y[i] = (uint8_t)add_one(p.a[i], p.b[i], p);
+        p.y[i] = (uint8_t)add_one_generic(p.a[i], p.b[i], p.q);
 }
 
 // ---- n-ary eltwise (eltwise.c:137-271) ---------------------------------------------------------
@@ -342,22 +323,16 @@ extern "C" int hipq_add_u8(const void *a, const void *b, void *y, size_t count, 
     HIPQ_REQUIRE(aligned16(a) && aligned16(b) && aligned16(y), "hipq_add_u8: buffers must be 16-byte aligned");
     if (count == 0)
         return 0;
-    if (ia0 > ia1) { // add.c:105-118
-        std::swap(ia0, ia1);
-        std::swap(iz0, iz1);
-        std::swap(a, b);
-    }
     AddArgs p;
-    int s0, s1;
-    hipq_quant_scale(ia0 / oa, 23, &p.m0, &s0);
-    hipq_quant_scale(ia1 / oa, 23, &p.m1, &s1);
-    p.sh = std::min(s0, s1) - 1;
-    p.s0 = s0 - p.sh, p.s1 = s1 - p.sh;
-    HIPQ_REQUIRE(valid_shift(p.sh) && valid_shift(p.s0) && valid_shift(p.s1),
-                 "hipq_add_u8: scales out of the fixed-point range (shifts %d, %d)", s0, s1);
+    HIPQ_REQUIRE(make_add_params(ia0, iz0, ia1, iz1, oa, oz, obits, &p.q),
+                 "hipq_add_u8: scales out of the fixed-point range");
     p.a = static_cast<const uint8_t *>(a), p.b = static_cast<const uint8_t *>(b), p.y = static_cast<uint8_t *>(y);
-    p.count = count, p.z0 = iz0, p.z1 = iz1, p.oz = oz, p.hi = (1 << obits) - 1;
-    hipLaunchKernelGGL(add_u8_kernel, dim3(grid_for(count / 16)), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+    p.count = count;
+    const dim3 grid(grid_for(count / 16)), block(256);
+    if (p.q.fast)
+        hipLaunchKernelGGL(add_u8_kernel<true>, grid, block, 0, static_cast<hipStream_t>(stream), p);
+    else
+        hipLaunchKernelGGL(add_u8_kernel<false>, grid, block, 0, static_cast<hipStream_t>(stream), p);
     return launch_status("add_u8_kernel");
 }
 

@@ -3,7 +3,9 @@
 #include <cstdarg>
 #include <cstdio>
 
-#include "hipq.h"
+#include <algorithm>
+
+#include "common.h"
 
 namespace hipq {
 
@@ -46,6 +48,26 @@ extern "C" void hipq_quant_scale(float x, int bits, uint32_t *mult, int *shift)
     }
     *mult = (uint32_t)(x * (float)(1ll << (bits - 1)));
     *shift = s + bits - 1;
+}
+
+bool hipq::make_add_params(float ia0, int iz0, float ia1, int iz1, float oa, int oz, int obits, AddParams *p)
+{
+    int s0, s1;
+    hipq_quant_scale(ia0 / oa, 23, &p->m0, &s0); // add.c:119-124
+    hipq_quant_scale(ia1 / oa, 23, &p->m1, &s1);
+    p->sh = std::min(s0, s1) - 1;
+    p->s0 = s0 - p->sh, p->s1 = s1 - p->sh;
+    p->z0 = iz0, p->z1 = iz1, p->oz = oz, p->hi = (1 << obits) - 1;
+    if (!valid_shift(p->sh) || !valid_shift(p->s0) || !valid_shift(p->s1))
+        return false;
+    p->fast = p->sh <= 22 && p->s0 <= 30 && p->s1 <= 30 && p->m0 < (1u << 23) && p->m1 < (1u << 23);
+    p->c0 = p->c1 = p->cadd = 0;
+    if (p->fast) {
+        p->c0 = (1 << (p->s0 - 1)) - iz0 * (int32_t)p->m0;
+        p->c1 = (1 << (p->s1 - 1)) - iz1 * (int32_t)p->m1;
+        p->cadd = (1 << (p->sh - 1)) + (oz << p->sh);
+    }
+    return true;
 }
 
 extern "C" int hipq_channel_stride(int C) { return C <= 4 ? 4 : (C + 15) / 16 * 16; }

@@ -37,6 +37,8 @@ _SIGS = {
     "hipq_conv2d_plan_destroy": (None, [C.c_void_p]),
     "hipq_conv2d_plan_kernel": (C.c_char_p, [C.c_void_p]),
     "hipq_conv2d_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+    "hipq_conv2d_run_add": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_float, C.c_int,
+                                      C.c_int, C.c_void_p, C.c_void_p]),
     "hipq_ip_reorder_weights": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 6),
     "hipq_add_u8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_float, C.c_int, C.c_float,
                               C.c_int, C.c_float, C.c_int, C.c_int, C.c_void_p]),
@@ -149,6 +151,12 @@ class Conv2d:
         if y is None:
             y = self.empty_output()
         check(lib().hipq_conv2d_run(self.handle, _ptr(x), _ptr(y), _ptr(acc), _stream()))
+        return y
+
+    def run_add(self, x, residual, residual_first, res_alpha, res_zp, oalpha, ozp, y, obits=8):
+        """y = add(conv(x), residual) in one launch (include/hipq.h: hipq_conv2d_run_add)."""
+        check(lib().hipq_conv2d_run_add(self.handle, _ptr(x), _ptr(residual), int(bool(residual_first)), res_alpha, res_zp,
+                                        oalpha, ozp, obits, _ptr(y), _stream()))
         return y
 
     def close(self):

@@ -12,8 +12,24 @@ from . import hipq
 
 
 class HipqExecutor:
-    def __init__(self, case):
+    """fuse_add: a convolution whose only consumer is a two-input add is launched with the add fused into its
+    epilogue (hipq_conv2d_run_add); the convolution's own output tensor is then never materialised."""
+
+    def __init__(self, case, fuse_add=False):
         self.case = case
+        self.fused = {}      # conv output name -> the add node that absorbs it
+        if fuse_add:
+            uses = {}
+            for node in case.nodes:
+                for i in node.inputs:
+                    uses.setdefault(i, []).append(node)
+            for node in case.nodes:
+                u = uses.get(node.output, [])
+                if (node.kind == "conv" and node.attrs["group"] == 1 and not node.attrs["relu"] and len(u) == 1
+                        and u[0].kind == "add" and u[0].inputs[0] != u[0].inputs[1] and node.output != case.output.name
+                        and not any(a is u[0] for a in self.fused.values())):  # one convolution per add
+                    self.fused[node.output] = u[0]  # launched at the add's position: both operands exist by then
+        self._pending = {}   # id(add node) -> the deferred convolution
         self.buf = {}        # tensor name -> device tensor
         self.steps = []      # (label, kernel name, callable, algorithmic ops, compulsory bytes)
         self.plans = []
@@ -34,7 +50,7 @@ class HipqExecutor:
             else:
                 out = torch.zeros((N, H, W, hipq.channel_stride(C)), dtype=torch.uint8, device="cuda")
             self.buf[y.name] = out
-            ins = [self.buf[i] for i in node.inputs]
+            ins = [self.buf.get(i) for i in node.inputs]
             a = node.attrs
             if node.kind == "quantize":
                 fn = (lambda i=ins[0], o=out, y=y: hipq.quantize_u8(i, o, y.alpha, y.zp))
@@ -48,8 +64,17 @@ class HipqExecutor:
                 plan = hipq.Conv2d(x.shape, case.weights[a["w"]], case.weights[a["b"]], a["pad"], a["stride"],
                                    a["group"], x.alpha, x.zp, a["walpha"], a["wzp"], y.alpha, y.zp, relu=a["relu"])
                 self.plans.append(plan)
-                fn = (lambda p=plan, i=ins[0], o=out: p(i, o))
                 nbytes = int(np.prod(x.shape)) + int(np.prod(y.shape)) + case.weights[a["w"]].size + 4 * a["K"]
+                if node.output in self.fused and plan.kernel.startswith("conv_mfma"):
+                    add = self.fused[node.output]
+                    other = [i for i in add.inputs if i != node.output][0]
+                    res_first = add.inputs[0] == other
+                    ot, st = T[other], T[add.output]
+                    self._pending[id(add)] = (plan, ins[0], other, res_first, ot, st, nbytes + int(np.prod(y.shape)))
+                    del self.buf[y.name]  # never materialised
+                    continue
+                self.fused.pop(node.output, None)
+                fn = (lambda p=plan, i=ins[0], o=out: p(i, o))
                 self._add(node, plan.kernel, fn, plan.ops, nbytes)
             elif node.kind == "ip":
                 x = xs[0]
@@ -73,6 +98,12 @@ class HipqExecutor:
                 fn = (lambda i=ins[0], o=out, x=x, y=y, a=a: hipq.pool_u8(i, o, x.shape[1], a["k"], a["pad"], a["stride"],
                                                                          a["method"], x.alpha, x.zp, y.alpha, y.zp))
                 self._add(node, "pool_u8_kernel", fn, 0, int(np.prod(x.shape)) + int(np.prod(y.shape)))
+            elif node.kind == "add" and id(node) in self._pending:
+                plan, xin, other, res_first, ot, st, nbytes = self._pending.pop(id(node))
+                fn = (lambda p=plan, i=xin, r=self.buf[other], rf=res_first, ot=ot, st=st, o=out:
+                      p.run_add(i, r, rf, ot.alpha, ot.zp, st.alpha, st.zp, o))
+                self.steps.append({"label": node.output, "kind": "conv+add", "kernel": plan.kernel + "+add", "fn": fn,
+                                   "ops": plan.ops, "bytes": nbytes})
             elif node.kind == "add":
                 fn = (lambda i=ins, o=out, xs=xs, y=y: hipq.add_u8(i[0], i[1], o, xs[0].alpha, xs[0].zp, xs[1].alpha,
                                                                  xs[1].zp, y.alpha, y.zp))

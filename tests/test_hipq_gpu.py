@@ -102,6 +102,41 @@ def test_conv_edge_cases():
     assert np.array_equal(y, want)
 
 
+def test_conv_with_fused_residual_add():
+    """hipq_conv2d_run_add == conv followed by the reference add, byte for byte: both operand orders, the 32-bit
+    fast form and the 64-bit form of the add (very unequal scales), every tile shape's epilogue, ragged tiles,
+    a narrow output (plain store path) and asymmetric weights."""
+    rng = np.random.default_rng(21)
+    shapes = [  # N, C, H, W, K, R, pad, stride
+        (2, 64, 14, 14, 256, 1, 0, 1), (1, 64, 9, 11, 64, 3, 1, 1), (3, 32, 10, 7, 48, 3, 1, 2), (1, 256, 5, 5, 512, 1, 0, 1),
+        (1, 16, 6, 6, 3, 3, 1, 1), (2, 128, 28, 28, 128, 3, 1, 1),
+    ]
+    for i, (N, C, H, W, K, R, pad, st) in enumerate(shapes):
+        x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+        w = rng.integers(0, 256, (K, C, R, R), dtype=np.uint8)
+        b = rng.integers(-30000, 30000, K).astype(np.int32)
+        for res_first, wzp, ratio in ((False, 128, 1.0), (True, 128, 1.7), (False, int(rng.integers(0, 256)), 3000.0),
+                                      (True, 128, 1 / 2500.0)):
+            q = (rand_q(rng), int(rng.integers(0, 256)), rand_q(rng), wzp, rand_q(rng, 1e-2, 1.0), int(rng.integers(0, 256)))
+            plan = hipq.Conv2d(x.shape, w, b, pad, st, 1, *q)
+            conv = orc.conv2d_u8(x, w, b, pad, st, 1, *q)
+            res = rng.integers(0, 256, conv.shape, dtype=np.uint8)
+            ra, rz = float(np.float32(q[4] * ratio)), int(rng.integers(0, 256))
+            oa, oz = float(np.float32(max(q[4], ra) * 1.3)), int(rng.integers(0, 256))
+            print("fused add case", i, x.shape, w.shape, res_first, ratio, plan.kernel, flush=True)
+            want = orc.add_u8(res, conv, ra, rz, q[4], q[5], oa, oz) if res_first else orc.add_u8(conv, res, q[4], q[5], ra, rz, oa, oz)
+            y = plan.empty_output()
+            plan.run_add(hipq.to_device_nhwc(x), hipq.to_device_nhwc(res), res_first, ra, rz, oa, oz, y)
+            torch.cuda.synchronize()
+            got = hipq.from_device_nhwc(y, K)
+            assert np.array_equal(got, want), (i, res_first, ratio, plan.kernel, int((got != want).sum()))
+    # a plan that does not run an MFMA kernel refuses, loudly
+    xdw = rng.integers(0, 256, (1, 32, 8, 8), dtype=np.uint8)
+    plan = hipq.Conv2d(xdw.shape, rng.integers(0, 256, (32, 1, 3, 3), dtype=np.uint8), None, 1, 1, 32, 0.02, 3, 0.01, 128, 0.05, 9)
+    with pytest.raises(hipq.HipqError, match="only the MFMA"):
+        plan.run_add(hipq.to_device_nhwc(xdw), hipq.to_device_nhwc(xdw), False, 0.05, 0, 0.07, 0, plan.empty_output())
+
+
 def test_conv_grouped_and_depthwise():
     rng = np.random.default_rng(13)
     kerns = set()
