@@ -20,6 +20,10 @@ sys.path.insert(0, ROOT)
 
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, TOP/s (published)
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s (published)
+# HBM bytes per launch of the dominant kernel family, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this very
+# command (profiles/conv_mfma_i8_resnet50_n64.md holds the counter readings and the copy-kernel scale factors).
+# A counter run cannot be made from inside the benchmark, so the figure is recorded here for the default workload.
+MEASURED_TRAFFIC = {("resnet50", 64, True): 35.07e6}
 
 
 def time_steps(fn, steps, warmup):
@@ -100,6 +104,9 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-fuse", action="store_true", help="run every residual add as its own kernel")
     ap.add_argument("--layers", action="store_true", help="print a per-layer table to stderr")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch a plain 256 MiB device copy (copy_bytes_kernel): the known-size reference that a "
+                         "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command is scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU's share of the batch: this build runs on a single GPU only "
@@ -128,6 +135,16 @@ def main():
     torch.cuda.synchronize()
     y = ex.output()
 
+    if args.calibrate_copy:
+        from nart_amd import hipq
+        n = 256 << 20
+        src = torch.zeros(n, dtype=torch.uint8, device="cuda")
+        dst = torch.empty(n, dtype=torch.uint8, device="cuda")
+        for _ in range(3):
+            hipq.check(hipq.lib().hipq_copy_bytes(src.data_ptr(), dst.data_ptr(), n, torch.cuda.current_stream().cuda_stream))
+        torch.cuda.synchronize()
+        del src, dst
+
     if args.no_graph:
         step = ex.run
     else:
@@ -155,6 +172,9 @@ def main():
         achieved = d["bytes"] / (d["ms"] * 1e-3) / 1e9
         roof = {"kernel": dom, "bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                 "frac": round(achieved / PEAK_HBM_GBS, 4), "traffic": None}
+    roof["traffic"] = MEASURED_TRAFFIC.get((args.workload, args.batch, not args.no_fuse))
+    roof["algorithmic_bytes_per_launch"] = round(d["bytes"] / d["launches"])
+    roof["algorithmic_ops_per_launch"] = round(d["ops"] / d["launches"]) if d["ops"] else None
     roof["launches_per_step"] = d["launches"]
     roof["avg_launch_us"] = round(d["ms"] / d["launches"] * 1e3, 2)
     roof["sum_kernel_ms"] = round(sum(kt), 4)
