@@ -181,7 +181,10 @@ __device__ static inline void conv_epilogue(const ConvArgs &a, v16i (&acc)[TN][T
                 *reinterpret_cast<uint32_t *>(lds + pl * OSTR + wn * (TN * 32) + tn * 32 + g * 8 + half * 4) = packed;
             }
     }
-    __syncthreads();
+    // own LDS writes complete, then the barrier: deliberately NOT __syncthreads(), whose fence would also wait for
+    // every vector-memory operation in flight
+    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0), vmcnt / expcnt untouched
+    __builtin_amdgcn_s_barrier();
     constexpr int LPR = BN / 16;   // lanes per pixel row
     constexpr int RPP = 256 / LPR; // rows per pass
     const int c16 = (tid % LPR) * 16;
@@ -924,7 +927,7 @@ static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_
     const bool aligned = a.in_cs % 64 == 0;
     // few slabs: two stages are all the pipeline can use, and the smaller LDS footprint lets more work-groups
     // share a CU, which is what hides the latency of such short kernels
-    const bool shallow = a.nslab <= 2;
+    const bool shallow = true; // two stages: deeper pipelines did not pay at these layer sizes, more resident work-groups do
 #define HIPQ_LAUNCH_DMA(NSV, WZ, AL) \
     hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, NSV, WZ, AL>), grid, block, 0, st, a)
     if (p->has_wzp) { // rare (asymmetric weights): generic addressing only
