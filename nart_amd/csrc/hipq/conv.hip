@@ -912,7 +912,11 @@ extern "C" void hipq_conv2d_plan_destroy(hipq_conv2d_plan *p)
 
 extern "C" const char *hipq_conv2d_plan_kernel(const hipq_conv2d_plan *p) { return p ? p->name.c_str() : ""; }
 
-template <int BM, int BN, int WM, int WN, int NS>
+// Two load stages everywhere: measured on the ResNet-50 layer shapes, deeper pipelines did not pay, while the smaller
+// LDS footprint lets four work-groups share a CU and overlap their load, multiply and store phases.
+constexpr int kStages = 2;
+
+template <int BM, int BN, int WM, int WN>
 static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_t st)
 {
     const int nblk = a.nbm * a.nbn;
@@ -922,31 +926,13 @@ static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_
             hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, true, true>), grid, block, 0, st, a);
         else
             hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, false, true>), grid, block, 0, st, a);
-        return;
-    }
-    const bool aligned = a.in_cs % 64 == 0;
-    // few slabs: two stages are all the pipeline can use, and the smaller LDS footprint lets more work-groups
-    // share a CU, which is what hides the latency of such short kernels
-    const bool shallow = true; // two stages: deeper pipelines did not pay at these layer sizes, more resident work-groups do
-#define HIPQ_LAUNCH_DMA(NSV, WZ, AL) \
-    hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, NSV, WZ, AL>), grid, block, 0, st, a)
-    if (p->has_wzp) { // rare (asymmetric weights): generic addressing only
-        if (shallow)
-            HIPQ_LAUNCH_DMA(2, true, false);
-        else
-            HIPQ_LAUNCH_DMA(NS, true, false);
-    } else if (aligned) {
-        if (shallow)
-            HIPQ_LAUNCH_DMA(2, false, true);
-        else
-            HIPQ_LAUNCH_DMA(NS, false, true);
+    } else if (p->has_wzp) { // rare (asymmetric weights): generic addressing only
+        hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, kStages, true, false>), grid, block, 0, st, a);
+    } else if (a.in_cs % 64 == 0) {
+        hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, kStages, false, true>), grid, block, 0, st, a);
     } else {
-        if (shallow)
-            HIPQ_LAUNCH_DMA(2, false, false);
-        else
-            HIPQ_LAUNCH_DMA(NS, false, false);
+        hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, kStages, false, false>), grid, block, 0, st, a);
     }
-#undef HIPQ_LAUNCH_DMA
 }
 
 static int run_conv(const hipq_conv2d_plan *p, ConvArgs &a, hipStream_t st);
@@ -989,11 +975,11 @@ static int run_conv(const hipq_conv2d_plan *p, ConvArgs &a, hipStream_t st)
     case kMfma:
     case kMfmaSmallC:
         switch (p->tile) {
-        case 0: launch_mfma<128, 128, 2, 2, 4>(p, a, st); break; // 4 x 16 KiB
-        case 1: launch_mfma<256, 64, 4, 1, 3>(p, a, st); break;  // 3 x 20 KiB
-        case 2: launch_mfma<128, 64, 2, 2, 4>(p, a, st); break;  // 4 x 12 KiB
-        case 3: launch_mfma<64, 128, 1, 4, 4>(p, a, st); break;
-        default: launch_mfma<64, 64, 2, 2, 4>(p, a, st); break;  // 4 x 8 KiB
+        case 0: launch_mfma<128, 128, 2, 2>(p, a, st); break;
+        case 1: launch_mfma<256, 64, 4, 1>(p, a, st); break;
+        case 2: launch_mfma<128, 64, 2, 2>(p, a, st); break;
+        case 3: launch_mfma<64, 128, 1, 4>(p, a, st); break;
+        default: launch_mfma<64, 64, 2, 2>(p, a, st); break;
         }
         break;
     case kDepthwise: {
