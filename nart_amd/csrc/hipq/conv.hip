@@ -73,7 +73,8 @@ struct ConvArgs {
     int fastq; // 1: the one-multiply requantisation is valid for q.shift
     int qt;    // shift - 32
     int qadd;  // 2^(qt-1) + zp * 2^qt
-    double inv_ohw, inv_ow; // 1 / (OH*OW), 1 / OW
+    double inv_ohw, inv_ow; // 1 / (OH*OW), 1 / OW (depthwise 3x3: 1 / work items per row, 1 / channel quads)
+    double inv_oh;          // 1 / OH
     const uint8_t *res; // fused residual add: the other operand (same layout as y), or nullptr
     int res_first;      // 1: the residual is input 0 of the add, the convolution's output input 1
     AddParams addq;
@@ -635,6 +636,187 @@ __global__ __launch_bounds__(256) void conv_mfma_dma_kernel(const ConvArgs a)
 }
 
 // ------------------------------------------------------------------------------------------------
+// Depthwise 3x3 (group == C == K, stride 1 or 2): HBM-bound on paper (16 bytes in, 16 bytes out per output pixel and
+// 16 channels), in practice bounded by vector ALU work, so the kernel is written for instruction count.
+// One thread owns 4 channels (one dword of the channels-last tensors) of a strip of 4 output pixels along W; a
+// wave covers 256 contiguous bytes per tap.  Bytes are re-centred as in the MFMA kernel (x ^ 0x80, w - 128).
+// Stride 1: per kernel row the six input columns of the strip are byte-transposed (8 v_perm_b32 per 4x4 block)
+// into per-channel dwords T0 = [x0 x1 x2 x3], T1 = [x2 x3 x4 x5]; outputs 0 / 1 are v_dot4_i32_i8 of T0 with the
+// packed weights [w0 w1 w2 0] / [0 w0 w1 w2], outputs 2 / 3 the same with T1.  Stride 2: each output gathers its
+// three taps with two v_perm_b32 into [x0 x1 x2 0].  bias + a * sum(w - 128) + 9ab is folded per channel; the
+// b * sum(x - 128) term (wzp != 128 only) is one more dot with ones.  Taps outside the image are loaded from a
+// clamped address (no divergent branch) and replaced by the byte izp.
+// A thread computes 2 output rows x 4 output columns x 4 channels, so that every loaded and transposed input row
+// serves up to three kernel rows of two output rows.
+// QMODE 0: 64-bit requantisation; 1: one-multiply form; 2: one-multiply form and clamp range exactly [0, 255]
+// (saturating packs instead of clamps).  DUMP: also write the int32 accumulators.
+template <int STRIDE, bool HAS_WZP, int QMODE, bool DUMP>
+__device__ static inline void depthwise3x3_body(const ConvArgs &a, int idx, int per_row, int cq, int ohp_count)
+{
+    constexpr int ROWS = 2;                      // output rows per thread
+    constexpr int NCOL = 3 * STRIDE + 3;         // input columns a strip of 4 outputs touches
+    constexpr int NIR = (ROWS - 1) * STRIDE + 3; // input rows the two output rows touch
+    const uint32_t *wtab = reinterpret_cast<const uint32_t *>(a.wpack); // [3 rows][2 alignments][cs] dwords
+    const int rowp = fast_div(idx, per_row, a.inv_ohw); // inv_ohw holds 1 / per_row for this kernel
+    const int rem = idx - rowp * per_row;
+    const int strip = fast_div(rem, cq, a.inv_ow), quad = rem - strip * cq; // inv_ow holds 1 / cq
+    const int n = fast_div(rowp, ohp_count, a.inv_oh), oh0 = (rowp - n * ohp_count) * ROWS; // inv_oh: 1 / row pairs per image
+    const int ow0 = strip * 4, iw0 = ow0 * STRIDE - a.pad_w, ih0 = oh0 * STRIDE - a.pad_h;
+    const int c0 = quad * 4;
+    const v4i bias = *reinterpret_cast<const v4i *>(a.bias2 + c0);
+    v4i wa[3], wb[3];
+#pragma unroll
+    for (int r = 0; r < 3; r++) {
+        wa[r] = *reinterpret_cast<const v4i *>(wtab + (r * 2 + 0) * a.in_cs + c0); // [w0 w1 w2 0] per channel
+        if (STRIDE == 1)
+            wb[r] = *reinterpret_cast<const v4i *>(wtab + (r * 2 + 1) * a.in_cs + c0); // [0 w0 w1 w2]
+    }
+    int32_t acc[ROWS][4][4], xsum[ROWS][4][4];
+#pragma unroll
+    for (int q = 0; q < ROWS; q++)
+#pragma unroll
+        for (int o = 0; o < 4; o++)
+#pragma unroll
+            for (int c = 0; c < 4; c++)
+                acc[q][o][c] = bias[c], xsum[q][o][c] = 0;
+    // 32-bit byte offsets from the tensor base (the host guarantees the tensor is smaller than 2 GiB)
+    const uint32_t nbase = (uint32_t)(n * a.H * a.W * a.in_cs + c0);
+    // threads whose whole NIR x NCOL footprint is inside the image (nearly all of them) skip the border logic
+    const bool interior = ih0 >= 0 && ih0 + NIR - 1 < a.H && iw0 >= 0 && iw0 + NCOL - 1 < a.W;
+    const uint32_t padx = a.padword ^ 0x80808080u;
+    // all loads first (NIR x NCOL dwords in flight per thread), arithmetic afterwards: the kernel lives on memory
+    // latency, not on occupancy
+    uint32_t colr[NIR][NCOL];
+#pragma unroll
+    for (int ir = 0; ir < NIR; ir++) {
+        uint32_t (&col)[NCOL] = colr[ir];
+        if (interior) {
+            const uint32_t rbase = nbase + (uint32_t)(((ih0 + ir) * a.W + iw0) * a.in_cs);
+#pragma unroll
+            for (int j = 0; j < NCOL; j++)
+                col[j] = *reinterpret_cast<const uint32_t *>(a.x + (rbase + (uint32_t)(j * a.in_cs))) ^ 0x80808080u;
+        } else {
+            // loaded from a clamped (always valid) address, then replaced by the pad byte where outside the image
+            const int ih = ih0 + ir;
+            const bool row_ok = (unsigned)ih < (unsigned)a.H;
+            const uint32_t rbase = nbase + (uint32_t)((ih < 0 ? 0 : (ih >= a.H ? a.H - 1 : ih)) * a.W * a.in_cs);
+#pragma unroll
+            for (int j = 0; j < NCOL; j++) {
+                const int iw = iw0 + j;
+                const uint32_t off = (uint32_t)((iw < 0 ? 0 : (iw >= a.W ? a.W - 1 : iw)) * a.in_cs);
+                const uint32_t v = *reinterpret_cast<const uint32_t *>(a.x + (rbase + off)) ^ 0x80808080u;
+                col[j] = (row_ok && (unsigned)iw < (unsigned)a.W) ? v : padx;
+            }
+        }
+    }
+#pragma unroll
+    for (int ir = 0; ir < NIR; ir++) {
+        const uint32_t (&col)[NCOL] = colr[ir];
+        if (STRIDE == 1) {
+#pragma unroll
+            for (int h = 0; h < 2; h++) { // columns 2h .. 2h+3 serve outputs 2h and 2h+1
+                const uint32_t A = col[2 * h], B = col[2 * h + 1], C = col[2 * h + 2], D = col[2 * h + 3];
+                // v_perm_b32(S0, S1, sel): selector bytes 0-3 pick from S1, 4-7 from S0
+                const uint32_t t0 = __builtin_amdgcn_perm(B, A, 0x05010400u), t1 = __builtin_amdgcn_perm(B, A, 0x07030602u);
+                const uint32_t t2 = __builtin_amdgcn_perm(D, C, 0x05010400u), t3 = __builtin_amdgcn_perm(D, C, 0x07030602u);
+                const uint32_t T[4] = {__builtin_amdgcn_perm(t2, t0, 0x05040100u), __builtin_amdgcn_perm(t2, t0, 0x07060302u),
+                                       __builtin_amdgcn_perm(t3, t1, 0x05040100u), __builtin_amdgcn_perm(t3, t1, 0x07060302u)};
+#pragma unroll
+                for (int q = 0; q < ROWS; q++) {
+                    const int kr = ir - q * STRIDE; // kernel row this input row is for output row q
+                    if (kr < 0 || kr > 2)
+                        continue;
+#pragma unroll
+                    for (int c = 0; c < 4; c++) {
+                        acc[q][2 * h][c] = __builtin_amdgcn_sdot4((int)T[c], wa[kr][c], acc[q][2 * h][c], false);
+                        acc[q][2 * h + 1][c] = __builtin_amdgcn_sdot4((int)T[c], wb[kr][c], acc[q][2 * h + 1][c], false);
+                        if (HAS_WZP) {
+                            xsum[q][2 * h][c] = __builtin_amdgcn_sdot4((int)T[c], 0x00010101, xsum[q][2 * h][c], false);
+                            xsum[q][2 * h + 1][c] = __builtin_amdgcn_sdot4((int)T[c], 0x01010100, xsum[q][2 * h + 1][c], false);
+                        }
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int o = 0; o < 4; o++) {
+                const uint32_t A = col[o * STRIDE], B = col[o * STRIDE + 1], C = col[o * STRIDE + 2];
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    // selector 0x0c gives a zero byte
+                    const uint32_t t = __builtin_amdgcn_perm(B, A, 0x0c0c0000u | ((4u + c) << 8) | (uint32_t)c);
+                    const uint32_t T = __builtin_amdgcn_perm(C, t, 0x0c000100u | ((4u + c) << 16));
+#pragma unroll
+                    for (int q = 0; q < ROWS; q++) {
+                        const int kr = ir - q * STRIDE;
+                        if (kr < 0 || kr > 2)
+                            continue;
+                        acc[q][o][c] = __builtin_amdgcn_sdot4((int)T, wa[kr][c], acc[q][o][c], false);
+                        if (HAS_WZP)
+                            xsum[q][o][c] = __builtin_amdgcn_sdot4((int)T, 0x00010101, xsum[q][o][c], false);
+                    }
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int q = 0; q < ROWS; q++) {
+        if (oh0 + q >= a.OH)
+            break;
+        const uint32_t obase = (uint32_t)((((n * a.OH + oh0 + q) * a.OW) + ow0) * a.out_cs + c0);
+#pragma unroll
+        for (int o = 0; o < 4; o++) {
+            if (ow0 + o >= a.OW)
+                break;
+            int32_t v[4];
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                v[c] = (int32_t)((uint32_t)acc[q][o][c] + (HAS_WZP ? (uint32_t)(a.bwz * xsum[q][o][c]) : 0u));
+                if (DUMP)
+                    a.acc_out[(size_t)(obase + o * a.out_cs) + c] = v[c];
+            }
+            uint32_t packed = 0;
+            if (QMODE == 2) {
+                int32_t r[4];
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                    r[c] = (__mulhi(v[c], (int)a.q.mult) + a.qadd) >> a.qt;
+                uint32_t p01, p23, b01, b23;
+                asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p01) : "v"(r[0]), "v"(r[1]));
+                asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(r[2]), "v"(r[3]));
+                asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
+                asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
+                packed = __builtin_amdgcn_perm(b23, b01, 0x05040100u); // low halves of both
+            } else {
+#pragma unroll
+                for (int c = 0; c < 4; c++)
+                    packed |= (uint32_t)conv_requant<QMODE == 1>(a, v[c]) << (8 * c);
+            }
+            *reinterpret_cast<uint32_t *>(a.y + (obase + (uint32_t)(o * a.out_cs))) = packed;
+        }
+    }
+}
+
+template <int STRIDE, bool HAS_WZP>
+__global__ __launch_bounds__(256) void conv_depthwise3x3_kernel(const ConvArgs a)
+{
+    const int cq = a.in_cs >> 2, nstrip = (a.OW + 3) >> 2, ohp = (a.OH + 1) >> 1;
+    const int per_row = nstrip * cq;
+    const int total = a.N * ohp * per_row; // the host guarantees it fits in 31 bits
+    const int qmode = a.fastq ? (a.lo == 0 && a.q.hi == 255 ? 2 : 1) : 0;
+    for (int idx = blockIdx.x * 256 + threadIdx.x; idx < total; idx += gridDim.x * 256) {
+        if (a.acc_out != nullptr)
+            depthwise3x3_body<STRIDE, HAS_WZP, 0, true>(a, idx, per_row, cq, ohp); // test path: exactness only
+        else if (qmode == 2)
+            depthwise3x3_body<STRIDE, HAS_WZP, 2, false>(a, idx, per_row, cq, ohp);
+        else if (qmode == 1)
+            depthwise3x3_body<STRIDE, HAS_WZP, 1, false>(a, idx, per_row, cq, ohp);
+        else
+            depthwise3x3_body<STRIDE, HAS_WZP, 0, false>(a, idx, per_row, cq, ohp);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // Depthwise (group == C == K): memory-bound; one thread = 4 channels of one output pixel.
 // Weights are stored tap-major as int16 (w - wzp needs 9 bits): wpack[tap][cs].
 __global__ __launch_bounds__(256) void conv_depthwise_kernel(const ConvArgs a)
@@ -722,7 +904,7 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const ConvArgs a)
 // host side
 using namespace hipq;
 
-enum ConvVariant { kMfma, kMfmaSmallC, kDepthwise, kDirect };
+enum ConvVariant { kMfma, kMfmaSmallC, kDepthwise3x3, kDepthwise, kDirect };
 
 // Tile shapes of the MFMA kernel: BM pixels x BN channels per work-group, waves arranged WM x WN.
 struct TileShape {
@@ -861,6 +1043,30 @@ extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t
         char nm[96];
         snprintf(nm, sizeof nm, "conv_mfma_i8_%dx%d%s%s", BM, BN, smallc ? "_c4" : "", p->has_wzp ? "_wzp" : "");
         p->name = nm;
+    } else if (d.group == d.C && d.K == d.C && d.in_cs == d.out_cs && d.R == 3 && d.S == 3 && d.stride_h == d.stride_w
+               && (d.stride_h == 1 || d.stride_h == 2)
+               && (long long)d.N * a.OH * ((a.OW + 3) / 4) * (d.in_cs / 4) < (1ll << 31)) {
+        p->variant = kDepthwise3x3;
+        p->has_wzp = boff != 0;
+        // weights: [kernel row][alignment][cs] dwords, {w0 - 128, w1 - 128, w2 - 128, 0} and {0, w0 - 128, w1 - 128, w2 - 128}
+        wbuf.assign((size_t)3 * 2 * d.in_cs * 4, 0);
+        bbuf.assign(d.in_cs, 0);
+        for (int c = 0; c < d.C; c++) {
+            long long wsum = 0;
+            for (int r = 0; r < 3; r++)
+                for (int t = 0; t < 3; t++) {
+                    const int ws = (int)w[(size_t)c * 9 + r * 3 + t] - 128;
+                    wsum += ws;
+                    wbuf[((size_t)(r * 2 + 0) * d.in_cs + c) * 4 + t] = (uint8_t)(int8_t)ws;
+                    wbuf[((size_t)(r * 2 + 1) * d.in_cs + c) * 4 + t + 1] = (uint8_t)(int8_t)ws;
+                }
+            const long long c0 = (bias ? (long long)bias[c] : 0) + (long long)aoff * wsum + 9ll * aoff * boff;
+            bbuf[c] = (int32_t)(uint32_t)(unsigned long long)c0;
+        }
+        a.inv_ohw = 1.0 / ((double)((a.OW + 3) / 4) * (d.in_cs / 4));
+        a.inv_ow = 1.0 / (double)(d.in_cs / 4);
+        a.inv_oh = 1.0 / (double)((a.OH + 1) / 2);
+        p->name = std::string("conv_depthwise3x3_u8_s") + (d.stride_h == 1 ? "1" : "2") + (p->has_wzp ? "_wzp" : "");
     } else if (d.group == d.C && d.K == d.C && d.in_cs == d.out_cs) {
         p->variant = kDepthwise;
         wbuf.assign((size_t)d.R * d.S * d.in_cs * 2, 0);
@@ -982,6 +1188,22 @@ static int run_conv(const hipq_conv2d_plan *p, ConvArgs &a, hipStream_t st)
         default: launch_mfma<64, 64, 2, 2>(p, a, st); break;
         }
         break;
+    case kDepthwise3x3: {
+        const size_t total = (size_t)a.N * ((a.OH + 1) / 2) * ((a.OW + 3) / 4) * (a.in_cs / 4);
+        const dim3 grid((unsigned)std::min<size_t>((total + 255) / 256, 256 * 64)), block(256);
+        if (p->d.stride_h == 1) {
+            if (p->has_wzp)
+                hipLaunchKernelGGL((conv_depthwise3x3_kernel<1, true>), grid, block, 0, st, a);
+            else
+                hipLaunchKernelGGL((conv_depthwise3x3_kernel<1, false>), grid, block, 0, st, a);
+        } else {
+            if (p->has_wzp)
+                hipLaunchKernelGGL((conv_depthwise3x3_kernel<2, true>), grid, block, 0, st, a);
+            else
+                hipLaunchKernelGGL((conv_depthwise3x3_kernel<2, false>), grid, block, 0, st, a);
+        }
+        break;
+    }
     case kDepthwise: {
         const size_t total = (size_t)a.P * (a.in_cs / 4);
         const unsigned blocks = (unsigned)std::min<size_t>((total + 255) / 256, 256 * 32);

@@ -44,40 +44,80 @@ struct EltArgs {
     uint32_t mult[HIPQ_MAX_ELTWISE_INPUTS];
     int shift[HIPQ_MAX_ELTWISE_INPUTS]; // shift[n] - s0
     int zp[HIPQ_MAX_ELTWISE_INPUTS];
-    int n_in, s0, oz, hi, is_max;
+    int cfast[HIPQ_MAX_ELTWISE_INPUTS]; // fast form: 2^(shift-1) - zp * mult
+    int n_in, s0, oz, hi, is_max, fast, cadd;
     uint8_t *y;
     size_t count;
 };
 
+// one partial term: input byte x of input n
+template <bool FAST>
+__device__ static inline int32_t eltwise_term(uint32_t x, int n, const EltArgs &p)
+{
+    if (FAST) // |mult * (x - zp)| < 2^30 and shift <= 30: 32-bit arithmetic is exact
+        return (__mul24((int)x, (int)p.mult[n]) + p.cfast[n]) >> p.shift[n];
+    return (int32_t)rshift_rn((int32_t)((uint32_t)((int32_t)x - p.zp[n]) * p.mult[n]), p.shift[n]);
+}
+
+template <bool FAST>
+__device__ static inline uint32_t eltwise_finish(int32_t t, const EltArgs &p)
+{
+    if (FAST)
+        return (uint32_t)sat_hi((t + p.cadd) >> p.s0, p.hi);
+    return (uint32_t)sat_hi((int32_t)(rshift_rn(t, p.s0) + p.oz), p.hi);
+}
+
+// NIN inputs and the operation known at compile time (register arrays stay in registers), 16 bytes per thread and input
+template <int NIN, bool FAST, bool IS_MAX>
 __global__ __launch_bounds__(256) void eltwise_u8_kernel(const EltArgs p)
 {
-    const size_t nvec = p.count / 4;
+    const size_t nvec = p.count / 16;
     const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nthr = (size_t)gridDim.x * blockDim.x;
-    for (size_t i = tid; i < nvec + (p.count & 3); i += nthr) {
-        const bool tail = i >= nvec;
-        const size_t base = tail ? nvec * 4 + (i - nvec) : i * 4;
-        const int ne = tail ? 1 : 4;
-        int32_t t[4];
-        for (int e = 0; e < 4; e++)
-            t[e] = p.is_max ? -1 : 0; // the reference's running maximum starts at 0xffffffff (eltwise.c:198)
-        for (int n = 0; n < p.n_in; n++) {
-            uint32_t v = tail ? p.in[n][base] : reinterpret_cast<const uint32_t *>(p.in[n])[i];
-            for (int e = 0; e < ne; e++) {
-                const int32_t pr = (int32_t)((uint32_t)((int32_t)((v >> (8 * e)) & 255) - p.zp[n]) * p.mult[n]);
-                const int64_t r = rshift_rn(pr, p.shift[n]);
-                if (p.is_max)
-                    t[e] = t[e] < (int32_t)r ? (int32_t)r : t[e];
-                else
-                    t[e] = (int32_t)(t[e] + r);
+    for (size_t i = tid; i < nvec; i += nthr) {
+        u32x4 v[NIN];
+#pragma unroll
+        for (int n = 0; n < NIN; n++)
+            v[n] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p.in[n]) + i);
+        u32x4 o;
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                int32_t t = IS_MAX ? -1 : 0; // the reference's running maximum starts at 0xffffffff (eltwise.c:198)
+#pragma unroll
+                for (int n = 0; n < NIN; n++) {
+                    const int32_t r = eltwise_term<FAST>((v[n][d] >> (8 * e)) & 255, n, p);
+                    t = IS_MAX ? (t < r ? r : t) : (int32_t)((uint32_t)t + (uint32_t)r);
+                }
+                w |= eltwise_finish<FAST>(t, p) << (8 * e);
             }
+            o[d] = w;
         }
-        uint32_t o = 0;
-        for (int e = 0; e < ne; e++)
-            o |= (uint32_t)sat_hi((int32_t)(rshift_rn(t[e], p.s0) + p.oz), p.hi) << (8 * e);
-        if (tail)
-            p.y[base] = (uint8_t)o;
-        else
-            reinterpret_cast<uint32_t *>(p.y)[i] = o;
+        reinterpret_cast<u32x4 *>(p.y)[i] = o;
+    }
+    for (size_t i = nvec * 16 + tid; i < p.count; i += nthr) {
+        int32_t t = IS_MAX ? -1 : 0;
+#pragma unroll
+        for (int n = 0; n < NIN; n++) {
+            const int32_t r = eltwise_term<false>(p.in[n][i], n, p);
+            t = IS_MAX ? (t < r ? r : t) : (int32_t)((uint32_t)t + (uint32_t)r);
+        }
+        p.y[i] = (uint8_t)eltwise_finish<false>(t, p);
+    }
+}
+
+// any number of inputs: one byte position at a time per input, no register arrays
+__global__ __launch_bounds__(256) void eltwise_u8_generic_kernel(const EltArgs p)
+{
+    const size_t tid = (size_t)blockIdx.x * blockDim.x + threadIdx.x, nthr = (size_t)gridDim.x * blockDim.x;
+    for (size_t i = tid; i < p.count; i += nthr) {
+        int32_t t = p.is_max ? -1 : 0;
+        for (int n = 0; n < p.n_in; n++) {
+            const int32_t r = eltwise_term<false>(p.in[n][i], n, p);
+            t = p.is_max ? (t < r ? r : t) : (int32_t)((uint32_t)t + (uint32_t)r);
+        }
+        p.y[i] = (uint8_t)eltwise_finish<false>(t, p);
     }
 }
 
@@ -204,6 +244,58 @@ __global__ __launch_bounds__(256) void pool_u8_kernel(const PoolArgs p)
     }
 }
 
+// Max pooling with a channel stride that is a multiple of 16: a thread owns 16 channels of one output pixel (128-bit
+// loads, one 128-bit store), 32-bit index arithmetic.  The byte-wise maxima are taken on the packed dwords.
+__device__ static inline uint32_t max_u8x4(uint32_t a, uint32_t b)
+{
+    // per byte: a >= b ? a : b, from the borrow of (a | 0x80) - (b & 0x7f) combined with the top bits
+    const uint32_t H = 0x80808080u;
+    const uint32_t d = (a | H) - (b & ~H);       // no borrow across bytes
+    const uint32_t ge = ((a & ~b) | (~(a ^ b) & d)) & H; // top bit set where a >= b
+    const uint32_t m = (ge >> 7) * 0xffu;        // 0xff in those bytes
+    return (a & m) | (b & ~m);
+}
+
+__global__ __launch_bounds__(256) void pool_max16_u8_kernel(const PoolArgs p, double inv_c16, double inv_ow, double inv_oh)
+{
+    const int c16n = p.cs >> 4;
+    const int total = p.N * p.OH * p.OW * c16n; // the host guarantees 31 bits
+    const int radd = (1 << (p.shift - 1)) + (p.oz << p.shift);
+    for (int idx = blockIdx.x * 256 + threadIdx.x; idx < total; idx += gridDim.x * 256) {
+        const int m = (int)((double)idx * inv_c16);
+        const int mm = m - (m * c16n > idx) + ((m + 1) * c16n <= idx), c0 = (idx - mm * c16n) * 16;
+        int row = (int)((double)mm * inv_ow);
+        row += ((row + 1) * p.OW <= mm) - (row * p.OW > mm);
+        const int ow = mm - row * p.OW;
+        int n = (int)((double)row * inv_oh);
+        n += ((n + 1) * p.OH <= row) - (n * p.OH > row);
+        const int oh = row - n * p.OH;
+        const int hs = max(oh * p.sh - p.ph, 0), ws = max(ow * p.sw - p.pw, 0);
+        const int he = min(oh * p.sh - p.ph + p.kh, p.H), we = min(ow * p.sw - p.pw + p.kw, p.W);
+        u32x4 mx = {0, 0, 0, 0};
+        for (int i = hs; i < he; i++)
+            for (int j = ws; j < we; j++) {
+                const u32x4 v = *reinterpret_cast<const u32x4 *>(p.x + (size_t)((n * p.H + i) * p.W + j) * p.cs + c0);
+#pragma unroll
+                for (int d = 0; d < 4; d++)
+                    mx[d] = max_u8x4(mx[d], v[d]);
+            }
+        u32x4 o;
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                // mult < 2^16, |max - zp| <= 255: the product fits 24 bits, shift <= 30 (host): 32-bit arithmetic is exact
+                const int32_t pr = __mul24((int)p.mult, (int)((mx[d] >> (8 * e)) & 255) - p.iz);
+                w |= (uint32_t)sat_hi((pr + radd) >> p.shift, p.hi) << (8 * e);
+            }
+            o[d] = w;
+        }
+        *reinterpret_cast<u32x4 *>(p.y + (size_t)mm * p.cs + c0) = o;
+    }
+}
+
 // ---- quantize (quantize.c:145-157): fp32 NCHW -> uint8 NHWC --------------------------------------
 // One thread produces the 4 channels of one dword of the output; reads are coalesced along W per
 // channel plane, writes along the pixel index.
@@ -241,6 +333,27 @@ __global__ __launch_bounds__(256) void quantize_u8_kernel(const QuantArgs p)
                 o |= quantize_one(p.x[((size_t)n * p.C + c) * hw + pix], p) << (8 * e);
         }
         *reinterpret_cast<uint32_t *>(p.y + ((size_t)n * hw + pix) * p.cs + q4 * 4) = o;
+    }
+}
+
+// Network inputs (C <= 4, channel stride 4): a thread converts 4 consecutive pixels, i.e. one 128-bit load per
+// channel plane and one 128-bit store; blockIdx.y is the image, so no 64-bit index arithmetic is needed.
+__global__ __launch_bounds__(256) void quantize_u8_c4_kernel(const QuantArgs p)
+{
+    const int hw = p.H * p.W, hw4 = hw >> 2; // the host checks hw % 4 == 0
+    const int n = blockIdx.y;
+    const float *xn = p.x + (size_t)n * p.C * hw;
+    u32x4 *yn = reinterpret_cast<u32x4 *>(p.y + (size_t)n * hw * 4);
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < hw4; i += gridDim.x * 256) {
+        u32x4 o = {0, 0, 0, 0};
+        for (int c = 0; c < p.C; c++) {
+            typedef float f32x4 __attribute__((ext_vector_type(4)));
+            const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(xn + (size_t)c * hw) + i);
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                o[e] |= quantize_one(v[e], p) << (8 * c);
+        }
+        yn[i] = o;
     }
 }
 
@@ -341,7 +454,7 @@ extern "C" int hipq_eltwise_u8(const void *const *in, int n_in, const float *coe
                                int obits, void *stream)
 {
     clear_error();
-    HIPQ_REQUIRE(in && ialpha && izp && y, "hipq_eltwise_u8: null pointer");
+    HIPQ_REQUIRE(in && ialpha && izp && y && aligned16(y), "hipq_eltwise_u8: null pointer or output not 16-byte aligned");
     HIPQ_REQUIRE(n_in >= 2 && n_in <= HIPQ_MAX_ELTWISE_INPUTS, "hipq_eltwise_u8: %d inputs (2..%d supported)", n_in,
                  HIPQ_MAX_ELTWISE_INPUTS);
     HIPQ_REQUIRE(operation == HIPQ_ELTWISE_SUM || operation == HIPQ_ELTWISE_MAX,
@@ -352,7 +465,7 @@ extern "C" int hipq_eltwise_u8(const void *const *in, int n_in, const float *coe
     memset(&p, 0, sizeof p);
     int smin = 127, sh[HIPQ_MAX_ELTWISE_INPUTS];
     for (int n = 0; n < n_in; n++) {
-        HIPQ_REQUIRE(in[n] && (reinterpret_cast<uintptr_t>(in[n]) & 3) == 0, "hipq_eltwise_u8: input %d unaligned", n);
+        HIPQ_REQUIRE(in[n] && aligned16(in[n]), "hipq_eltwise_u8: input %d is null or not 16-byte aligned", n);
         hipq_quant_scale((coeff ? coeff[n] : 1.0f) * ialpha[n] / oa, 23, &p.mult[n], &sh[n]);
         smin = std::min(smin, sh[n]);
         p.in[n] = static_cast<const uint8_t *>(in[n]);
@@ -366,8 +479,36 @@ extern "C" int hipq_eltwise_u8(const void *const *in, int n_in, const float *coe
     }
     p.n_in = n_in, p.oz = oz, p.hi = (1 << obits) - 1, p.is_max = operation == HIPQ_ELTWISE_MAX;
     p.y = static_cast<uint8_t *>(y), p.count = count;
-    hipLaunchKernelGGL(eltwise_u8_kernel, dim3(grid_for(count / 4 + 4)), dim3(256), 0,
-                       static_cast<hipStream_t>(stream), p);
+    // 32-bit form: every product below 2^30 (22-bit multipliers), shifts within a word, the sum of n terms and
+    // the folded rounding / zero-point constant without overflow
+    p.fast = p.s0 <= 20 && n_in <= 4;
+    for (int n = 0; n < n_in; n++) {
+        p.fast = p.fast && p.shift[n] <= 30 && p.mult[n] < (1u << 23) && (reinterpret_cast<uintptr_t>(in[n]) & 15) == 0;
+        p.cfast[n] = p.fast ? (1 << (p.shift[n] - 1)) - p.zp[n] * (int32_t)p.mult[n] : 0;
+    }
+    p.fast = p.fast && (reinterpret_cast<uintptr_t>(y) & 15) == 0;
+    p.cadd = p.fast ? (1 << (p.s0 - 1)) + (oz << p.s0) : 0;
+    const dim3 grid(grid_for(count / 16 + 1)), block(256);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define HIPQ_ELT(NIN)                                                                          \
+    if (p.fast && p.is_max)                                                                    \
+        hipLaunchKernelGGL((eltwise_u8_kernel<NIN, true, true>), grid, block, 0, st, p);       \
+    else if (p.fast)                                                                           \
+        hipLaunchKernelGGL((eltwise_u8_kernel<NIN, true, false>), grid, block, 0, st, p);      \
+    else if (p.is_max)                                                                         \
+        hipLaunchKernelGGL((eltwise_u8_kernel<NIN, false, true>), grid, block, 0, st, p);      \
+    else                                                                                       \
+        hipLaunchKernelGGL((eltwise_u8_kernel<NIN, false, false>), grid, block, 0, st, p)
+    if (n_in == 2) {
+        HIPQ_ELT(2);
+    } else if (n_in == 3) {
+        HIPQ_ELT(3);
+    } else if (n_in == 4) {
+        HIPQ_ELT(4);
+    } else {
+        hipLaunchKernelGGL(eltwise_u8_generic_kernel, dim3(grid_for(count)), block, 0, st, p);
+    }
+#undef HIPQ_ELT
     return launch_status("eltwise_u8_kernel");
 }
 
@@ -405,6 +546,14 @@ extern "C" int hipq_pool_u8(const void *x, void *y, int N, int C, int H, int W, 
     hipq_quant_scale(ia / oa, 16, &p.mult, &p.shift);
     p.mult &= 0xffff; // get_quant_scale_int16 stores the multiplier in a uint16_t
     HIPQ_REQUIRE(valid_shift(p.shift), "hipq_pool_u8: scale out of the fixed-point range");
+    if (!p.is_avg && cs % 16 == 0 && p.shift <= 22 && (long long)N * OH * OW * (cs / 16) < (1ll << 31)
+        && (long long)N * H * W * cs < (1ll << 31) && (reinterpret_cast<uintptr_t>(x) & 15) == 0
+        && (reinterpret_cast<uintptr_t>(y) & 15) == 0) {
+        const size_t total16 = (size_t)N * OH * OW * (cs / 16);
+        hipLaunchKernelGGL(pool_max16_u8_kernel, dim3(grid_for(total16)), dim3(256), 0, static_cast<hipStream_t>(stream), p,
+                           1.0 / (cs / 16), 1.0 / OW, 1.0 / OH);
+        return launch_status("pool_max16_u8_kernel");
+    }
     const size_t total = (size_t)N * OH * OW * (cs / 4);
     hipLaunchKernelGGL(pool_u8_kernel, dim3(grid_for(total)), dim3(256), 0, static_cast<hipStream_t>(stream), p);
     return launch_status("pool_u8_kernel");
@@ -420,6 +569,12 @@ extern "C" int hipq_quantize_u8(const float *x, void *y, int N, int C, int H, in
     p.alpha = oa;
     p.beta = -(oa * (float)oz); // quantize.c:152
     p.hi = (float)((1 << obits) - 1);
+    if (cs == 4 && (H * W) % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0
+        && N <= 65535) {
+        const unsigned bx = (unsigned)std::min((H * W / 4 + 255) / 256, 1024);
+        hipLaunchKernelGGL(quantize_u8_c4_kernel, dim3(bx, N), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+        return launch_status("quantize_u8_c4_kernel");
+    }
     const size_t total = (size_t)N * H * W * (cs / 4);
     hipLaunchKernelGGL(quantize_u8_kernel, dim3(grid_for(total)), dim3(256), 0, static_cast<hipStream_t>(stream), p);
     return launch_status("quantize_u8_kernel");

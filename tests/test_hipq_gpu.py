@@ -197,6 +197,19 @@ def test_elementwise():
         assert np.array_equal(got, orc.eltwise_u8([a, b], ia[:2], iz[:2], oa, oz, 1, coeff=[0.5, 1.75]))
         got = hipq.relu_u8(ta, ty, ia[0], iz[0], oa, oz).cpu().numpy()
         assert np.array_equal(got, orc.relu_u8(a, ia[0], iz[0], oa, oz)), ("relu", n)
+        # very unequal scales: shifts beyond the 32-bit forms of add / eltwise (64-bit path), and 4 / 6 inputs
+        wide = [ia[0], float(np.float32(ia[0] * 3.0e-4)), float(np.float32(ia[0] * 40.0))]
+        got = hipq.add_u8(ta, tb, ty, wide[0], iz[0], wide[1], iz[1], wide[0], oz).cpu().numpy()
+        assert np.array_equal(got, orc.add_u8(a, b, wide[0], iz[0], wide[1], iz[1], wide[0], oz)), ("add wide", n)
+        got = hipq.eltwise_u8([ta, tb, tc], ty, wide, iz, wide[0], oz, 1).cpu().numpy()
+        assert np.array_equal(got, orc.eltwise_u8([a, b, c], wide, iz, wide[0], oz, 1)), ("eltwise wide", n)
+        for k in (4, 6):
+            ins = [a, b, c, a[::-1].copy(), b[::-1].copy(), c[::-1].copy()][:k]
+            tins = [torch.from_numpy(v).cuda() for v in ins]
+            iak, izk = (ia * 2)[:k], (iz * 2)[:k]
+            for operation in (1, 2):
+                got = hipq.eltwise_u8(tins, ty, iak, izk, oa, oz, operation).cpu().numpy()
+                assert np.array_equal(got, orc.eltwise_u8(ins, iak, izk, oa, oz, operation)), ("eltwise", k, n, operation)
 
 
 def test_pool():
