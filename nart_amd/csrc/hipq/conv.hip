@@ -222,6 +222,63 @@ __device__ static inline void conv_epilogue(const ConvArgs &a, v16i (&acc)[TN][T
         fused(std::false_type{});
 }
 
+// Epilogue with the residual add applied in the accumulator layout.  The residual tile [BM][BN] was fetched into
+// LDS by the load unit at kernel start (chunk c of row r at chunk c ^ ((r >> 1) & (BN/16 - 1))), so its latency is
+// long gone; each lane reads the dword holding its 4 channels.  Requires the one-multiply requantisation and the
+// 32-bit form of the add (the host checks).  Per element: the convolution's clamped result minus its zero point is
+// clamp(q, lo - zp, hi - zp) with q = (mulhi(acc, mult) + 2^(t-1)) >> t; the add's terms are (d * m + c) >> s; the sum
+// is clamped and packed.  Bit-identical to storing the convolution's bytes and running the add on them.
+template <int BM, int BN, int WM, int WN, int TM, int TN>
+__device__ static inline void conv_epilogue_fused_add(const ConvArgs &a, v16i (&acc)[TN][TM], uint8_t *lds_out,
+                                                      const uint8_t *lds_res, int bm, int bn, int wm, int wn)
+{
+    constexpr int OSTR = BN + 16, CMASK = BN / 16 - 1;
+    const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5;
+    const AddParams &q = a.addq;
+    // operand order of the add: the convolution is input 1 when the residual comes first
+    const int mc = (int)(a.res_first ? q.m1 : q.m0), sc = a.res_first ? q.s1 : q.s0;
+    const int mr = (int)(a.res_first ? q.m0 : q.m1), sr = a.res_first ? q.s0 : q.s1, cr = a.res_first ? q.c0 : q.c1;
+    const int rc = 1 << (sc - 1);                    // rounding of the convolution's term (its zero point cancels)
+    const int qround = 1 << (a.qt - 1);
+    const int dlo = a.lo - a.q.zp, dhi = a.q.hi - a.q.zp; // clamp range of (conv byte - conv zero point)
+#pragma unroll
+    for (int tm = 0; tm < TM; tm++) {
+        const int pl = wm * (TM * 32) + tm * 32 + (lane & 31);
+        const int rsw = (pl >> 1) & CMASK;
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const int chl = wn * (TN * 32) + tn * 32 + g * 8 + half * 4;
+                const uint32_t rv = *reinterpret_cast<const uint32_t *>(lds_res + pl * BN + (((chl >> 4) ^ rsw) << 4) + (chl & 15));
+                uint32_t packed = 0;
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    int32_t d = (__mulhi(acc[tn][tm][g * 4 + e], (int)a.q.mult) + qround) >> a.qt;
+                    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(d) : "v"(d), "s"(dlo), "v"(dhi));
+                    const int32_t t0 = (__mul24(d, mc) + rc) >> sc;
+                    const int32_t t1 = (__mul24((int)((rv >> (8 * e)) & 255), mr) + cr) >> sr;
+                    int32_t y = (t0 + t1 + q.cadd) >> q.sh;
+                    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(y) : "v"(y), "s"(0), "v"(q.hi));
+                    packed |= (uint32_t)y << (8 * e);
+                }
+                *reinterpret_cast<uint32_t *>(lds_out + pl * OSTR + chl) = packed;
+            }
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    constexpr int LPR = BN / 16, RPP = 256 / LPR;
+    const int c16 = (tid % LPR) * 16;
+    if (bn * BN + c16 >= a.out_cs)
+        return;
+#pragma unroll
+    for (int r = tid / LPR; r < BM; r += RPP) {
+        const int m = bm * BM + r;
+        if (m < a.P)
+            *reinterpret_cast<v4i *>(a.y + (size_t)m * a.out_cs + bn * BN + c16) = *reinterpret_cast<const v4i *>(lds_out + r * OSTR + c16);
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // MFMA implicit-GEMM kernel.  SMALLC: input has channel stride 4 (C <= 4, e.g. the RGB stem); then one
 // 16-byte piece is 4 horizontally adjacent taps x 4 channels and k = (r, s padded to 4, c4).
@@ -428,14 +485,17 @@ typedef __attribute__((address_space(3))) void *lptr_t;
 
 // ALIGNED: in_cs is a multiple of 64, so a slab never straddles two taps; the source addresses then advance by
 // a wave-uniform offset and the bounds tests are redone only when the tap changes.
-template <int BM, int BN, int WM, int WN, int NS, bool HAS_WZP, bool ALIGNED>
+// FUSED: the residual add runs in the accumulator layout on a residual tile prefetched into LDS (see
+// conv_epilogue_fused_add); only instantiated for ALIGNED && !HAS_WZP.
+template <int BM, int BN, int WM, int WN, int NS, bool HAS_WZP, bool ALIGNED, bool FUSED = false>
 __global__ __launch_bounds__(256) void conv_mfma_dma_kernel(const ConvArgs a)
 {
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     constexpr int NPB = BM / 64, NPA = BN / 64, LPS = NPA + NPB; // loads per thread and stage
     constexpr int STAGE = (BM + BN) * 64;
     constexpr int OSTR = BN + 16;
-    constexpr int LDS_BYTES = NS * STAGE > BM * OSTR ? NS * STAGE : BM * OSTR;
+    constexpr int STAGES_BYTES = NS * STAGE > BM * OSTR ? NS * STAGE : BM * OSTR;
+    constexpr int LDS_BYTES = STAGES_BYTES + (FUSED ? BM * BN : 0); // the residual tile follows the stages
     static_assert(WM * WN == 4 && TM >= 1 && TN >= 1 && NPB >= 1 && NPA >= 1 && NS >= 2, "tile shape");
     static_assert((NS - 2) * LPS <= 63, "vmcnt range");
     __shared__ __attribute__((aligned(1024))) uint8_t lds[LDS_BYTES];
@@ -543,6 +603,17 @@ __global__ __launch_bounds__(256) void conv_mfma_dma_kernel(const ConvArgs a)
     // first the stage loads, then the (ordinary) loads of the folded bias: the bias loads are YOUNGER than the
     // first NS-1 slabs, which makes the very first wait below conservative (it also waits for slabs 1..NS-2) and
     // every later one exact; in exchange the bias latency overlaps with the activations' on their way from HBM
+    if (FUSED) {
+        // the residual tile first: these loads are the oldest, so every counted wait below covers them as well
+        constexpr int NPR = BM * BN / 4096, CPR = BN / 16;
+#pragma unroll
+        for (int j = 0; j < NPR; j++) {
+            const int sl = tid + 256 * j, r = sl / CPR, c = (sl % CPR) ^ ((r >> 1) & (CPR - 1));
+            const int m = bm * BM + r;
+            const uint8_t *src = (m < a.P && bn * BN + c * 16 < a.out_cs) ? a.res + (size_t)m * a.out_cs + bn * BN + c * 16 : a.padbuf;
+            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(lds + STAGES_BYTES + wave_off + j * 4096), 16, 0, 0);
+        }
+    }
     for (int s = 0; s < NS - 1 && s < a.nslab; s++)
         issue(s);
 
@@ -627,6 +698,10 @@ __global__ __launch_bounds__(256) void conv_mfma_dma_kernel(const ConvArgs a)
             colsum[tm] = a.bwz * (colsum[tm] + __shfl_xor(colsum[tm], 32));
     }
     __syncthreads(); // every wave has finished reading the last stage; no load is in flight any more
+    if (FUSED) {
+        conv_epilogue_fused_add<BM, BN, WM, WN, TM, TN>(a, acc, lds, lds + STAGES_BYTES, bm, bn, wm, wn);
+        return;
+    }
     if (a.fastq && a.lo == 0 && a.q.hi == 255)
         conv_epilogue<BM, BN, WM, WN, HAS_WZP, true, true, TM, TN>(a, acc, colsum, lds, bm, bn, wm, wn);
     else if (a.fastq)
@@ -1118,9 +1193,12 @@ extern "C" void hipq_conv2d_plan_destroy(hipq_conv2d_plan *p)
 
 extern "C" const char *hipq_conv2d_plan_kernel(const hipq_conv2d_plan *p) { return p ? p->name.c_str() : ""; }
 
-// Two load stages everywhere: measured on the ResNet-50 layer shapes, deeper pipelines did not pay, while the smaller
-// LDS footprint lets four work-groups share a CU and overlap their load, multiply and store phases.
+// Load stages.  Short reductions (few slabs) run with two stages: the smaller LDS footprint lets four work-groups
+// share a CU and overlap their load, multiply and store phases.  Long reductions (3x3 layers, wide 1x1 layers) run
+// with four (three for the largest tile): measured inside the whole network, where a layer's input comes from HBM
+// or the last-level cache rather than from a warm L2, the deeper stream is worth 10 % of the ResNet-50 step.
 constexpr int kStages = 2;
+constexpr int kDeepFrom = 8; // slabs
 
 template <int BM, int BN, int WM, int WN>
 static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_t st)
@@ -1134,8 +1212,17 @@ static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_
             hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, false, true>), grid, block, 0, st, a);
     } else if (p->has_wzp) { // rare (asymmetric weights): generic addressing only
         hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, kStages, true, false>), grid, block, 0, st, a);
+    } else if (a.in_cs % 64 == 0 && a.res != nullptr && a.fastq && a.addq.fast && a.acc_out == nullptr && (a.out_cs & 15) == 0) {
+        // residual add in the accumulator layout, residual tile prefetched into LDS
+        if (a.nslab >= kDeepFrom)
+            hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, 3, false, true, true>), grid, block, 0, st, a);
+        else
+            hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, kStages, false, true, true>), grid, block, 0, st, a);
     } else if (a.in_cs % 64 == 0) {
-        hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, kStages, false, true>), grid, block, 0, st, a);
+        if (a.nslab >= kDeepFrom)
+            hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, (BM + BN >= 320 ? 3 : 4), false, true>), grid, block, 0, st, a);
+        else
+            hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, kStages, false, true>), grid, block, 0, st, a);
     } else {
         hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, kStages, false, false>), grid, block, 0, st, a);
     }
