@@ -296,6 +296,58 @@ __global__ __launch_bounds__(256) void pool_max16_u8_kernel(const PoolArgs p, do
     }
 }
 
+// Global average pooling (one window = the whole image, no padding) with a channel stride that is a multiple of 16.
+// A work-group of 256 threads covers 64 groups of 16 channels of one image; the pixels are dealt to 4 thread groups,
+// each thread sums its pixels on packed 16-bit lanes (at most 256 pixels per thread), the 4 partial sums meet in LDS.
+__global__ __launch_bounds__(256) void pool_gavg16_u8_kernel(const PoolArgs p, uint32_t mult, int shift)
+{
+    __shared__ int32_t part[3][64][17];
+    const int c16n = p.cs >> 4, hw = p.H * p.W;
+    const int n = blockIdx.y, chunk = blockIdx.x * 64 + (threadIdx.x & 63), pg = threadIdx.x >> 6;
+    const bool live = chunk < c16n;
+    uint32_t ev[4] = {0, 0, 0, 0}, od[4] = {0, 0, 0, 0};
+    if (live) {
+        const uint8_t *src = p.x + (size_t)n * hw * p.cs + chunk * 16;
+        for (int i = pg; i < hw; i += 4) {
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(src + (size_t)i * p.cs);
+#pragma unroll
+            for (int d = 0; d < 4; d++) {
+                ev[d] += v[d] & 0x00ff00ffu;
+                od[d] += (v[d] >> 8) & 0x00ff00ffu;
+            }
+        }
+    }
+    int32_t sum[16];
+#pragma unroll
+    for (int d = 0; d < 4; d++) {
+        sum[4 * d + 0] = ev[d] & 0xffff, sum[4 * d + 1] = od[d] & 0xffff;
+        sum[4 * d + 2] = ev[d] >> 16, sum[4 * d + 3] = od[d] >> 16;
+    }
+    if (pg > 0) {
+#pragma unroll
+        for (int e = 0; e < 16; e++)
+            part[pg - 1][threadIdx.x & 63][e] = sum[e];
+    }
+    __syncthreads();
+    if (pg == 0 && live) {
+        u32x4 o;
+#pragma unroll
+        for (int d = 0; d < 4; d++) {
+            uint32_t w = 0;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int k = 4 * d + e;
+                const int32_t t = sum[k] + part[0][threadIdx.x][k] + part[1][threadIdx.x][k] + part[2][threadIdx.x][k] -
+                                  hw * p.iz;
+                const int32_t pr = (int32_t)(mult * (uint32_t)t);
+                w |= (uint32_t)sat_hi((int32_t)(rshift_rn(pr, shift) + p.oz), p.hi) << (8 * e);
+            }
+            o[d] = w;
+        }
+        *reinterpret_cast<u32x4 *>(p.y + (size_t)n * p.cs + chunk * 16) = o;
+    }
+}
+
 // ---- quantize (quantize.c:145-157): fp32 NCHW -> uint8 NHWC --------------------------------------
 // One thread produces the 4 channels of one dword of the output; reads are coalesced along W per
 // channel plane, writes along the pixel index.
@@ -553,6 +605,17 @@ extern "C" int hipq_pool_u8(const void *x, void *y, int N, int C, int H, int W, 
         hipLaunchKernelGGL(pool_max16_u8_kernel, dim3(grid_for(total16)), dim3(256), 0, static_cast<hipStream_t>(stream), p,
                            1.0 / (cs / 16), 1.0 / OW, 1.0 / OH);
         return launch_status("pool_max16_u8_kernel");
+    }
+    if (p.is_avg && OH == 1 && OW == 1 && ph == 0 && pw == 0 && kh >= H && kw >= W && cs % 16 == 0 && H * W <= 1024
+        && N <= 65535 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0) {
+        uint32_t mult;
+        int shift;
+        hipq_quant_scale(p.ia_over_oa / (float)(uint32_t)(H * W), 16, &mult, &shift); // pool.c:211-216
+        if (valid_shift(shift)) {
+            hipLaunchKernelGGL(pool_gavg16_u8_kernel, dim3((cs / 16 + 63) / 64, N), dim3(256), 0,
+                               static_cast<hipStream_t>(stream), p, mult, shift);
+            return launch_status("pool_gavg16_u8_kernel");
+        }
     }
     const size_t total = (size_t)N * OH * OW * (cs / 4);
     hipLaunchKernelGGL(pool_u8_kernel, dim3(grid_for(total)), dim3(256), 0, static_cast<hipStream_t>(stream), p);

@@ -215,7 +215,10 @@ def test_elementwise():
 def test_pool():
     rng = np.random.default_rng(16)
     cases = [(2, 64, 112, 112, 3, 1, 2, 0, False), (2, 64, 13, 13, 3, 1, 2, 0, True), (3, 40, 7, 7, 7, 0, 1, 1, True),
-             (1, 20, 9, 11, 3, 1, 2, 1, True), (1, 3, 8, 8, 2, 0, 2, 1, False), (2, 17, 10, 10, (3, 2), (1, 0), (2, 1), 1, True)]
+             (1, 20, 9, 11, 3, 1, 2, 1, True), (1, 3, 8, 8, 2, 0, 2, 1, False), (2, 17, 10, 10, (3, 2), (1, 0), (2, 1), 1, True),
+             # global average windows: the one-work-group-per-image kernel, its 1024-pixel limit and the generic fallback
+             (5, 2048, 7, 7, 7, 0, 1, 1, False), (2, 1280, 7, 7, 7, 0, 7, 1, True), (2, 200, 32, 32, 32, 0, 1, 1, False),
+             (1, 16, 33, 33, 33, 0, 1, 1, False), (2, 1040, 5, 3, (5, 3), 0, 1, 1, False)]
     for N, C, H, W, k, pad, st, method, ceil_mode in cases:
         x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
         q = (rand_q(rng), int(rng.integers(0, 256)), rand_q(rng), int(rng.integers(0, 256)))
