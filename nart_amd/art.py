@@ -189,8 +189,9 @@ class Op:
         assert ok, "op_setting_array_set(%#x) refused" % item
         return self
 
-    def set_quant(self, ialpha=None, izp=None, walpha=None, wzp=None, oalpha=None, ozp=None, bits=8):
+    def set_quant(self, ialpha=None, izp=None, walpha=None, wzp=None, oalpha=None, ozp=None, bits=8, obits=None):
         """The SETTING_QUANT_* arrays every quant op reads (e.g. conv_2d.c:42-69)."""
+        obits = bits if obits is None else obits
         if ialpha is not None:
             ia = np.atleast_1d(np.asarray(ialpha, dtype=np.float32))
             self.set_array(SETTING_QUANT_IALPHA, dtFLOAT32, ia)
@@ -203,7 +204,7 @@ class Op:
         if oalpha is not None:
             self.set_array(SETTING_QUANT_OALPHA, dtFLOAT32, [oalpha])
             self.set_array(SETTING_QUANT_OZERO_POINT, dtUINT8, [ozp])
-            self.set_array(SETTING_QUANT_OBITS, dtUINT8, [bits])
+            self.set_array(SETTING_QUANT_OBITS, dtUINT8, [obits])
         return self
 
     def config(self):
@@ -301,12 +302,16 @@ class Workspace:
         op.set_single(SETTING_POOL_CEIL_MODE, dtBOOL, int(ceil_mode))
         return op.set_quant(**q).config()
 
-    def quantize(self, x, oalpha, ozp, bits=8):
+    def quantize(self, x, oalpha, ozp, bits=8, qtype=None):
         op = self.new_op(OP_QUANT_QUANTIZE, [x])
+        if qtype is not None:  # SETTING_QUANT_DEFAULT / _BIASED / _SYMMETRIC (quant_op_settings.h:38-41)
+            op.set_single(SETTING_QUANT_QTYPE, dtINT32, qtype)
         return op.set_quant(oalpha=oalpha, ozp=ozp, bits=bits).config()
 
-    def dequantize(self, x, ialpha, izp, bits=8):
+    def dequantize(self, x, ialpha, izp, bits=8, qtype=None):
         op = self.new_op(OP_QUANT_DEQUANTIZE, [x])
+        if qtype is not None:
+            op.set_single(SETTING_QUANT_QTYPE, dtINT32, qtype)
         return op.set_quant(ialpha=ialpha, izp=izp, bits=bits).config()
 
     def reshape_flatten(self, x, axis=1):

@@ -166,6 +166,50 @@ def dequantize_u8(x, ialpha, izp):
     return y
 
 
+def conv2d_i8(x, w, bias, pad, stride, group, ialpha, walpha, oalpha, obits=8, return_acc=False):
+    x = np.ascontiguousarray(x, np.int8)
+    w = np.ascontiguousarray(w, np.int8)
+    bias = None if bias is None else np.ascontiguousarray(bias, np.int32)
+    N, Cc, H, W = x.shape
+    K, _, R, S = w.shape
+    (ph, pw), (sh, sw) = _pair(pad), _pair(stride)
+    OH, OW = conv_out_dim(H, ph, R, sh), conv_out_dim(W, pw, S, sw)
+    y = np.empty((N, K, OH, OW), np.int8)
+    acc = np.empty((N, K, OH, OW), np.int32) if return_acc else None
+    lib().orc_conv2d_i8(_p(x), _p(w), _p(bias), _p(y), _p(acc), N, Cc, H, W, K, R, S, ph, pw, sh, sw, group,
+                        _f(ialpha), _f(walpha), _f(oalpha), int(obits))
+    return (y, acc) if return_acc else y
+
+
+def ip_i8(x, w, bias, ialpha, walpha, oalpha, obits=8, return_acc=False):
+    x = np.ascontiguousarray(x, np.int8)
+    w = np.ascontiguousarray(w, np.int8)
+    bias = None if bias is None else np.ascontiguousarray(bias, np.int32)
+    M = x.shape[0]
+    Kd = int(np.prod(x.shape[1:]))
+    Nout = w.shape[0]
+    assert int(np.prod(w.shape[1:])) == Kd
+    y = np.empty((M, Nout), np.int8)
+    acc = np.empty((M, Nout), np.int32) if return_acc else None
+    lib().orc_ip_i8(_p(x), _p(w), _p(bias), _p(y), _p(acc), M, Kd, Nout, _f(ialpha), _f(walpha), _f(oalpha),
+                    int(obits))
+    return (y, acc) if return_acc else y
+
+
+def quantize_i8(x, oalpha, obits=8):
+    x = np.ascontiguousarray(x, np.float32)
+    y = np.empty(x.shape, np.int8)
+    lib().orc_quantize_i8(_p(x), _p(y), C.c_size_t(x.size), _f(oalpha), int(obits))
+    return y
+
+
+def dequantize_i8(x, ialpha):
+    x = np.ascontiguousarray(x, np.int8)
+    y = np.empty(x.shape, np.float32)
+    lib().orc_dequantize_i8(_p(x), _p(y), C.c_size_t(x.size), _f(ialpha))
+    return y
+
+
 class XorShift:
     """The generator of the recorded conv known answers (state 0x9E3779B97F4A7C15 at the start of a case)."""
 

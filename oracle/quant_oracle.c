@@ -390,6 +390,102 @@ void orc_dequantize_u8(const uint8_t *x, float *y, size_t count, float ialpha, i
         y[i] = (float)((int)x[i] - izp) * ialpha; /* dequantize.c:121 */
 }
 
+/* ---- int8 symmetric variants (no zero points) --------------------------------------------------- */
+
+/* ssaturate_int_by_bits — quant_helper.h:43-47: clip to +-(2^bits - 1), then the implicit conversion of the
+ * int result to the int8_t return type (two's complement truncation; with bits = 8 values beyond +-127 wrap). */
+int8_t orc_ssat_bits(int32_t x, int bits)
+{
+    const int32_t m = (1 << bits) - 1;
+    const int32_t c = x > m ? m : (x < -m ? -m : x);
+    return (int8_t)(uint8_t)((uint32_t)c & 255u);
+}
+
+static inline int8_t requant_acc_i8(int32_t acc, uint32_t mult, int shift, int obits)
+{
+    /* conv_2d_int8_impl.c:148-172, ip.cpp:268-272: the int64 result of rshift_rn is passed to an int32_t parameter */
+    return orc_ssat_bits((int32_t)orc_rshift_rn((int64_t)acc * (int64_t)mult, shift), obits);
+}
+
+/* op_conv_2d_i8xi8_run — conv_2d_int8_impl.c:34-174 with im2col_i8 (utils/im2col.cpp:22-116: out-of-image taps
+ * are 0) and the portable branch of gemm_i8xi8 (gemm/default/gemm.c:257-303: int32 += int8 * int8). */
+void orc_conv2d_i8(const int8_t *x, const int8_t *w, const int32_t *bias, int8_t *y, int32_t *acc_out, int N,
+                   int C, int H, int W, int K, int R, int S, int pad_h, int pad_w, int stride_h, int stride_w,
+                   int group, float ialpha, float walpha, float oalpha, int obits)
+{
+    const int OH = orc_conv_out_dim(H, pad_h, R, stride_h);
+    const int OW = orc_conv_out_dim(W, pad_w, S, stride_w);
+    const int cg = C / group, kg = K / group;
+    uint32_t mult;
+    int shift;
+    orc_quant_scale(ialpha * walpha / oalpha, 32, &mult, &shift);
+    for (int n = 0; n < N; n++)
+        for (int k = 0; k < K; k++) {
+            const int g = k / kg;
+            for (int oh = 0; oh < OH; oh++)
+                for (int ow = 0; ow < OW; ow++) {
+                    uint32_t acc = bias ? (uint32_t)bias[k] : 0u;
+                    for (int c = 0; c < cg; c++)
+                        for (int r = 0; r < R; r++) {
+                            const int ih = oh * stride_h - pad_h + r;
+                            if (ih < 0 || ih >= H)
+                                continue;
+                            for (int s = 0; s < S; s++) {
+                                const int iw = ow * stride_w - pad_w + s;
+                                if (iw < 0 || iw >= W)
+                                    continue;
+                                const int32_t xv = x[(((size_t)n * C + (size_t)g * cg + c) * H + ih) * W + iw];
+                                const int32_t wv = w[(((size_t)k * cg + c) * R + r) * S + s];
+                                acc += (uint32_t)(xv * wv);
+                            }
+                        }
+                    const size_t o = (((size_t)n * K + k) * OH + oh) * OW + ow;
+                    if (acc_out)
+                        acc_out[o] = (int32_t)acc;
+                    y[o] = requant_acc_i8((int32_t)acc, mult, shift, obits);
+                }
+        }
+}
+
+/* op_quant_ip_i8xi8_run — ip.cpp:211-274. */
+void orc_ip_i8(const int8_t *x, const int8_t *w, const int32_t *bias, int8_t *y, int32_t *acc_out, int M,
+               int Kdim, int Nout, float ialpha, float walpha, float oalpha, int obits)
+{
+    uint32_t mult;
+    int shift;
+    orc_quant_scale(ialpha * walpha / oalpha, 32, &mult, &shift);
+    for (int m = 0; m < M; m++)
+        for (int n = 0; n < Nout; n++) {
+            uint32_t acc = bias ? (uint32_t)bias[n] : 0u;
+            for (int k = 0; k < Kdim; k++)
+                acc += (uint32_t)((int32_t)x[(size_t)m * Kdim + k] * (int32_t)w[(size_t)n * Kdim + k]);
+            if (acc_out)
+                acc_out[(size_t)m * Nout + n] = (int32_t)acc;
+            y[(size_t)m * Nout + n] = requant_acc_i8((int32_t)acc, mult, shift, obits);
+        }
+}
+
+/* op_quantize_run_i8 — quantize.c:159-185: alpha = (float)(1.0 / oalpha) (a double division), the product is
+ * fp32, round() is the C library's (half away from zero), the double -> int conversion of clip()'s argument is
+ * x86-64's cvttsd2si: values outside int32 (and NaN) become INT32_MIN. */
+void orc_quantize_i8(const float *x, int8_t *y, size_t count, float oalpha, int obits)
+{
+    const float alpha = (float)(1. / (double)oalpha);
+    const int l = (int)((1l << (obits - 1)) - 1);
+    for (size_t i = 0; i < count; i++) {
+        const double r = round((double)(x[i] * alpha));
+        const int32_t v = (r >= -2147483648.0 && r < 2147483648.0) ? (int32_t)r : INT32_MIN;
+        y[i] = (int8_t)(v > l ? l : (v < -l ? -l : v));
+    }
+}
+
+/* op_dequantize_run_i8 — dequantize.c:125-136. */
+void orc_dequantize_i8(const int8_t *x, float *y, size_t count, float ialpha)
+{
+    for (size_t i = 0; i < count; i++)
+        y[i] = (float)x[i] * ialpha;
+}
+
 uint64_t orc_fnv1a64(const uint8_t *p, size_t n)
 {
     uint64_t h = 1469598103934665603ull;

@@ -94,6 +94,21 @@ void orc_quantize_u8(const float *x, uint8_t *y, size_t count, float oalpha, int
 /* op_dequantize_run_u8 — dequantize.c:111-123. */
 void orc_dequantize_u8(const uint8_t *x, float *y, size_t count, float ialpha, int izp);
 
+/* ---- int8 symmetric variants: no zero points, outputs clipped to +-(2^obits - 1) and truncated to int8 ---- */
+/* ssaturate_int_by_bits — quant_helper.h:43-47. */
+int8_t orc_ssat_bits(int32_t x, int bits);
+/* op_conv_2d_i8xi8_run — conv_2d_int8_impl.c:34-174 (x86-64 branch: gemm_i8xi8, i.e. ibits or wbits == 8). */
+void orc_conv2d_i8(const int8_t *x, const int8_t *w, const int32_t *bias, int8_t *y, int32_t *acc_out, int N,
+                   int C, int H, int W, int K, int R, int S, int pad_h, int pad_w, int stride_h, int stride_w,
+                   int group, float ialpha, float walpha, float oalpha, int obits);
+/* op_quant_ip_i8xi8_run — ip.cpp:211-274. */
+void orc_ip_i8(const int8_t *x, const int8_t *w, const int32_t *bias, int8_t *y, int32_t *acc_out, int M,
+               int Kdim, int Nout, float ialpha, float walpha, float oalpha, int obits);
+/* op_quantize_run_i8 — quantize.c:159-185. */
+void orc_quantize_i8(const float *x, int8_t *y, size_t count, float oalpha, int obits);
+/* op_dequantize_run_i8 — dequantize.c:125-136. */
+void orc_dequantize_i8(const int8_t *x, float *y, size_t count, float ialpha);
+
 /* FNV-1a-64 over a byte buffer (the checksum the recorded known answers use). */
 uint64_t orc_fnv1a64(const uint8_t *p, size_t n);
 

@@ -82,3 +82,37 @@ def quantize_u8(ws, x, oalpha, ozp):
 
 def dequantize_u8(ws, x, ialpha, izp):
     return _run(ws.dequantize(ws.tensor(x), ialpha, izp))
+
+
+# ---- int8 symmetric variants (zero points are ignored by these operators; 0 is passed) ----------
+def conv2d_i8(ws, x, w, bias, pad, stride, group, ialpha, walpha, oalpha, obits=8):
+    """Without a bias tensor the reference accumulates into an int32 buffer it never clears
+    (conv_2d_int8_impl.c:82-93 initialises it only when there are three inputs), which is only right on
+    never-touched pages; a bias of zeros states the intended result."""
+    q = _q(ialpha=ialpha, izp=0, walpha=walpha, wzp=0, oalpha=oalpha, ozp=0, obits=obits)
+    if bias is None and ws.name.startswith("quant"):
+        bias = np.zeros(w.shape[0], np.int32)
+    tb = ws.tensor(np.asarray(bias, np.int32)) if bias is not None else None
+    tw = ws.tensor(np.asarray(w, np.int8))
+    # the reference sizes its accumulator buffer for one image (conv_2d_int8_impl.c:28, :77): feed it one at a time
+    per_image = ws.name.startswith("quant")
+    x = np.asarray(x, np.int8)
+    chunks = [x[i:i + 1] for i in range(x.shape[0])] if per_image else [x]
+    return np.concatenate([_run(ws.conv2d(ws.tensor(xc), tw, tb, pad, stride, group, q)) for xc in chunks], 0)
+
+
+def ip_i8(ws, x, w, bias, ialpha, walpha, oalpha, obits=8):
+    q = _q(ialpha=ialpha, izp=0, walpha=walpha, wzp=0, oalpha=oalpha, ozp=0, obits=obits)
+    if x.ndim == 2:
+        x = x.reshape(x.shape[0], x.shape[1], 1, 1)
+    tb = ws.tensor(np.asarray(bias, np.int32)) if bias is not None else None
+    return _run(ws.ip(ws.tensor(np.asarray(x, np.int8)), ws.tensor(np.asarray(w, np.int8)), tb, q))
+
+
+def quantize_i8(ws, x, oalpha, obits=8):
+    return _run(ws.quantize(ws.tensor(np.asarray(x, np.float32)), oalpha, 0, bits=obits, qtype=2))
+
+
+def dequantize_i8(ws, x, ialpha, ibits=8):
+    # the operator is chosen from (qtype, ibits), not from the tensor's dtype (dequantize.c:141-161)
+    return _run(ws.dequantize(ws.tensor(np.asarray(x, np.int8)), ialpha, 0, bits=ibits, qtype=2))

@@ -161,6 +161,57 @@ def test_quantize_dequantize_vs_reference(ref_ws):
         assert np.array_equal(orc.dequantize_u8(want, oa, oz).view(np.uint32), d.view(np.uint32))
 
 
+def test_int8_conv_vs_reference(ref_ws):
+    """op_conv_2d_i8xi8_run with the portable gemm_i8xi8 (ibits == wbits == 8; the lower-bit GEMMs are not
+    implemented outside aarch64).  7x7 kernels take the reference's region-split im2col and are left out."""
+    rng = np.random.default_rng(21)
+    for it in range(50):
+        grp = int(rng.choice([1, 1, 1, 2, 4]))
+        C = grp * int(rng.integers(1, 9))
+        K = grp * int(rng.integers(1, 9))
+        if it % 10 == 0:
+            grp = C = K = int(rng.integers(2, 12))
+        R, S = int(rng.integers(1, 6)), int(rng.integers(1, 6))
+        H, W = int(rng.integers(R, R + 12)), int(rng.integers(S, S + 12))
+        pad = (int(rng.integers(0, R)), int(rng.integers(0, S)))
+        st = (int(rng.integers(1, 4)), int(rng.integers(1, 4)))
+        N = int(rng.integers(1, 4))
+        x = rng.integers(-128, 128, (N, C, H, W), dtype=np.int8)
+        w = rng.integers(-128, 128, (K, C // grp, R, S), dtype=np.int8)
+        b = rng.integers(-20000, 20000, K).astype(np.int32) if it % 4 else None
+        q = (rand_q(rng), rand_q(rng), rand_q(rng, 1e-2, 1.0))
+        obits = int(rng.choice([8, 8, 7, 4]))
+        want = refrun.conv2d_i8(ref_ws, x, w, b, pad, st, grp, *q, obits=obits)
+        got = orc.conv2d_i8(x, w, b, pad, st, grp, *q, obits=obits)
+        assert want.dtype == np.int8 and np.array_equal(got, want), (it, x.shape, w.shape, pad, st, grp, q, obits)
+
+
+def test_int8_ip_vs_reference(ref_ws):
+    rng = np.random.default_rng(22)
+    for it in range(25):
+        M, Kd, No = int(rng.integers(1, 6)), int(rng.integers(1, 400)), int(rng.integers(1, 50))
+        x = rng.integers(-128, 128, (M, Kd), dtype=np.int8)
+        w = rng.integers(-128, 128, (No, Kd), dtype=np.int8)
+        b = rng.integers(-50000, 50000, No).astype(np.int32) if it % 3 else None
+        q = (rand_q(rng), rand_q(rng), rand_q(rng, 1e-2, 1.0))
+        obits = int(rng.choice([8, 7]))
+        assert np.array_equal(orc.ip_i8(x, w, b, *q, obits=obits), refrun.ip_i8(ref_ws, x, w, b, *q, obits=obits)), (it, q)
+
+
+def test_int8_quantize_dequantize_vs_reference(ref_ws):
+    rng = np.random.default_rng(23)
+    for it in range(12):
+        oa = rand_q(rng, 5e-3, 0.1)
+        obits = int(rng.choice([8, 8, 7, 6, 4, 3, 2]))
+        x = (rng.standard_normal((2, 3, 20, 20)) * 60 * oa).astype(np.float32)
+        x.flat[:600] = (np.arange(600, dtype=np.float32) * 0.5 - 150) * np.float32(oa)  # ties of both signs, both clips
+        x.flat[600:606] = [3e9, -3e9, 1e30, -1e30, np.inf, -np.inf]  # beyond int32: the conversion's sentinel
+        want = refrun.quantize_i8(ref_ws, x, oa, obits)
+        assert want.dtype == np.int8 and np.array_equal(orc.quantize_i8(x, oa, obits), want), (it, oa, obits)
+        d = refrun.dequantize_i8(ref_ws, want, oa, obits)
+        assert np.array_equal(orc.dequantize_i8(want, oa).view(np.uint32), d.view(np.uint32))
+
+
 # ----------------------------------------------------------------------------------------------
 # 3. committed golden outputs of the compiled reference
 def test_golden_outputs():
@@ -189,6 +240,28 @@ def test_golden_outputs():
         else:
             raise AssertionError(kind)
         assert got.shape == want.shape, name
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), name
+
+
+def test_golden_outputs_int8():
+    g = np.load(os.path.join(GOLD, "quant_ops_int8.npz"))
+    meta = json.loads(bytes(g["meta"]).decode())
+    assert len(meta) == 10
+    for name, m in meta.items():
+        kind, a = m["kind"], m["args"]
+        ins = [g["%s.in%d" % (name, i)] for i in range(m["n_in"])]
+        want = g[name + ".out"]
+        if kind == "conv":
+            got = orc.conv2d_i8(ins[0], ins[1], ins[2], a["pad"], a["stride"], a["group"], *a["q"], obits=a["obits"])
+        elif kind == "ip":
+            got = orc.ip_i8(ins[0], ins[1], ins[2], *a["q"], obits=a["obits"])
+        elif kind == "quantize":
+            got = orc.quantize_i8(ins[0], *a["q"], obits=a["obits"])
+        elif kind == "dequantize":
+            got = orc.dequantize_i8(ins[0], *a["q"])
+        else:
+            raise AssertionError(kind)
+        assert got.shape == want.shape and got.dtype == want.dtype, name
         assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), name
 
 
@@ -310,3 +383,52 @@ def test_pool_closed_forms():
     # global average, same scales: round-half-up mean to within the 15-bit multiplier's precision
     y = orc.pool_u8(x, 6, 0, 1, 1, True, 0.05, 0, 0.05, 0).astype(np.float64).ravel()
     assert np.max(np.abs(y - x.reshape(6, 36).mean(axis=1))) <= 0.51
+
+
+def test_int8_conv_against_int64_tensordot():
+    """Signed conv: zero padding, no zero points, clip to +-(2^obits - 1) then two's complement truncation."""
+    rng = np.random.default_rng(31)
+    for it in range(12):
+        grp = int(rng.choice([1, 2]))
+        C, K = grp * int(rng.integers(1, 6)), grp * int(rng.integers(1, 6))
+        R, S = int(rng.integers(1, 4)), int(rng.integers(1, 4))
+        H, W = int(rng.integers(R, 9)), int(rng.integers(S, 9))
+        ph, pw, sh, sw = int(rng.integers(0, R)), int(rng.integers(0, S)), int(rng.integers(1, 3)), int(rng.integers(1, 3))
+        x = rng.integers(-128, 128, (2, C, H, W), dtype=np.int8)
+        w = rng.integers(-128, 128, (K, C // grp, R, S), dtype=np.int8)
+        b = rng.integers(-5000, 5000, K).astype(np.int32)
+        ia, wa, oa = rand_q(rng), rand_q(rng), rand_q(rng, 1e-2, 1.0)
+        obits = int(rng.choice([8, 7, 5]))
+        y, acc = orc.conv2d_i8(x, w, b, (ph, pw), (sh, sw), grp, ia, wa, oa, obits, return_acc=True)
+        OH, OW = (H + 2 * ph - R) // sh + 1, (W + 2 * pw - S) // sw + 1
+        xp = np.pad(x.astype(np.int64), ((0, 0), (0, 0), (ph, ph), (pw, pw)))
+        ref = np.zeros((2, K, OH, OW), np.int64) + b[None, :, None, None]
+        cg, kg = C // grp, K // grp
+        for g in range(grp):
+            for r in range(R):
+                for s in range(S):
+                    win = xp[:, g * cg:(g + 1) * cg, r:r + sh * (OH - 1) + 1:sh, s:s + sw * (OW - 1) + 1:sw]
+                    ref[:, g * kg:(g + 1) * kg] += np.einsum("nchw,kc->nkhw", win, w[g * kg:(g + 1) * kg, :, r, s].astype(np.int64))
+        assert np.array_equal(acc, ref)
+        mult, shift = orc.quant_scale(np.float32(ia) * np.float32(wa) / np.float32(oa), 32)
+        m = (1 << obits) - 1
+        q = np.array([int(Fraction(int(v) * mult, 1 << shift) + Fraction(1, 2)) if (int(v) * mult) % (1 << shift) == 0
+                      else (int(v) * mult + (1 << (shift - 1))) >> shift for v in ref.ravel()], dtype=np.int64)
+        want = (np.clip(q, -m, m) & 255).astype(np.uint8).view(np.int8).reshape(ref.shape)
+        assert np.array_equal(y, want), (it, obits)
+
+
+def test_int8_quantize_formula():
+    """clip(round_half_away(fp32(x * fp32(1/alpha))), +-(2^(bits-1) - 1)); dequantize is one fp32 product."""
+    rng = np.random.default_rng(32)
+    for bits in (8, 7, 4, 2):
+        oa = np.float32(rand_q(rng, 5e-3, 0.1))
+        x = (rng.standard_normal(4000) * 80 * oa).astype(np.float32)
+        inv = np.float32(1.0 / np.float64(oa))
+        p = (x * inv).astype(np.float64)
+        r = np.sign(p) * np.floor(np.abs(p) + 0.5)
+        lim = (1 << (bits - 1)) - 1
+        want = np.clip(r, -lim, lim).astype(np.int8)
+        got = orc.quantize_i8(x, oa, bits)
+        assert np.array_equal(got, want), bits
+        assert np.array_equal(orc.dequantize_i8(got, oa), got.astype(np.float32) * oa)
