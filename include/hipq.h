@@ -34,13 +34,15 @@
 extern "C" {
 #endif
 
-#define HIPQ_ABI_VERSION 1
+#define HIPQ_ABI_VERSION 2
 
 #define HIPQ_ELTWISE_SUM 1 /* SETTING_ELTWISE_OP_SUM */
 #define HIPQ_ELTWISE_MAX 2 /* SETTING_ELTWISE_OP_MAX */
 #define HIPQ_POOL_MAX 0    /* SETTING_POOL_MAX */
 #define HIPQ_POOL_AVE 1    /* SETTING_POOL_AVE */
 #define HIPQ_MAX_ELTWISE_INPUTS 8
+#define HIPQ_DTYPE_U8 0
+#define HIPQ_DTYPE_I8 1
 
 int hipq_abi_version(void);
 const char *hipq_last_error(void);
@@ -68,6 +70,12 @@ typedef struct hipq_conv2d_desc {
     int32_t obits;            /* output saturates to [0, 2^obits - 1] */
     int32_t relu;             /* 1: y = max(y, ozp) after requantisation (== a following quant relu
                                  op with equal in/out scale and zero point, src/op/relu.c:76-115) */
+    int32_t dtype;            /* HIPQ_DTYPE_U8 (0): asymmetric uint8 tensors, op_conv_2d_u8xu8_run.
+                                 HIPQ_DTYPE_I8: int8 symmetric x, w and y, op_conv_2d_i8xi8_run
+                                 (src/op/conv_2d_int8_impl.c:34-174) / op_quant_ip_i8xi8_run (src/op/ip.cpp:211-274):
+                                 zero points are ignored, taps outside the image are 0, y is
+                                 clip(v, -(2^obits - 1), 2^obits - 1) truncated to int8 (ssaturate_int_by_bits,
+                                 quant_helper.h:43-47; obits = 8 wraps beyond +-127 exactly as the reference does) */
 } hipq_conv2d_desc;
 
 typedef struct hipq_conv2d_plan hipq_conv2d_plan;
@@ -140,6 +148,14 @@ int hipq_quantize_u8(const float *x_nchw, void *y_nhwc, int N, int C, int H, int
 /* op_dequantize_run_u8 — src/op/dequantize.c:111-123: x uint8 NHWC, y fp32 dense NCHW. */
 int hipq_dequantize_u8(const void *x_nhwc, float *y_nchw, int N, int C, int H, int W, int cs,
                        float ialpha, int izp, void *stream);
+
+/* op_quantize_run_i8 — src/op/quantize.c:159-185 (qtype SYMMETRIC, 2..8 bits): y int8 NHWC,
+ * y = clip(round(x * (float)(1.0 / oalpha)), -(2^(obits-1) - 1), 2^(obits-1) - 1). */
+int hipq_quantize_i8(const float *x_nchw, void *y_nhwc, int N, int C, int H, int W, int cs,
+                     float oalpha, int obits, void *stream);
+/* op_dequantize_run_i8 — src/op/dequantize.c:125-136: x int8 NHWC, y = x * ialpha, fp32 dense NCHW. */
+int hipq_dequantize_i8(const void *x_nhwc, float *y_nchw, int N, int C, int H, int W, int cs,
+                       float ialpha, void *stream);
 
 /* A plain device-to-device copy kernel of known size; the calibration reference for HBM counters. */
 int hipq_copy_bytes(const void *src, void *dst, size_t count, void *stream);

@@ -68,6 +68,8 @@ struct ConvArgs {
     int bwz;          // b = 128 - wzp
     int izp, wzp;     // for the non-MFMA kernels
     uint32_t padword; // byte izp in all four lanes
+    uint32_t xmask;   // MFMA kernels: 0x80808080 re-centres uint8 activations, 0 leaves int8 activations alone
+    int sx;           // other kernels: bytes are read as (byte ^ sx) - zero point; 0x80 with zero points 128 == int8
     Requant q;
     int lo;    // lower clamp: ozp when ReLU is fused, else 0
     int fastq; // 1: the one-multiply requantisation is valid for q.shift
@@ -109,6 +111,13 @@ __device__ static inline int32_t conv_requant(const ConvArgs &a, int32_t v)
     return out;
 }
 
+// Pack the low bytes of four values into a dword (three v_perm_b32 / v_or_b32; works for negative values, whose
+// low byte is their two's complement int8).
+__device__ static inline uint32_t pack_low_bytes(int32_t r0, int32_t r1, int32_t r2, int32_t r3)
+{
+    return __builtin_amdgcn_perm((uint32_t)r1, (uint32_t)r0, 0x0c0c0400u) | __builtin_amdgcn_perm((uint32_t)r3, (uint32_t)r2, 0x04000c0cu);
+}
+
 template <int BM, int BN, int WM, int WN, bool HAS_WZP, bool FAST, bool PLAIN_SAT, int TM, int TN>
 __device__ static inline void conv_epilogue(const ConvArgs &a, v16i (&acc)[TN][TM], int (&colsum)[TM], uint8_t *lds,
                                             int bm, int bn, int wm, int wn)
@@ -131,14 +140,15 @@ __device__ static inline void conv_epilogue(const ConvArgs &a, v16i (&acc)[TN][T
                     const int ko = ch0 + tn * 32 + g * 8 + half * 4;
                     if (ko >= a.out_cs)
                         continue;
-                    uint32_t packed = 0;
+                    int32_t rq[4];
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         const int32_t v = (int32_t)((uint32_t)acc[tn][tm][g * 4 + e] + (HAS_WZP ? (uint32_t)colsum[tm] : 0u));
                         if (a.acc_out)
                             a.acc_out[(size_t)m * a.out_cs + ko + e] = v;
-                        packed |= (uint32_t)conv_requant<FAST>(a, v) << (8 * e);
+                        rq[e] = conv_requant<FAST>(a, v);
                     }
+                    uint32_t packed = pack_low_bytes(rq[0], rq[1], rq[2], rq[3]);
                     if (a.res) {
                         const uint32_t rv = *reinterpret_cast<const uint32_t *>(a.res + (size_t)m * a.out_cs + ko);
                         packed = a.res_first ? add_dword<false>(rv, packed, a.addq) : add_dword<false>(packed, rv, a.addq);
@@ -173,11 +183,13 @@ __device__ static inline void conv_epilogue(const ConvArgs &a, v16i (&acc)[TN][T
                     asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
                     packed = (b01 & 0xffffu) | (b23 << 16);
                 } else {
+                    int32_t rq[4];
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         const int32_t v = (int32_t)((uint32_t)acc[tn][tm][g * 4 + e] + (HAS_WZP ? (uint32_t)colsum[tm] : 0u));
-                        packed |= (uint32_t)conv_requant<FAST>(a, v) << (8 * e);
+                        rq[e] = conv_requant<FAST>(a, v);
                     }
+                    packed = pack_low_bytes(rq[0], rq[1], rq[2], rq[3]);
                 }
                 *reinterpret_cast<uint32_t *>(lds + pl * OSTR + wn * (TN * 32) + tn * 32 + g * 8 + half * 4) = packed;
             }
@@ -428,7 +440,7 @@ __global__ __launch_bounds__(256) void conv_mfma_kernel(const ConvArgs a)
                 af[tn] = *reinterpret_cast<const v4i *>(buf + arow + tn * 2048 + fo);
 #pragma unroll
             for (int tm = 0; tm < TM; tm++)
-                bf[tm] = *reinterpret_cast<const v4i *>(buf + brow + tm * 2048 + fo) ^ (int)0x80808080;
+                bf[tm] = *reinterpret_cast<const v4i *>(buf + brow + tm * 2048 + fo) ^ (int)a.xmask;
 #pragma unroll
             for (int tn = 0; tn < TN; tn++)
 #pragma unroll
@@ -660,7 +672,7 @@ __global__ __launch_bounds__(256) void conv_mfma_dma_kernel(const ConvArgs a)
     auto multiply = [&](v4i(&af)[TN], v4i(&bf)[TM]) {
 #pragma unroll
         for (int tm = 0; tm < TM; tm++)
-            bf[tm] ^= (int)0x80808080;
+            bf[tm] ^= (int)a.xmask;
 #pragma unroll
         for (int tn = 0; tn < TN; tn++)
 #pragma unroll
@@ -921,7 +933,7 @@ __global__ __launch_bounds__(256) void conv_depthwise_kernel(const ConvArgs a)
                 const int16_t *wp = wq + (size_t)(r * a.S + s) * a.in_cs + c0;
 #pragma unroll
                 for (int e = 0; e < 4; e++)
-                    acc[e] += ((int)((xv >> (8 * e)) & 255) - a.izp) * (int)wp[e];
+                    acc[e] += ((int)(((xv >> (8 * e)) & 255) ^ (uint32_t)a.sx) - a.izp) * (int)wp[e];
             }
         }
         uint32_t packed = 0;
@@ -929,9 +941,7 @@ __global__ __launch_bounds__(256) void conv_depthwise_kernel(const ConvArgs a)
         for (int e = 0; e < 4; e++) {
             if (a.acc_out)
                 a.acc_out[(size_t)m * a.out_cs + c0 + e] = acc[e];
-            int32_t r = requant_acc(acc[e], a.q);
-            r = r < a.lo ? a.lo : r;
-            packed |= (uint32_t)r << (8 * e);
+            packed |= (uint32_t)(conv_requant<false>(a, acc[e]) & 255) << (8 * e);
         }
         *reinterpret_cast<uint32_t *>(a.y + (size_t)m * a.out_cs + c0) = packed;
     }
@@ -962,14 +972,12 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const ConvArgs a)
                 const uint8_t *xp = a.x + ((size_t)(n * a.H + ih) * a.W + iw) * a.in_cs + g * cg;
                 const uint8_t *wp = a.wpack + ((size_t)k * cg * a.R + r) * a.S + s;
                 for (int c = 0; c < cg; c++)
-                    acc += (uint32_t)(((int)xp[c] - a.izp) * ((int)wp[(size_t)c * a.R * a.S] - a.wzp));
+                    acc += (uint32_t)(((int)(xp[c] ^ a.sx) - a.izp) * ((int)(wp[(size_t)c * a.R * a.S] ^ a.sx) - a.wzp));
             }
         }
         if (a.acc_out)
             a.acc_out[(size_t)m * a.out_cs + k] = (int32_t)acc;
-        int32_t r = requant_acc((int32_t)acc, a.q);
-        r = r < a.lo ? a.lo : r;
-        a.y[(size_t)m * a.out_cs + k] = (uint8_t)r;
+        a.y[(size_t)m * a.out_cs + k] = (uint8_t)conv_requant<false>(a, (int32_t)acc);
     }
 }
 
@@ -1036,6 +1044,11 @@ extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t
     HIPQ_REQUIRE(d.izp >= 0 && d.izp <= 255 && d.wzp >= 0 && d.wzp <= 255 && d.ozp >= 0 && d.ozp <= 255,
                  "conv: zero points must be in 0..255");
     HIPQ_REQUIRE(d.obits >= 1 && d.obits <= 8, "conv: obits must be in 1..8");
+    HIPQ_REQUIRE(d.dtype == HIPQ_DTYPE_U8 || d.dtype == HIPQ_DTYPE_I8, "conv: dtype must be HIPQ_DTYPE_U8 or HIPQ_DTYPE_I8");
+    // int8 symmetric tensors (op_conv_2d_i8xi8_run, conv_2d_int8_impl.c:34-174): no zero points, out-of-image taps
+    // are 0, the result is clipped to +-(2^obits - 1) and stored as the low byte.  An int8 byte b is the uint8 byte
+    // b ^ 0x80 with zero point 128, which is how the kernels that are not specialised read it.
+    const bool sgn = d.dtype == HIPQ_DTYPE_I8;
 
     auto *p = new hipq_conv2d_plan();
     p->d = d;
@@ -1046,7 +1059,9 @@ extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t
     a.in_cs = d.in_cs, a.out_cs = d.out_cs;
     a.OH = conv_out_dim(d.H, d.pad_h, d.R, d.stride_h);
     a.OW = conv_out_dim(d.W, d.pad_w, d.S, d.stride_w);
-    a.izp = d.izp, a.wzp = d.wzp;
+    a.izp = sgn ? 128 : d.izp, a.wzp = sgn ? 128 : d.wzp;
+    a.sx = sgn ? 0x80 : 0;
+    a.xmask = sgn ? 0u : 0x80808080u;
     const long long P = (long long)d.N * a.OH * a.OW;
     if (P <= 0 || P * (long long)d.out_cs >= (1ll << 31) || (long long)d.N * d.H * d.W * d.in_cs >= (1ll << 31)) {
         delete p;
@@ -1054,9 +1069,9 @@ extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t
     }
     a.P = (int)P;
     hipq_quant_scale(d.ialpha * d.walpha / d.oalpha, 32, &a.q.mult, &a.q.shift);
-    a.q.zp = d.ozp;
+    a.q.zp = sgn ? 0 : d.ozp;
     a.q.hi = (1 << d.obits) - 1;
-    a.lo = d.relu ? d.ozp : 0;
+    a.lo = sgn ? (d.relu ? 0 : -a.q.hi) : (d.relu ? d.ozp : 0);
     if (!valid_shift(a.q.shift)) {
         delete p;
         return fail("conv: requantisation shift %d outside 1..62 (scale %g)", a.q.shift,
@@ -1064,11 +1079,14 @@ extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t
     }
     a.fastq = a.q.shift >= 33 && a.q.shift <= 52;
     a.qt = a.fastq ? a.q.shift - 32 : 1;
-    a.qadd = a.fastq ? (1 << (a.qt - 1)) + (d.ozp << a.qt) : 0;
+    a.qadd = a.fastq ? (1 << (a.qt - 1)) + (a.q.zp << a.qt) : 0;
     a.inv_ohw = 1.0 / ((double)a.OH * a.OW);
     a.inv_ow = 1.0 / (double)a.OW;
-    a.padword = 0x01010101u * (uint32_t)d.izp;
-    const int aoff = 128 - d.izp, boff = 128 - d.wzp;
+    const int pad_byte = sgn ? 0 : d.izp; // the byte an out-of-image tap reads
+    a.padword = 0x01010101u * (uint32_t)pad_byte;
+    const int aoff = 128 - a.izp, boff = 128 - a.wzp; // both 0 for int8
+    // weight byte -> signed value relative to 128 (uint8) or the int8 value itself
+    auto wval = [&](uint8_t b) { return sgn ? (int)(int8_t)b : (int)b - 128; };
     a.bwz = boff;
 
     const int cg = d.C / d.group;
@@ -1105,7 +1123,7 @@ extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t
                         c = kp % d.in_cs, r = tap / d.S, s = tap % d.S;
                     }
                     if (s < d.S && c < d.C)
-                        ws = (int)w[(((size_t)ko * d.C + c) * d.R + r) * d.S + s] - 128;
+                        ws = wval(w[(((size_t)ko * d.C + c) * d.R + r) * d.S + s]);
                 }
                 wsum += ws;
                 const int slab = kp >> 6, chunk = ((kp >> 4) & 3) ^ ((ko >> 2) & 3);
@@ -1116,11 +1134,12 @@ extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t
             bbuf[ko] = (int32_t)(uint32_t)(unsigned long long)c0;
         }
         pad_off = wbuf.size();
-        wbuf.resize(pad_off + 64, (uint8_t)d.izp); // source of out-of-image taps
+        wbuf.resize(pad_off + 64, (uint8_t)pad_byte); // source of out-of-image taps
         char nm[96];
-        snprintf(nm, sizeof nm, "conv_mfma_i8_%dx%d%s%s", BM, BN, smallc ? "_c4" : "", p->has_wzp ? "_wzp" : "");
+        snprintf(nm, sizeof nm, "conv_mfma_i8_%dx%d%s%s%s", BM, BN, smallc ? "_c4" : "", p->has_wzp ? "_wzp" : "",
+                 sgn ? "_signed" : "");
         p->name = nm;
-    } else if (d.group == d.C && d.K == d.C && d.in_cs == d.out_cs && d.R == 3 && d.S == 3 && d.stride_h == d.stride_w
+    } else if (!sgn && d.group == d.C && d.K == d.C && d.in_cs == d.out_cs && d.R == 3 && d.S == 3 && d.stride_h == d.stride_w
                && (d.stride_h == 1 || d.stride_h == 2)
                && (long long)d.N * a.OH * ((a.OW + 3) / 4) * (d.in_cs / 4) < (1ll << 31)) {
         p->variant = kDepthwise3x3;
@@ -1150,18 +1169,18 @@ extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t
         int16_t *wq = reinterpret_cast<int16_t *>(wbuf.data());
         for (int c = 0; c < d.C; c++)
             for (int t = 0; t < d.R * d.S; t++)
-                wq[(size_t)t * d.in_cs + c] = (int16_t)((int)w[(size_t)c * d.R * d.S + t] - d.wzp);
+                wq[(size_t)t * d.in_cs + c] = (int16_t)(wval(w[(size_t)c * d.R * d.S + t]) + boff);
         bbuf.assign(d.in_cs, 0);
         for (int c = 0; c < d.C; c++)
             bbuf[c] = bias ? bias[c] : 0;
-        p->name = "conv_depthwise_u8";
+        p->name = sgn ? "conv_depthwise_i8" : "conv_depthwise_u8";
     } else {
         p->variant = kDirect;
         wbuf.assign(w, w + (size_t)d.K * cg * d.R * d.S);
         bbuf.assign(d.K, 0);
         for (int k = 0; k < d.K; k++)
             bbuf[k] = bias ? bias[k] : 0;
-        p->name = "conv_direct_u8";
+        p->name = sgn ? "conv_direct_i8" : "conv_direct_u8";
     }
 
     hipError_t e = hipMalloc(&p->d_w, wbuf.size());
@@ -1250,6 +1269,7 @@ extern "C" int hipq_conv2d_run_add(const hipq_conv2d_plan *p, const void *x, con
     HIPQ_REQUIRE(p && x && y && residual, "hipq_conv2d_run_add: null argument");
     HIPQ_REQUIRE(p->variant == kMfma || p->variant == kMfmaSmallC,
                  "hipq_conv2d_run_add: only the MFMA convolution kernels fuse the add (this plan runs %s)", p->name.c_str());
+    HIPQ_REQUIRE(p->d.dtype == HIPQ_DTYPE_U8, "hipq_conv2d_run_add: the fused add exists for uint8 tensors only (op_quant_add_run)");
     HIPQ_REQUIRE(res_zp >= 0 && res_zp <= 255 && ozp >= 0 && ozp <= 255 && obits >= 1 && obits <= 8,
                  "hipq_conv2d_run_add: zero points must be in 0..255, obits in 1..8");
     ConvArgs a = p->args;

@@ -356,6 +356,7 @@ struct QuantArgs {
     uint8_t *y;
     int N, C, H, W, cs;
     float alpha, beta, hi;
+    int lim; // int8 variant: alpha holds fp32(1 / oalpha), the result is clipped to +-lim
 };
 
 __device__ static inline uint32_t quantize_one(float x, const QuantArgs &p)
@@ -368,6 +369,23 @@ __device__ static inline uint32_t quantize_one(float x, const QuantArgs &p)
     return (uint32_t)(uint8_t)((double)q + 0.5); // saturate_float_by_bits: +0.5 in double, truncate
 }
 
+// op_quantize_run_i8 (quantize.c:159-185): clip(round(x * fp32(1 / oalpha)), -lim, lim).  The product is fp32, round()
+// is the C library's on a double (half away from zero), and clip() takes an int: the reference's x86-64 conversion
+// turns everything outside int32 (and NaN) into INT32_MIN, which then clips to -lim.
+__device__ static inline uint32_t quantize_one_i8(float x, const QuantArgs &p)
+{
+    const double r = round((double)__fmul_rn(x, p.alpha));
+    const int v = (r >= -2147483648.0 && r < 2147483648.0) ? (int)r : INT32_MIN;
+    return (uint32_t)min(max(v, -p.lim), p.lim) & 255u;
+}
+
+template <bool SIGNED>
+__device__ static inline uint32_t quantize_any(float x, const QuantArgs &p)
+{
+    return SIGNED ? quantize_one_i8(x, p) : quantize_one(x, p);
+}
+
+template <bool SIGNED>
 __global__ __launch_bounds__(256) void quantize_u8_kernel(const QuantArgs p)
 {
     const int cq = p.cs >> 2;
@@ -382,7 +400,7 @@ __global__ __launch_bounds__(256) void quantize_u8_kernel(const QuantArgs p)
         for (int e = 0; e < 4; e++) {
             const int c = q4 * 4 + e;
             if (c < p.C)
-                o |= quantize_one(p.x[((size_t)n * p.C + c) * hw + pix], p) << (8 * e);
+                o |= quantize_any<SIGNED>(p.x[((size_t)n * p.C + c) * hw + pix], p) << (8 * e);
         }
         *reinterpret_cast<uint32_t *>(p.y + ((size_t)n * hw + pix) * p.cs + q4 * 4) = o;
     }
@@ -390,6 +408,7 @@ __global__ __launch_bounds__(256) void quantize_u8_kernel(const QuantArgs p)
 
 // Network inputs (C <= 4, channel stride 4): a thread converts 4 consecutive pixels, i.e. one 128-bit load per
 // channel plane and one 128-bit store; blockIdx.y is the image, so no 64-bit index arithmetic is needed.
+template <bool SIGNED>
 __global__ __launch_bounds__(256) void quantize_u8_c4_kernel(const QuantArgs p)
 {
     const int hw = p.H * p.W, hw4 = hw >> 2; // the host checks hw % 4 == 0
@@ -403,7 +422,7 @@ __global__ __launch_bounds__(256) void quantize_u8_c4_kernel(const QuantArgs p)
             const f32x4 v = __builtin_nontemporal_load(reinterpret_cast<const f32x4 *>(xn + (size_t)c * hw) + i);
 #pragma unroll
             for (int e = 0; e < 4; e++)
-                o[e] |= quantize_one(v[e], p) << (8 * c);
+                o[e] |= quantize_any<SIGNED>(v[e], p) << (8 * c);
         }
         yn[i] = o;
     }
@@ -416,6 +435,7 @@ struct DequantArgs {
     int N, C, H, W, cs;
     float alpha;
     int zp;
+    int sgn; // 1: the bytes are int8 and there is no zero point (op_dequantize_run_i8, dequantize.c:125-136)
 };
 
 __global__ __launch_bounds__(256) void dequantize_u8_kernel(const DequantArgs p)
@@ -425,7 +445,8 @@ __global__ __launch_bounds__(256) void dequantize_u8_kernel(const DequantArgs p)
          idx += (size_t)gridDim.x * blockDim.x) {
         const size_t pix = idx % hw, rest = idx / hw;
         const int c = (int)(rest % p.C), n = (int)(rest / p.C);
-        const int v = (int)p.x[((size_t)n * hw + pix) * p.cs + c] - p.zp;
+        const uint8_t b = p.x[((size_t)n * hw + pix) * p.cs + c];
+        const int v = p.sgn ? (int)(int8_t)b : (int)b - p.zp;
         p.y[idx] = __fmul_rn((float)v, p.alpha);
     }
 }
@@ -622,37 +643,69 @@ extern "C" int hipq_pool_u8(const void *x, void *y, int N, int C, int H, int W, 
     return launch_status("pool_u8_kernel");
 }
 
-extern "C" int hipq_quantize_u8(const float *x, void *y, int N, int C, int H, int W, int cs, float oa, int oz, int obits,
-                                void *stream)
+static int launch_quantize(const char *who, bool sgn, const float *x, void *y, int N, int C, int H, int W, int cs, float oa,
+                           int oz, int obits, void *stream)
 {
     clear_error();
-    HIPQ_REQUIRE(x && y && N > 0 && C > 0 && H > 0 && W > 0 && cs >= C && cs % 4 == 0, "hipq_quantize_u8: bad argument");
+    HIPQ_REQUIRE(x && y && N > 0 && C > 0 && H > 0 && W > 0 && cs >= C && cs % 4 == 0, "%s: bad argument", who);
+    HIPQ_REQUIRE(obits >= 1 && obits <= 8, "%s: obits must be in 1..8", who);
     QuantArgs p;
     p.x = x, p.y = static_cast<uint8_t *>(y), p.N = N, p.C = C, p.H = H, p.W = W, p.cs = cs;
-    p.alpha = oa;
-    p.beta = -(oa * (float)oz); // quantize.c:152
+    p.alpha = sgn ? (float)(1. / (double)oa) : oa; // quantize.c:166: a double division, rounded to fp32
+    p.beta = -(oa * (float)oz);                    // quantize.c:152
     p.hi = (float)((1 << obits) - 1);
+    p.lim = (1 << (obits - 1)) - 1;
+    const hipStream_t st = static_cast<hipStream_t>(stream);
     if (cs == 4 && (H * W) % 4 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) == 0
         && N <= 65535) {
         const unsigned bx = (unsigned)std::min((H * W / 4 + 255) / 256, 1024);
-        hipLaunchKernelGGL(quantize_u8_c4_kernel, dim3(bx, N), dim3(256), 0, static_cast<hipStream_t>(stream), p);
-        return launch_status("quantize_u8_c4_kernel");
+        if (sgn)
+            hipLaunchKernelGGL(quantize_u8_c4_kernel<true>, dim3(bx, N), dim3(256), 0, st, p);
+        else
+            hipLaunchKernelGGL(quantize_u8_c4_kernel<false>, dim3(bx, N), dim3(256), 0, st, p);
+        return launch_status(sgn ? "quantize_i8_c4_kernel" : "quantize_u8_c4_kernel");
     }
     const size_t total = (size_t)N * H * W * (cs / 4);
-    hipLaunchKernelGGL(quantize_u8_kernel, dim3(grid_for(total)), dim3(256), 0, static_cast<hipStream_t>(stream), p);
-    return launch_status("quantize_u8_kernel");
+    if (sgn)
+        hipLaunchKernelGGL(quantize_u8_kernel<true>, dim3(grid_for(total)), dim3(256), 0, st, p);
+    else
+        hipLaunchKernelGGL(quantize_u8_kernel<false>, dim3(grid_for(total)), dim3(256), 0, st, p);
+    return launch_status(sgn ? "quantize_i8_kernel" : "quantize_u8_kernel");
+}
+
+extern "C" int hipq_quantize_u8(const float *x, void *y, int N, int C, int H, int W, int cs, float oa, int oz, int obits,
+                                void *stream)
+{
+    return launch_quantize("hipq_quantize_u8", false, x, y, N, C, H, W, cs, oa, oz, obits, stream);
+}
+
+extern "C" int hipq_quantize_i8(const float *x, void *y, int N, int C, int H, int W, int cs, float oa, int obits, void *stream)
+{
+    return launch_quantize("hipq_quantize_i8", true, x, y, N, C, H, W, cs, oa, 0, obits, stream);
+}
+
+static int launch_dequantize(const char *who, int sgn, const void *x, float *y, int N, int C, int H, int W, int cs, float ia,
+                             int iz, void *stream)
+{
+    clear_error();
+    HIPQ_REQUIRE(x && y && N > 0 && C > 0 && H > 0 && W > 0 && cs >= C, "%s: bad argument", who);
+    DequantArgs p;
+    p.x = static_cast<const uint8_t *>(x), p.y = y, p.N = N, p.C = C, p.H = H, p.W = W, p.cs = cs, p.alpha = ia, p.zp = iz;
+    p.sgn = sgn;
+    hipLaunchKernelGGL(dequantize_u8_kernel, dim3(grid_for((size_t)N * C * H * W)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), p);
+    return launch_status(sgn ? "dequantize_i8_kernel" : "dequantize_u8_kernel");
 }
 
 extern "C" int hipq_dequantize_u8(const void *x, float *y, int N, int C, int H, int W, int cs, float ia, int iz,
                                   void *stream)
 {
-    clear_error();
-    HIPQ_REQUIRE(x && y && N > 0 && C > 0 && H > 0 && W > 0 && cs >= C, "hipq_dequantize_u8: bad argument");
-    DequantArgs p;
-    p.x = static_cast<const uint8_t *>(x), p.y = y, p.N = N, p.C = C, p.H = H, p.W = W, p.cs = cs, p.alpha = ia, p.zp = iz;
-    hipLaunchKernelGGL(dequantize_u8_kernel, dim3(grid_for((size_t)N * C * H * W)), dim3(256), 0,
-                       static_cast<hipStream_t>(stream), p);
-    return launch_status("dequantize_u8_kernel");
+    return launch_dequantize("hipq_dequantize_u8", 0, x, y, N, C, H, W, cs, ia, iz, stream);
+}
+
+extern "C" int hipq_dequantize_i8(const void *x, float *y, int N, int C, int H, int W, int cs, float ia, void *stream)
+{
+    return launch_dequantize("hipq_dequantize_i8", 1, x, y, N, C, H, W, cs, ia, 0, stream);
 }
 
 static int layout_args(LayoutArgs &p, const void *src, void *dst, int N, int C, int H, int W, int cs)

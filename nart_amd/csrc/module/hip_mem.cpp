@@ -183,7 +183,7 @@ void hip_mem_tag(tensor_t *t)
     const int nd = t->shape.dim_size;
     hip_layout_t layout = HIP_LAYOUT_RAW;
     int N = 0, C = 0, H = 1, W = 1;
-    if (t->dtype == dtUINT8 && (nd == 4 || nd == 2)) {
+    if ((t->dtype == dtUINT8 || t->dtype == dtINT8) && (nd == 4 || nd == 2)) { // one byte per element either way
         layout = HIP_LAYOUT_NHWC_U8;
         N = (int)t->shape.dim[0], C = (int)t->shape.dim[1];
         if (nd == 4)

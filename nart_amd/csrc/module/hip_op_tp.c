@@ -32,10 +32,23 @@ static tensor_t *one_output(op_t *op, uint32_t dtype)
     return &op->output_tensors[0];
 }
 
-/* quantize.c:51-81 maps (qtype << 8 | bits) to an output dtype; this module implements the uint8 rows */
+/* quantize.c:40-86 maps (qtype << 8 | bits) to an output dtype; this module implements the uint8 and int8 rows
+ * (prepare rejects the others).  The qtype setting sits right after op_t in the module's quantize struct. */
 static bool infer_quantize(op_t *op)
 {
-    one_output(op, dtUINT8);
+    int32_t qtype = 0;
+    uint8_t *bits = NULL;
+    size_t n = 0;
+    uint32_t dt = dtUINT8;
+    if (op_setting_single_get(op, SETTING_QUANT_QTYPE, dtINT32, &qtype)
+        && op_setting_array_get(op, SETTING_QUANT_OBITS, dtUINT8, &n, &bits) && n >= 1) {
+        const int32_t key = qtype << 8 | bits[0];
+        if (key >= 0x0202 && key <= 0x0208 && key != 0x0205)
+            dt = dtINT8;
+    }
+    if (op->output_size == 1)
+        op->output_tensors[0].dtype = dt; /* settings may have changed since the first inference */
+    one_output(op, dt);
     return true;
 }
 

@@ -58,12 +58,15 @@ void destroy_nothing(op_t *) {}
 const void *in_ptr(op_t *op, int i) { return hip_mem_dev_in(op->input_tensors[i]->mem, op_stream(op)); }
 void *out_ptr(op_t *op) { return hip_mem_dev_out(op->output_tensors[0].mem, op_stream(op)); }
 
-void require_hip_u8(op_t *op, size_t n_act)
+// allow_i8: conv_2d, ip and dequantize also exist for int8 symmetric tensors (conv_2d.c:120-141, ip.cpp:312-331,
+// dequantize.c:156-163); every other operator of the reference module is uint8 only.
+void require_hip_u8(op_t *op, size_t n_act, bool allow_i8 = false)
 {
     for (size_t i = 0; i < n_act; ++i) {
-        if (op->input_tensors[i]->dtype != dtUINT8) {
-            fprintf(stderr, "[hip module] %s: input %zu has dtype %u; only uint8 activations are implemented\n",
-                    op->entry->tp->name, i, op->input_tensors[i]->dtype);
+        const uint32_t dt = op->input_tensors[i]->dtype;
+        if (dt != dtUINT8 && !(allow_i8 && dt == dtINT8)) {
+            fprintf(stderr, "[hip module] %s: input %zu has dtype %u; this operator is implemented for uint8%s activations\n",
+                    op->entry->tp->name, i, dt, allow_i8 ? " and int8" : "");
             abort(); // the reference aborts on unsupported dtypes as well (conv_2d.c:143-145)
         }
         HIPM_CHECK(is_hip_mem(op->input_tensors[i]->mem));
@@ -142,14 +145,19 @@ void build_plan(op_t *op, const hipq_conv2d_desc &d, const uint8_t *w, const voi
 const uint8_t *host_weights(op_t *op)
 {
     tensor_t *w = op->input_tensors[1];
-    HIPM_CHECK(w->dtype == dtUINT8);
+    HIPM_CHECK(w->dtype == op->input_tensors[0]->dtype); // u8 x u8 or i8 x i8, as in the reference
     return static_cast<const uint8_t *>(is_hip_mem(w->mem) ? hip_mem_host_in(w->mem) : mem_cpu_data(w->mem));
 }
+
+// int8 tensors select the symmetric operators.  The reference picks special low-bit GEMMs that exist on aarch64 only
+// when ibits and wbits are both below 8 (conv_2d.c:121-139, ip.cpp:313-318); their results equal the plain int8
+// product for in-range values, which is what runs here.
+int signed_dtype(op_t *op) { return op->input_tensors[0]->dtype == dtINT8 ? HIPQ_DTYPE_I8 : HIPQ_DTYPE_U8; }
 
 void conv_prepare(op_t *op)
 {
     conv_op_t *c = reinterpret_cast<conv_op_t *>(op);
-    require_hip_u8(op, 1);
+    require_hip_u8(op, 1, true);
     alloc_and_tag(op);
     const shape_t &xs = op->input_tensors[0]->shape;
     const hip_mem_t *xm = as_hip(op->input_tensors[0]->mem), *ym = as_hip(op->output_tensors[0].mem);
@@ -166,16 +174,18 @@ void conv_prepare(op_t *op)
     d.izp = c->qi.zp[0], d.wzp = c->qw.zp[0], d.ozp = c->qo.zp[0];
     d.obits = c->qo.bits[0];
     d.relu = 0; // the reference CPU module ignores SETTING_CONV_2D_RELU_FLAG (conv_2d.c:27-70); so does this one
+    d.dtype = signed_dtype(op);
     build_plan(op, d, host_weights(op), op->input_tensors[1]->mem);
 }
 
 void ip_prepare(op_t *op)
 {
     conv_op_t *c = reinterpret_cast<conv_op_t *>(op);
-    require_hip_u8(op, 1);
+    require_hip_u8(op, 1, true);
     alloc_and_tag(op);
     const hip_mem_t *xm = as_hip(op->input_tensors[0]->mem), *ym = as_hip(op->output_tensors[0].mem);
     HIPM_CHECK(xm->layout == HIP_LAYOUT_NHWC_U8 && ym->layout == HIP_LAYOUT_NHWC_U8);
+    const int dtype = signed_dtype(op);
     // the input's true geometry is the producer's (a flatten/reshape in between does not move bytes)
     const int M = xm->N, kd = xm->H * xm->W * xm->cs;
     const size_t kin = (size_t)xm->C * xm->H * xm->W;
@@ -186,7 +196,7 @@ void ip_prepare(op_t *op)
     if (xm->H * xm->W > 1 || xm->cs != xm->C) { // (c,h,w) order of the reference -> (h,w,c) with channel stride
         reordered.resize((size_t)c->num_output * kd);
         HIPM_HIPQ(hipq_ip_reorder_weights(w, reordered.data(), (int)c->num_output, xm->C, xm->H, xm->W, xm->cs,
-                                          c->qw.zp[0]));
+                                          dtype == HIPQ_DTYPE_I8 ? 0 : c->qw.zp[0])); // pad channels weigh nothing
         w = reordered.data();
     }
     hipq_conv2d_desc d;
@@ -197,6 +207,7 @@ void ip_prepare(op_t *op)
     d.ialpha = c->qi.alpha[0], d.walpha = c->qw.alpha[0], d.oalpha = c->qo.alpha[0];
     d.izp = c->qi.zp[0], d.wzp = c->qw.zp[0], d.ozp = c->qo.zp[0];
     d.obits = c->qo.bits[0];
+    d.dtype = dtype;
     build_plan(op, d, w, op->input_tensors[1]->mem);
 }
 
@@ -394,19 +405,34 @@ void quantize_run(op_t *op)
     int d[4];
     dims4(op->input_tensors[0], d);
     const hip_mem_t *y = as_hip(op->output_tensors[0].mem);
-    HIPM_HIPQ(hipq_quantize_u8(static_cast<const float *>(in_ptr(op, 0)), out_ptr(op), d[0], d[1], d[2], d[3], y->cs,
-                               q->q.alpha[0], q->q.zp[0], q->q.bits[0], op_stream(op)));
+    if (op->output_tensors[0].dtype == dtINT8)
+        HIPM_HIPQ(hipq_quantize_i8(static_cast<const float *>(in_ptr(op, 0)), out_ptr(op), d[0], d[1], d[2], d[3], y->cs,
+                                   q->q.alpha[0], q->q.bits[0], op_stream(op)));
+    else
+        HIPM_HIPQ(hipq_quantize_u8(static_cast<const float *>(in_ptr(op, 0)), out_ptr(op), d[0], d[1], d[2], d[3], y->cs,
+                                   q->q.alpha[0], q->q.zp[0], q->q.bits[0], op_stream(op)));
+}
+
+// (qtype << 8 | bits) rows of quantize.c:233-262 / dequantize.c:150-167 that exist here: 1 = uint8, 2 = int8
+int qdq_row(int32_t key)
+{
+    if (key == 0x0008 || key == 0x0108)
+        return 1;
+    if (key >= 0x0202 && key <= 0x0208 && key != 0x0205)
+        return 2;
+    return 0;
 }
 
 void quantize_prepare(op_t *op)
 {
     qdq_op_t *q = reinterpret_cast<qdq_op_t *>(op);
     HIPM_CHECK(op->input_tensors[0]->dtype == dtFLOAT32 && is_hip_mem(op->input_tensors[0]->mem));
-    const int32_t key = q->qtype << 8 | q->q.bits[0];
-    if (key != 0x0008 && key != 0x0108) { // quantize.c:233-262: this module implements the uint8 rows
+    const int row = qdq_row(q->qtype << 8 | q->q.bits[0]);
+    if (row == 0) { // the 16- and 32-bit rows of quantize.c:233-262 are not implemented
         fprintf(stderr, "[hip module] quantization for %d bits with type %d is not implemented\n", q->q.bits[0], q->qtype);
         abort();
     }
+    HIPM_CHECK(op->output_tensors[0].dtype == (row == 2 ? dtINT8 : dtUINT8));
     const int nd = op->input_tensors[0]->shape.dim_size;
     HIPM_CHECK(nd == 4 || nd == 2);
     hip_mem_tag(op->input_tensors[0]);
@@ -425,19 +451,22 @@ void dequantize_run(op_t *op)
 {
     qdq_op_t *q = reinterpret_cast<qdq_op_t *>(op);
     const hip_mem_t *x = as_hip(op->input_tensors[0]->mem);
-    HIPM_HIPQ(hipq_dequantize_u8(in_ptr(op, 0), static_cast<float *>(out_ptr(op)), x->N, x->C, x->H, x->W, x->cs,
-                                 q->q.alpha[0], q->q.zp[0], op_stream(op)));
+    if (qdq_row(q->qtype << 8 | q->q.bits[0]) == 2) // chosen from the settings, not from the tensor's dtype (dequantize.c:141-163)
+        HIPM_HIPQ(hipq_dequantize_i8(in_ptr(op, 0), static_cast<float *>(out_ptr(op)), x->N, x->C, x->H, x->W, x->cs,
+                                     q->q.alpha[0], op_stream(op)));
+    else
+        HIPM_HIPQ(hipq_dequantize_u8(in_ptr(op, 0), static_cast<float *>(out_ptr(op)), x->N, x->C, x->H, x->W, x->cs,
+                                     q->q.alpha[0], q->q.zp[0], op_stream(op)));
 }
 
 void dequantize_prepare(op_t *op)
 {
     qdq_op_t *q = reinterpret_cast<qdq_op_t *>(op);
-    const int32_t key = q->qtype << 8 | q->q.bits[0];
-    if (key != 0x0008 && key != 0x0108) { // dequantize.c:150-167
+    if (qdq_row(q->qtype << 8 | q->q.bits[0]) == 0) { // dequantize.c:150-167
         fprintf(stderr, "[hip module] dequantization for %d bits with type %d is not implemented\n", q->q.bits[0], q->qtype);
         abort();
     }
-    require_hip_u8(op, 1);
+    require_hip_u8(op, 1, true);
     alloc_and_tag(op);
     HIPM_CHECK(as_hip(op->input_tensors[0]->mem)->layout == HIP_LAYOUT_NHWC_U8);
     op->run_func = dequantize_run;

@@ -22,7 +22,10 @@ class ConvDesc(C.Structure):  # hipq_conv2d_desc
     _fields_ = [(n, C.c_int32) for n in ("N", "C", "H", "W", "K", "R", "S", "pad_h", "pad_w", "stride_h",
                                          "stride_w", "group", "in_cs", "out_cs")] \
         + [(n, C.c_float) for n in ("ialpha", "walpha", "oalpha")] \
-        + [(n, C.c_int32) for n in ("izp", "wzp", "ozp", "obits", "relu")]
+        + [(n, C.c_int32) for n in ("izp", "wzp", "ozp", "obits", "relu", "dtype")]
+
+
+DTYPE_U8, DTYPE_I8 = 0, 1
 
 
 # every symbol include/hipq.h declares, with its signature
@@ -50,6 +53,8 @@ _SIGS = {
                                                                           C.c_int, C.c_void_p]),
     "hipq_quantize_u8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_float, C.c_int, C.c_int, C.c_void_p]),
     "hipq_dequantize_u8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_float, C.c_int, C.c_void_p]),
+    "hipq_quantize_i8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_float, C.c_int, C.c_void_p]),
+    "hipq_dequantize_i8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_float, C.c_void_p]),
     "hipq_copy_bytes": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
 }
 EXPORTS = tuple(_SIGS)
@@ -100,7 +105,8 @@ def conv_out_dim(i, pad, k, stride):
 def to_device_nhwc(x_nchw):
     """numpy uint8 [N,C,H,W] -> CUDA uint8 [N,H,W,cs] (channels-last, padded channel stride)."""
     import torch
-    x = np.ascontiguousarray(x_nchw, np.uint8)
+    x = np.ascontiguousarray(x_nchw)
+    x = x.view(np.uint8) if x.dtype == np.int8 else np.ascontiguousarray(x, np.uint8)  # int8 travels as its bytes
     N, Cc, H, W = x.shape
     cs = channel_stride(Cc)
     src = torch.from_numpy(x).cuda()
@@ -122,16 +128,17 @@ class Conv2d:
     """A convolution plan (weights packed and resident on the device) plus its launch."""
 
     def __init__(self, x_shape, w, bias, pad, stride, group, ialpha, izp, walpha, wzp, oalpha, ozp, obits=8,
-                 relu=False, in_cs=None, out_cs=None):
+                 relu=False, in_cs=None, out_cs=None, dtype=DTYPE_U8):
+        """dtype=DTYPE_I8: int8 symmetric tensors (w is an int8 array, zero points are ignored)."""
         N, Cc, H, W = x_shape
-        w = np.ascontiguousarray(w, np.uint8)
+        w = np.ascontiguousarray(w, np.int8 if dtype == DTYPE_I8 else np.uint8)
         K, _, R, S = w.shape
         ph, pw = (pad, pad) if np.isscalar(pad) else pad
         sh, sw = (stride, stride) if np.isscalar(stride) else stride
         d = ConvDesc(N=N, C=Cc, H=H, W=W, K=K, R=R, S=S, pad_h=ph, pad_w=pw, stride_h=sh, stride_w=sw, group=group,
                      in_cs=in_cs or channel_stride(Cc), out_cs=out_cs or channel_stride(K),
                      ialpha=ialpha, walpha=walpha, oalpha=oalpha, izp=izp, wzp=wzp, ozp=ozp, obits=obits,
-                     relu=int(relu))
+                     relu=int(relu), dtype=dtype)
         self.desc = d
         self.OH, self.OW = conv_out_dim(H, ph, R, sh), conv_out_dim(W, pw, S, sw)
         b = None if bias is None else np.ascontiguousarray(bias, np.int32)
@@ -209,6 +216,18 @@ def quantize_u8(x_nchw, y, oalpha, ozp, obits=8):
     N, Cc, H, W = x_nchw.shape
     check(lib().hipq_quantize_u8(_ptr(x_nchw), _ptr(y), N, Cc, H, W, y.shape[-1], oalpha, ozp, obits, _stream()))
     return y
+
+
+def quantize_i8(x_nchw, y, oalpha, obits=8):
+    N, Cc, H, W = x_nchw.shape
+    check(lib().hipq_quantize_i8(_ptr(x_nchw), _ptr(y), N, Cc, H, W, y.shape[-1], oalpha, obits, _stream()))
+    return y
+
+
+def dequantize_i8(x, y_nchw, ialpha):
+    N, Cc, H, W = y_nchw.shape
+    check(lib().hipq_dequantize_i8(_ptr(x), _ptr(y_nchw), N, Cc, H, W, x.shape[-1], ialpha, _stream()))
+    return y_nchw
 
 
 def dequantize_u8(x, y_nchw, ialpha, izp):

@@ -274,3 +274,116 @@ def test_full_size_properties():
     for i in (0, 63):
         want = orc.conv2d_u8(x[i:i + 1], w, b, 1, 1, 1, *q)
         assert np.array_equal(y[i:i + 1], want)
+
+
+# ---- int8 symmetric variants (op_conv_2d_i8xi8_run, op_quant_ip_i8xi8_run, op_quantize_run_i8, op_dequantize_run_i8) ----
+def run_conv_i8(x, w, b, pad, stride, group, q, obits=8, in_cs=None):
+    ia, wa, oa = q
+    plan = hipq.Conv2d(x.shape, w, b, pad, stride, group, ia, 0, wa, 0, oa, 0, obits=obits, dtype=hipq.DTYPE_I8, in_cs=in_cs)
+    xd = hipq.to_device_nhwc(x)
+    acc = torch.zeros((x.shape[0], plan.OH, plan.OW, plan.desc.out_cs), dtype=torch.int32, device="cuda")
+    yd = plan(xd, acc=acc)
+    torch.cuda.synchronize()
+    y = hipq.from_device_nhwc(yd, w.shape[0]).view(np.int8)
+    return y, acc.cpu().numpy()[..., :w.shape[0]].transpose(0, 3, 1, 2), plan.kernel
+
+
+def test_conv_int8():
+    """Every kernel variant with int8 tensors: MFMA tiles (DMA-fed and the small-C stem form), depthwise, grouped;
+    obits 8 (clip to +-255, then two's complement wrap), 7 and 4; with and without bias; ragged tiles and paddings."""
+    rng = np.random.default_rng(41)
+    kerns = set()
+    cases = [  # N, C, H, W, K, R, S, pad, stride, group
+        (2, 64, 14, 14, 64, 3, 3, 1, 1, 1), (1, 64, 9, 11, 128, 1, 1, 0, 1, 1), (3, 32, 10, 7, 48, 3, 3, 1, 2, 1),
+        (1, 16, 12, 12, 24, 5, 3, (1, 2), 1, 1), (2, 128, 7, 7, 256, 1, 1, 0, 2, 1), (1, 3, 33, 29, 64, 7, 7, 3, 2, 1),
+        (2, 3, 16, 16, 16, 3, 3, 1, 1, 1), (1, 256, 6, 6, 64, 3, 3, 1, 1, 1), (2, 32, 9, 9, 32, 3, 3, 1, 1, 32),
+        (1, 48, 10, 10, 48, 3, 3, 1, 2, 48), (1, 24, 8, 8, 24, 5, 5, 2, 1, 24), (1, 8, 9, 9, 12, 3, 3, (2, 0), (1, 2), 2),
+        (2, 512, 7, 7, 512, 3, 3, 1, 1, 1), (4, 256, 14, 14, 1024, 1, 1, 0, 1, 1),
+    ]
+    for i, (N, C, H, W, K, R, S, pad, st, grp) in enumerate(cases):
+        x = rng.integers(-128, 128, (N, C, H, W), dtype=np.int8)
+        w = rng.integers(-128, 128, (K, C // grp, R, S), dtype=np.int8)
+        b = rng.integers(-30000, 30000, K).astype(np.int32) if i % 3 else None
+        for obits in (8, 7, 4):
+            q = (rand_q(rng), rand_q(rng), rand_q(rng, 1e-2, 1.0))
+            print("int8 conv case", i, x.shape, w.shape, pad, st, grp, q, obits, flush=True)
+            want_y, want_acc = orc.conv2d_i8(x, w, b, pad, st, grp, *q, obits=obits, return_acc=True)
+            y, acc, kern = run_conv_i8(x, w, b, pad, st, grp, q, obits)
+            kerns.add(kern)
+            assert np.array_equal(acc, want_acc), (i, kern, "accumulators differ", int((acc != want_acc).sum()))
+            assert np.array_equal(y, want_y), (i, kern, obits, "outputs differ", int((y != want_y).sum()))
+    assert any("mfma" in k and "_c4" in k for k in kerns) and any("depthwise_i8" in k for k in kerns) \
+        and any("direct_i8" in k for k in kerns), kerns
+    # extremes: -128 * -128 over a long reduction, and outputs that wrap with obits = 8
+    x = np.full((1, 512, 3, 3), -128, np.int8)
+    w = np.full((16, 512, 3, 3), -128, np.int8)
+    for oa in (0.5, 40.0):
+        want = orc.conv2d_i8(x, w, None, 1, 1, 1, 0.01, 0.01, oa, 8)
+        y, _, _ = run_conv_i8(x, w, None, 1, 1, 1, (0.01, 0.01, oa), 8)
+        assert np.array_equal(y, want)
+    assert want.min() < -100 or want.max() > 100
+    with pytest.raises(hipq.HipqError):  # the fused residual add is a uint8 operator
+        plan = hipq.Conv2d((1, 64, 4, 4), np.zeros((64, 64, 1, 1), np.int8), None, 0, 1, 1, 0.1, 0, 0.1, 0, 0.1, 0,
+                           dtype=hipq.DTYPE_I8)
+        t = torch.zeros((1, 4, 4, 64), dtype=torch.uint8, device="cuda")
+        plan.run_add(t, t, False, 0.1, 0, 0.1, 0, t.clone())
+
+
+def test_ip_int8():
+    rng = np.random.default_rng(42)
+    for M, Kd, No, obits in ((1, 64, 10, 8), (7, 300, 33, 7), (128, 4096, 256, 8), (5, 2048, 1000, 7)):
+        x = rng.integers(-128, 128, (M, Kd), dtype=np.int8)
+        w = rng.integers(-128, 128, (No, Kd), dtype=np.int8)
+        b = rng.integers(-50000, 50000, No).astype(np.int32)
+        q = (rand_q(rng), rand_q(rng), rand_q(rng, 1e-1, 10.0))
+        want_y, want_acc = orc.ip_i8(x, w, b, *q, obits=obits, return_acc=True)
+        y, acc, kern = run_conv_i8(x.reshape(M, Kd, 1, 1), w.reshape(No, Kd, 1, 1), b, 0, 1, 1, q, obits)
+        assert np.array_equal(acc.reshape(M, No), want_acc), (M, Kd, No, kern)
+        assert np.array_equal(y.reshape(M, No), want_y), (M, Kd, No, kern)
+
+
+def test_quantize_dequantize_int8():
+    rng = np.random.default_rng(43)
+    for shape in ((2, 3, 224, 224), (1, 16, 9, 9), (4, 1000, 1, 1), (2, 3, 7, 5)):
+        for obits in (8, 7, 4, 2):
+            oa = rand_q(rng, 5e-3, 0.1)
+            x = (rng.standard_normal(shape) * 60 * oa).astype(np.float32)
+            n = min(600, x.size - 8)
+            x.flat[:n] = (np.arange(n, dtype=np.float32) * 0.5 - 150) * np.float32(oa)  # ties of both signs, both clips
+            x.flat[n:n + 6] = [3e9, -3e9, 1e30, -1e30, np.inf, -np.inf]                 # beyond int32: the conversion's sentinel
+            xd = torch.from_numpy(x).cuda()
+            cs = hipq.channel_stride(shape[1])
+            yd = torch.empty((shape[0], shape[2], shape[3], cs), dtype=torch.uint8, device="cuda")
+            hipq.quantize_i8(xd, yd, oa, obits)
+            want = orc.quantize_i8(x, oa, obits)
+            got = hipq.from_device_nhwc(yd, shape[1]).view(np.int8)
+            assert np.array_equal(got, want), (shape, obits, int((got != want).sum()))
+            fd = torch.empty(shape, dtype=torch.float32, device="cuda")
+            hipq.dequantize_i8(yd, fd, oa)
+            assert np.array_equal(fd.cpu().numpy().view(np.uint32), orc.dequantize_i8(want, oa).view(np.uint32))
+
+
+def test_golden_int8_outputs_on_gpu():
+    """The compiled reference's recorded int8 outputs, reproduced by the HIP kernels."""
+    g = np.load(os.path.join(HERE, "golden", "quant_ops_int8.npz"))
+    meta = json.loads(bytes(g["meta"]).decode())
+    for name, m in meta.items():
+        kind, a = m["kind"], m["args"]
+        ins = [g["%s.in%d" % (name, i)] for i in range(m["n_in"])]
+        want = g[name + ".out"]
+        if kind == "conv":
+            got, _, _ = run_conv_i8(ins[0], ins[1], ins[2], a["pad"], a["stride"], a["group"], a["q"], a["obits"])
+        elif kind == "ip":
+            M, Kd = ins[0].shape
+            got, _, _ = run_conv_i8(ins[0].reshape(M, Kd, 1, 1), ins[1].reshape(-1, Kd, 1, 1), ins[2], 0, 1, 1, a["q"], a["obits"])
+            got = got.reshape(want.shape)
+        elif kind == "quantize":
+            N, Cc, H, W = ins[0].shape
+            yd = torch.empty((N, H, W, hipq.channel_stride(Cc)), dtype=torch.uint8, device="cuda")
+            hipq.quantize_i8(torch.from_numpy(ins[0]).cuda(), yd, a["q"][0], a["obits"])
+            got = hipq.from_device_nhwc(yd, Cc).view(np.int8)
+        else:
+            fd = torch.empty(ins[0].shape, dtype=torch.float32, device="cuda")
+            hipq.dequantize_i8(hipq.to_device_nhwc(ins[0]), fd, a["q"][0])
+            got = fd.cpu().numpy()
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), name

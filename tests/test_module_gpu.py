@@ -107,6 +107,41 @@ def test_single_ops_through_the_op_api(own_rt):
     ws.delete()
 
 
+def test_int8_ops_through_the_op_api(own_rt):
+    """quantize (symmetric) -> conv (int8) -> flatten -> ip (int8) -> dequantize on the hip workspace, every
+    stage against the oracle; the operators are chosen from the tensor dtype / the qtype setting as in the reference
+    (conv_2d.c:113-146, ip.cpp:297-336, quantize.c:233-262, dequantize.c:141-167)."""
+    import refrun
+    from oracle import orc
+    ws = own_rt.workspace("hip")
+    rng = np.random.default_rng(12)
+    xf = (rng.standard_normal((3, 16, 10, 10)) * 2).astype(np.float32)
+    w = rng.integers(-128, 128, (24, 16, 3, 3), dtype=np.int8)
+    b = rng.integers(-5000, 5000, 24).astype(np.int32)
+    wf = rng.integers(-128, 128, (10, 24 * 5 * 5), dtype=np.int8)
+    bf = rng.integers(-5000, 5000, 10).astype(np.int32)
+    qz = ws.quantize(ws.tensor(xf), 0.03, 0, bits=8, qtype=2).prepare().run()
+    xq = orc.quantize_i8(xf, 0.03, 8)
+    assert qz.output(0).dtype == np.int8 and same_bits(qz.output(0).numpy(), xq)
+    q = dict(ialpha=0.03, izp=0, walpha=0.004, wzp=0, oalpha=0.2, ozp=0, obits=7)
+    conv = ws.conv2d(qz.output(0), ws.tensor(w), ws.tensor(b), 1, 2, 1, q).prepare().run()
+    yc = orc.conv2d_i8(xq, w, b, 1, 2, 1, 0.03, 0.004, 0.2, 7)
+    assert conv.output(0).dtype == np.int8 and same_bits(conv.output(0).numpy(), yc)
+    flat = ws.reshape_flatten(conv.output(0)).prepare().run()
+    q2 = dict(ialpha=0.2, izp=0, walpha=0.002, wzp=0, oalpha=0.9, ozp=0, obits=7)
+    ip = ws.ip(flat.output(0), ws.tensor(wf), ws.tensor(bf), q2).prepare().run()
+    yi = orc.ip_i8(yc.reshape(3, -1), wf, bf, 0.2, 0.002, 0.9, 7)
+    assert same_bits(ip.output(0).numpy().reshape(yi.shape), yi)
+    dq = ws.dequantize(ip.output(0), 0.9, 0, bits=8, qtype=2).prepare().run()
+    assert same_bits(dq.output(0).numpy().reshape(yi.shape), orc.dequantize_i8(yi, 0.9))
+    # the same through refrun's helpers (the signatures the reference workspace is driven with)
+    assert same_bits(refrun.conv2d_i8(ws, xq, w, None, (1, 0), (1, 2), 1, 0.03, 0.004, 0.2, 8),
+                     orc.conv2d_i8(xq, w, None, (1, 0), (1, 2), 1, 0.03, 0.004, 0.2, 8))
+    for o in (dq, ip, flat, conv, qz):
+        o.delete()
+    ws.delete()
+
+
 @pytest.mark.skipif(not (os.path.exists(REF_SO) and os.path.exists(HIP_FOR_REF)),
                     reason="reference runtime / module built against its headers not present")
 def test_module_plugs_into_the_reference_runtime():
