@@ -105,8 +105,19 @@ def build_module(force=False, nart_tree=None, out_name="libart_module_hip.so"):
     return [out]
 
 
+def build_tools(force=False):
+    """nart_promark, the command-line runner (counterpart of the reference's tools/promark.cpp); finds libart.so and
+    the case modules next to itself."""
+    src = _glob("tools", (".cpp",))
+    out = os.path.join(LIB, "nart_promark")
+    if src and (force or not _newer(out, src + [os.path.join(INC, "art", "art.h")])):
+        _run(["g++", "-O2", "-std=c++17", "-Wall", "-I" + INC, "-o", out] + src +
+             ["-L" + LIB, "-lart", "-ldl", "-Wl,--disable-new-dtags", "-Wl,-rpath,$ORIGIN"])
+    return [out] if src else []
+
+
 def build_all(force=False):
-    return [build_hipq(force)] + build_art(force)
+    return [build_hipq(force)] + build_art(force) + build_tools(force)
 
 
 if __name__ == "__main__":

@@ -529,6 +529,13 @@ ART_PUBLIC void hip_workspace_set_stream(workspace_t *w, void *stream)
     ws->own_stream = false;
 }
 
+// Blocks until everything the workspace has launched is done; runners that time a run call it (operators return
+// as soon as their kernels are queued).
+ART_PUBLIC void hip_workspace_synchronize(workspace_t *w)
+{
+    HIPM_HIP(hipStreamSynchronize(reinterpret_cast<hip_workspace_t *>(w)->stream));
+}
+
 #define HIP_ENTRY(TP, T, CONFIG, DESTROY, PREPARE) {&TP, alloc_op<T>, CONFIG, DESTROY, dealloc_op, PREPARE}
 
 ART_PUBLIC op_tp_entry_t hip_op_table[] = {

@@ -142,6 +142,32 @@ def test_int8_ops_through_the_op_api(own_rt):
     ws.delete()
 
 
+def test_command_line_runner(tmp_path):
+    """nart_promark loads an engine file with the `hip` workspace named in a JSON configuration, reshapes the batch
+    (-b), times runs (-n, with and without copies), reads the input from a file (-i) and writes nart-out-<name>.bin
+    (-s) — the reference runner's contract (tools/promark.cpp:192-522).  The saved output must be the oracle's."""
+    import subprocess
+    tool = os.path.join(LIB, "nart_promark")
+    case = cases.resnet18(N=1, hw=64)
+    (tmp_path / "engine.bin").write_bytes(engine.write_engine(case))
+    (tmp_path / "cfg.json").write_text('{"workspaces": {"hip": {}}, "input_workspace": "hip"}')
+    big = cases.resnet18(N=3, hw=64)  # what -b 3 turns the case into
+    x = casecpu.random_input(big, 5)
+    npdt = {"u8": np.uint8, "f32": np.float32}
+    np.ascontiguousarray(x, npdt[big.input.dtype]).tofile(tmp_path / "in.bin")
+    shown = {"u8": "UINT8", "f32": "FLOAT32"}[big.input.dtype] + " " + ", ".join(str(d) for d in big.input.shape)
+    for extra in ([], ["-y"], ["-d"]):
+        r = subprocess.run([tool, "-m", "engine.bin", "-c", "cfg.json", "-n", "3", "-b", "3", "-i", "in.bin", "-s"] + extra,
+                           cwd=tmp_path, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
+        assert r.returncode == 0, r.stderr[-2000:]
+        assert "average cost" in r.stdout and "Process 2 : cost" in r.stdout and shown in r.stdout, r.stdout
+        name = "nart-out-" + case.output.name.replace("/", "_") + ".bin"
+        got = np.fromfile(tmp_path / name, dtype=npdt[big.output.dtype]).reshape(big.output.shape)
+        want = casecpu.run_case(big, x)[big.output.name]
+        assert same_bits(got, want), extra
+        os.remove(tmp_path / name)
+
+
 @pytest.mark.skipif(not (os.path.exists(REF_SO) and os.path.exists(HIP_FOR_REF)),
                     reason="reference runtime / module built against its headers not present")
 def test_module_plugs_into_the_reference_runtime():
