@@ -256,6 +256,8 @@ bool op_setting_array_get(const op_t *op, uint32_t item, uint32_t dtype, size_t 
 #define OP_RELU     OP_DECLARE(OP_GROUP_CODE_DEFAULT, 0x0101)
 #define OP_POOL     OP_DECLARE(OP_GROUP_CODE_DEFAULT, 0x0102)
 #define OP_IP       OP_DECLARE(OP_GROUP_CODE_DEFAULT, 0x0104)
+#define OP_CONCAT   OP_DECLARE(OP_GROUP_CODE_DEFAULT, 0x0106)
+#define OP_SOFTMAX  OP_DECLARE(OP_GROUP_CODE_DEFAULT, 0x010B)
 #define OP_ELTWISE  OP_DECLARE(OP_GROUP_CODE_DEFAULT, 0x010C)
 #define OP_RESHAPE  OP_DECLARE(OP_GROUP_CODE_DEFAULT, 0x010E)
 #define OP_QUANT_QUANTIZE   OP_DECLARE(OP_GROUP_CODE_QUANT, 0x80000000u) /* quant_op_tp.h:23 */
@@ -263,6 +265,7 @@ bool op_setting_array_get(const op_t *op, uint32_t item, uint32_t dtype, size_t 
 
 /* shared op types of the generic ops: shape inference lives in the core (art/src/op.c) */
 extern const op_tp_t op_conv_2d_tp, op_ip_tp, op_pool_tp, op_relu_tp, op_add_tp, op_eltwise_tp, op_reshape_tp;
+extern const op_tp_t op_concat_tp, op_softmax_tp;
 
 /* setting ids (op_settings.h, quant_op_settings.h:24-40) */
 enum {
@@ -281,6 +284,8 @@ enum {
     SETTING_ELTWISE_OPERATION = 1, SETTING_ELTWISE_COEFF = 2, SETTING_ELTWISE_RELU_FLAG = 3,
     SETTING_ELTWISE_OP_PROD = 0, SETTING_ELTWISE_OP_SUM = 1, SETTING_ELTWISE_OP_MAX = 2
 };
+enum { SETTING_CONCAT_AXIS = 1 };  /* op_settings.h:74 */
+enum { SETTING_SOFTMAX_AXIS = 1 }; /* op_settings.h:89 */
 enum { SETTING_RESHAPE_DIMS = 1, SETTING_RESHAPE_DIM_SIZE = 2, SETTING_RESHAPE_AXIS = 3, SETTING_RESHAPE_NUM_AXES = 4 };
 #define SETTING_QUANT(code) ((uint32_t)((OP_GROUP_CODE_QUANT << 16) | (code)))
 #define SETTING_QUANT_IALPHA      SETTING_QUANT(0x0101)

@@ -134,6 +134,15 @@ int hipq_eltwise_u8(const void *const *in, int n_in, const float *coeff, const f
 int hipq_relu_u8(const void *x, void *y, size_t count, float ialpha, int izp, float oalpha, int ozp,
                  int obits, void *stream);
 
+/* op_quant_concat_run — src/op/concat.c:82-124: concatenation along the channels with a per-input rescale.
+ * in[j]: NHWC with channels[j] channels (stride hipq_channel_stride(channels[j])); y: NHWC with the summed
+ * channel count; npix = N*H*W. */
+int hipq_concat_u8(const void *const *in, int n_in, const int *channels, const float *ialpha,
+                   const uint8_t *izp, void *y, size_t npix, float oalpha, int ozp, int obits, void *stream);
+/* op_quant_softmax_run — src/op/softmax.c:89-122, over the channels of every pixel (axis 1 of NCHW). */
+int hipq_softmax_u8(const void *x, void *y, size_t npix, int C, int cs, float ialpha, int izp,
+                    float oalpha, int ozp, int obits, void *stream);
+
 /* ---- pooling: op_quant_pool_max_run / op_quant_pool_average_run — src/op/pool.c:96-249.
  * x: NHWC [N,H,W,cs], y: NHWC [N,OH,OW,cs]; OH, OW as inferred by art/src/op.c:903-967. */
 int hipq_pool_u8(const void *x, void *y, int N, int C, int H, int W, int OH, int OW, int cs, int kh,

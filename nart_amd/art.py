@@ -34,6 +34,8 @@ OP_POOL = 0x0102
 OP_IP = 0x0104
 OP_ELTWISE = 0x010C
 OP_RESHAPE = 0x010E
+OP_CONCAT, OP_SOFTMAX = 0x0106, 0x010B
+SETTING_CONCAT_AXIS = SETTING_SOFTMAX_AXIS = 1
 OP_QUANT_QUANTIZE = (OP_GROUP_QUANT << 32) | 0x80000000   # quant_op_tp.h:23
 OP_QUANT_DEQUANTIZE = (OP_GROUP_QUANT << 32) | 0x80000001  # quant_op_tp.h:24
 
@@ -313,6 +315,16 @@ class Workspace:
         if qtype is not None:
             op.set_single(SETTING_QUANT_QTYPE, dtINT32, qtype)
         return op.set_quant(ialpha=ialpha, izp=izp, bits=bits).config()
+
+    def concat(self, ins, q, axis=1):
+        op = self.new_op(OP_CONCAT, list(ins))
+        op.set_single(SETTING_CONCAT_AXIS, dtUINT32, axis)
+        return op.set_quant(**q).config()
+
+    def softmax(self, x, q, axis=1):
+        op = self.new_op(OP_SOFTMAX, [x])
+        op.set_single(SETTING_SOFTMAX_AXIS, dtUINT32, axis)
+        return op.set_quant(**q).config()
 
     def reshape_flatten(self, x, axis=1):
         """Caffe-style flatten expressed as `reshape` (dims [0,-1] from `axis` on)."""

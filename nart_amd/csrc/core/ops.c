@@ -169,6 +169,27 @@ static bool infer_reshape(op_t *op)
     return tensor_reshape(y, axis + (int)n, full);
 }
 
+/* ---- concat (op.c:872-901): all dims equal except `axis`, which adds up ---------------------------------------- */
+static bool infer_concat(op_t *op)
+{
+    const uint32_t axis = get_u32(op, SETTING_CONCAT_AXIS);
+    ART_CHECK(op->input_size >= 2);
+    const tensor_t *x0 = op->input_tensors[0];
+    ART_CHECK((int)axis < x0->shape.dim_size);
+    uint32_t total = x0->shape.dim[axis];
+    for (size_t i = 1; i < op->input_size; ++i) {
+        const tensor_t *xi = op->input_tensors[i];
+        ART_CHECK(xi->shape.dim_size == x0->shape.dim_size && xi->dtype == x0->dtype);
+        for (int j = 0; j < x0->shape.dim_size; ++j)
+            ART_CHECK(j == (int)axis || xi->shape.dim[j] == x0->shape.dim[j]);
+        total += xi->shape.dim[axis];
+    }
+    tensor_t *y = single_output(op, false);
+    y->shape = x0->shape;
+    y->shape.dim[axis] = total;
+    return true;
+}
+
 /* ---- the op-type objects ------------------------------------------------------------------------------------------- */
 #define C_REQ(i, t) {.item = i, .dtype = t, .ctp = ENUM_SETTING_CONSTRAINT_REQUIRED, .name = #i}
 #define C_OPT(i, t, member, dft) \
@@ -219,3 +240,11 @@ ART_PUBLIC const op_tp_t op_reshape_tp = { /* op.c:2691-2703 */
     .max_output_size = 1, .infer_output_func = infer_reshape,
     .constraints = {C_REP(SETTING_RESHAPE_DIMS, dtINT32), C_OPT(SETTING_RESHAPE_AXIS, dtINT32, i32, 0),
                     C_OPT(SETTING_RESHAPE_NUM_AXES, dtINT32, i32, -1), C_END()}};
+
+ART_PUBLIC const op_tp_t op_concat_tp = { /* op.c:2614-2624 */
+    .op_tp_code = OP_CONCAT, .name = "concat", .min_input_size = 2, .max_input_size = 0xffff, .min_output_size = 1,
+    .max_output_size = 1, .infer_output_func = infer_concat, .constraints = {C_REQ(SETTING_CONCAT_AXIS, dtUINT32), C_END()}};
+
+ART_PUBLIC const op_tp_t op_softmax_tp = { /* op.c:2544-2560 */
+    .op_tp_code = OP_SOFTMAX, .name = "softmax", .min_input_size = 1, .max_input_size = 1, .min_output_size = 1,
+    .max_output_size = 1, .infer_output_func = infer_unary, .constraints = {C_OPT(SETTING_SOFTMAX_AXIS, dtUINT32, u32, 1), C_END()}};

@@ -348,6 +348,91 @@ __global__ __launch_bounds__(256) void pool_gavg16_u8_kernel(const PoolArgs p, u
     }
 }
 
+// ---- concat along the channels (op_quant_concat_run, concat.c:82-124) ----------------------------------------------
+// Output pixel p, channel c comes from input j with off[j] <= c < off[j+1]; every input has its own rescale
+// y = sat(rrn(mult_j * (x - zp_j), shift_j) + oz) with a 16-bit multiplier.  One thread writes one dword (4 channels)
+// of the output; when the 4 channels come from one input at a dword-aligned offset they are read as one dword.
+struct ConcatArgs {
+    const uint8_t *in[HIPQ_MAX_ELTWISE_INPUTS];
+    int off[HIPQ_MAX_ELTWISE_INPUTS + 1]; // first output channel of each input; off[n_in] = total channels
+    int cs[HIPQ_MAX_ELTWISE_INPUTS];      // channel stride of each input
+    uint32_t mult[HIPQ_MAX_ELTWISE_INPUTS];
+    int shift[HIPQ_MAX_ELTWISE_INPUTS];
+    int zp[HIPQ_MAX_ELTWISE_INPUTS];
+    int n_in, oz, hi, cs_out;
+    uint8_t *y;
+    size_t npix;
+};
+
+__device__ static inline uint32_t concat_one(uint32_t x, int j, const ConcatArgs &p)
+{
+    const int32_t pr = (int32_t)p.mult[j] * ((int32_t)x - p.zp[j]); // 16-bit * 9-bit
+    return (uint32_t)sat_hi((int32_t)(rshift_rn(pr, p.shift[j]) + p.oz), p.hi);
+}
+
+__global__ __launch_bounds__(256) void concat_u8_kernel(const ConcatArgs p)
+{
+    const int cq = p.cs_out >> 2;
+    const size_t total = p.npix * cq;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (size_t)gridDim.x * blockDim.x) {
+        const size_t pix = idx / cq;
+        const int c0 = (int)(idx - pix * cq) * 4;
+        uint32_t o = 0;
+        int j = 0;
+        while (j + 1 < p.n_in && c0 >= p.off[j + 1])
+            j++;
+        if (c0 + 3 < p.off[j + 1] && ((c0 - p.off[j]) & 3) == 0) {
+            const uint32_t v = *reinterpret_cast<const uint32_t *>(p.in[j] + pix * p.cs[j] + (c0 - p.off[j]));
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                o |= concat_one((v >> (8 * e)) & 255, j, p) << (8 * e);
+        } else {
+            for (int e = 0; e < 4; e++) {
+                const int c = c0 + e;
+                if (c >= p.off[p.n_in])
+                    break; // pad channels of the output stay zero
+                while (c >= p.off[j + 1])
+                    j++;
+                o |= concat_one(p.in[j][pix * p.cs[j] + (c - p.off[j])], j, p) << (8 * e);
+            }
+        }
+        *reinterpret_cast<uint32_t *>(p.y + pix * p.cs_out + c0) = o;
+    }
+}
+
+// ---- softmax over the channels (op_quant_softmax_run, softmax.c:89-122) -------------------------------------------
+// e(x) = fp32(exp(double(fp32(ialpha * (x - izp))))) takes 256 values: the host tabulates them with the C library's
+// exp, the very call the reference makes.  A thread owns a pixel: it sums its channels in fp32 in channel order (the
+// reference's order), then y = saturate_float_by_bits(e / sum / oalpha + ozp) with IEEE fp32 divisions.
+struct SoftmaxArgs {
+    const uint8_t *x;
+    uint8_t *y;
+    size_t npix;
+    int C, cs;
+    float oalpha, ozp, hi;
+    float table[256];
+};
+
+__global__ __launch_bounds__(256) void softmax_u8_kernel(const SoftmaxArgs p)
+{
+    __shared__ float tab[256];
+    tab[threadIdx.x] = p.table[threadIdx.x];
+    __syncthreads();
+    for (size_t pix = (size_t)blockIdx.x * blockDim.x + threadIdx.x; pix < p.npix; pix += (size_t)gridDim.x * blockDim.x) {
+        const uint8_t *xr = p.x + pix * p.cs;
+        uint8_t *yr = p.y + pix * p.cs;
+        float sum = 0.f;
+        for (int c = 0; c < p.C; c++)
+            sum = __fadd_rn(sum, tab[xr[c]]);
+        for (int c = 0; c < p.C; c++) {
+            const float q = __fadd_rn(__fdiv_rn(__fdiv_rn(tab[xr[c]], sum), p.oalpha), p.ozp);
+            yr[c] = q > p.hi ? (uint8_t)p.hi : (q < 0 ? (uint8_t)0 : (uint8_t)((double)q + 0.5));
+        }
+        for (int c = p.C; c < p.cs; c++)
+            yr[c] = 0;
+    }
+}
+
 // ---- quantize (quantize.c:145-157): fp32 NCHW -> uint8 NHWC --------------------------------------
 // One thread produces the 4 channels of one dword of the output; reads are coalesced along W per
 // channel plane, writes along the pixel index.
@@ -599,6 +684,53 @@ extern "C" int hipq_relu_u8(const void *x, void *y, size_t count, float ia, int 
     p.iz = iz, p.oz = oz, p.hi = (1 << obits) - 1;
     hipLaunchKernelGGL(relu_u8_kernel, dim3(grid_for(count / 16)), dim3(256), 0, static_cast<hipStream_t>(stream), p);
     return launch_status("relu_u8_kernel");
+}
+
+extern "C" int hipq_concat_u8(const void *const *in, int n_in, const int *channels, const float *ialpha, const uint8_t *izp,
+                              void *y, size_t npix, float oa, int oz, int obits, void *stream)
+{
+    clear_error();
+    HIPQ_REQUIRE(in && channels && ialpha && izp && y, "hipq_concat_u8: null pointer");
+    HIPQ_REQUIRE(n_in >= 2 && n_in <= HIPQ_MAX_ELTWISE_INPUTS, "hipq_concat_u8: %d inputs (2..%d supported)", n_in,
+                 HIPQ_MAX_ELTWISE_INPUTS);
+    HIPQ_REQUIRE(obits >= 1 && obits <= 8, "hipq_concat_u8: obits must be in 1..8");
+    if (npix == 0)
+        return 0;
+    ConcatArgs p;
+    memset(&p, 0, sizeof p);
+    for (int j = 0; j < n_in; j++) {
+        HIPQ_REQUIRE(in[j] && channels[j] > 0, "hipq_concat_u8: input %d is null or has no channels", j);
+        p.in[j] = static_cast<const uint8_t *>(in[j]);
+        p.off[j + 1] = p.off[j] + channels[j];
+        p.cs[j] = hipq_channel_stride(channels[j]);
+        hipq_quant_scale(ialpha[j] / oa, 16, &p.mult[j], &p.shift[j]); // concat.c:104-108
+        p.mult[j] &= 0xffff;
+        HIPQ_REQUIRE(valid_shift(p.shift[j]), "hipq_concat_u8: scale of input %d out of the fixed-point range", j);
+        p.zp[j] = izp[j];
+    }
+    p.n_in = n_in, p.oz = oz, p.hi = (1 << obits) - 1, p.cs_out = hipq_channel_stride(p.off[n_in]);
+    p.y = static_cast<uint8_t *>(y), p.npix = npix;
+    hipLaunchKernelGGL(concat_u8_kernel, dim3(grid_for(npix * (p.cs_out / 4))), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+    return launch_status("concat_u8_kernel");
+}
+
+extern "C" int hipq_softmax_u8(const void *x, void *y, size_t npix, int C, int cs, float ia, int iz, float oa, int oz, int obits,
+                               void *stream)
+{
+    clear_error();
+    HIPQ_REQUIRE(x && y && C > 0 && cs >= C, "hipq_softmax_u8: bad argument");
+    HIPQ_REQUIRE(obits >= 1 && obits <= 8, "hipq_softmax_u8: obits must be in 1..8");
+    if (npix == 0)
+        return 0;
+    SoftmaxArgs p;
+    p.x = static_cast<const uint8_t *>(x), p.y = static_cast<uint8_t *>(y), p.npix = npix, p.C = C, p.cs = cs;
+    p.oalpha = oa, p.ozp = (float)oz, p.hi = (float)((1 << obits) - 1);
+    for (int v = 0; v < 256; v++) {
+        const float arg = ia * (float)(v - iz);        // softmax.c:112: an fp32 product ...
+        p.table[v] = (float)std::exp((double)arg);     // ... passed to the double exp, stored as fp32
+    }
+    hipLaunchKernelGGL(softmax_u8_kernel, dim3(grid_for(npix)), dim3(256), 0, static_cast<hipStream_t>(stream), p);
+    return launch_status("softmax_u8_kernel");
 }
 
 extern "C" int hipq_pool_u8(const void *x, void *y, int N, int C, int H, int W, int OH, int OW, int cs, int kh, int kw,

@@ -17,6 +17,7 @@ extern "C" {
 #include "art/quant/quant_op_tp.h"
 // the shared op types of the generic ops live in libart (art/src/op.c:2252-2703)
 extern const op_tp_t op_conv_2d_tp, op_ip_tp, op_pool_tp, op_relu_tp, op_add_tp, op_eltwise_tp, op_reshape_tp;
+extern const op_tp_t op_concat_tp, op_softmax_tp;
 }
 #define ART_PUBLIC __attribute__((visibility("default")))
 #else

@@ -325,6 +325,87 @@ void relu_prepare(op_t *op)
     op->run_func = relu_run;
 }
 
+// ---- concat / softmax (uint8 only, along the channels) --------------------------------------------------------------------
+struct axis_op_t {
+    op_t o;
+    uint32_t axis;
+    QSet qi, qo;
+};
+
+void concat_config(op_t *op)
+{
+    axis_op_t *a = reinterpret_cast<axis_op_t *>(op);
+    HIPM_CHECK(op_setting_single_get(op, SETTING_CONCAT_AXIS, dtUINT32, &a->axis));
+    READ_I(op, &a->qi);
+    READ_O(op, &a->qo);
+    HIPM_CHECK(a->qi.n >= op->input_size);
+}
+
+void concat_run(op_t *op)
+{
+    axis_op_t *a = reinterpret_cast<axis_op_t *>(op);
+    const void *in[HIPQ_MAX_ELTWISE_INPUTS];
+    int ch[HIPQ_MAX_ELTWISE_INPUTS];
+    for (size_t i = 0; i < op->input_size; ++i) {
+        in[i] = in_ptr(op, (int)i);
+        ch[i] = as_hip(op->input_tensors[i]->mem)->C;
+    }
+    const hip_mem_t *y = as_hip(op->output_tensors[0].mem);
+    HIPM_HIPQ(hipq_concat_u8(in, (int)op->input_size, ch, a->qi.alpha, a->qi.zp, out_ptr(op), (size_t)y->N * y->H * y->W,
+                             a->qo.alpha[0], a->qo.zp[0], a->qo.bits[0], op_stream(op)));
+}
+
+void concat_prepare(op_t *op)
+{
+    axis_op_t *a = reinterpret_cast<axis_op_t *>(op);
+    HIPM_CHECK(op->input_size <= HIPQ_MAX_ELTWISE_INPUTS);
+    require_hip_u8(op, op->input_size);
+    alloc_and_tag(op);
+    // the reference's loop copies image by image, input by input (concat.c:99-121): that is a concatenation along
+    // dimension 1 whatever the axis setting says, so only axis 1 has a meaning to reproduce
+    if (a->axis != 1) {
+        fprintf(stderr, "[hip module] concat along axis %u is not implemented (channels only)\n", a->axis);
+        abort();
+    }
+    const hip_mem_t *y = as_hip(op->output_tensors[0].mem);
+    HIPM_CHECK(y->layout == HIP_LAYOUT_NHWC_U8);
+    for (size_t i = 0; i < op->input_size; ++i) {
+        const hip_mem_t *x = as_hip(op->input_tensors[i]->mem);
+        HIPM_CHECK(x->layout == HIP_LAYOUT_NHWC_U8 && x->N == y->N && x->H == y->H && x->W == y->W);
+    }
+    op->run_func = concat_run;
+}
+
+void softmax_config(op_t *op)
+{
+    axis_op_t *a = reinterpret_cast<axis_op_t *>(op);
+    HIPM_CHECK(op_setting_single_get(op, SETTING_SOFTMAX_AXIS, dtUINT32, &a->axis));
+    READ_I(op, &a->qi);
+    READ_O(op, &a->qo);
+}
+
+void softmax_run(op_t *op)
+{
+    axis_op_t *a = reinterpret_cast<axis_op_t *>(op);
+    const hip_mem_t *x = as_hip(op->input_tensors[0]->mem);
+    HIPM_HIPQ(hipq_softmax_u8(in_ptr(op, 0), out_ptr(op), (size_t)x->N * x->H * x->W, x->C, x->cs, a->qi.alpha[0], a->qi.zp[0],
+                              a->qo.alpha[0], a->qo.zp[0], a->qo.bits[0], op_stream(op)));
+}
+
+void softmax_prepare(op_t *op)
+{
+    axis_op_t *a = reinterpret_cast<axis_op_t *>(op);
+    require_hip_u8(op, 1);
+    alloc_and_tag(op);
+    same_geometry(op);
+    if (a->axis != 1) { // other axes would need a strided walk over the channels-last device layout
+        fprintf(stderr, "[hip module] softmax along axis %u is not implemented (channels only)\n", a->axis);
+        abort();
+    }
+    HIPM_CHECK(as_hip(op->input_tensors[0]->mem)->layout == HIP_LAYOUT_NHWC_U8);
+    op->run_func = softmax_run;
+}
+
 // ---- pool ----------------------------------------------------------------------------------------------------------
 struct pool_op_t {
     op_t o;
@@ -548,6 +629,8 @@ ART_PUBLIC op_tp_entry_t hip_op_table[] = {
     HIP_ENTRY(op_eltwise_tp, ew_op_t, eltwise_config, destroy_nothing, eltwise_prepare),
     HIP_ENTRY(op_pool_tp, pool_op_t, pool_config, destroy_nothing, pool_prepare),
     HIP_ENTRY(op_reshape_tp, ew_op_t, reshape_config, destroy_nothing, reshape_prepare),
+    HIP_ENTRY(op_concat_tp, axis_op_t, concat_config, destroy_nothing, concat_prepare),
+    HIP_ENTRY(op_softmax_tp, axis_op_t, softmax_config, destroy_nothing, softmax_prepare),
     {nullptr, nullptr, nullptr, nullptr, nullptr, nullptr},
 };
 

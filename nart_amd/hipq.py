@@ -49,6 +49,10 @@ _SIGS = {
                                   C.c_size_t, C.c_int, C.c_float, C.c_int, C.c_int, C.c_void_p]),
     "hipq_relu_u8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_float, C.c_int, C.c_float, C.c_int,
                                C.c_int, C.c_void_p]),
+    "hipq_concat_u8": (C.c_int, [C.POINTER(C.c_void_p), C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t,
+                                 C.c_float, C.c_int, C.c_int, C.c_void_p]),
+    "hipq_softmax_u8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int, C.c_int, C.c_float, C.c_int, C.c_float,
+                                  C.c_int, C.c_int, C.c_void_p]),
     "hipq_pool_u8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 14 + [C.c_float, C.c_int, C.c_float, C.c_int,
                                                                           C.c_int, C.c_void_p]),
     "hipq_quantize_u8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_float, C.c_int, C.c_int, C.c_void_p]),
@@ -198,6 +202,24 @@ def eltwise_u8(ins, y, ialpha, izp, oalpha, ozp, operation=1, coeff=None, obits=
 
 def relu_u8(x, y, ialpha, izp, oalpha, ozp, obits=8):
     check(lib().hipq_relu_u8(_ptr(x), _ptr(y), x.numel(), ialpha, izp, oalpha, ozp, obits, _stream()))
+    return y
+
+
+def concat_u8(ins, channels, y, ialpha, izp, oalpha, ozp, obits=8):
+    n = len(ins)
+    ptrs = (C.c_void_p * n)(*[t.data_ptr() for t in ins])
+    ch = np.ascontiguousarray(channels, np.int32)
+    ia = np.ascontiguousarray(ialpha, np.float32)
+    iz = np.ascontiguousarray(izp, np.uint8)
+    N, H, W, _ = y.shape
+    check(lib().hipq_concat_u8(ptrs, n, C.c_void_p(ch.ctypes.data), C.c_void_p(ia.ctypes.data), C.c_void_p(iz.ctypes.data),
+                               _ptr(y), N * H * W, oalpha, ozp, obits, _stream()))
+    return y
+
+
+def softmax_u8(x, y, Cc, ialpha, izp, oalpha, ozp, obits=8):
+    N, H, W, cs = x.shape
+    check(lib().hipq_softmax_u8(_ptr(x), _ptr(y), N * H * W, Cc, cs, ialpha, izp, oalpha, ozp, obits, _stream()))
     return y
 
 

@@ -166,6 +166,33 @@ def dequantize_u8(x, ialpha, izp):
     return y
 
 
+def concat_u8(ins, ialpha, izp, oalpha, ozp, obits=8):
+    """Concatenation along dimension 1 with per-input rescaling (the reference ignores `axis`, concat.c:99-121)."""
+    ins = [np.ascontiguousarray(a, np.uint8) for a in ins]
+    n = len(ins)
+    N = ins[0].shape[0]
+    per = (C.c_size_t * n)(*[a.size // N for a in ins])
+    ptrs = (C.c_void_p * n)(*[a.ctypes.data for a in ins])
+    ia = np.ascontiguousarray(ialpha, np.float32)
+    iz = np.ascontiguousarray(izp, np.uint8)
+    shape = list(ins[0].shape)
+    shape[1] = sum(a.shape[1] for a in ins)
+    y = np.empty(shape, np.uint8)
+    lib().orc_concat_u8(ptrs, n, per, _p(ia), _p(iz), _p(y), N, _f(oalpha), int(ozp), int(obits))
+    return y
+
+
+def softmax_u8(x, axis, ialpha, izp, oalpha, ozp, obits=8):
+    x = np.ascontiguousarray(x, np.uint8)
+    ch = x.shape[axis]
+    outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+    inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    y = np.empty(x.shape, np.uint8)
+    lib().orc_softmax_u8(_p(x), _p(y), C.c_size_t(outer), C.c_size_t(ch), C.c_size_t(inner), _f(ialpha), int(izp),
+                         _f(oalpha), int(ozp), int(obits))
+    return y
+
+
 def conv2d_i8(x, w, bias, pad, stride, group, ialpha, walpha, oalpha, obits=8, return_acc=False):
     x = np.ascontiguousarray(x, np.int8)
     w = np.ascontiguousarray(w, np.int8)

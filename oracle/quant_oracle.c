@@ -390,6 +390,51 @@ void orc_dequantize_u8(const uint8_t *x, float *y, size_t count, float ialpha, i
         y[i] = (float)((int)x[i] - izp) * ialpha; /* dequantize.c:121 */
 }
 
+/* op_quant_concat_run — concat.c:82-124: whatever `axis` says, the loop copies image by image and input by input,
+ * i.e. it concatenates along dimension 1; every input is rescaled: (mult, shift) = gqs(ialpha_j / oalpha, 16),
+ * y = sat(rrn(mult * (x - izp_j), shift) + ozp).  mult is a uint16_t, the product an int. */
+void orc_concat_u8(const uint8_t *const *in, int n_in, const size_t *per_image, const float *ialpha,
+                   const uint8_t *izp, uint8_t *y, int N, float oalpha, int ozp, int obits)
+{
+    for (int n = 0; n < N; n++)
+        for (int j = 0; j < n_in; j++) {
+            uint32_t mult;
+            int shift;
+            orc_quant_scale(ialpha[j] / oalpha, 16, &mult, &shift);
+            mult &= 0xffff;
+            const uint8_t *src = in[j] + (size_t)n * per_image[j];
+            for (size_t k = 0; k < per_image[j]; k++) {
+                const int32_t p = (int32_t)mult * ((int32_t)src[k] - (int32_t)izp[j]);
+                *y++ = orc_sat_bits((int32_t)(orc_rshift_rn(p, shift) + ozp), obits);
+            }
+        }
+}
+
+/* op_quant_softmax_run — softmax.c:89-122: e = (float)exp((double)(ialpha * (x - izp))) (the argument is an fp32
+ * product, exp is the C library's double routine), the sum runs in fp32 in channel order, and
+ * y = saturate_float_by_bits(e / sum / oalpha + ozp) with every operation in fp32. */
+void orc_softmax_u8(const uint8_t *x, uint8_t *y, size_t outer, size_t ch, size_t inner, float ialpha, int izp,
+                    float oalpha, int ozp, int obits)
+{
+    const float hi = (float)((1 << obits) - 1);
+    float *e = (float *)malloc(sizeof(float) * (ch ? ch : 1));
+    for (size_t o = 0; o < outer; o++)
+        for (size_t i = 0; i < inner; i++) {
+            float sum = 0.f;
+            for (size_t c = 0; c < ch; c++) {
+                const size_t idx = (o * ch + c) * inner + i;
+                e[c] = (float)exp((double)(ialpha * (float)((int)x[idx] - izp)));
+                sum += e[c];
+            }
+            for (size_t c = 0; c < ch; c++) {
+                const size_t idx = (o * ch + c) * inner + i;
+                const float q = e[c] / sum / oalpha + (float)ozp;
+                y[idx] = q > hi ? (uint8_t)hi : (q < 0 ? 0 : (uint8_t)((double)q + 0.5));
+            }
+        }
+    free(e);
+}
+
 /* ---- int8 symmetric variants (no zero points) --------------------------------------------------- */
 
 /* ssaturate_int_by_bits — quant_helper.h:43-47: clip to +-(2^bits - 1), then the implicit conversion of the

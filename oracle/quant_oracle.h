@@ -94,6 +94,13 @@ void orc_quantize_u8(const float *x, uint8_t *y, size_t count, float oalpha, int
 /* op_dequantize_run_u8 — dequantize.c:111-123. */
 void orc_dequantize_u8(const uint8_t *x, float *y, size_t count, float ialpha, int izp);
 
+/* op_quant_concat_run — concat.c:82-124.  per_image[j] = elements of input j per image (C_j*H*W). */
+void orc_concat_u8(const uint8_t *const *in, int n_in, const size_t *per_image, const float *ialpha,
+                   const uint8_t *izp, uint8_t *y, int N, float oalpha, int ozp, int obits);
+/* op_quant_softmax_run — softmax.c:89-122 over [outer, ch, inner]. */
+void orc_softmax_u8(const uint8_t *x, uint8_t *y, size_t outer, size_t ch, size_t inner, float ialpha, int izp,
+                    float oalpha, int ozp, int obits);
+
 /* ---- int8 symmetric variants: no zero points, outputs clipped to +-(2^obits - 1) and truncated to int8 ---- */
 /* ssaturate_int_by_bits — quant_helper.h:43-47. */
 int8_t orc_ssat_bits(int32_t x, int bits);

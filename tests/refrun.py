@@ -76,6 +76,15 @@ def pool_u8(ws, x, kernel, pad, stride, method, ceil_mode, ialpha, izp, oalpha, 
     return _run(ws.pool(ws.tensor(x), kernel, pad, stride, method, ceil_mode, q))
 
 
+def concat_u8(ws, ins, ialpha, izp, oalpha, ozp, axis=1):
+    q = _q(ialpha=list(ialpha), izp=list(izp), oalpha=oalpha, ozp=ozp)
+    return _run(ws.concat([ws.tensor(a) for a in ins], q, axis))
+
+
+def softmax_u8(ws, x, axis, ialpha, izp, oalpha, ozp):
+    return _run(ws.softmax(ws.tensor(x), _q(ialpha=ialpha, izp=izp, oalpha=oalpha, ozp=ozp), axis))
+
+
 def quantize_u8(ws, x, oalpha, ozp):
     return _run(ws.quantize(ws.tensor(np.asarray(x, np.float32)), oalpha, ozp))
 

@@ -120,13 +120,14 @@ def _check_hip_table(rt, lib):
     core.workspace_support_op.restype = C.c_bool
     core.workspace_support_op.argtypes = [C.POINTER(art.workspace_t), C.c_uint64, C.c_bool]
     g = art.OP_GROUP_QUANT << 32
-    for code in (art.OP_CONV_2D, art.OP_IP, art.OP_POOL, art.OP_RELU, art.OP_ADD, art.OP_ELTWISE, art.OP_RESHAPE):
+    for code in (art.OP_CONV_2D, art.OP_IP, art.OP_POOL, art.OP_RELU, art.OP_ADD, art.OP_ELTWISE, art.OP_RESHAPE,
+                 art.OP_CONCAT, art.OP_SOFTMAX):
         assert core.workspace_support_op(ws.ptr, g | code, True), hex(code)      # strict: group 6
         assert not core.workspace_support_op(ws.ptr, (2 << 32) | code, True)      # another module's group
         assert core.workspace_support_op(ws.ptr, (2 << 32) | code, False)         # by op code alone
     assert core.workspace_support_op(ws.ptr, art.OP_QUANT_QUANTIZE, False)
     assert core.workspace_support_op(ws.ptr, art.OP_QUANT_DEQUANTIZE, True)
-    assert not core.workspace_support_op(ws.ptr, g | 0x010B, False)               # softmax: not in the table
+    assert not core.workspace_support_op(ws.ptr, g | 0x010D, False)               # scale (op_tp.h:61): not in the table
     # configure a conv and a pool through the public API and read back the inferred shapes
     x = rt.tensor(dtype=np.uint8, shape=(2, 64, 56, 56))
     w = rt.tensor(np.zeros((128, 64, 3, 3), np.uint8))

@@ -276,6 +276,32 @@ def test_full_size_properties():
         assert np.array_equal(y[i:i + 1], want)
 
 
+def test_concat_softmax():
+    rng = np.random.default_rng(44)
+    for it in range(12):
+        n_in = int(rng.integers(2, 9))
+        N, H, W = int(rng.integers(1, 4)), int(rng.integers(1, 9)), int(rng.integers(1, 9))
+        chans = [int(rng.choice([1, 3, 4, 7, 16, 20, 64, 100])) for _ in range(n_in)]
+        if it == 0:
+            N, H, W, chans = 4, 28, 28, [64, 128, 32, 32]  # an inception-style block: every piece dword-aligned
+        ins = [rng.integers(0, 256, (N, c, H, W), dtype=np.uint8) for c in chans]
+        ia, iz = [rand_q(rng) for _ in ins], [int(rng.integers(0, 256)) for _ in ins]
+        oa, oz = rand_q(rng), int(rng.integers(0, 256))
+        want = orc.concat_u8(ins, ia, iz, oa, oz)
+        yd = torch.full((N, H, W, hipq.channel_stride(sum(chans))), 0xAB, dtype=torch.uint8, device="cuda")
+        hipq.concat_u8([hipq.to_device_nhwc(a) for a in ins], chans, yd, ia, iz, oa, oz)
+        assert np.array_equal(hipq.from_device_nhwc(yd, sum(chans)), want), (it, chans)
+        assert int(yd[..., sum(chans):].max().item() if yd.shape[-1] > sum(chans) else 0) == 0  # pad channels cleared
+    for it, shape in enumerate([(64, 1000, 1, 1), (2, 21, 33, 17), (1, 2, 5, 5), (3, 7, 1, 9), (5, 300, 2, 2)]):
+        x = rng.integers(0, 256, shape, dtype=np.uint8)
+        q = (rand_q(rng, 1e-2, 0.2), int(rng.integers(0, 256)), float(np.float32(1.0 / 255)), int(rng.integers(0, 3)))
+        want = orc.softmax_u8(x, 1, *q)
+        xd = hipq.to_device_nhwc(x)
+        yd = torch.empty_like(xd)
+        hipq.softmax_u8(xd, yd, shape[1], *q)
+        assert np.array_equal(hipq.from_device_nhwc(yd, shape[1]), want), (it, shape, q)
+
+
 # ---- int8 symmetric variants (op_conv_2d_i8xi8_run, op_quant_ip_i8xi8_run, op_quantize_run_i8, op_dequantize_run_i8) ----
 def run_conv_i8(x, w, b, pad, stride, group, q, obits=8, in_cs=None):
     ia, wa, oa = q

@@ -107,6 +107,20 @@ def test_single_ops_through_the_op_api(own_rt):
     ws.delete()
 
 
+def test_concat_softmax_through_the_op_api(own_rt):
+    import refrun
+    from oracle import orc
+    ws = own_rt.workspace("hip")
+    rng = np.random.default_rng(13)
+    ins = [rng.integers(0, 256, (2, c, 6, 5), dtype=np.uint8) for c in (16, 5, 32)]
+    ia, iz = [0.02, 0.05, 0.011], [3, 128, 250]
+    assert same_bits(refrun.concat_u8(ws, ins, ia, iz, 0.03, 17), orc.concat_u8(ins, ia, iz, 0.03, 17))
+    x = rng.integers(0, 256, (4, 1000), dtype=np.uint8)
+    got = refrun.softmax_u8(ws, x.reshape(4, 1000, 1, 1), 1, 0.07, 140, 1.0 / 255, 0)
+    assert same_bits(got.reshape(4, 1000), orc.softmax_u8(x, 1, 0.07, 140, 1.0 / 255, 0))
+    ws.delete()
+
+
 def test_int8_ops_through_the_op_api(own_rt):
     """quantize (symmetric) -> conv (int8) -> flatten -> ip (int8) -> dequantize on the hip workspace, every
     stage against the oracle; the operators are chosen from the tensor dtype / the qtype setting as in the reference

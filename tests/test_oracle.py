@@ -161,6 +161,26 @@ def test_quantize_dequantize_vs_reference(ref_ws):
         assert np.array_equal(orc.dequantize_u8(want, oa, oz).view(np.uint32), d.view(np.uint32))
 
 
+def test_concat_softmax_vs_reference(ref_ws):
+    rng = np.random.default_rng(24)
+    for it in range(20):
+        n_in = int(rng.integers(2, 5))
+        N, H, W = int(rng.integers(1, 4)), int(rng.integers(1, 7)), int(rng.integers(1, 7))
+        ins = [rng.integers(0, 256, (N, int(rng.integers(1, 20)), H, W), dtype=np.uint8) for _ in range(n_in)]
+        ia, iz = [rand_q(rng) for _ in ins], [int(rng.integers(0, 256)) for _ in ins]
+        oa, oz = rand_q(rng), int(rng.integers(0, 256))
+        want = refrun.concat_u8(ref_ws, ins, ia, iz, oa, oz)
+        assert np.array_equal(orc.concat_u8(ins, ia, iz, oa, oz), want), (it, ia, iz, oa, oz)
+    for it in range(20):
+        shape = [(int(rng.integers(1, 4)), int(rng.integers(2, 40)), int(rng.integers(1, 6)), int(rng.integers(1, 6))),
+                 (int(rng.integers(1, 5)), int(rng.integers(2, 1200)), 1, 1)][it % 2]
+        axis = 1 if it % 4 else int(rng.integers(1, 4))
+        x = rng.integers(0, 256, shape, dtype=np.uint8)
+        q = (rand_q(rng, 1e-2, 0.2), int(rng.integers(0, 256)), float(np.float32(1.0 / 255)), int(rng.integers(0, 3)))
+        want = refrun.softmax_u8(ref_ws, x, axis, *q)
+        assert np.array_equal(orc.softmax_u8(x, axis, *q), want), (it, shape, axis, q)
+
+
 def test_int8_conv_vs_reference(ref_ws):
     """op_conv_2d_i8xi8_run with the portable gemm_i8xi8 (ibits == wbits == 8; the lower-bit GEMMs are not
     implemented outside aarch64).  7x7 kernels take the reference's region-split im2col and are left out."""
@@ -432,3 +452,26 @@ def test_int8_quantize_formula():
         got = orc.quantize_i8(x, oa, bits)
         assert np.array_equal(got, want), bits
         assert np.array_equal(orc.dequantize_i8(got, oa), got.astype(np.float32) * oa)
+
+
+def test_concat_and_softmax_closed_forms():
+    rng = np.random.default_rng(33)
+    a, b = rng.integers(0, 256, (2, 3, 4, 5), dtype=np.uint8), rng.integers(0, 256, (2, 6, 4, 5), dtype=np.uint8)
+    # equal scales and zero points: a plain concatenation along the channels
+    assert np.array_equal(orc.concat_u8([a, b], [0.05, 0.05], [9, 9], 0.05, 9), np.concatenate([a, b], 1))
+    # otherwise each piece is the affine map round_half_up((x - z) * m / 2^s) + oz of its input, saturated
+    ia, iz, oa, oz = [0.02, 0.07], [100, 3], 0.04, 50
+    y = orc.concat_u8([a, b], ia, iz, oa, oz)
+    for piece, src, al, z in ((y[:, :3], a, ia[0], iz[0]), (y[:, 3:], b, ia[1], iz[1])):
+        m, s = orc.quant_scale(np.float32(al) / np.float32(oa), 16)
+        want = np.clip(((src.astype(np.int64) - z) * m + (1 << (s - 1)) >> s) + oz, 0, 255)
+        assert np.array_equal(piece, want.astype(np.uint8))
+    # softmax: within one step of the real-valued softmax of the dequantized input, and each pixel sums to ~1/oalpha
+    x = rng.integers(0, 256, (3, 10, 2, 2), dtype=np.uint8)
+    y = orc.softmax_u8(x, 1, 0.05, 128, 1.0 / 255, 0)
+    z = 0.05 * (x.astype(np.float64) - 128)
+    p = np.exp(z) / np.exp(z).sum(1, keepdims=True)
+    assert np.abs(y.astype(np.float64) - p * 255).max() <= 0.5 + 1e-3
+    # along another axis the same numbers appear with the axes swapped
+    xt = np.ascontiguousarray(x.transpose(0, 2, 1, 3))
+    assert np.array_equal(orc.softmax_u8(xt, 2, 0.05, 128, 1.0 / 255, 0).transpose(0, 2, 1, 3), y)
