@@ -1,16 +1,17 @@
-// Quantized uint8 convolution for gfx950: implicit GEMM on the int8 MFMA units.
+// Quantized convolution for gfx950: implicit GEMM on the int8 MFMA units (uint8 asymmetric and int8 symmetric tensors).
 //
 // Computes, bit for bit, what the reference CPU module computes in op_conv_2d_u8xu8_run
 // (art/modules/quant/src/op/conv_2d_uint8_impl.c:39-165):
 //     acc[n,k,oh,ow] = bias[k] + sum_{c,r,s} (x[n,c,ih,iw] - izp) * (w[k,c,r,s] - wzp)     (int32, wrapping)
 //     y = sat( (int32)( floor((acc * mult + 2^(shift-1)) / 2^shift) + ozp ) )
+// and, for int8 tensors, op_conv_2d_i8xi8_run (conv_2d_int8_impl.c:34-174): no zero points, the result clipped to
+// +-(2^obits - 1) and truncated to a byte.
 //
 // Mapping to the hardware
 //   * GEMM view: D[kout][pixel] = sum_k A[kout][k] * B[k][pixel], k = (r, s, c) with c fastest, so that
 //     16 consecutive k are 16 consecutive channels = one 128-bit load from the NHWC activation tensor.
-//   * v_mfma_i32_32x32x32_i8 multiplies SIGNED bytes.  Activations and weights are unsigned with zero
-//     points, so both are re-centred: xs = x - 128 (a byte-wise XOR with 0x80), ws = w - 128, and with
-//     a = 128 - izp, b = 128 - wzp
+//   * v_mfma_i32_32x32x32_i8 multiplies SIGNED bytes.  uint8 activations and weights have zero points, so both
+//     are re-centred: xs = x - 128 (a byte-wise XOR with 0x80), ws = w - 128, and with a = 128 - izp, b = 128 - wzp
 //         sum (x - izp)(w - wzp) = sum xs*ws + b * sum xs + a * sum ws + Kp*a*b.
 //     The last two terms are per-output-channel constants folded, with the bias, into `bias2` at setup;
 //     the accumulators START at bias2, so the epilogue adds nothing.  The second term is per pixel and
@@ -18,22 +19,26 @@
 //     (template flag HAS_WZP).  Taps that fall outside the image read the byte izp (xs = -a), which makes
 //     their (x - izp) exactly zero; k slots that exist only because of padding (pad channels, tail of the
 //     last 64-byte slab) carry the weight wzp (ws = -b), which makes their contribution zero whatever
-//     activation byte happens to sit there.
+//     activation byte happens to sit there.  int8 tensors need none of this: the XOR mask is 0, a = b = 0.
 //   * A work-group of 4 waves computes a BM pixels x BN channels tile, 64 bytes of k ("slab") at a time.
-//     Both operands go through LDS: the weight slab [BN][64] is a straight copy of the pre-packed weights
-//     (coalesced, L2 resident), the activation slab [BM][64] is gathered 16 bytes per lane.  Rows are 64
-//     bytes without padding; the four 16-byte chunks of a row are stored at chunk ^ ((row >> 2) & 3), which
-//     makes both the 128-bit stores and the MFMA fragment reads bank-conflict free.  The weights are
-//     packed in that order on the host, so the copy is linear.  Two LDS stages; the global loads of slab
-//     i+1 are in flight while slab i is multiplied.
+//     Both operands go through LDS and are put there by the load unit itself (global_load_lds_dwordx4: no VGPR
+//     staging, no LDS store instructions): the weight slab [BN][64] is a straight copy of the pre-packed
+//     weights, the activation slab [BM][64] is gathered 16 bytes per lane.  Rows are 64 bytes without padding;
+//     the four 16-byte chunks of a row sit at chunk ^ ((row >> 2) & 3), which keeps the MFMA fragment reads
+//     bank-conflict free; the weights are packed in that order on the host.  Two stages for short reductions
+//     (more work-groups per CU, whose load, multiply and store phases overlap), three or four for long ones.
 //   * Epilogue.  mult = m * 2^7 with m < 2^24, and for 33 <= shift <= 52 (every realistic scale)
 //         floor((acc*mult + 2^(shift-1)) / 2^shift) + zp == (mulhi(acc, mult) + 2^(t-1) + zp*2^t) >> t,  t = shift-32
 //     because the low 32 bits of the product cannot carry across the floor.  That is one v_mul_hi_i32, one
-//     add, one shift and one clamp per output instead of a 64-bit multiply-add-shift.  Other shifts take
+//     add, one shift and a saturating pack per output instead of a 64-bit multiply-add-shift.  Other shifts take
 //     the 64-bit path.  Each lane then holds 4 consecutive channels of one pixel per accumulator quad;
 //     the packed dwords are transposed through LDS so that every pixel's channels leave as 128-bit stores.
+//     A residual add can run here as well (hipq_conv2d_run_add): in the accumulator layout, against a residual
+//     tile that the load unit fetched into LDS while the reduction ran.
 //   * Work-groups are renumbered so that each of the 8 XCDs (round-robin dispatch) gets a contiguous
 //     range of pixel tiles: neighbouring tiles share input halos and weight slabs in that XCD's L2.
+//   * Other shapes: C <= 4 inputs (the RGB stem) use a register-staged variant of the same tile computation,
+//     depthwise 3x3 a dot-product kernel, remaining depthwise / grouped shapes plain per-output kernels.
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
