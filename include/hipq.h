@@ -95,6 +95,14 @@ void hipq_conv2d_plan_destroy(hipq_conv2d_plan *plan);
 const char *hipq_conv2d_plan_kernel(const hipq_conv2d_plan *plan);
 
 /*
+ * Tuning hook (no counterpart in the reference): choose the work-group tile (index: 0 128x128, 1 256x64, 2 128x64,
+ * 3 64x128, 4 64x64 pixels x channels; -1 keeps the current one) and the number of load stages (2..4; 0 = the
+ * built-in rule) of a plan that runs the DMA-fed MFMA kernel.  Every choice computes identical results; callers that
+ * can time a whole network (nart_amd/runner.py) search the choices per layer.  Other plans return an error.
+ */
+int hipq_conv2d_plan_select(hipq_conv2d_plan *plan, int tile, int stages);
+
+/*
  * Run: op_conv_2d_u8xu8_run — src/op/conv_2d_uint8_impl.c:39-165 (im2col src/utils/im2col.cpp:487,
  * GEMM src/gemm/default/gemm.c:306).  x, y: device NHWC.  acc_out: optional device int32
  * [N*OH*OW, out_cs] that receives the raw accumulators (bias included), NULL to skip.

@@ -654,14 +654,18 @@ __global__ __launch_bounds__(256) void conv_mfma_dma_kernel(const ConvArgs a)
 
 
     // Fragment reads run one k-step (32 bytes of k) ahead of the MFMAs that consume them, so the LDS latency
-    // hides behind the matrix pipe.  make_ready(i) = slab i has landed for every wave, and the stage that
-    // slab i+NS-1 will occupy has been read for the last time by every wave.
+    // hides behind the matrix pipe.  make_ready(i) = slab i has landed for every wave, and every wave's reads of the
+    // stage that slab i+NS-1 will occupy (the stage of slab i-1) have returned their data.
     int st_comp = 0;
     auto make_ready = [&](int i) {
         if (i + NS - 2 <= a.nslab - 1)
             wait_vmcnt<(NS - 2) * LPS>(); // slabs i+1 .. i+NS-2 may still be in flight
         else
             wait_vmcnt<0>();
+        // This wave's fragment reads of slab i-1 must have RETURNED, not merely been issued, before the barrier lets any
+        // wave refill that stage: the load unit's LDS writes are not ordered against another wave's pending ds_reads.
+        // (The reads were issued a whole multiply() ago, so the wait is normally free.)
+        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0), vmcnt / expcnt untouched
         __builtin_amdgcn_s_barrier();
         if (i + NS - 1 < a.nslab)
             issue(i + NS - 1);
@@ -1005,7 +1009,8 @@ struct hipq_conv2d_plan {
     hipq_conv2d_desc d;
     ConvArgs args;
     ConvVariant variant;
-    int tile; // index into kTiles
+    int tile;       // index into kTiles
+    int stages = 0; // load stages of the DMA kernel; 0 = the built-in rule
     bool has_wzp;
     void *d_w = nullptr, *d_bias = nullptr;
     std::string name;
@@ -1219,12 +1224,39 @@ extern "C" void hipq_conv2d_plan_destroy(hipq_conv2d_plan *p)
 
 extern "C" const char *hipq_conv2d_plan_kernel(const hipq_conv2d_plan *p) { return p ? p->name.c_str() : ""; }
 
+extern "C" int hipq_conv2d_plan_select(hipq_conv2d_plan *p, int tile, int stages)
+{
+    clear_error();
+    HIPQ_REQUIRE(p, "hipq_conv2d_plan_select: null plan");
+    HIPQ_REQUIRE(p->variant == kMfma, "hipq_conv2d_plan_select: only the DMA-fed MFMA kernel has variants (this plan runs %s)",
+                 p->name.c_str());
+    HIPQ_REQUIRE(tile >= -1 && tile < kNumTiles && (stages == 0 || (stages >= 2 && stages <= 4)),
+                 "hipq_conv2d_plan_select: tile must be -1 (keep) or 0..%d, stages 0 (built-in rule) or 2..4", kNumTiles - 1);
+    if (tile >= 0) {
+        p->tile = tile;
+        p->args.nbm = (p->args.P + kTiles[tile].bm - 1) / kTiles[tile].bm;
+        p->args.nbn = (p->d.out_cs + kTiles[tile].bn - 1) / kTiles[tile].bn;
+        char nm[96];
+        snprintf(nm, sizeof nm, "conv_mfma_i8_%dx%d%s%s", kTiles[tile].bm, kTiles[tile].bn, p->has_wzp ? "_wzp" : "",
+                 p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
+        p->name = nm;
+    }
+    p->stages = stages;
+    return 0;
+}
+
 // Load stages.  Short reductions (few slabs) run with two stages: the smaller LDS footprint lets four work-groups
 // share a CU and overlap their load, multiply and store phases.  Long reductions (3x3 layers, wide 1x1 layers) run
 // with four (three for the largest tile): measured inside the whole network, where a layer's input comes from HBM
 // or the last-level cache rather than from a warm L2, the deeper stream is worth 10 % of the ResNet-50 step.
 constexpr int kStages = 2;
 constexpr int kDeepFrom = 8; // slabs
+
+template <int BM, int BN, int WM, int WN, int NS, bool FUSED>
+static void launch_dma_aligned(const dim3 grid, const ConvArgs &a, hipStream_t st)
+{
+    hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, NS, false, true, FUSED>), grid, dim3(256), 0, st, a);
+}
 
 template <int BM, int BN, int WM, int WN>
 static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_t st)
@@ -1240,15 +1272,21 @@ static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_
         hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, kStages, true, false>), grid, block, 0, st, a);
     } else if (a.in_cs % 64 == 0 && a.res != nullptr && a.fastq && a.addq.fast && a.acc_out == nullptr && (a.out_cs & 15) == 0) {
         // residual add in the accumulator layout, residual tile prefetched into LDS
-        if (a.nslab >= kDeepFrom)
-            hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, 3, false, true, true>), grid, block, 0, st, a);
+        const int ns = p->stages ? p->stages : (a.nslab >= kDeepFrom ? 3 : kStages);
+        if (ns >= 4)
+            launch_dma_aligned<BM, BN, WM, WN, 4, true>(grid, a, st);
+        else if (ns == 3)
+            launch_dma_aligned<BM, BN, WM, WN, 3, true>(grid, a, st);
         else
-            hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, kStages, false, true, true>), grid, block, 0, st, a);
+            launch_dma_aligned<BM, BN, WM, WN, 2, true>(grid, a, st);
     } else if (a.in_cs % 64 == 0) {
-        if (a.nslab >= kDeepFrom)
-            hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, (BM + BN >= 320 ? 3 : 4), false, true>), grid, block, 0, st, a);
+        const int ns = p->stages ? p->stages : (a.nslab >= kDeepFrom ? (BM + BN >= 320 ? 3 : 4) : kStages);
+        if (ns >= 4)
+            launch_dma_aligned<BM, BN, WM, WN, 4, false>(grid, a, st);
+        else if (ns == 3)
+            launch_dma_aligned<BM, BN, WM, WN, 3, false>(grid, a, st);
         else
-            hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, kStages, false, true>), grid, block, 0, st, a);
+            launch_dma_aligned<BM, BN, WM, WN, 2, false>(grid, a, st);
     } else {
         hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, kStages, false, false>), grid, block, 0, st, a);
     }

@@ -6,6 +6,7 @@ is no host fallback — loading fails loudly if the library has not been built.
 """
 import ctypes as C
 import os
+import re
 
 import numpy as np
 
@@ -26,6 +27,7 @@ class ConvDesc(C.Structure):  # hipq_conv2d_desc
 
 
 DTYPE_U8, DTYPE_I8 = 0, 1
+TILE_INDEX = {"128x128": 0, "256x64": 1, "128x64": 2, "64x128": 3, "64x64": 4}  # hipq_conv2d_plan_select
 
 
 # every symbol include/hipq.h declares, with its signature
@@ -39,6 +41,7 @@ _SIGS = {
     "hipq_conv2d_plan_create": (C.c_int, [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p)]),
     "hipq_conv2d_plan_destroy": (None, [C.c_void_p]),
     "hipq_conv2d_plan_kernel": (C.c_char_p, [C.c_void_p]),
+    "hipq_conv2d_plan_select": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
     "hipq_conv2d_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "hipq_conv2d_run_add": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_float, C.c_int,
                                       C.c_int, C.c_void_p, C.c_void_p]),
@@ -151,7 +154,15 @@ class Conv2d:
                                             C.c_void_p(b.ctypes.data) if b is not None else None, C.byref(h)))
         self.handle = h
         self.kernel = lib().hipq_conv2d_plan_kernel(h).decode()
+        m = re.match(r"conv_mfma_i8_(\d+x\d+)", self.kernel)
+        self._tile0 = TILE_INDEX.get(m.group(1), -1) if m else -1  # the built-in choice, for the tuner to return to
         self.ops = 2 * N * K * self.OH * self.OW * (Cc // group) * R * S
+
+    def select(self, tile=-1, stages=0):
+        """Tuning hook: work-group tile index and load stages of the MFMA kernel (include/hipq.h)."""
+        check(lib().hipq_conv2d_plan_select(self.handle, tile, stages))
+        self.kernel = lib().hipq_conv2d_plan_kernel(self.handle).decode()
+        return self
 
     def empty_output(self):
         import torch

@@ -76,6 +76,7 @@ class HipqExecutor:
                 self.fused.pop(node.output, None)
                 fn = (lambda p=plan, i=ins[0], o=out: p(i, o))
                 self._add(node, plan.kernel, fn, plan.ops, nbytes)
+                self.steps[-1]["plan"] = plan
             elif node.kind == "ip":
                 x = xs[0]
                 Nn, Cc, Hh, Ww = x.shape
@@ -103,7 +104,7 @@ class HipqExecutor:
                 fn = (lambda p=plan, i=xin, r=self.buf[other], rf=res_first, ot=ot, st=st, o=out:
                       p.run_add(i, r, rf, ot.alpha, ot.zp, st.alpha, st.zp, o))
                 self.steps.append({"label": node.output, "kind": "conv+add", "kernel": plan.kernel + "+add", "fn": fn,
-                                   "ops": plan.ops, "bytes": nbytes})
+                                   "ops": plan.ops, "bytes": nbytes, "plan": plan})
             elif node.kind == "add":
                 fn = (lambda i=ins, o=out, xs=xs, y=y: hipq.add_u8(i[0], i[1], o, xs[0].alpha, xs[0].zp, xs[1].alpha,
                                                                  xs[1].zp, y.alpha, y.zp))
@@ -136,6 +137,61 @@ class HipqExecutor:
     def run(self):
         for s in self.steps:
             s["fn"]()
+
+    # ---- tuning ----------------------------------------------------------------------------------
+    TILES = (0, 2, 3, 4)   # 128x128, 128x64, 64x128, 64x64 (include/hipq.h: hipq_conv2d_plan_select)
+    STAGES = (2, 3, 4)
+
+    def _time_window(self, lo, hi, reps):
+        """Replays steps[lo:hi] from a HIP graph `reps` times; returns microseconds per replay."""
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for s in self.steps[lo:hi]:
+                s["fn"]()
+        for _ in range(3):
+            g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps * 1e3
+
+    def tune(self, reps=20, before=2, after=1, verbose=False):
+        """Per-layer search over the MFMA convolution's tile shapes and load stages, timed inside the network: each
+        candidate is measured as part of a replayed window of its neighbouring operators, because a kernel timed
+        alone on warm inputs ranks the variants differently from the same kernel between its producer and its
+        consumer.  Every variant computes the same bytes; only the launch shape changes."""
+        self.run()
+        torch.cuda.synchronize()
+        chosen = {}
+        for k, s in enumerate(self.steps):
+            plan = s.get("plan")
+            if plan is None or not plan.kernel.startswith("conv_mfma") or "_c4" in plan.kernel or "_wzp" in plan.kernel:
+                continue
+            if plan.desc.in_cs % 64:
+                continue  # the generic-addressing kernel has a single variant
+            lo, hi = max(0, k - before), min(len(self.steps), k + 1 + after)
+            base = self._time_window(lo, hi, reps)
+            best, best_t = (-1, 0), base
+            for tile in self.TILES:
+                for st in self.STAGES:
+                    plan.select(tile, st)
+                    t = min(self._time_window(lo, hi, reps) for _ in range(2))
+                    if t < best_t * 0.985:  # only move for a clear win
+                        best, best_t = (tile, st), t
+            if best[0] >= 0:
+                plan.select(*best)
+            else:  # back to the built-in choice
+                plan.select(plan._tile0, 0)
+            s["kernel"] = plan.kernel + ("+add" if s["kind"] == "conv+add" else "")
+            chosen[s["label"]] = (best, round(base, 2), round(best_t, 2))
+            if verbose:
+                print("tune %-12s %-28s window %.1f -> %.1f us  choice %s" % (s["label"], plan.kernel, base, best_t, best), flush=True)
+        return chosen
 
     def capture(self):
         """Record one pass into a HIP graph (kernel nodes only: no memsets, no allocations)."""

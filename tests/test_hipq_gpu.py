@@ -276,6 +276,41 @@ def test_full_size_properties():
         assert np.array_equal(y[i:i + 1], want)
 
 
+def test_conv_plan_variants_are_bit_identical():
+    """hipq_conv2d_plan_select: every work-group tile and stage count of the MFMA kernel gives the bytes of the
+    built-in choice, with and without the fused residual add; plans without variants refuse."""
+    rng = np.random.default_rng(45)
+    shapes = [(2, 64, 14, 14, 64, 3, 1, 1), (1, 128, 9, 11, 256, 1, 0, 1), (3, 64, 10, 7, 48, 3, 1, 2), (1, 256, 12, 12, 128, 3, 1, 1),
+              (2, 1024, 7, 7, 256, 1, 0, 1), (1, 192, 20, 20, 320, 1, 0, 1)]
+    for N, C, H, W, K, R, pad, st in shapes:
+        x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+        w = rng.integers(0, 256, (K, C, R, R), dtype=np.uint8)
+        b = rng.integers(-30000, 30000, K).astype(np.int32)
+        q = (rand_q(rng), int(rng.integers(0, 256)), rand_q(rng), 128, rand_q(rng, 1e-2, 1.0), int(rng.integers(0, 256)))
+        want = orc.conv2d_u8(x, w, b, pad, st, 1, *q)
+        plan = hipq.Conv2d(x.shape, w, b, pad, st, 1, *q)
+        xd = hipq.to_device_nhwc(x)
+        res = rng.integers(0, 256, want.shape, dtype=np.uint8)
+        rd = hipq.to_device_nhwc(res)
+        want_add = orc.add_u8(want, res, q[4], q[5], 0.07, 33, 0.1, 5)
+        for tile in (0, 1, 2, 3, 4):
+            for stages in (0, 2, 3, 4):
+                plan.select(tile, stages)
+                yd = plan(xd)
+                assert np.array_equal(hipq.from_device_nhwc(yd, K), want), (x.shape, w.shape, tile, stages, plan.kernel)
+                if K % 16 == 0:
+                    zd = torch.empty_like(yd)
+                    plan.run_add(xd, rd, False, 0.07, 33, 0.1, 5, zd)
+                    assert np.array_equal(hipq.from_device_nhwc(zd, K), want_add), ("add", x.shape, tile, stages, plan.kernel)
+    dw = hipq.Conv2d((1, 32, 8, 8), rng.integers(0, 256, (32, 1, 3, 3), dtype=np.uint8), None, 1, 1, 32, 0.1, 3, 0.1, 128, 0.1, 0)
+    with pytest.raises(hipq.HipqError):
+        dw.select(0, 2)
+    with pytest.raises(hipq.HipqError):
+        plan.select(7, 2)
+    with pytest.raises(hipq.HipqError):
+        plan.select(0, 5)
+
+
 def test_concat_softmax():
     rng = np.random.default_rng(44)
     for it in range(12):
