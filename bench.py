@@ -104,6 +104,9 @@ def main():
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-fuse", action="store_true", help="run every residual add as its own kernel")
     ap.add_argument("--layers", action="store_true", help="print a per-layer table to stderr")
+    ap.add_argument("--tune", action="store_true",
+                    help="before timing, let the executor search tile shape / load stages per convolution inside the network "
+                         "(HipqExecutor.tune); off by default: the built-in choice is what a NART runner gets")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch a plain 256 MiB device copy (copy_bytes_kernel): the known-size reference that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command is scaled by")
@@ -145,6 +148,8 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    if args.tune:
+        ex.tune()
     if args.no_graph:
         step = ex.run
     else:
@@ -196,7 +201,7 @@ def main():
            "ms_per_step": round(ms, 4), "wall_ms_per_step": round(wall_ms, 4), "higher_is_better": True,
            "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
            "config": {"workload": case.name, "batch": args.batch, "input": list(case.input.shape),
-                      "operators": len(case.nodes), "graph_replay": not args.no_graph, "fused_residual_adds": len(ex.fused),
+                      "operators": len(case.nodes), "graph_replay": not args.no_graph, "tuned": bool(args.tune), "fused_residual_adds": len(ex.fused),
                       "conv_fc_gop_per_step": round(case.conv_ops() / 1e9, 2)},
            "conv_tops_whole_step": round(case.conv_ops() / (ms * 1e-3) / 1e12, 2),
            "roofline": roof, "kernel_families": families}
