@@ -96,8 +96,8 @@ const char *hipq_conv2d_plan_kernel(const hipq_conv2d_plan *plan);
 
 /*
  * Tuning hook (no counterpart in the reference): choose the work-group tile (index: 0 128x128, 1 256x64, 2 128x64,
- * 3 64x128, 4 64x64 pixels x channels; -1 keeps the current one) and the number of load stages (2..4; 0 = the
- * built-in rule) of a plan that runs the DMA-fed MFMA kernel.  Every choice computes identical results; callers that
+ * 3 64x128, 4 64x64 pixels x channels; -1 keeps the current one) and the number of load stages (2..4, or 8 for the
+ * 64x128 / 64x64 tiles — other tiles then use 4; 0 = the built-in rule) of a plan that runs the DMA-fed MFMA kernel.  Every choice computes identical results; callers that
  * can time a whole network (nart_amd/runner.py) search the choices per layer.  Other plans return an error.
  */
 int hipq_conv2d_plan_select(hipq_conv2d_plan *plan, int tile, int stages);

@@ -1036,6 +1036,8 @@ static int choose_tile(long long P, int out_cs, bool expand)
         return count(2) >= 1024 ? 2 : 4; // 128x64, or 64x64 for small images
     if (expand && P >= 8000)
         return 4; // short reduction, wide output: store-bound, many small work-groups overlap best
+    if (count(3) <= 64)
+        return 4; // a handful of tiles (fully-connected layers): the smallest tile, to put more CUs on the weight stream
     return count(0) >= 200 ? 0 : 3;      // 128x128, or 64x128 when that leaves most CUs idle
 }
 
@@ -1230,8 +1232,8 @@ extern "C" int hipq_conv2d_plan_select(hipq_conv2d_plan *p, int tile, int stages
     HIPQ_REQUIRE(p, "hipq_conv2d_plan_select: null plan");
     HIPQ_REQUIRE(p->variant == kMfma, "hipq_conv2d_plan_select: only the DMA-fed MFMA kernel has variants (this plan runs %s)",
                  p->name.c_str());
-    HIPQ_REQUIRE(tile >= -1 && tile < kNumTiles && (stages == 0 || (stages >= 2 && stages <= 4)),
-                 "hipq_conv2d_plan_select: tile must be -1 (keep) or 0..%d, stages 0 (built-in rule) or 2..4", kNumTiles - 1);
+    HIPQ_REQUIRE(tile >= -1 && tile < kNumTiles && (stages == 0 || (stages >= 2 && stages <= 4) || stages == 8),
+                 "hipq_conv2d_plan_select: tile must be -1 (keep) or 0..%d, stages 0 (built-in rule), 2..4 or 8", kNumTiles - 1);
     if (tile >= 0) {
         p->tile = tile;
         p->args.nbm = (p->args.P + kTiles[tile].bm - 1) / kTiles[tile].bm;
@@ -1280,8 +1282,13 @@ static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_
         else
             launch_dma_aligned<BM, BN, WM, WN, 2, true>(grid, a, st);
     } else if (a.in_cs % 64 == 0) {
-        const int ns = p->stages ? p->stages : (a.nslab >= kDeepFrom ? (BM + BN >= 320 ? 3 : 4) : kStages);
-        if (ns >= 4)
+        // Few tiles, long reduction (fully-connected layers at small batch): the weights stream from HBM through a
+        // handful of CUs, and only the bytes each of them keeps in flight cover the memory latency: eight stages.
+        const bool stream = nblk <= 128 && a.nslab >= 16 && BM + BN <= 192;
+        const int ns = p->stages ? p->stages : stream ? 8 : (a.nslab >= kDeepFrom ? (BM + BN >= 320 ? 3 : 4) : kStages);
+        if (ns >= 8 && BM + BN <= 192)
+            launch_dma_aligned<BM, BN, WM, WN, (BM + BN <= 192 ? 8 : 4), false>(grid, a, st);
+        else if (ns >= 4)
             launch_dma_aligned<BM, BN, WM, WN, 4, false>(grid, a, st);
         else if (ns == 3)
             launch_dma_aligned<BM, BN, WM, WN, 3, false>(grid, a, st);

@@ -294,7 +294,7 @@ def test_conv_plan_variants_are_bit_identical():
         rd = hipq.to_device_nhwc(res)
         want_add = orc.add_u8(want, res, q[4], q[5], 0.07, 33, 0.1, 5)
         for tile in (0, 1, 2, 3, 4):
-            for stages in (0, 2, 3, 4):
+            for stages in (0, 2, 3, 4, 8):
                 plan.select(tile, stages)
                 yd = plan(xd)
                 assert np.array_equal(hipq.from_device_nhwc(yd, K), want), (x.shape, w.shape, tile, stages, plan.kernel)
