@@ -131,3 +131,27 @@ def test_full_size_resnet50_is_reproducible_and_exact():
                 continue
             got, want = ex.fetch(node.output)[i:i + 1], vals[node.output]
             assert np.array_equal(np.ascontiguousarray(got).view(np.uint8), want.view(np.uint8)), (i, node.kind, node.output)
+
+
+@pytest.mark.parametrize("build", [lambda: cases.mobilenet_v2(N=64), lambda: cases.resnet18(N=64)], ids=["mobilenetv2", "resnet18"])
+def test_full_size_reruns_are_identical(build):
+    """Batch-64 passes of the other two networks (depthwise kernels, the generic-addressing MFMA kernel, the unfused
+    add): every tensor of every rerun equals the first run's, eager and replayed from a graph."""
+    case = build()
+    ex = HipqExecutor(case, fuse_add=True)
+    ex.set_input(case_oracle.random_input(case, seed=10))
+    ex.run()
+    torch.cuda.synchronize()
+    first = {k: v.clone() for k, v in ex.buf.items()}
+    for it in range(8):
+        ex.run()
+        torch.cuda.synchronize()
+        for s in ex.steps:
+            k = s["label"]
+            assert torch.equal(first[k], ex.buf[k]), "run %d: %s (%s) differs from the first run in %d bytes" % (
+                it, k, s["kernel"], int((first[k] != ex.buf[k]).sum().item()))
+    ex.capture()
+    for it in range(4):
+        ex.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(first[case.output.name], ex.buf[case.output.name]), "graph replay %d" % it
