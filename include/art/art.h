@@ -333,7 +333,32 @@ void parade_prepare(parade_t *parade);
 void parade_run(parade_t *parade);
 bool parade_apply_reshape(parade_t *parade);
 
-/* ---- engine file reader (serialize.h:27-75; format: serialize_v1.c:26-95) --------------------------------- */
+/* Input pre-processing description that a version-2 engine file may attach to an input (transform.h:25-73).  The
+ * runtime only carries it for the caller's image pipeline (parade.c:128-153); nothing here applies it. */
+typedef struct frame_t frame_t;
+typedef struct pixel_t {
+    float r, g, b;
+} pixel_t;
+typedef struct transform_param_t {
+    const char *tensor_name;
+    uint32_t operators;
+    size_t batch;
+    frame_t **frames;
+    int32_t tensor_type;
+    int32_t (*rois)[4];
+    int32_t (*dst_rois)[4];
+    float (*mats)[3][3];
+    pixel_t means, stds, paddings;
+} transform_param_t;
+typedef struct transform_tensor_t { /* what an input tensor with with_transform == 1 really is */
+    tensor_t tensor;
+    size_t capacity;
+    transform_param_t param;
+} transform_tensor_t;
+bool parade_get_transfrom_param(parade_t *parade, size_t *count, transform_param_t *params); /* sic, parade.h:40 */
+void parade_set_transfrom_param(parade_t *parade, transform_param_t *params);
+
+/* ---- engine file reader (serialize.h:27-75; formats: serialize_v1.c:26-95, serialize_v2.c:25-98) --------------------------------- */
 typedef size_t (*nart_buffer_read_func)(size_t sz, void *data, void *param);
 typedef struct buffer_t buffer_t;
 buffer_t *nart_buffer_new(size_t buffer_size);

@@ -1,7 +1,7 @@
 /*
  * A small host core implementing the art C API (include/art/art.h): element types, host memory,
  * tensors, typed settings, operator life cycle, op lookup in a module's table, the parade (ordered op
- * list) and the version-1 engine file reader.  It exists so that the `hip` case module can be loaded and
+ * list) and the engine file reader (versions 1 and 2).  It exists so that the `hip` case module can be loaded and
  * driven where a NART installation is not available; it follows the behaviour of the reference core
  * (art/src/{data_type,mem,tensor,settings,op,module,parade,serialize,serialize_v1}.c) for the parts a
  * quantized CNN case uses and makes no attempt to cover the rest of NART.
@@ -640,7 +640,7 @@ ART_PUBLIC size_t nart_buffer_read(buffer_t *b, size_t sz, void *out)
     return done;
 }
 
-/* ---- engine file, version 1 (layout: serialize_v1.c:26-95; reader :203-340) ----------------------------------- */
+/* ---- engine file, versions 1 and 2 (layouts: serialize_v1.c:26-95, serialize_v2.c:25-98; readers :203-340) ----------------------------------- */
 static int32_t rd_i32(buffer_t *b)
 {
     int32_t v = 0;
@@ -750,7 +750,53 @@ static void rd_setting(op_t *op, buffer_t *b)
     free(m);
 }
 
-static parade_t *read_parade_v1(buffer_t *b, const deserialize_param_t *param)
+/* version 2 (serialize_v2.c:25-98, :215-249): every input declaration is followed by a flag and, if it is set, by the
+ * pre-processing parameters {operators, frame type, mean, std, padding}; the tensor then is a transform_tensor_t */
+static tensor_t *rd_input_transform(buffer_t *b, tensor_t *plain)
+{
+    if (rd_i32(b) == 0)
+        return plain;
+    transform_tensor_t *tt = (transform_tensor_t *)calloc(1, sizeof(transform_tensor_t));
+    tt->tensor = *plain; /* takes over mem and name */
+    free(plain);
+    tt->tensor.with_transform = 1;
+    tt->param.operators = (uint32_t)rd_i32(b);
+    (void)rd_i32(b); /* frame type: read and dropped, as in the reference */
+    pixel_t *px[3] = {&tt->param.means, &tt->param.stds, &tt->param.paddings};
+    for (int i = 0; i < 3; ++i)
+        ART_CHECK(nart_buffer_read(b, sizeof(pixel_t), px[i]) == sizeof(pixel_t));
+    return &tt->tensor;
+}
+
+ART_PUBLIC bool parade_get_transfrom_param(parade_t *parade, size_t *count, transform_param_t *params)
+{
+    if (parade == NULL)
+        return false;
+    if (count != NULL)
+        *count = parade->input_tensor_count;
+    if (params != NULL) { /* the reference returns input 0's block unconditionally (parade.c:128-138) */
+        if (parade->input_tensor_count == 0 || !parade->input_tensors[0]->with_transform)
+            return false;
+        *params = ((transform_tensor_t *)parade->input_tensors[0])->param;
+    }
+    return true;
+}
+
+ART_PUBLIC void parade_set_transfrom_param(parade_t *parade, transform_param_t *params)
+{
+    for (size_t i = 0; parade != NULL && params != NULL && params->tensor_name != NULL && i < parade->input_tensor_count; ++i) {
+        tensor_t *t = parade->input_tensors[i];
+        if (t->name != NULL && strncmp(params->tensor_name, t->name, 64) == 0) {
+            if (t->with_transform) {
+                ((transform_tensor_t *)t)->param = *params;
+                return;
+            }
+            printf("tensor [%s] found, but with no transform flag\n", params->tensor_name);
+        }
+    }
+}
+
+static parade_t *read_parade(buffer_t *b, const deserialize_param_t *param, uint32_t version)
 {
     parade_t *p = parade_new();
     int32_t n_tensors = rd_i32(b);
@@ -760,8 +806,12 @@ static parade_t *read_parade_v1(buffer_t *b, const deserialize_param_t *param)
 
     int32_t n_in = rd_i32(b);
     p->input_tensors = (tensor_t **)calloc((size_t)n_in + 1, sizeof(tensor_t *));
-    for (int32_t i = 0; i < n_in; ++i)
-        tab[cur++] = p->input_tensors[p->input_tensor_count++] = rd_tensor_decl(b, param->input_mem_tp);
+    for (int32_t i = 0; i < n_in; ++i) {
+        tensor_t *t = rd_tensor_decl(b, param->input_mem_tp);
+        if (version >= 2)
+            t = rd_input_transform(b, t);
+        tab[cur++] = p->input_tensors[p->input_tensor_count++] = t;
+    }
 
     int32_t n_w = rd_i32(b);
     p->weight_tensors = (tensor_t **)calloc((size_t)n_w + 1, sizeof(tensor_t *));
@@ -827,7 +877,7 @@ ART_PUBLIC parade_t *deserialize_parade(buffer_t *b, const deserialize_param_t *
     uint32_t version = (uint32_t)rd_i32(b); /* head: version, name (serialize.c:143-160) */
     char *name = rd_string(b);
     free(name);
-    if (version != 1)
-        ART_FATAL("engine file version %u is not supported by this core (only version 1)\n", version);
-    return read_parade_v1(b, param);
+    if (version != 1 && version != 2)
+        ART_FATAL("engine file version %u is not supported by this core (versions 1 and 2)\n", version);
+    return read_parade(b, param, version);
 }

@@ -69,9 +69,11 @@ def _quant(ialpha=None, izp=None, walpha=None, wzp=None, oalpha=None, ozp=None, 
     return out
 
 
-def write_engine(case):
+def write_engine(case, version=1, transform=None):
     """Serialise a Case (nart_amd/cases.py).  A conv with relu=True becomes conv_2d followed by a relu op with
-    equal scales and zero point — the reference CPU module has no fused ReLU."""
+    equal scales and zero point — the reference CPU module has no fused ReLU.
+    version=2 writes the format of serialize_v2.c:25-98: each input is followed by a flag and, with
+    transform = (operators, frame_type, mean_rgb, std_rgb, padding_rgb), by that pre-processing block."""
     T = case.tensors
     index = {case.input.name: 0}
     inputs = [case.input]
@@ -120,10 +122,16 @@ def write_engine(case):
         index[y.name] = nxt
         nxt += 1
 
-    out = [_i32(1), _str(case.name), _i32(nxt)]
+    assert version in (1, 2) and (transform is None or version == 2)
+    out = [_i32(version), _str(case.name), _i32(nxt)]
     out.append(_i32(len(inputs)))
     for t in inputs:
         out += [struct.pack("<I", art.dtFLOAT32 if t.dtype == "f32" else art.dtUINT8), _str(t.name), _shape(t.shape)]
+        if version == 2:
+            out.append(_i32(1 if transform else 0))
+            if transform:
+                oprs, frame_type, mean, std, pad = transform
+                out += [struct.pack("<Ii", oprs, frame_type), struct.pack("<9f", *mean, *std, *pad)]
     out.append(_i32(len(weights)))
     for name, arr in weights:
         arr = np.ascontiguousarray(arr)
@@ -177,6 +185,23 @@ class Parade:
         core.nart_buffer_delete(buf)
         assert self.ptr, "deserialize_parade failed"
         core.parade_prepare(self.ptr)
+
+    def transform_param(self):
+        """(operators, means, stds, paddings) of input 0's pre-processing block (parade_get_transfrom_param, parade.c:128-138;
+        only meaningful for a version-2 file whose input carries one)."""
+        class Pixel(C.Structure):
+            _fields_ = [("r", C.c_float), ("g", C.c_float), ("b", C.c_float)]
+
+        class Param(C.Structure):  # transform_param_t, transform.h:54-67
+            _fields_ = [("tensor_name", C.c_char_p), ("operators", C.c_uint32), ("batch", C.c_size_t), ("frames", C.c_void_p),
+                        ("tensor_type", C.c_int32), ("rois", C.c_void_p), ("dst_rois", C.c_void_p), ("mats", C.c_void_p),
+                        ("means", Pixel), ("stds", Pixel), ("paddings", Pixel)]
+        f = self.rt.core.parade_get_transfrom_param
+        f.restype, f.argtypes = C.c_bool, [C.c_void_p, C.POINTER(C.c_size_t), C.POINTER(Param)]
+        n, prm = C.c_size_t(), Param()
+        assert f(self.ptr, C.byref(n), C.byref(prm))
+        px = lambda q: (q.r, q.g, q.b)  # noqa: E731
+        return prm.operators, px(prm.means), px(prm.stds), px(prm.paddings)
 
     def _tensors(self, getter):
         n, arr = C.c_size_t(), C.POINTER(C.POINTER(art.tensor_t))()

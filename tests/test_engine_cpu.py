@@ -43,6 +43,25 @@ def test_engine_file_runs_on_reference_runtime():
         p.delete()
 
 
+@needs_ref
+def test_version2_engine_file_on_reference_runtime():
+    """The writer's version-2 files (serialize_v2.c:25-98): with and without the pre-processing block on the input."""
+    rt = art.Runtime(REF_SO)
+    case = cases.resnet18(N=1, hw=96)
+    x = casecpu.random_input(case, 3)
+    want = casecpu.run_case(case, x)[case.output.name]
+    tf = (0x11, 2, (1.5, 2.5, 3.5), (0.25, 0.5, 0.75), (7.0, 8.0, 9.0))
+    for transform in (None, tf):
+        ws = rt.workspace("quant")
+        p = engine.Parade(rt, engine.write_engine(case, version=2, transform=transform), [ws])
+        casecpu.zero_reference_conv_scratch(p)
+        got = p.forward(x).reshape(case.output.shape)
+        assert np.array_equal(got.view(np.uint8), want.view(np.uint8))
+        if transform:
+            assert p.transform_param() == (0x11, (1.5, 2.5, 3.5), (0.25, 0.5, 0.75), (7.0, 8.0, 9.0))
+        p.delete()
+
+
 def _probe_source():
     return r'''
 #include <stdio.h>
@@ -54,6 +73,7 @@ def _probe_source():
 #include "art/op_settings.h"
 #include "art/parade.h"
 #include "art/serialize.h"
+#include "art/transform.h"
 #else
 #include "art/art.h"
 #endif
@@ -72,6 +92,8 @@ int main(void) {
     S(op_t); O(op_t, workspace); O(op_t, input_size); O(op_t, input_tensors); O(op_t, output_tensors); O(op_t, run_func);
     O(op_t, setting); S(workspace_t); S(module_t); O(module_t, name_func); O(module_t, new_func); O(module_t, op_tp_entry);
     S(deserialize_param_t); O(deserialize_param_t, input_mem_tp);
+    S(pixel_t); S(transform_param_t); O(transform_param_t, operators); O(transform_param_t, mats); O(transform_param_t, means);
+    O(transform_param_t, paddings); S(transform_tensor_t); O(transform_tensor_t, capacity); O(transform_tensor_t, param);
     printf("codes %llx %llx %llx %llx %llx %llx %llx %llx %llx\n", (unsigned long long)OP_CONV_2D, (unsigned long long)OP_IP,
            (unsigned long long)OP_POOL, (unsigned long long)OP_RELU, (unsigned long long)OP_ADD, (unsigned long long)OP_ELTWISE,
            (unsigned long long)OP_RESHAPE, 0ull, 0ull);

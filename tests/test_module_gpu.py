@@ -56,6 +56,23 @@ def test_engine_file_runs_on_hip_workspace(own_rt):
     ws.delete()
 
 
+def test_version2_engine_file(own_rt):
+    """Version-2 engine files (an optional pre-processing block after every input declaration) load on the repo's core
+    and run on the hip workspace; the block is handed back unchanged."""
+    ws = own_rt.workspace("hip")
+    case = cases.resnet18(N=2, hw=96)
+    x = casecpu.random_input(case, 4)
+    want = casecpu.run_case(case, x)[case.output.name]
+    tf = (0x11, 2, (1.5, 2.5, 3.5), (0.25, 0.5, 0.75), (7.0, 8.0, 9.0))
+    for transform in (None, tf):
+        p = engine.Parade(own_rt, engine.write_engine(case, version=2, transform=transform), [ws])
+        assert same_bits(p.forward(x).reshape(case.output.shape), want)
+        if transform:
+            assert p.transform_param() == (0x11, (1.5, 2.5, 3.5), (0.25, 0.5, 0.75), (7.0, 8.0, 9.0))
+        p.delete()
+    ws.delete()
+
+
 def test_prepare_twice_and_batch_reshape(own_rt):
     """parade_apply_reshape re-infers every shape and calls prepare again (art/src/parade.c:199-215): plans and
     device buffers must follow the new batch size."""
