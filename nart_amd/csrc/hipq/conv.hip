@@ -1083,7 +1083,9 @@ extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t
     hipq_quant_scale(d.ialpha * d.walpha / d.oalpha, 32, &a.q.mult, &a.q.shift);
     a.q.zp = sgn ? 0 : d.ozp;
     a.q.hi = (1 << d.obits) - 1;
-    a.lo = sgn ? (d.relu ? 0 : -a.q.hi) : (d.relu ? d.ozp : 0);
+    // fused ReLU: max(y, ozp); a zero point beyond the saturation value (obits < 8) leaves only that value, as the
+    // reference's relu applied to the saturated convolution output would
+    a.lo = sgn ? (d.relu ? 0 : -a.q.hi) : (d.relu ? std::min(d.ozp, a.q.hi) : 0);
     if (!valid_shift(a.q.shift)) {
         delete p;
         return fail("conv: requantisation shift %d outside 1..62 (scale %g)", a.q.shift,

@@ -146,6 +146,10 @@ def pool_u8(x, kernel, pad, stride, method, ceil_mode, ialpha, izp, oalpha, ozp,
     (kh, kw), (ph, pw), (sh, sw) = _pair(kernel), _pair(pad), _pair(stride)
     OH = pool_out_dim(H, ph, kh, sh, ceil_mode, ph or pw)
     OW = pool_out_dim(W, pw, kw, sw, ceil_mode, ph or pw)
+    if (OH - 1) * sh - ph >= H + ph or (OW - 1) * sw - pw >= W + pw:
+        # an empty last window (ceil mode without padding): the average's divisor is 0 and the reference's scale search
+        # (quant_helper.h:60-118) never ends on the infinite scale
+        raise ValueError("pool_u8: a window lies outside the image")
     y = np.empty((N, Cc, OH, OW), np.uint8)
     lib().orc_pool_u8(_p(x), _p(y), N, Cc, H, W, OH, OW, kh, kw, ph, pw, sh, sw, int(method),
                       _f(ialpha), int(izp), _f(oalpha), int(ozp), int(obits))

@@ -100,6 +100,13 @@ def test_conv_edge_cases():
     y, _, _ = run_conv(x, w, None, 1, 1, 1, q, relu=True, want_acc=False)
     want = orc.relu_u8(orc.conv2d_u8(x, w, None, 1, 1, 1, *q), 0.05, 90, 0.05, 90)
     assert np.array_equal(y, want)
+    # fewer output bits, with a zero point inside and beyond the saturation value (then only that value remains)
+    for obits, ozp in ((4, 9), (4, 200), (7, 127), (7, 128)):
+        q = (0.02, 100, 0.005, 128, 0.05, ozp)
+        plan = hipq.Conv2d(x.shape, w, None, 1, 1, 1, *q, obits=obits, relu=True)
+        got = hipq.from_device_nhwc(plan(hipq.to_device_nhwc(x)), 16)
+        want = orc.relu_u8(orc.conv2d_u8(x, w, None, 1, 1, 1, *q, obits=obits), 0.05, ozp, 0.05, ozp, obits)
+        assert np.array_equal(got, want), (obits, ozp)
 
 
 def test_conv_with_fused_residual_add():
