@@ -101,6 +101,14 @@ const char *hipq_conv2d_plan_kernel(const hipq_conv2d_plan *plan);
  * can time a whole network (nart_amd/runner.py) search the choices per layer.  Other plans return an error.
  */
 int hipq_conv2d_plan_select(hipq_conv2d_plan *plan, int tile, int stages);
+/*
+ * Tuning hook (no counterpart in the reference): 3x3 / stride 1 / pad 1 convolutions whose input channel stride is a
+ * multiple of 64 can run a kernel that loads each input tile with its halo once and forms the nine taps from LDS
+ * (kernel name "..._halo") instead of streaming every tap from memory.  mode 1 (the default) uses it for 64-channel
+ * inputs up to 63 pixels wide, where it is faster; mode 2 also for 128, 256 and 512 channels (128-channel tiles, images up
+ * to 31 pixels wide); mode 0 never.  Identical results in every mode.  Plans that do not run the MFMA kernel return an error.
+ */
+int hipq_conv2d_plan_halo(hipq_conv2d_plan *plan, int mode);
 
 /*
  * Run: op_conv_2d_u8xu8_run — src/op/conv_2d_uint8_impl.c:39-165 (im2col src/utils/im2col.cpp:487,

@@ -732,6 +732,217 @@ __global__ __launch_bounds__(256) void conv_mfma_dma_kernel(const ConvArgs a)
 }
 
 // ------------------------------------------------------------------------------------------------
+// 3x3, stride 1, pad 1 convolutions (in_cs a multiple of 64).  The nine taps of an output pixel read nine shifted copies
+// of the same input bytes, so instead of streaming one 64-byte slab per pixel and tap, the work-group loads, per
+// 64-channel slab, the pixels [m0 - W - 1, m0 + BM + W] of the flattened (n, h, w) index space ONCE (a "halo tile" of
+// BM + 2W + 2 rows of 64 bytes) and forms the pixel fragments of tap (dr, ds) by reading row r + W + 1 + dr*W + ds of it.
+// A tap outside the image would find a wrong neighbour there (the flat index runs on into the previous row or image):
+// such lanes read a row of pad bytes instead, chosen by a 9-bit mask computed once per lane.  Weight slabs are streamed as
+// in conv_mfma_dma_kernel, in the order (channel slab, tap) - slab tap * (in_cs / 64) + channel slab of the packed
+// weights; int32 accumulation does not depend on the order.  The LDS fill per k-step drops from (BM + BN) * 64 bytes to
+// BN * 64 + (BM + 2W + 2) * 64 / 9, and all bytes a tile touches first are requested at once.
+// The halo tiles of ALL channel slabs are requested when the work-group starts (NAB = in_cs / 64 buffers): a halo that
+// arrives from HBM in the middle of the weight stream would hold up every younger weight slab behind it, because a wave's
+// loads complete in order.  NPH: halo rows / 64 (>= BM + 2W + 2 rows, the host checks).
+template <int BM, int BN, int WM, int WN, int NS, int NPH, int NAB>
+__global__ __launch_bounds__(256) void conv3x3_halo_kernel(const ConvArgs a)
+{
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int NPA = BN / 64; // weight loads per thread and slab
+    constexpr int WSTAGE = BN * 64;
+    constexpr int ABUF = NPH * 64 * 64;
+    constexpr int A_OFF = NS * WSTAGE;
+    constexpr int PAD_OFF = A_OFF + NAB * ABUF; // 64 pad bytes
+    constexpr int OSTR = BN + 16;
+    constexpr int LDS_BYTES = PAD_OFF + 64 > BM * OSTR ? PAD_OFF + 64 : BM * OSTR;
+    static_assert(WM * WN == 4 && TM >= 1 && TN >= 1 && NS >= 2 && NS <= 9, "tile shape");
+    static_assert((NS - 2) * NPA <= 63, "vmcnt range");
+    static_assert(LDS_BYTES <= 160 * 1024, "LDS");
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[LDS_BYTES];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave % WM, wn = wave / WM;
+    const int nblk = a.nbm * a.nbn;
+    const int L = (int)(blockIdx.x % 8) * (int)(gridDim.x / 8) + (int)(blockIdx.x / 8);
+    if (L >= nblk)
+        return;
+    const int bm = L / a.nbn, bn = L % a.nbn;
+    const int nc = a.in_cs >> 6;
+    const int m0 = bm * BM;
+
+    // ---- halo source: LDS slot tid (+256 j) = phys chunk (tid & 3) of halo row (tid >> 2) + 64 j
+    const int chunk16 = ((tid & 3) ^ ((tid >> 4) & 3)) * 16;
+    if (tid < 16)
+        *reinterpret_cast<uint32_t *>(lds + PAD_OFF + tid * 4) = a.padword; // visible after the first barrier
+    const int hrows = BM + 2 * a.W + 2;
+    const uint8_t *hp[NPH];
+#pragma unroll
+    for (int j = 0; j < NPH; j++) {
+        const int row = (tid >> 2) + 64 * j, q = m0 - a.W - 1 + row;
+        hp[j] = (row < hrows && q >= 0 && q < a.P) ? a.x + (size_t)q * a.in_cs + chunk16 : nullptr;
+    }
+    const int wave_off = __builtin_amdgcn_readfirstlane(wave) * 1024;
+    auto issue_halo = [&](int cs) {
+        uint8_t *dst = lds + A_OFF + cs * ABUF + wave_off;
+#pragma unroll
+        for (int j = 0; j < NPH; j++) {
+            const uint8_t *src = hp[j] ? hp[j] + cs * 64 : a.padbuf;
+            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(dst + j * 4096), 16, 0, 0);
+        }
+    };
+    const uint8_t *wsrc = a.wpack + (size_t)bn * BN * 64 + tid * 16;
+    const size_t wslab = (size_t)a.kout_pad * 64;
+    int st_issue = 0, wi_t = 0, wi_cs = 0; // next weight slab to issue: (channel slab, tap), and its stage
+    auto issue_w = [&]() {
+        uint8_t *st = lds + st_issue * WSTAGE + wave_off;
+        st_issue = st_issue + 1 == NS ? 0 : st_issue + 1;
+        const uint8_t *ws = wsrc + (size_t)(wi_t * nc + wi_cs) * wslab;
+#pragma unroll
+        for (int j = 0; j < NPA; j++)
+            __builtin_amdgcn_global_load_lds((gptr_t)(ws + j * 4096), (lptr_t)(st + j * 4096), 16, 0, 0);
+        if (++wi_t == 9) {
+            wi_t = 0;
+            ++wi_cs;
+        }
+    };
+
+    // ---- this lane's pixel rows and their tap masks
+    const int half = lane >> 5;
+    int hr0[TM], vm[TM];
+    const int hw = a.H * a.W;
+#pragma unroll
+    for (int tm = 0; tm < TM; tm++) {
+        const int r = wm * (TM * 32) + tm * 32 + (lane & 31), m = m0 + r;
+        hr0[tm] = r + a.W + 1;
+        int mask = 0;
+        if (m < a.P) {
+            const int n = fast_div(m, hw, a.inv_ohw), rem = m - n * hw;
+            const int oh = fast_div(rem, a.W, a.inv_ow), ow = rem - oh * a.W;
+#pragma unroll
+            for (int t = 0; t < 9; t++) {
+                const int ih = oh + t / 3 - 1, iw = ow + t % 3 - 1;
+                mask |= ((unsigned)ih < (unsigned)a.H && (unsigned)iw < (unsigned)a.W) ? 1 << t : 0;
+            }
+        }
+        vm[tm] = mask;
+    }
+
+#pragma unroll
+    for (int cs = 0; cs < NAB; cs++)
+        issue_halo(cs);
+    for (int s = 0; s < NS - 1 && s < a.nslab; s++)
+        issue_w();
+
+    const int ch0 = bn * BN + wn * (TN * 32);
+    v16i acc[TN][TM];
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const v4i bias = *reinterpret_cast<const v4i *>(a.bias2 + ch0 + tn * 32 + g * 8 + (lane >> 5) * 4);
+#pragma unroll
+            for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    acc[tn][tm][g * 4 + e] = bias[e];
+        }
+    int colsum[TM];
+#pragma unroll
+    for (int tm = 0; tm < TM; tm++)
+        colsum[tm] = 0;
+
+    // ready(i): weight slab i has landed (and with it every halo, which are older), every wave's reads of step i-1 have
+    // returned; then the freed weight stage is refilled.
+    auto make_ready = [&](int i) {
+        if (i + NS - 2 <= a.nslab - 1)
+            wait_vmcnt<(NS - 2) * NPA>();
+        else
+            wait_vmcnt<0>();
+        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): this wave's fragment reads (and the pad row's store) are done
+        __builtin_amdgcn_s_barrier();
+        if (i + NS - 1 < a.nslab)
+            issue_w();
+    };
+
+    const int swz = (lane >> 2) & 3;
+    const int foff0 = (lane & 31) * 64 + (((0 + half) ^ swz) << 4);
+    const int foff1 = (lane & 31) * 64 + (((2 + half) ^ swz) << 4);
+    const int arow = wn * (TN * 32) * 64;
+    int rt = 0, rs = 0, shift = -a.W - 1, a_off = A_OFF; // tap being read, its column, its row shift, its halo buffer
+    // LDS address of this lane's bytes [16 half, 16 half + 16) of the current tap's halo row, or of the pad row where the
+    // tap lies outside the image (branch-free: the mask is 0 / -1); bytes [32 + 16 half, ...) are at that address ^ 32.
+    const int padc = PAD_OFF + (half << 4);
+    int adr[TM];
+    auto tap_addresses = [&]() {
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++) {
+            const int hr = hr0[tm] + shift;
+            const int x = a_off + (hr << 6) + ((((hr >> 2) ^ half) & 3) << 4);
+            const int inside = __builtin_amdgcn_sbfe(vm[tm], rt, 1);
+            adr[tm] = padc ^ ((x ^ padc) & inside);
+        }
+    };
+    auto read_frags = [&](v4i(&af)[TN], v4i(&bf)[TM], const uint8_t *wbuf, int kk) {
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++)
+            af[tn] = *reinterpret_cast<const v4i *>(wbuf + arow + tn * 2048 + (kk ? foff1 : foff0));
+        if (kk == 0)
+            tap_addresses();
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+            bf[tm] = *reinterpret_cast<const v4i *>(lds + (adr[tm] ^ (kk << 4)));
+    };
+    auto next_tap = [&]() {
+        ++shift;
+        if (++rs == 3) {
+            rs = 0;
+            shift += a.W - 3;
+        }
+        if (++rt == 9) {
+            rt = 0;
+            shift = -a.W - 1;
+            a_off += ABUF;
+        }
+    };
+    auto multiply = [&](v4i(&af)[TN], v4i(&bf)[TM]) {
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+            bf[tm] ^= (int)a.xmask;
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+            for (int tm = 0; tm < TM; tm++)
+                acc[tn][tm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[tn], bf[tm], acc[tn][tm], 0, 0, 0);
+    };
+
+    int st_comp = 0;
+    v4i af0[TN], bf0[TM], af1[TN], bf1[TM];
+    make_ready(0);
+    read_frags(af0, bf0, lds, 0);
+    for (int i = 0; i + 1 < a.nslab; i++) {
+        const uint8_t *buf = lds + st_comp * WSTAGE;
+        st_comp = st_comp + 1 == NS ? 0 : st_comp + 1;
+        read_frags(af1, bf1, buf, 2);
+        next_tap();
+        multiply(af0, bf0);
+        make_ready(i + 1);
+        read_frags(af0, bf0, lds + st_comp * WSTAGE, 0);
+        multiply(af1, bf1);
+    }
+    read_frags(af1, bf1, lds + st_comp * WSTAGE, 2);
+    multiply(af0, bf0);
+    multiply(af1, bf1);
+
+    __syncthreads(); // every wave has finished reading; no load is in flight any more
+    if (a.fastq && a.lo == 0 && a.q.hi == 255)
+        conv_epilogue<BM, BN, WM, WN, false, true, true, TM, TN>(a, acc, colsum, lds, bm, bn, wm, wn);
+    else if (a.fastq)
+        conv_epilogue<BM, BN, WM, WN, false, true, false, TM, TN>(a, acc, colsum, lds, bm, bn, wm, wn);
+    else
+        conv_epilogue<BM, BN, WM, WN, false, false, false, TM, TN>(a, acc, colsum, lds, bm, bn, wm, wn);
+}
+
+// ------------------------------------------------------------------------------------------------
 // Depthwise 3x3 (group == C == K, stride 1 or 2): HBM-bound on paper (16 bytes in, 16 bytes out per output pixel and
 // 16 channels), in practice bounded by vector ALU work, so the kernel is written for instruction count.
 // One thread owns 4 channels (one dword of the channels-last tensors) of a strip of 4 output pixels along W; a
@@ -1011,10 +1222,35 @@ struct hipq_conv2d_plan {
     ConvVariant variant;
     int tile;       // index into kTiles
     int stages = 0; // load stages of the DMA kernel; 0 = the built-in rule
+    int halo = 1; // 3x3 / stride 1 / pad 1 layers, halo-tile kernel: 0 never, 1 built-in rule, 2 wherever it applies
     bool has_wzp;
     void *d_w = nullptr, *d_bias = nullptr;
     std::string name;
 };
+
+// conv3x3_halo_kernel: 3x3, stride 1, pad 1, 64-byte channel slabs, weight zero point 128 (or int8), and a halo of
+// BM + 2W + 2 pixel rows within the BM + 128 rows the kernel holds; not for the 256-pixel tile.
+static bool halo_applies(const hipq_conv2d_plan *p)
+{
+    const hipq_conv2d_desc &d = p->d;
+    if (!(p->halo && p->variant == kMfma && !p->has_wzp && d.in_cs % 64 == 0 && d.R == 3 && d.S == 3 && d.stride_h == 1
+          && d.stride_w == 1 && d.pad_h == 1 && d.pad_w == 1 && d.W <= 63 && kTiles[p->tile].bm <= 128))
+        return false;
+    const int nc = d.in_cs / 64, bm = kTiles[p->tile].bm;
+    if (nc == 1)
+        return true;
+    // Several channel slabs (all halo tiles resident at once): measured slower than the streaming kernel on 14x14 and
+    // 7x7 images and equal on 28x28, so only on request.
+    return p->halo == 2 && (nc == 2 || nc == 4 || nc == 8) && kTiles[p->tile].bn == 128 && bm + 2 * d.W + 2 <= bm + 64;
+}
+
+static void set_mfma_name(hipq_conv2d_plan *p, bool smallc)
+{
+    char nm[96];
+    snprintf(nm, sizeof nm, "conv_mfma_i8_%dx%d%s%s%s%s", kTiles[p->tile].bm, kTiles[p->tile].bn, smallc ? "_c4" : "",
+             p->has_wzp ? "_wzp" : "", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "", halo_applies(p) ? "_halo" : "");
+    p->name = nm;
+}
 
 static int conv_out_dim(int in, int pad, int k, int stride)
 {
@@ -1149,10 +1385,9 @@ extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t
         }
         pad_off = wbuf.size();
         wbuf.resize(pad_off + 64, (uint8_t)pad_byte); // source of out-of-image taps
-        char nm[96];
-        snprintf(nm, sizeof nm, "conv_mfma_i8_%dx%d%s%s%s", BM, BN, smallc ? "_c4" : "", p->has_wzp ? "_wzp" : "",
-                 sgn ? "_signed" : "");
-        p->name = nm;
+        static const bool no_halo = getenv("HIPQ_NO_HALO") != nullptr; // for A/B measurements
+        p->halo = no_halo ? 0 : 1;
+        set_mfma_name(p, smallc);
     } else if (!sgn && d.group == d.C && d.K == d.C && d.in_cs == d.out_cs && d.R == 3 && d.S == 3 && d.stride_h == d.stride_w
                && (d.stride_h == 1 || d.stride_h == 2)
                && (long long)d.N * a.OH * ((a.OW + 3) / 4) * (d.in_cs / 4) < (1ll << 31)) {
@@ -1240,12 +1475,21 @@ extern "C" int hipq_conv2d_plan_select(hipq_conv2d_plan *p, int tile, int stages
         p->tile = tile;
         p->args.nbm = (p->args.P + kTiles[tile].bm - 1) / kTiles[tile].bm;
         p->args.nbn = (p->d.out_cs + kTiles[tile].bn - 1) / kTiles[tile].bn;
-        char nm[96];
-        snprintf(nm, sizeof nm, "conv_mfma_i8_%dx%d%s%s", kTiles[tile].bm, kTiles[tile].bn, p->has_wzp ? "_wzp" : "",
-                 p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
-        p->name = nm;
+        set_mfma_name(p, false);
     }
     p->stages = stages;
+    return 0;
+}
+
+extern "C" int hipq_conv2d_plan_halo(hipq_conv2d_plan *p, int mode)
+{
+    clear_error();
+    HIPQ_REQUIRE(p, "hipq_conv2d_plan_halo: null plan");
+    HIPQ_REQUIRE(p->variant == kMfma, "hipq_conv2d_plan_halo: only the DMA-fed MFMA kernel has variants (this plan runs %s)",
+                 p->name.c_str());
+    HIPQ_REQUIRE(mode >= 0 && mode <= 2, "hipq_conv2d_plan_halo: mode must be 0 (never), 1 (built-in rule) or 2 (wherever it applies)");
+    p->halo = mode;
+    set_mfma_name(p, false);
     return 0;
 }
 
@@ -1262,11 +1506,62 @@ static void launch_dma_aligned(const dim3 grid, const ConvArgs &a, hipStream_t s
     hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, NS, false, true, FUSED>), grid, dim3(256), 0, st, a);
 }
 
+// Weight stages of the halo kernel beside nab halo buffers of nph * 64 rows: as many as leave two work-groups to a CU
+// (80 KB each), at most 8; where the halo buffers alone leave fewer than 4, one work-group per CU and 7 stages.
+constexpr int halo_stages(int bn, int nph, int nab)
+{
+    const int n = (80 * 1024 - 64 - nab * nph * 4096) / (bn * 64);
+    return n > 8 ? 8 : n < 4 ? 7 : n;
+}
+
+// The halo-tile kernel serves 3x3 / stride 1 / pad 1 layers whose halo (BM + 2W + 2 pixel rows) fits BM + 128 LDS rows
+// (one channel slab) or BM + 64 rows (2, 4 or 8 channel slabs; 128x128 and 64x128 tiles).
+template <int BM, int BN, int WM, int WN>
+static bool launch_halo(const hipq_conv2d_plan *p, const ConvArgs &a, const dim3 grid, hipStream_t st)
+{
+    if constexpr (BM > 128) {
+        return false;
+    } else {
+        if (!halo_applies(p) || a.res != nullptr) // the fused residual add stays with the streaming kernel
+            return false;
+        constexpr int N0 = BM / 64 + 1;
+        const bool wide = BM + 2 * a.W + 2 > N0 * 64;
+        const int nc = a.in_cs / 64;
+        const dim3 block(256);
+        if (nc == 1) {
+            // a single channel slab has nine steps in all
+            if (wide)
+                hipLaunchKernelGGL((conv3x3_halo_kernel<BM, BN, WM, WN, 4, N0 + 1, 1>), grid, block, 0, st, a);
+            else
+                hipLaunchKernelGGL((conv3x3_halo_kernel<BM, BN, WM, WN, 4, N0, 1>), grid, block, 0, st, a);
+            return true;
+        }
+        if constexpr (BN == 128) {
+            // A step is 128-256 clocks of MFMA work against a load latency of well over a thousand, so the weight stream
+            // runs as deep as LDS allows (a weight stage is only BN * 64 bytes here).
+            if (wide)
+                return false;
+            if (nc == 2)
+                hipLaunchKernelGGL((conv3x3_halo_kernel<BM, BN, WM, WN, halo_stages(BN, N0, 2), N0, 2>), grid, block, 0, st, a);
+            else if (nc == 4)
+                hipLaunchKernelGGL((conv3x3_halo_kernel<BM, BN, WM, WN, halo_stages(BN, N0, 4), N0, 4>), grid, block, 0, st, a);
+            else if (nc == 8)
+                hipLaunchKernelGGL((conv3x3_halo_kernel<BM, BN, WM, WN, halo_stages(BN, N0, 8), N0, 8>), grid, block, 0, st, a);
+            else
+                return false;
+            return true;
+        }
+        return false;
+    }
+}
+
 template <int BM, int BN, int WM, int WN>
 static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_t st)
 {
     const int nblk = a.nbm * a.nbn;
     const dim3 grid((nblk + 7) / 8 * 8), block(256);
+    if (p->variant == kMfma && launch_halo<BM, BN, WM, WN>(p, a, grid, st))
+        return;
     if (p->variant == kMfmaSmallC) {
         if (p->has_wzp)
             hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, true, true>), grid, block, 0, st, a);

@@ -42,6 +42,7 @@ _SIGS = {
     "hipq_conv2d_plan_destroy": (None, [C.c_void_p]),
     "hipq_conv2d_plan_kernel": (C.c_char_p, [C.c_void_p]),
     "hipq_conv2d_plan_select": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
+    "hipq_conv2d_plan_halo": (C.c_int, [C.c_void_p, C.c_int]),
     "hipq_conv2d_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "hipq_conv2d_run_add": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_float, C.c_int,
                                       C.c_int, C.c_void_p, C.c_void_p]),
@@ -161,6 +162,13 @@ class Conv2d:
     def select(self, tile=-1, stages=0):
         """Tuning hook: work-group tile index and load stages of the MFMA kernel (include/hipq.h)."""
         check(lib().hipq_conv2d_plan_select(self.handle, tile, stages))
+        self.kernel = lib().hipq_conv2d_plan_kernel(self.handle).decode()
+        return self
+
+    def halo(self, mode=1):
+        """Tuning hook: the halo-tile kernel of 3x3 stride-1 layers: 0 never, 1 built-in rule, 2 wherever it applies
+        (include/hipq.h)."""
+        check(lib().hipq_conv2d_plan_halo(self.handle, int(mode)))
         self.kernel = lib().hipq_conv2d_plan_kernel(self.handle).decode()
         return self
 

@@ -318,6 +318,58 @@ def test_conv_plan_variants_are_bit_identical():
         plan.select(0, 5)
 
 
+def test_conv3x3_halo_kernel_matches_the_streaming_kernel_and_the_oracle():
+    """3x3 / stride 1 / pad 1 layers load a pixel tile with its halo once and read the nine taps from LDS: every tile
+    shape, one and several channel slabs, images narrower and wider than a tile, several images per tile (taps must
+    not leak across image or row borders), ragged last tiles, int8 tensors."""
+    rng = np.random.default_rng(46)
+    shapes = [(2, 64, 56, 56, 64), (3, 64, 5, 7, 48), (1, 128, 28, 28, 128), (5, 192, 3, 3, 80), (2, 256, 14, 14, 256), (7, 64, 1, 1, 16),
+              (1, 64, 2, 63, 64), (4, 512, 7, 7, 512), (3, 128, 9, 31, 200), (1, 64, 40, 62, 32), (1, 128, 6, 32, 64)]
+    for N, C, H, W, K in shapes:
+        print("halo case", N, C, H, W, K, flush=True)
+        x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+        w = rng.integers(0, 256, (K, C, 3, 3), dtype=np.uint8)
+        b = rng.integers(-30000, 30000, K).astype(np.int32)
+        q = (rand_q(rng), int(rng.integers(0, 256)), rand_q(rng), 128, rand_q(rng, 1e-2, 1.0), int(rng.integers(0, 256)))
+        want, want_acc = orc.conv2d_u8(x, w, b, 1, 1, 1, *q, return_acc=True)
+        plan = hipq.Conv2d(x.shape, w, b, 1, 1, 1, *q)
+        assert plan.kernel.endswith("_halo") == (C == 64), plan.kernel  # the built-in rule: single channel slab only
+        plan.halo(2)
+        xd = hipq.to_device_nhwc(x)
+        for tile in (0, 2, 3, 4):
+            plan.select(tile, 0)
+            # one channel slab: every tile; 2, 4 or 8 slabs: the 128-channel tiles, images up to 31 pixels wide
+            applies = C == 64 or (C in (128, 256, 512) and tile in (0, 3) and W <= 31)
+            assert plan.kernel.endswith("_halo") == applies, (plan.kernel, x.shape, tile)
+            assert np.array_equal(hipq.from_device_nhwc(plan(xd), K), want), (x.shape, K, tile, plan.kernel)
+        plan.select(3, 0)
+        acc = torch.empty((N, H, W, plan.desc.out_cs), dtype=torch.int32, device="cuda")
+        plan(xd, acc=acc)
+        assert np.array_equal(acc.cpu().numpy()[..., :K].transpose(0, 3, 1, 2), want_acc)
+        plan.halo(0)
+        assert not plan.kernel.endswith("_halo")
+        assert np.array_equal(hipq.from_device_nhwc(plan(xd), K), want)
+        plan.select(1, 0).halo(2)  # the 256-pixel tile has no halo variant
+        assert not plan.kernel.endswith("_halo")
+        assert np.array_equal(hipq.from_device_nhwc(plan(xd), K), want)
+        # int8 tensors: zero padding
+        xs, ws = x.view(np.int8), w.view(np.int8)
+        want8 = orc.conv2d_i8(xs, ws, b, 1, 1, 1, q[0], q[2], q[4], 7)
+        p8 = hipq.Conv2d(x.shape, ws, b, 1, 1, 1, q[0], 0, q[2], 0, q[4], 0, obits=7, dtype=hipq.DTYPE_I8)
+        p8.select(0, 0).halo(2)
+        assert p8.kernel.endswith("_halo") == (C == 64 or (C in (128, 256, 512) and W <= 31)), p8.kernel
+        assert np.array_equal(hipq.from_device_nhwc(p8(hipq.to_device_nhwc(xs)), K).view(np.int8), want8), (x.shape, K)
+    # not eligible: stride 2, pad 0, wide images, asymmetric weights
+    for kw in (dict(stride=2), dict(pad=0), dict(W=64), dict(wzp=100)):
+        W_ = kw.get("W", 16)
+        x = rng.integers(0, 256, (1, 64, 16, W_), dtype=np.uint8)
+        w = rng.integers(0, 256, (64, 64, 3, 3), dtype=np.uint8)
+        plan = hipq.Conv2d(x.shape, w, None, kw.get("pad", 1), kw.get("stride", 1), 1, 0.02, 7, 0.005, kw.get("wzp", 128), 0.05, 3)
+        assert not plan.kernel.endswith("_halo"), (kw, plan.kernel)
+        want = orc.conv2d_u8(x, w, None, kw.get("pad", 1), kw.get("stride", 1), 1, 0.02, 7, 0.005, kw.get("wzp", 128), 0.05, 3)
+        assert np.array_equal(hipq.from_device_nhwc(plan(hipq.to_device_nhwc(x)), 64), want), kw
+
+
 def test_concat_softmax():
     rng = np.random.default_rng(44)
     for it in range(12):
