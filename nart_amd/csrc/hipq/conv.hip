@@ -745,7 +745,7 @@ __global__ __launch_bounds__(256) void conv_mfma_dma_kernel(const ConvArgs a)
 // arrives from HBM in the middle of the weight stream would hold up every younger weight slab behind it, because a wave's
 // loads complete in order.  NPH: halo rows / 64 (>= BM + 2W + 2 rows, the host checks).
 template <int BM, int BN, int WM, int WN, int NS, int NPH, int NAB>
-__global__ __launch_bounds__(256) void conv3x3_halo_kernel(const ConvArgs a)
+__global__ __launch_bounds__(256) void conv_mfma_halo_kernel(const ConvArgs a)
 {
     constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
     constexpr int NPA = BN / 64; // weight loads per thread and slab
@@ -1228,7 +1228,7 @@ struct hipq_conv2d_plan {
     std::string name;
 };
 
-// conv3x3_halo_kernel: 3x3, stride 1, pad 1, 64-byte channel slabs, weight zero point 128 (or int8), and a halo of
+// conv_mfma_halo_kernel: 3x3, stride 1, pad 1, 64-byte channel slabs, weight zero point 128 (or int8), and a halo of
 // BM + 2W + 2 pixel rows within the BM + 128 rows the kernel holds; not for the 256-pixel tile.
 static bool halo_applies(const hipq_conv2d_plan *p)
 {
@@ -1531,9 +1531,9 @@ static bool launch_halo(const hipq_conv2d_plan *p, const ConvArgs &a, const dim3
         if (nc == 1) {
             // a single channel slab has nine steps in all
             if (wide)
-                hipLaunchKernelGGL((conv3x3_halo_kernel<BM, BN, WM, WN, 4, N0 + 1, 1>), grid, block, 0, st, a);
+                hipLaunchKernelGGL((conv_mfma_halo_kernel<BM, BN, WM, WN, 4, N0 + 1, 1>), grid, block, 0, st, a);
             else
-                hipLaunchKernelGGL((conv3x3_halo_kernel<BM, BN, WM, WN, 4, N0, 1>), grid, block, 0, st, a);
+                hipLaunchKernelGGL((conv_mfma_halo_kernel<BM, BN, WM, WN, 4, N0, 1>), grid, block, 0, st, a);
             return true;
         }
         if constexpr (BN == 128) {
@@ -1542,11 +1542,11 @@ static bool launch_halo(const hipq_conv2d_plan *p, const ConvArgs &a, const dim3
             if (wide)
                 return false;
             if (nc == 2)
-                hipLaunchKernelGGL((conv3x3_halo_kernel<BM, BN, WM, WN, halo_stages(BN, N0, 2), N0, 2>), grid, block, 0, st, a);
+                hipLaunchKernelGGL((conv_mfma_halo_kernel<BM, BN, WM, WN, halo_stages(BN, N0, 2), N0, 2>), grid, block, 0, st, a);
             else if (nc == 4)
-                hipLaunchKernelGGL((conv3x3_halo_kernel<BM, BN, WM, WN, halo_stages(BN, N0, 4), N0, 4>), grid, block, 0, st, a);
+                hipLaunchKernelGGL((conv_mfma_halo_kernel<BM, BN, WM, WN, halo_stages(BN, N0, 4), N0, 4>), grid, block, 0, st, a);
             else if (nc == 8)
-                hipLaunchKernelGGL((conv3x3_halo_kernel<BM, BN, WM, WN, halo_stages(BN, N0, 8), N0, 8>), grid, block, 0, st, a);
+                hipLaunchKernelGGL((conv_mfma_halo_kernel<BM, BN, WM, WN, halo_stages(BN, N0, 8), N0, 8>), grid, block, 0, st, a);
             else
                 return false;
             return true;
