@@ -37,6 +37,8 @@
 //     tile that the load unit fetched into LDS while the reduction ran.
 //   * Work-groups are renumbered so that each of the 8 XCDs (round-robin dispatch) gets a contiguous
 //     range of pixel tiles: neighbouring tiles share input halos and weight slabs in that XCD's L2.
+//   * 3x3 / stride 1 / pad 1 layers with 64 input channels run conv_mfma_halo_kernel: the input tile is loaded once
+//     with its halo and the nine taps are read from LDS at shifted rows, instead of one slab per tap from memory.
 //   * Other shapes: C <= 4 inputs (the RGB stem) use a register-staged variant of the same tile computation,
 //     depthwise 3x3 a dot-product kernel, remaining depthwise / grouped shapes plain per-output kernels.
 #include <algorithm>
