@@ -234,8 +234,7 @@ def mobilenet_v2(N=64, seed=22, hw=224):
             y = x
             if t != 1:
                 y = c.conv(y, cin * t, 1, relu=True, ozp=int(c.rng.integers(0, 64)))
-            y = c.conv(y, y.shape[1], 3, stride=stride, group=y.shape[1], relu=True, ozp=int(c.rng.integers(0, 64)),
-                       wzp=int(c.rng.integers(100, 156)), w_lo=0)
+            y = c.conv(y, y.shape[1], 3, stride=stride, group=y.shape[1], relu=True, ozp=int(c.rng.integers(0, 64)))
             y = c.conv(y, cout, 1, ozp=rz())
             x = c.add(x, y, implicit_relu=False, ozp=rz()) if (stride == 1 and cin == cout) else y
             cin = cout

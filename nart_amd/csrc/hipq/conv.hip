@@ -502,8 +502,9 @@ __device__ static inline void wait_vmcnt()
 typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
 
-// ALIGNED: in_cs is a multiple of 64, so a slab never straddles two taps; the source addresses then advance by
-// a wave-uniform offset and the bounds tests are redone only when the tap changes.
+// ALIGNED: a slab never straddles two taps (in_cs a multiple of 64, or a 1x1 kernel with any in_cs, whose last slab
+// may be partial); the source addresses then advance by a wave-uniform offset and the bounds tests are redone only
+// when the tap changes.
 // FUSED: the residual add runs in the accumulator layout on a residual tile prefetched into LDS (see
 // conv_epilogue_fused_add); only instantiated for ALIGNED && !HAS_WZP.
 template <int BM, int BN, int WM, int WN, int NS, bool HAS_WZP, bool ALIGNED, bool FUSED = false>
@@ -576,6 +577,7 @@ __global__ __launch_bounds__(256) void conv_mfma_dma_kernel(const ConvArgs a)
     const uint8_t *wsrc = a.wpack + (size_t)bn * BN * 64 + tid * 16;
     const int wave_off = __builtin_amdgcn_readfirstlane(wave) * 1024;
     const size_t wslab = (size_t)a.kout_pad * 64;
+    const bool pad_last = ALIGNED && chunk16 + 64 * (a.nslab - 1) >= a.in_cs * a.R * a.S; // only ever true for 1x1 kernels
 
     int st_issue = 0; // stage the next issue() fills; stages are used round-robin
     auto issue = [&](int slab) {
@@ -587,9 +589,12 @@ __global__ __launch_bounds__(256) void conv_mfma_dma_kernel(const ConvArgs a)
             __builtin_amdgcn_global_load_lds((gptr_t)(ws + j * 4096), (lptr_t)(st + j * 4096), 16, 0, 0);
         if (ALIGNED) {
             const int off = tap_off + tap_c;
+            // 1x1 kernels whose channel stride is not a multiple of 64: the chunks of the last slab that lie beyond the
+            // pixel's own bytes (their weights are pad slots) come from the pad buffer, not from the next pixel
+            const bool skip = pad_last && slab == a.nslab - 1;
 #pragma unroll
             for (int j = 0; j < NPB; j++) {
-                const uint8_t *src = lp_in[j] ? lp_ptr[j] + off : a.padbuf;
+                const uint8_t *src = lp_in[j] && !skip ? lp_ptr[j] + off : a.padbuf;
                 __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(st + BN * 64 + j * 4096), 16, 0, 0);
             }
             tap_c += 64;
@@ -1564,6 +1569,10 @@ static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_
     const dim3 grid((nblk + 7) / 8 * 8), block(256);
     if (p->variant == kMfma && launch_halo<BM, BN, WM, WN>(p, a, grid, st))
         return;
+    // "aligned" addressing: a 64-byte slab never straddles two taps.  True when a pixel's channels are whole slabs, and
+    // for 1x1 kernels with any channel stride (a multiple of 16): there is one tap, and the pad chunks of the last
+    // slab (beyond the pixel's own bytes) are read from the pad buffer.
+    const bool aligned = a.in_cs % 64 == 0 || (a.R == 1 && a.S == 1 && a.in_cs % 16 == 0);
     if (p->variant == kMfmaSmallC) {
         if (p->has_wzp)
             hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, true, true>), grid, block, 0, st, a);
@@ -1571,7 +1580,7 @@ static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_
             hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, false, true>), grid, block, 0, st, a);
     } else if (p->has_wzp) { // rare (asymmetric weights): generic addressing only
         hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, kStages, true, false>), grid, block, 0, st, a);
-    } else if (a.in_cs % 64 == 0 && a.res != nullptr && a.fastq && a.addq.fast && a.acc_out == nullptr && (a.out_cs & 15) == 0) {
+    } else if (aligned && a.res != nullptr && a.fastq && a.addq.fast && a.acc_out == nullptr && (a.out_cs & 15) == 0) {
         // residual add in the accumulator layout, residual tile prefetched into LDS
         const int ns = p->stages ? p->stages : (a.nslab >= kDeepFrom ? 3 : kStages);
         if (ns >= 4)
@@ -1580,7 +1589,7 @@ static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_
             launch_dma_aligned<BM, BN, WM, WN, 3, true>(grid, a, st);
         else
             launch_dma_aligned<BM, BN, WM, WN, 2, true>(grid, a, st);
-    } else if (a.in_cs % 64 == 0) {
+    } else if (aligned) {
         // Few tiles, long reduction (fully-connected layers at small batch): the weights stream from HBM through a
         // handful of CUs, and only the bytes each of them keeps in flight cover the memory latency: eight stages.
         const bool stream = nblk <= 128 && a.nslab >= 16 && BM + BN <= 192;

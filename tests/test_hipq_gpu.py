@@ -288,7 +288,10 @@ def test_conv_plan_variants_are_bit_identical():
     built-in choice, with and without the fused residual add; plans without variants refuse."""
     rng = np.random.default_rng(45)
     shapes = [(2, 64, 14, 14, 64, 3, 1, 1), (1, 128, 9, 11, 256, 1, 0, 1), (3, 64, 10, 7, 48, 3, 1, 2), (1, 256, 12, 12, 128, 3, 1, 1),
-              (2, 1024, 7, 7, 256, 1, 0, 1), (1, 192, 20, 20, 320, 1, 0, 1)]
+              (2, 1024, 7, 7, 256, 1, 0, 1), (1, 192, 20, 20, 320, 1, 0, 1),
+              # 1x1 kernels whose channel stride is not a multiple of 64: partial last slab
+              (2, 96, 9, 9, 24, 1, 0, 1), (1, 16, 12, 12, 96, 1, 0, 1), (1, 144, 7, 7, 32, 1, 0, 1), (3, 160, 5, 5, 320, 1, 0, 1),
+              (1, 32, 10, 10, 192, 1, 0, 2), (1, 20, 6, 6, 16, 1, 0, 1)]
     for N, C, H, W, K, R, pad, st in shapes:
         x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
         w = rng.integers(0, 256, (K, C, R, R), dtype=np.uint8)
