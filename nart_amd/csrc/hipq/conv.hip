@@ -950,6 +950,103 @@ __global__ __launch_bounds__(256) void conv_mfma_halo_kernel(const ConvArgs a)
 }
 
 // ------------------------------------------------------------------------------------------------
+// Pointwise (1x1, stride 1) convolutions with at most 64 input and 256 output channels.  Such layers are memory-bound
+// (an expansion writes 4 to 16 bytes per byte it reads), and the tile machinery above - LDS staging of the activations,
+// a barrier per slab, a transposing epilogue - is pure overhead for them.  Here a WAVE owns a strip of 32 pixels:
+//   * its pixel fragments come straight from global memory: lane (p, h) loads bytes [32 s + 16 h, +16) of pixel p for
+//     k-step s - a pixel's channels are contiguous, so that IS the MFMA operand;
+//   * the weights (at most 16 KB, in the packed order of the tile kernels) and the folded bias sit in LDS for the life of
+//     the work-group, which loops over strips;
+//   * the rows of each 32-channel block are permuted: MFMA row i computes channel 16 ((i >> 2) & 1) + 4 (i >> 3) + (i & 3)
+//     of the block, so the 16 accumulators of lane (p, h) are the 16 CONSECUTIVE channels 16 h .. 16 h + 15 of the block
+//     and leave as one 128-bit store: no transpose, no barrier;
+// The fused residual add stays with the tile kernels: applied to packed bytes in this layout it costs more vector
+// arithmetic than their accumulator-layout form, and the layer becomes VALU-bound (measured 49 against 31 us).
+// NKS: k-steps of 32 bytes (1: up to 32 input channels, 2: up to 64).  PLAIN_SAT: clamp range exactly [0, 255].
+// Requires the one-multiply requantisation (the host checks).
+template <int NKS, bool PLAIN_SAT>
+__device__ static inline void pointwise_strips(const ConvArgs &a, const uint8_t *lds)
+{
+    constexpr int MAXB = 8; // 32-channel blocks
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, p = lane & 31;
+    const int nb = (a.out_cs + 31) >> 5, nstrips = (a.P + 31) >> 5;
+    const int prow = 16 * ((p >> 2) & 1) + 4 * (p >> 3) + (p & 3); // the channel (within a block) MFMA row p stands for
+    const int32_t *lbias = reinterpret_cast<const int32_t *>(lds + 256 * 64);
+    for (int strip = blockIdx.x * 4 + wave; strip < nstrips; strip += gridDim.x * 4) {
+        const int m = strip * 32 + p;
+        const bool ok = m < a.P;
+        v4i bf[NKS];
+#pragma unroll
+        for (int s = 0; s < NKS; s++) {
+            const int kb = 32 * s + 16 * half;
+            bf[s] = v4i{0, 0, 0, 0}; // k slots beyond the input channels carry zero weights
+            if (ok && kb < a.in_cs)
+                bf[s] = *reinterpret_cast<const v4i *>(a.x + (size_t)m * a.in_cs + kb) ^ (int)a.xmask;
+        }
+        const size_t orow = (size_t)m * a.out_cs + 16 * half;
+#pragma unroll
+        for (int b = 0; b < MAXB; b++) {
+            if (b >= nb)
+                break;
+            v16i acc;
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const v4i bv = *reinterpret_cast<const v4i *>(lbias + b * 32 + 16 * half + 4 * g);
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    acc[g * 4 + e] = bv[e];
+            }
+            const int ko = b * 32 + prow;
+#pragma unroll
+            for (int s = 0; s < NKS; s++) {
+                const v4i af = *reinterpret_cast<const v4i *>(lds + ko * 64 + (((2 * s + half) ^ ((ko >> 2) & 3)) << 4));
+                acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf[s], acc, 0, 0, 0);
+            }
+            u32x4 cv;
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                if (PLAIN_SAT) {
+                    int32_t r[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        r[e] = (__mulhi(acc[g * 4 + e], (int)a.q.mult) + a.qadd) >> a.qt;
+                    uint32_t p01, p23, b01, b23;
+                    asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p01) : "v"(r[0]), "v"(r[1]));
+                    asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(r[2]), "v"(r[3]));
+                    asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
+                    asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
+                    cv[g] = (b01 & 0xffffu) | (b23 << 16);
+                } else {
+                    int32_t rq[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        rq[e] = conv_requant<true>(a, acc[g * 4 + e]);
+                    cv[g] = pack_low_bytes(rq[0], rq[1], rq[2], rq[3]);
+                }
+            }
+            if (ok && b * 32 + 16 * half < a.out_cs)
+                *reinterpret_cast<u32x4 *>(a.y + orow + b * 32) = cv;
+        }
+    }
+}
+
+template <int NKS>
+__global__ __launch_bounds__(256) void conv_mfma_pointwise_kernel(const ConvArgs a)
+{
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[256 * 64 + 256 * 4]; // weights [kout_pad <= 256][64], folded bias
+    const int tid = threadIdx.x;
+    for (int i = tid * 16; i < a.kout_pad * 64; i += 256 * 16)
+        *reinterpret_cast<v4i *>(lds + i) = *reinterpret_cast<const v4i *>(a.wpack + i);
+    for (int i = tid; i < a.kout_pad; i += 256)
+        reinterpret_cast<int32_t *>(lds + 256 * 64)[i] = a.bias2[i];
+    __syncthreads();
+    if (a.lo == 0 && a.q.hi == 255)
+        pointwise_strips<NKS, true>(a, lds);
+    else
+        pointwise_strips<NKS, false>(a, lds);
+}
+
+// ------------------------------------------------------------------------------------------------
 // Depthwise 3x3 (group == C == K, stride 1 or 2): HBM-bound on paper (16 bytes in, 16 bytes out per output pixel and
 // 16 channels), in practice bounded by vector ALU work, so the kernel is written for instruction count.
 // One thread owns 4 channels (one dword of the channels-last tensors) of a strip of 4 output pixels along W; a
@@ -1229,7 +1326,7 @@ struct hipq_conv2d_plan {
     ConvVariant variant;
     int tile;       // index into kTiles
     int stages = 0; // load stages of the DMA kernel; 0 = the built-in rule
-    int halo = 1; // 3x3 / stride 1 / pad 1 layers, halo-tile kernel: 0 never, 1 built-in rule, 2 wherever it applies
+    int special = 1; // the halo-tile and pointwise kernels: 0 never, 1 built-in rule, 2 wherever they apply
     bool has_wzp;
     void *d_w = nullptr, *d_bias = nullptr;
     std::string name;
@@ -1240,7 +1337,7 @@ struct hipq_conv2d_plan {
 static bool halo_applies(const hipq_conv2d_plan *p)
 {
     const hipq_conv2d_desc &d = p->d;
-    if (!(p->halo && p->variant == kMfma && !p->has_wzp && d.in_cs % 64 == 0 && d.R == 3 && d.S == 3 && d.stride_h == 1
+    if (!(p->special && p->variant == kMfma && !p->has_wzp && d.in_cs % 64 == 0 && d.R == 3 && d.S == 3 && d.stride_h == 1
           && d.stride_w == 1 && d.pad_h == 1 && d.pad_w == 1 && d.W <= 63 && kTiles[p->tile].bm <= 128))
         return false;
     const int nc = d.in_cs / 64, bm = kTiles[p->tile].bm;
@@ -1248,14 +1345,26 @@ static bool halo_applies(const hipq_conv2d_plan *p)
         return true;
     // Several channel slabs (all halo tiles resident at once): measured slower than the streaming kernel on 14x14 and
     // 7x7 images and equal on 28x28, so only on request.
-    return p->halo == 2 && (nc == 2 || nc == 4 || nc == 8) && kTiles[p->tile].bn == 128 && bm + 2 * d.W + 2 <= bm + 64;
+    return p->special == 2 && (nc == 2 || nc == 4 || nc == 8) && kTiles[p->tile].bn == 128 && bm + 2 * d.W + 2 <= bm + 64;
+}
+
+// conv_mfma_pointwise_kernel: 1x1, stride 1, no padding, at most 64 input and 256 output channels, weight zero point
+// 128 (or int8), one-multiply requantisation.
+static bool pointwise_applies(const hipq_conv2d_plan *p)
+{
+    const hipq_conv2d_desc &d = p->d;
+    return p->special && p->variant == kMfma && !p->has_wzp && d.R == 1 && d.S == 1 && d.stride_h == 1 && d.stride_w == 1
+        && d.pad_h == 0 && d.pad_w == 0 && d.in_cs % 16 == 0 && d.in_cs <= 64 && p->args.kout_pad <= 256 && p->args.fastq;
 }
 
 static void set_mfma_name(hipq_conv2d_plan *p, bool smallc)
 {
     char nm[96];
-    snprintf(nm, sizeof nm, "conv_mfma_i8_%dx%d%s%s%s%s", kTiles[p->tile].bm, kTiles[p->tile].bn, smallc ? "_c4" : "",
-             p->has_wzp ? "_wzp" : "", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "", halo_applies(p) ? "_halo" : "");
+    if (pointwise_applies(p))
+        snprintf(nm, sizeof nm, "conv_mfma_i8_pointwise%s", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
+    else
+        snprintf(nm, sizeof nm, "conv_mfma_i8_%dx%d%s%s%s%s", kTiles[p->tile].bm, kTiles[p->tile].bn, smallc ? "_c4" : "",
+                 p->has_wzp ? "_wzp" : "", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "", halo_applies(p) ? "_halo" : "");
     p->name = nm;
 }
 
@@ -1393,7 +1502,7 @@ extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t
         pad_off = wbuf.size();
         wbuf.resize(pad_off + 64, (uint8_t)pad_byte); // source of out-of-image taps
         static const bool no_halo = getenv("HIPQ_NO_HALO") != nullptr; // for A/B measurements
-        p->halo = no_halo ? 0 : 1;
+        p->special = no_halo ? 0 : 1;
         set_mfma_name(p, smallc);
     } else if (!sgn && d.group == d.C && d.K == d.C && d.in_cs == d.out_cs && d.R == 3 && d.S == 3 && d.stride_h == d.stride_w
                && (d.stride_h == 1 || d.stride_h == 2)
@@ -1488,14 +1597,14 @@ extern "C" int hipq_conv2d_plan_select(hipq_conv2d_plan *p, int tile, int stages
     return 0;
 }
 
-extern "C" int hipq_conv2d_plan_halo(hipq_conv2d_plan *p, int mode)
+extern "C" int hipq_conv2d_plan_special(hipq_conv2d_plan *p, int mode)
 {
     clear_error();
-    HIPQ_REQUIRE(p, "hipq_conv2d_plan_halo: null plan");
-    HIPQ_REQUIRE(p->variant == kMfma, "hipq_conv2d_plan_halo: only the DMA-fed MFMA kernel has variants (this plan runs %s)",
+    HIPQ_REQUIRE(p, "hipq_conv2d_plan_special: null plan");
+    HIPQ_REQUIRE(p->variant == kMfma, "hipq_conv2d_plan_special: only the DMA-fed MFMA kernel has variants (this plan runs %s)",
                  p->name.c_str());
-    HIPQ_REQUIRE(mode >= 0 && mode <= 2, "hipq_conv2d_plan_halo: mode must be 0 (never), 1 (built-in rule) or 2 (wherever it applies)");
-    p->halo = mode;
+    HIPQ_REQUIRE(mode >= 0 && mode <= 2, "hipq_conv2d_plan_special: mode must be 0 (never), 1 (built-in rule) or 2 (wherever they apply)");
+    p->special = mode;
     set_mfma_name(p, false);
     return 0;
 }
@@ -1569,6 +1678,16 @@ static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_
     const dim3 grid((nblk + 7) / 8 * 8), block(256);
     if (p->variant == kMfma && launch_halo<BM, BN, WM, WN>(p, a, grid, st))
         return;
+    if (pointwise_applies(p) && a.acc_out == nullptr && a.res == nullptr) {
+        // persistent work-groups (four waves, a strip of 32 pixels each per turn), five to a CU
+        const int nstrips = (a.P + 31) / 32, want = (nstrips + 3) / 4;
+        const dim3 pgrid(want < 1280 ? want : 1280);
+        if (a.in_cs <= 32)
+            hipLaunchKernelGGL(conv_mfma_pointwise_kernel<1>, pgrid, block, 0, st, a);
+        else
+            hipLaunchKernelGGL(conv_mfma_pointwise_kernel<2>, pgrid, block, 0, st, a);
+        return;
+    }
     // "aligned" addressing: a 64-byte slab never straddles two taps.  True when a pixel's channels are whole slabs, and
     // for 1x1 kernels with any channel stride (a multiple of 16): there is one tap, and the pad chunks of the last
     // slab (beyond the pixel's own bytes) are read from the pad buffer.

@@ -42,7 +42,7 @@ _SIGS = {
     "hipq_conv2d_plan_destroy": (None, [C.c_void_p]),
     "hipq_conv2d_plan_kernel": (C.c_char_p, [C.c_void_p]),
     "hipq_conv2d_plan_select": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
-    "hipq_conv2d_plan_halo": (C.c_int, [C.c_void_p, C.c_int]),
+    "hipq_conv2d_plan_special": (C.c_int, [C.c_void_p, C.c_int]),
     "hipq_conv2d_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "hipq_conv2d_run_add": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_float, C.c_int,
                                       C.c_int, C.c_void_p, C.c_void_p]),
@@ -165,10 +165,10 @@ class Conv2d:
         self.kernel = lib().hipq_conv2d_plan_kernel(self.handle).decode()
         return self
 
-    def halo(self, mode=1):
-        """Tuning hook: the halo-tile kernel of 3x3 stride-1 layers: 0 never, 1 built-in rule, 2 wherever it applies
-        (include/hipq.h)."""
-        check(lib().hipq_conv2d_plan_halo(self.handle, int(mode)))
+    def special(self, mode=1):
+        """Tuning hook: the halo-tile (3x3 stride 1) and pointwise (small 1x1) kernels: 0 never, 1 built-in rule,
+        2 wherever they apply (include/hipq.h)."""
+        check(lib().hipq_conv2d_plan_special(self.handle, int(mode)))
         self.kernel = lib().hipq_conv2d_plan_kernel(self.handle).decode()
         return self
 

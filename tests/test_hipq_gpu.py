@@ -291,7 +291,9 @@ def test_conv_plan_variants_are_bit_identical():
               (2, 1024, 7, 7, 256, 1, 0, 1), (1, 192, 20, 20, 320, 1, 0, 1),
               # 1x1 kernels whose channel stride is not a multiple of 64: partial last slab
               (2, 96, 9, 9, 24, 1, 0, 1), (1, 16, 12, 12, 96, 1, 0, 1), (1, 144, 7, 7, 32, 1, 0, 1), (3, 160, 5, 5, 320, 1, 0, 1),
-              (1, 32, 10, 10, 192, 1, 0, 2), (1, 20, 6, 6, 16, 1, 0, 1)]
+              (1, 32, 10, 10, 192, 1, 0, 2), (1, 20, 6, 6, 16, 1, 0, 1),
+              # the pointwise kernel: ragged strips, 1 and 2 k-steps, partial channel blocks, the widest output
+              (3, 64, 7, 9, 256, 1, 0, 1), (1, 48, 5, 5, 40, 1, 0, 1), (2, 8, 3, 11, 16, 1, 0, 1), (1, 64, 33, 31, 64, 1, 0, 1)]
     for N, C, H, W, K, R, pad, st in shapes:
         x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
         w = rng.integers(0, 256, (K, C, R, R), dtype=np.uint8)
@@ -303,6 +305,17 @@ def test_conv_plan_variants_are_bit_identical():
         res = rng.integers(0, 256, want.shape, dtype=np.uint8)
         rd = hipq.to_device_nhwc(res)
         want_add = orc.add_u8(want, res, q[4], q[5], 0.07, 33, 0.1, 5)
+        if plan.kernel.endswith("pointwise"):  # small 1x1 layers: the pointwise kernel first, then the tile kernels
+            assert R == 1 and C <= 64 and K <= 256, plan.kernel
+            assert np.array_equal(hipq.from_device_nhwc(plan(xd), K), want), (x.shape, w.shape, plan.kernel)
+            if K % 16 == 0:
+                zd = plan.empty_output()
+                plan.run_add(xd, rd, False, 0.07, 33, 0.1, 5, zd)
+                assert np.array_equal(hipq.from_device_nhwc(zd, K), want_add), ("add", x.shape, plan.kernel)
+                plan.run_add(xd, rd, True, 0.07, 33, 0.1, 5, zd)
+                assert np.array_equal(hipq.from_device_nhwc(zd, K), orc.add_u8(res, want, 0.07, 33, q[4], q[5], 0.1, 5)), ("add first", x.shape)
+            plan.special(0)
+            assert not plan.kernel.endswith("pointwise")
         for tile in (0, 1, 2, 3, 4):
             for stages in (0, 2, 3, 4, 8):
                 plan.select(tile, stages)
@@ -337,7 +350,7 @@ def test_conv3x3_halo_kernel_matches_the_streaming_kernel_and_the_oracle():
         want, want_acc = orc.conv2d_u8(x, w, b, 1, 1, 1, *q, return_acc=True)
         plan = hipq.Conv2d(x.shape, w, b, 1, 1, 1, *q)
         assert plan.kernel.endswith("_halo") == (C == 64), plan.kernel  # the built-in rule: single channel slab only
-        plan.halo(2)
+        plan.special(2)
         xd = hipq.to_device_nhwc(x)
         for tile in (0, 2, 3, 4):
             plan.select(tile, 0)
@@ -349,17 +362,17 @@ def test_conv3x3_halo_kernel_matches_the_streaming_kernel_and_the_oracle():
         acc = torch.empty((N, H, W, plan.desc.out_cs), dtype=torch.int32, device="cuda")
         plan(xd, acc=acc)
         assert np.array_equal(acc.cpu().numpy()[..., :K].transpose(0, 3, 1, 2), want_acc)
-        plan.halo(0)
+        plan.special(0)
         assert not plan.kernel.endswith("_halo")
         assert np.array_equal(hipq.from_device_nhwc(plan(xd), K), want)
-        plan.select(1, 0).halo(2)  # the 256-pixel tile has no halo variant
+        plan.select(1, 0).special(2)  # the 256-pixel tile has no halo variant
         assert not plan.kernel.endswith("_halo")
         assert np.array_equal(hipq.from_device_nhwc(plan(xd), K), want)
         # int8 tensors: zero padding
         xs, ws = x.view(np.int8), w.view(np.int8)
         want8 = orc.conv2d_i8(xs, ws, b, 1, 1, 1, q[0], q[2], q[4], 7)
         p8 = hipq.Conv2d(x.shape, ws, b, 1, 1, 1, q[0], 0, q[2], 0, q[4], 0, obits=7, dtype=hipq.DTYPE_I8)
-        p8.select(0, 0).halo(2)
+        p8.select(0, 0).special(2)
         assert p8.kernel.endswith("_halo") == (C == 64 or (C in (128, 256, 512) and W <= 31)), p8.kernel
         assert np.array_equal(hipq.from_device_nhwc(p8(hipq.to_device_nhwc(xs)), K).view(np.int8), want8), (x.shape, K)
     # not eligible: stride 2, pad 0, wide images, asymmetric weights
