@@ -39,6 +39,8 @@
 //     range of pixel tiles: neighbouring tiles share input halos and weight slabs in that XCD's L2.
 //   * 3x3 / stride 1 / pad 1 layers with 64 input channels run conv_mfma_halo_kernel: the input tile is loaded once
 //     with its halo and the nine taps are read from LDS at shifted rows, instead of one slab per tap from memory.
+//   * 1x1 / stride 1 layers with at most 64 input and 256 output channels run conv_mfma_pointwise_kernel: a wave per
+//     strip of 32 pixels, pixel fragments straight from global memory, no LDS staging of activations, no barriers.
 //   * Other shapes: C <= 4 inputs (the RGB stem) use a register-staged variant of the same tile computation,
 //     depthwise 3x3 a dot-product kernel, remaining depthwise / grouped shapes plain per-output kernels.
 #include <algorithm>
