@@ -1356,7 +1356,8 @@ static bool pointwise_applies(const hipq_conv2d_plan *p)
 {
     const hipq_conv2d_desc &d = p->d;
     return p->special && p->variant == kMfma && !p->has_wzp && d.R == 1 && d.S == 1 && d.stride_h == 1 && d.stride_w == 1
-        && d.pad_h == 0 && d.pad_w == 0 && d.in_cs % 16 == 0 && d.in_cs <= 64 && p->args.kout_pad <= 256 && p->args.fastq;
+        && d.pad_h == 0 && d.pad_w == 0 && d.in_cs % 16 == 0 && d.in_cs <= 64 && d.out_cs % 16 == 0 && p->args.kout_pad <= 256
+        && p->args.fastq;
 }
 
 static void set_mfma_name(hipq_conv2d_plan *p, bool smallc)

@@ -293,7 +293,9 @@ def test_conv_plan_variants_are_bit_identical():
               (2, 96, 9, 9, 24, 1, 0, 1), (1, 16, 12, 12, 96, 1, 0, 1), (1, 144, 7, 7, 32, 1, 0, 1), (3, 160, 5, 5, 320, 1, 0, 1),
               (1, 32, 10, 10, 192, 1, 0, 2), (1, 20, 6, 6, 16, 1, 0, 1),
               # the pointwise kernel: ragged strips, 1 and 2 k-steps, partial channel blocks, the widest output
-              (3, 64, 7, 9, 256, 1, 0, 1), (1, 48, 5, 5, 40, 1, 0, 1), (2, 8, 3, 11, 16, 1, 0, 1), (1, 64, 33, 31, 64, 1, 0, 1)]
+              (3, 64, 7, 9, 256, 1, 0, 1), (1, 48, 5, 5, 40, 1, 0, 1), (2, 8, 3, 11, 16, 1, 0, 1), (1, 64, 33, 31, 64, 1, 0, 1),
+              # four output channels or fewer: a 4-byte channel stride, which the pointwise kernel's 16-byte stores must not get
+              (2, 32, 9, 9, 3, 1, 0, 1), (1, 17, 6, 5, 1, 1, 0, 1)]
     for N, C, H, W, K, R, pad, st in shapes:
         x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
         w = rng.integers(0, 256, (K, C, R, R), dtype=np.uint8)
@@ -305,6 +307,7 @@ def test_conv_plan_variants_are_bit_identical():
         res = rng.integers(0, 256, want.shape, dtype=np.uint8)
         rd = hipq.to_device_nhwc(res)
         want_add = orc.add_u8(want, res, q[4], q[5], 0.07, 33, 0.1, 5)
+        assert not (K <= 4 and "pointwise" in plan.kernel), plan.kernel
         if plan.kernel.endswith("pointwise"):  # small 1x1 layers: the pointwise kernel first, then the tile kernels
             assert R == 1 and C <= 64 and K <= 256, plan.kernel
             assert np.array_equal(hipq.from_device_nhwc(plan(xd), K), want), (x.shape, w.shape, plan.kernel)
