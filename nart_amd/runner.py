@@ -172,8 +172,10 @@ class HipqExecutor:
             plan = s.get("plan")
             if plan is None or not plan.kernel.startswith("conv_mfma") or "_c4" in plan.kernel or "_wzp" in plan.kernel:
                 continue
-            if plan.desc.in_cs % 64:
+            if plan.desc.in_cs % 64 and not (plan.desc.R == 1 and plan.desc.S == 1):
                 continue  # the generic-addressing kernel has a single variant
+            if plan.kernel.endswith("pointwise") and s["kind"] != "conv+add":
+                continue  # the pointwise kernel has no tile or stages (the fused add runs a tile kernel)
             lo, hi = max(0, k - before), min(len(self.steps), k + 1 + after)
             base = self._time_window(lo, hi, reps)
             best, best_t = (-1, 0), base
