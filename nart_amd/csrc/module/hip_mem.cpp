@@ -37,6 +37,7 @@ static void hm_free(mem_t *mm)
     m->host = m->dev = m->stage = nullptr;
     m->host_cap = m->dev_cap = m->stage_cap = m->size = 0;
     m->host_valid = m->dev_valid = false;
+    m->pending = nullptr;
 }
 
 static void hm_delete(mem_t *mm)
@@ -103,6 +104,7 @@ static void upload(hip_mem_t *m, hipStream_t st)
 static void *hm_cpu_data(const mem_t *mm)
 {
     hip_mem_t *m = as_hip(const_cast<mem_t *>(mm));
+    hip_mem_settle(m);
     if (m->dev_valid && !m->host_valid) {
         HIPM_HIP(hipDeviceSynchronize()); // the producing kernels run on a workspace stream
         download(m);
@@ -116,6 +118,7 @@ static void *hm_cpu_data(const mem_t *mm)
 const void *hip_mem_host_in(mem_t *mm)
 {
     hip_mem_t *m = as_hip(mm);
+    hip_mem_settle(m);
     if (m->dev_valid && !m->host_valid) {
         HIPM_HIP(hipDeviceSynchronize());
         download(m);
@@ -128,6 +131,7 @@ const void *hip_mem_host_in(mem_t *mm)
 const void *hip_mem_dev_in(mem_t *mm, hipStream_t st)
 {
     hip_mem_t *m = as_hip(mm);
+    hip_mem_settle(m);
     if (!m->dev_valid) {
         ensure_host(m); // never-written memory reads as zeros
         m->host_valid = true;
@@ -139,6 +143,7 @@ const void *hip_mem_dev_in(mem_t *mm, hipStream_t st)
 void *hip_mem_dev_out(mem_t *mm, hipStream_t)
 {
     hip_mem_t *m = as_hip(mm);
+    m->pending = nullptr; // about to be overwritten: a deferred producer's result is dead
     grow_dev(&m->dev, &m->dev_cap, dev_bytes(m));
     m->dev_valid = true;
     m->host_valid = false;
@@ -191,6 +196,7 @@ void hip_mem_tag(tensor_t *t)
     }
     if (layout != m->layout || N != m->N || C != m->C || H != m->H || W != m->W) {
         // geometry changed (first use, or a batch reshape): what the device holds is no longer addressable
+        hip_mem_settle(m);
         if (m->dev_valid && !m->host_valid && m->dev)
             download(m);
         m->dev_valid = false;

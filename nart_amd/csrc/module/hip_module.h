@@ -83,7 +83,22 @@ struct hip_mem_t {
     hip_layout_t layout;
     int N, C, H, W, cs; // geometry for HIP_LAYOUT_NHWC_U8
     bool host_valid, dev_valid;
+    // Deferred producer.  A convolution whose only reader is an add does not launch at its own run(): it leaves this
+    // hook, and the add runs both as one fused kernel (hip_ops.cpp).  Whoever else asks for the contents first - the
+    // host, another workspace, a re-run - makes the hook launch the plain convolution into `dev` (hip_mem_settle).
+    void (*pending)(void *ctx);
+    void *pending_ctx;
 };
+
+// make the device contents current: run the deferred producer, if any
+static inline void hip_mem_settle(hip_mem_t *m)
+{
+    if (m->pending) {
+        void (*f)(void *) = m->pending;
+        m->pending = nullptr;
+        f(m->pending_ctx);
+    }
+}
 
 extern const mem_tp hip_mem_tp_st;
 

@@ -6,7 +6,9 @@
 // folded per-channel constants, which the reference recomputes on every run) and selects the run function;
 // `run` only launches kernels on the workspace stream.
 #include <cstring>
+#include <map>
 #include <new>
+#include <set>
 #include <vector>
 
 #include "hip_module.h"
@@ -45,6 +47,8 @@ void alloc_and_tag(op_t *op)
     }
 }
 
+void forget_reader(op_t *op);
+
 template <class T>
 op_t *alloc_op(workspace_t *)
 {
@@ -52,11 +56,34 @@ op_t *alloc_op(workspace_t *)
     return reinterpret_cast<op_t *>(p);
 }
 
-void dealloc_op(op_t *op) { free(op); }
+void dealloc_op(op_t *op)
+{
+    // forget what the operator read (the registry of the convolution + add fusion, below)
+    forget_reader(op);
+    free(op);
+}
 void destroy_nothing(op_t *) {}
 
 const void *in_ptr(op_t *op, int i) { return hip_mem_dev_in(op->input_tensors[i]->mem, op_stream(op)); }
 void *out_ptr(op_t *op) { return hip_mem_dev_out(op->output_tensors[0].mem, op_stream(op)); }
+
+// Which operators of this workspace read which memory, collected as the operators are prepared (every prepare of the
+// pass has run before the first run()).  A convolution asks it whether an add is the ONLY reader of its output.
+typedef std::map<const mem_t *, std::set<const op_t *>> reader_map;
+
+// keyed by workspace (the runtime is single-threaded, art/include/art/workspace.h has no locking either)
+std::map<const workspace_t *, reader_map> g_readers;
+long g_fused_adds = 0; // launches of the fused kernel so far (hip_module_fused_adds)
+
+reader_map &readers_of(op_t *op) { return g_readers[op->workspace]; }
+
+void forget_reader(op_t *op)
+{
+    const auto it = g_readers.find(op->workspace);
+    if (it != g_readers.end())
+        for (auto &kv : it->second)
+            kv.second.erase(op);
+}
 
 // allow_i8: conv_2d, ip and dequantize also exist for int8 symmetric tensors (conv_2d.c:120-141, ip.cpp:312-331,
 // dequantize.c:156-163); every other operator of the reference module is uint8 only.
@@ -71,6 +98,7 @@ void require_hip_u8(op_t *op, size_t n_act, bool allow_i8 = false)
         }
         HIPM_CHECK(is_hip_mem(op->input_tensors[i]->mem));
         hip_mem_tag(op->input_tensors[i]);
+        readers_of(op)[op->input_tensors[i]->mem].insert(op);
     }
 }
 
@@ -82,6 +110,7 @@ struct conv_op_t {
     hipq_conv2d_plan *plan;
     hipq_conv2d_desc desc; // what the plan was built for (re-used when prepare is called again unchanged)
     const void *w_seen;    // identity of the weights the plan was packed from
+    int defer;             // 0 undecided, 1 leave the launch to the add that reads the output, -1 launch at run()
 };
 
 void conv_config(op_t *op)
@@ -116,15 +145,54 @@ void conv_destroy(op_t *op)
     c->plan = nullptr;
 }
 
+// ---- convolution + add fusion ------------------------------------------------------------------------------------
+// In a residual network the expanding convolution's output is read by the add and by nothing else.  Such a
+// convolution does not launch at its own run(): it leaves a hook on its output memory, and the add's run() launches
+// hipq_conv2d_run_add - the convolution with the add in its epilogue, bit-identical to the two operators - so the
+// convolution's output is never written or read.  Anything else that asks for that memory (the host through
+// mem_cpu_data, a foreign workspace through mem_data) settles the hook first, which launches the plain convolution.
+void conv_launch_plain(void *ctx)
+{
+    op_t *op = static_cast<op_t *>(ctx);
+    conv_op_t *c = reinterpret_cast<conv_op_t *>(op);
+    hip_mem_t *ym = as_hip(op->output_tensors[0].mem);
+    HIPM_HIPQ(hipq_conv2d_run(c->plan, in_ptr(op, 0), ym->dev, nullptr, op_stream(op)));
+}
+
+bool add_is_only_reader(op_t *op)
+{
+    static const bool off = getenv("NART_HIP_NO_FUSION") != nullptr;
+    conv_op_t *c = reinterpret_cast<conv_op_t *>(op);
+    if (off || c->desc.dtype != HIPQ_DTYPE_U8 || strncmp(hipq_conv2d_plan_kernel(c->plan), "conv_mfma", 9) != 0)
+        return false; // hipq_conv2d_run_add exists for the uint8 MFMA plans
+    const reader_map &rm = readers_of(op);
+    const auto it = rm.find(op->output_tensors[0].mem);
+    if (it == rm.end() || it->second.size() != 1)
+        return false;
+    const op_t *r = *it->second.begin();
+    return r->entry->tp == &op_add_tp && r->workspace == op->workspace && r->input_size == 2
+        && r->input_tensors[0]->mem != r->input_tensors[1]->mem;
+}
+
 void conv_run(op_t *op)
 {
     conv_op_t *c = reinterpret_cast<conv_op_t *>(op);
+    if (c->defer == 0)
+        c->defer = add_is_only_reader(op) ? 1 : -1;
+    if (c->defer == 1) {
+        hip_mem_t *ym = as_hip(op->output_tensors[0].mem);
+        (void)out_ptr(op); // the buffer exists and the device side is the current one - once the hook has run
+        ym->pending = conv_launch_plain;
+        ym->pending_ctx = op;
+        return;
+    }
     HIPM_HIPQ(hipq_conv2d_run(c->plan, in_ptr(op, 0), out_ptr(op), nullptr, op_stream(op)));
 }
 
 void build_plan(op_t *op, const hipq_conv2d_desc &d, const uint8_t *w, const void *w_id)
 {
     conv_op_t *c = reinterpret_cast<conv_op_t *>(op);
+    c->defer = 0; // decided at the next run, when every operator of the pass has been prepared
     if (c->plan && memcmp(&c->desc, &d, sizeof d) == 0 && c->w_seen == w_id)
         return; // prepare is called again after a reshape (art/src/parade.c:199-215): nothing changed
     hipq_conv2d_plan_destroy(c->plan);
@@ -249,6 +317,26 @@ void add_config(op_t *op)
 void add_run(op_t *op)
 {
     ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    for (int i = 0; i < 2; ++i) {
+        hip_mem_t *m = as_hip(op->input_tensors[i]->mem);
+        if (m->pending != conv_launch_plain)
+            continue;
+        // input i is a convolution that left its launch to this add (conv_run): run both as one kernel, provided the
+        // add reads the convolution's output with the scale it was written with
+        op_t *cop = static_cast<op_t *>(m->pending_ctx);
+        conv_op_t *c = reinterpret_cast<conv_op_t *>(cop);
+        const int o = 1 - i;
+        if (e->qi.alpha[i] != c->desc.oalpha || e->qi.zp[i] != c->desc.ozp)
+            break;
+        const void *res = in_ptr(op, o); // settles the other input if it is deferred as well
+        const void *x = in_ptr(cop, 0);
+        if (hipq_conv2d_run_add(c->plan, x, res, o == 0, e->qi.alpha[o], e->qi.zp[o], e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0],
+                                out_ptr(op), op_stream(op)) == 0) {
+            ++g_fused_adds;
+            return; // the convolution's own output stays unwritten; its hook stays for whoever asks
+        }
+        break;      // parameters outside the fused kernel's range: the plain path below settles the hook
+    }
     HIPM_HIPQ(hipq_add_u8(in_ptr(op, 0), in_ptr(op, 1), out_ptr(op), e->bytes, e->qi.alpha[0], e->qi.zp[0], e->qi.alpha[1],
                           e->qi.zp[1], e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0], op_stream(op)));
 }
@@ -564,6 +652,7 @@ void ws_delete(workspace_t *w)
     hip_workspace_t *ws = reinterpret_cast<hip_workspace_t *>(w);
     if (ws->own_stream && ws->stream)
         (void)hipStreamDestroy(ws->stream);
+    g_readers.erase(w);
     free(ws);
 }
 
@@ -599,6 +688,9 @@ static workspace_t *ws_new(const setting_entry_t *settings)
 }
 
 // Extra entry points for runners that own a stream already (graph capture, event timing).
+// How many add operators have run fused into the convolution that produces one of their inputs (diagnostics, tests).
+ART_PUBLIC long hip_module_fused_adds(void) { return g_fused_adds; }
+
 ART_PUBLIC void *hip_workspace_stream(workspace_t *w) { return reinterpret_cast<hip_workspace_t *>(w)->stream; }
 
 ART_PUBLIC void hip_workspace_set_stream(workspace_t *w, void *stream)

@@ -124,6 +124,56 @@ def test_single_ops_through_the_op_api(own_rt):
     ws.delete()
 
 
+def test_convolution_and_add_run_as_one_kernel(own_rt):
+    """A convolution whose output only an add reads leaves its launch to that add (one fused kernel, the convolution's
+    output is never written); whoever asks for the elided tensor afterwards gets it computed on demand.  Results are
+    those of the two operators run one after the other; a convolution with a second reader is not deferred."""
+    import ctypes as C
+    from oracle import orc
+    fused = own_rt.libs[1].hip_module_fused_adds
+    fused.restype = C.c_long
+    ws = own_rt.workspace("hip")
+    rng = np.random.default_rng(21)
+    x = rng.integers(0, 256, (2, 64, 9, 11), dtype=np.uint8)
+    w = rng.integers(0, 256, (128, 64, 1, 1), dtype=np.uint8)
+    b = rng.integers(-5000, 5000, 128).astype(np.int32)
+    r = rng.integers(0, 256, (2, 128, 9, 11), dtype=np.uint8)
+    q = dict(ialpha=0.031, izp=77, walpha=0.0042, wzp=128, oalpha=0.09, ozp=13)
+    want_c = orc.conv2d_u8(x, w, b, 0, 1, 1, 0.031, 77, 0.0042, 128, 0.09, 13)
+    for conv_first in (True, False):
+        tx, tr = ws.tensor(x), ws.tensor(r)
+        conv = ws.conv2d(tx, ws.tensor(w), ws.tensor(b), 0, 1, 1, q).prepare()
+        ins = [conv.output(0), tr] if conv_first else [tr, conv.output(0)]
+        qa = dict(ialpha=[0.09, 0.05] if conv_first else [0.05, 0.09], izp=[13, 200] if conv_first else [200, 13], oalpha=0.12, ozp=31)
+        add = ws.add(ins[0], ins[1], qa).prepare()
+        want_a = orc.add_u8(want_c, r, 0.09, 13, 0.05, 200, 0.12, 31) if conv_first else orc.add_u8(r, want_c, 0.05, 200, 0.09, 13, 0.12, 31)
+        n0 = fused()
+        for _ in range(2):  # the second pass defers and fuses again
+            conv.run()
+            add.run()
+            assert same_bits(add.output(0).numpy(), want_a), conv_first
+        assert fused() == n0 + 2
+        assert same_bits(conv.output(0).numpy(), want_c)  # elided so far: computed now
+        # new input through the host mirror, then only the convolution: the deferred launch happens when the output is read
+        x2 = rng.integers(0, 256, x.shape, dtype=np.uint8)
+        tx.write(x2)
+        conv.run()
+        assert same_bits(conv.output(0).numpy(), orc.conv2d_u8(x2, w, b, 0, 1, 1, 0.031, 77, 0.0042, 128, 0.09, 13))
+        tx.write(x)
+        # a second reader: no deferral from now on (decided at prepare + first run), results unchanged
+        relu = ws.relu(conv.output(0), dict(ialpha=0.09, izp=13, oalpha=0.05, ozp=3)).prepare()
+        conv.prepare()
+        n1 = fused()
+        conv.run()
+        add.run()
+        relu.run()
+        assert fused() == n1
+        assert same_bits(add.output(0).numpy(), want_a) and same_bits(relu.output(0).numpy(), orc.relu_u8(want_c, 0.09, 13, 0.05, 3))
+        for o in (relu, add, conv):
+            o.delete()
+    ws.delete()
+
+
 def test_concat_softmax_through_the_op_api(own_rt):
     import refrun
     from oracle import orc
