@@ -196,7 +196,10 @@ void hip_mem_tag(tensor_t *t)
     }
     if (layout != m->layout || N != m->N || C != m->C || H != m->H || W != m->W) {
         // geometry changed (first use, or a batch reshape): what the device holds is no longer addressable
-        hip_mem_settle(m);
+        if (m->pending) { // a convolution that never launched: there is nothing to keep
+            m->pending = nullptr;
+            m->dev_valid = false;
+        }
         if (m->dev_valid && !m->host_valid && m->dev)
             download(m);
         m->dev_valid = false;

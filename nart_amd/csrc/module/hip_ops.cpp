@@ -141,6 +141,10 @@ void ip_config(op_t *op)
 void conv_destroy(op_t *op)
 {
     conv_op_t *c = reinterpret_cast<conv_op_t *>(op);
+    // a launch left to an add (conv_run) must not outlive the plan: the output's memory may, as a view's
+    if (op->output_size > 0 && op->output_tensors != nullptr && op->output_tensors[0].mem != nullptr
+        && is_hip_mem(op->output_tensors[0].mem) && as_hip(op->output_tensors[0].mem)->pending_ctx == op)
+        as_hip(op->output_tensors[0].mem)->pending = nullptr;
     hipq_conv2d_plan_destroy(c->plan);
     c->plan = nullptr;
 }
