@@ -125,6 +125,15 @@ int hipq_conv2d_run(const hipq_conv2d_plan *plan, const void *x, void *y, int32_
                     void *stream);
 
 /*
+ * Convolution with a ReLU fused into its epilogue, for a plan created with relu = 0: y = max(conv(x), ozp), which is
+ * bit-identical to hipq_conv2d_run followed by hipq_relu_u8 with input and output scale and zero point equal to the
+ * plan's oalpha / ozp and the plan's obits (op_conv_2d_u8xu8_run, then op_quant_relu_run — src/op/relu.c:76-115: with
+ * equal scales the multiplier is exactly one).  The same as running a plan created with relu = 1; a caller that learns
+ * only at run time that a ReLU follows (the art module) does not need a second plan.  uint8 plans only.
+ */
+int hipq_conv2d_run_relu(const hipq_conv2d_plan *plan, const void *x, void *y, void *stream);
+
+/*
  * Convolution with the residual add fused into its epilogue: y = add(conv(x), residual), bit-identical to
  * hipq_conv2d_run followed by hipq_add_u8 on the stored bytes (op_conv_2d_u8xu8_run, then op_quant_add_run —
  * src/op/add.c:83-148), but the convolution's own uint8 result never travels to memory.  `residual` has the

@@ -1742,6 +1742,19 @@ extern "C" int hipq_conv2d_run(const hipq_conv2d_plan *p, const void *x, void *y
     return run_conv(p, a, static_cast<hipStream_t>(stream));
 }
 
+extern "C" int hipq_conv2d_run_relu(const hipq_conv2d_plan *p, const void *x, void *y, void *stream)
+{
+    clear_error();
+    HIPQ_REQUIRE(p && x && y, "hipq_conv2d_run_relu: null argument");
+    HIPQ_REQUIRE(p->d.dtype == HIPQ_DTYPE_U8, "hipq_conv2d_run_relu: uint8 plans only (op_quant_relu_run is a uint8 operator)");
+    ConvArgs a = p->args;
+    a.x = static_cast<const uint8_t *>(x);
+    a.y = static_cast<uint8_t *>(y);
+    a.acc_out = nullptr;
+    a.lo = std::min(p->d.ozp, a.q.hi); // what plan creation sets for relu = 1
+    return run_conv(p, a, static_cast<hipStream_t>(stream));
+}
+
 extern "C" int hipq_conv2d_run_add(const hipq_conv2d_plan *p, const void *x, const void *residual, int residual_is_input0,
                                    float res_alpha, int res_zp, float oalpha, int ozp, int obits, void *y, void *stream)
 {

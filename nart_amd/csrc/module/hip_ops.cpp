@@ -73,7 +73,7 @@ typedef std::map<const mem_t *, std::set<const op_t *>> reader_map;
 
 // keyed by workspace (the runtime is single-threaded, art/include/art/workspace.h has no locking either)
 std::map<const workspace_t *, reader_map> g_readers;
-long g_fused_adds = 0; // launches of the fused kernel so far (hip_module_fused_adds)
+long g_fused_adds = 0, g_fused_relus = 0; // fused launches so far (hip_module_fused_adds / _relus)
 
 reader_map &readers_of(op_t *op) { return g_readers[op->workspace]; }
 
@@ -110,7 +110,7 @@ struct conv_op_t {
     hipq_conv2d_plan *plan;
     hipq_conv2d_desc desc; // what the plan was built for (re-used when prepare is called again unchanged)
     const void *w_seen;    // identity of the weights the plan was packed from
-    int defer;             // 0 undecided, 1 leave the launch to the add that reads the output, -1 launch at run()
+    int defer;             // 0 undecided, 1 leave the launch to the add / relu that reads the output, -1 launch at run()
 };
 
 void conv_config(op_t *op)
@@ -149,11 +149,13 @@ void conv_destroy(op_t *op)
     c->plan = nullptr;
 }
 
-// ---- convolution + add fusion ------------------------------------------------------------------------------------
-// In a residual network the expanding convolution's output is read by the add and by nothing else.  Such a
-// convolution does not launch at its own run(): it leaves a hook on its output memory, and the add's run() launches
-// hipq_conv2d_run_add - the convolution with the add in its epilogue, bit-identical to the two operators - so the
-// convolution's output is never written or read.  Anything else that asks for that memory (the host through
+// ---- convolution + add / relu fusion -----------------------------------------------------------------------------
+// In a residual network the expanding convolution's output is read by the add and by nothing else; where the converter
+// emits ReLU as an operator of its own (the CPU module ignores the convolution's relu flag, conv_2d.c:27-70), the
+// convolution's output is read by that relu and by nothing else.  Such a convolution does not launch at its own run():
+// it leaves a hook on its output memory, and the reader's run() launches hipq_conv2d_run_add / hipq_conv2d_run_relu - the
+// convolution with the add / the clamp in its epilogue, bit-identical to the two operators - so the convolution's
+// output is never written or read.  Anything else that asks for that memory (the host through
 // mem_cpu_data, a foreign workspace through mem_data) settles the hook first, which launches the plain convolution.
 void conv_launch_plain(void *ctx)
 {
@@ -163,26 +165,32 @@ void conv_launch_plain(void *ctx)
     HIPM_HIPQ(hipq_conv2d_run(c->plan, in_ptr(op, 0), ym->dev, nullptr, op_stream(op)));
 }
 
-bool add_is_only_reader(op_t *op)
+// 1: the only reader of the convolution's output is an add or a relu of this workspace that can take over the launch
+bool sole_reader_fuses(op_t *op)
 {
     static const bool off = getenv("NART_HIP_NO_FUSION") != nullptr;
     conv_op_t *c = reinterpret_cast<conv_op_t *>(op);
-    if (off || c->desc.dtype != HIPQ_DTYPE_U8 || strncmp(hipq_conv2d_plan_kernel(c->plan), "conv_mfma", 9) != 0)
-        return false; // hipq_conv2d_run_add exists for the uint8 MFMA plans
+    if (off || c->desc.dtype != HIPQ_DTYPE_U8)
+        return false;
     const reader_map &rm = readers_of(op);
     const auto it = rm.find(op->output_tensors[0].mem);
     if (it == rm.end() || it->second.size() != 1)
         return false;
     const op_t *r = *it->second.begin();
-    return r->entry->tp == &op_add_tp && r->workspace == op->workspace && r->input_size == 2
-        && r->input_tensors[0]->mem != r->input_tensors[1]->mem;
+    if (r->workspace != op->workspace)
+        return false;
+    if (r->entry->tp == &op_relu_tp)
+        return true; // any plan runs with the ReLU clamp (hipq_conv2d_run_relu)
+    // hipq_conv2d_run_add exists for the MFMA plans
+    return r->entry->tp == &op_add_tp && r->input_size == 2 && r->input_tensors[0]->mem != r->input_tensors[1]->mem
+        && strncmp(hipq_conv2d_plan_kernel(c->plan), "conv_mfma", 9) == 0;
 }
 
 void conv_run(op_t *op)
 {
     conv_op_t *c = reinterpret_cast<conv_op_t *>(op);
     if (c->defer == 0)
-        c->defer = add_is_only_reader(op) ? 1 : -1;
+        c->defer = sole_reader_fuses(op) ? 1 : -1;
     if (c->defer == 1) {
         hip_mem_t *ym = as_hip(op->output_tensors[0].mem);
         (void)out_ptr(op); // the buffer exists and the device side is the current one - once the hook has run
@@ -403,6 +411,19 @@ void relu_config(op_t *op)
 void relu_run(op_t *op)
 {
     ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    hip_mem_t *m = as_hip(op->input_tensors[0]->mem);
+    if (m->pending == conv_launch_plain) {
+        // the input is a convolution that left its launch to this relu (conv_run).  With equal scales and zero points
+        // on both sides the relu is max(x, zp): the convolution's lower clamp.
+        op_t *cop = static_cast<op_t *>(m->pending_ctx);
+        conv_op_t *c = reinterpret_cast<conv_op_t *>(cop);
+        if (e->qi.alpha[0] == c->desc.oalpha && e->qi.zp[0] == c->desc.ozp && e->qo.alpha[0] == c->desc.oalpha
+            && e->qo.zp[0] == c->desc.ozp && e->qo.bits[0] == c->desc.obits
+            && hipq_conv2d_run_relu(c->plan, in_ptr(cop, 0), out_ptr(op), op_stream(op)) == 0) {
+            ++g_fused_relus;
+            return;
+        }
+    }
     HIPM_HIPQ(hipq_relu_u8(in_ptr(op, 0), out_ptr(op), e->bytes, e->qi.alpha[0], e->qi.zp[0], e->qo.alpha[0], e->qo.zp[0],
                            e->qo.bits[0], op_stream(op)));
 }
@@ -694,6 +715,7 @@ static workspace_t *ws_new(const setting_entry_t *settings)
 // Extra entry points for runners that own a stream already (graph capture, event timing).
 // How many add operators have run fused into the convolution that produces one of their inputs (diagnostics, tests).
 ART_PUBLIC long hip_module_fused_adds(void) { return g_fused_adds; }
+ART_PUBLIC long hip_module_fused_relus(void) { return g_fused_relus; }
 
 ART_PUBLIC void *hip_workspace_stream(workspace_t *w) { return reinterpret_cast<hip_workspace_t *>(w)->stream; }
 

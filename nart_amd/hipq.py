@@ -43,6 +43,7 @@ _SIGS = {
     "hipq_conv2d_plan_kernel": (C.c_char_p, [C.c_void_p]),
     "hipq_conv2d_plan_select": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
     "hipq_conv2d_plan_special": (C.c_int, [C.c_void_p, C.c_int]),
+    "hipq_conv2d_run_relu": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "hipq_conv2d_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "hipq_conv2d_run_add": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_float, C.c_int,
                                       C.c_int, C.c_void_p, C.c_void_p]),
@@ -181,6 +182,13 @@ class Conv2d:
         if y is None:
             y = self.empty_output()
         check(lib().hipq_conv2d_run(self.handle, _ptr(x), _ptr(y), _ptr(acc), _stream()))
+        return y
+
+    def run_relu(self, x, y=None):
+        """y = max(conv(x), ozp) from a plan created without relu (include/hipq.h: hipq_conv2d_run_relu)."""
+        if y is None:
+            y = self.empty_output()
+        check(lib().hipq_conv2d_run_relu(self.handle, _ptr(x), _ptr(y), _stream()))
         return y
 
     def run_add(self, x, residual, residual_first, res_alpha, res_zp, oalpha, ozp, y, obits=8):

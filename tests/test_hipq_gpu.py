@@ -337,6 +337,35 @@ def test_conv_plan_variants_are_bit_identical():
         plan.select(0, 5)
 
 
+def test_relu_decided_at_run_time():
+    """hipq_conv2d_run_relu on a plan created without relu == a plan created with relu == convolution, then the relu
+    operator with the convolution's output scale on both sides; every kernel family, obits below 8 included."""
+    rng = np.random.default_rng(47)
+    kerns = set()
+    #         N, C,  H,  W,  K,  R, pad, stride, group
+    shapes = [(2, 64, 12, 12, 64, 3, 1, 1, 1), (1, 32, 9, 9, 96, 1, 0, 1, 1), (2, 256, 7, 7, 128, 1, 0, 1, 1), (1, 3, 20, 20, 32, 3, 1, 2, 1),
+              (2, 48, 10, 10, 48, 3, 1, 1, 48), (1, 32, 9, 9, 32, 3, 1, 2, 32), (1, 24, 7, 7, 24, 5, 2, 1, 24), (1, 16, 8, 8, 32, 3, 1, 1, 4)]
+    for N, C, H, W, K, R, pad, st, g in shapes:
+        x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+        w = rng.integers(0, 256, (K, C // g, R, R), dtype=np.uint8)
+        b = rng.integers(-20000, 20000, K).astype(np.int32)
+        for obits, ozp in ((8, 40), (8, 0), (7, 100), (4, 200)):
+            q = (rand_q(rng), int(rng.integers(0, 256)), rand_q(rng), 128, rand_q(rng, 1e-2, 0.5), ozp)
+            plain = hipq.Conv2d(x.shape, w, b, pad, st, g, *q, obits=obits)
+            fused = hipq.Conv2d(x.shape, w, b, pad, st, g, *q, obits=obits, relu=True)
+            kerns.add(plain.kernel)
+            xd = hipq.to_device_nhwc(x)
+            want = orc.relu_u8(orc.conv2d_u8(x, w, b, pad, st, g, *q, obits=obits), q[4], ozp, q[4], ozp, obits)
+            assert np.array_equal(hipq.from_device_nhwc(plain.run_relu(xd), K), want), (plain.kernel, obits, ozp)
+            assert np.array_equal(hipq.from_device_nhwc(fused(xd), K), want), (fused.kernel, obits, ozp)
+    assert any("halo" in k for k in kerns) and any("pointwise" in k for k in kerns) and any("_c4" in k for k in kerns)
+    assert any("depthwise3x3" in k for k in kerns) and "conv_depthwise_u8" in kerns and "conv_direct_u8" in kerns
+    p8 = hipq.Conv2d((1, 16, 4, 4), rng.integers(-128, 128, (16, 16, 1, 1), dtype=np.int8), None, 0, 1, 1, 0.1, 0, 0.1, 0, 0.1, 0,
+                     dtype=hipq.DTYPE_I8)
+    with pytest.raises(hipq.HipqError, match="uint8 plans only"):
+        p8.run_relu(hipq.to_device_nhwc(np.zeros((1, 16, 4, 4), np.int8)))
+
+
 def test_conv3x3_halo_kernel_matches_the_streaming_kernel_and_the_oracle():
     """3x3 / stride 1 / pad 1 layers load a pixel tile with its halo once and read the nine taps from LDS: every tile
     shape, one and several channel slabs, images narrower and wider than a tile, several images per tile (taps must

@@ -174,6 +174,36 @@ def test_convolution_and_add_run_as_one_kernel(own_rt):
     ws.delete()
 
 
+def test_convolution_and_relu_run_as_one_kernel(own_rt):
+    """A convolution whose output only a relu with the same scale and zero point on both sides reads leaves its launch
+    to that relu (the clamp moves into the convolution's epilogue); other relus run as operators of their own."""
+    import ctypes as C
+    from oracle import orc
+    fused = own_rt.libs[1].hip_module_fused_relus
+    fused.restype = C.c_long
+    ws = own_rt.workspace("hip")
+    rng = np.random.default_rng(22)
+    for (Cc, K, R, pad, g) in ((32, 96, 1, 0, 1), (48, 48, 3, 1, 48), (64, 64, 3, 1, 1)):
+        x = rng.integers(0, 256, (2, Cc, 10, 9), dtype=np.uint8)
+        w = rng.integers(0, 256, (K, Cc // g, R, R), dtype=np.uint8)
+        b = rng.integers(-5000, 5000, K).astype(np.int32)
+        q = dict(ialpha=0.031, izp=77, walpha=0.0042, wzp=128, oalpha=0.09, ozp=60)
+        want_c = orc.conv2d_u8(x, w, b, pad, 1, g, 0.031, 77, 0.0042, 128, 0.09, 60)
+        for same in (True, False):
+            conv = ws.conv2d(ws.tensor(x), ws.tensor(w), ws.tensor(b), pad, 1, g, q).prepare()
+            qr = dict(ialpha=0.09, izp=60, oalpha=0.09 if same else 0.05, ozp=60 if same else 3)
+            relu = ws.relu(conv.output(0), qr).prepare()
+            n0 = fused()
+            conv.run()
+            relu.run()
+            assert same_bits(relu.output(0).numpy(), orc.relu_u8(want_c, 0.09, 60, qr["oalpha"], qr["ozp"])), (Cc, K, same)
+            assert fused() == n0 + (1 if same else 0)
+            assert same_bits(conv.output(0).numpy(), want_c)
+            relu.delete()
+            conv.delete()
+    ws.delete()
+
+
 def test_concat_softmax_through_the_op_api(own_rt):
     import refrun
     from oracle import orc
