@@ -165,6 +165,8 @@ void conv_launch_plain(void *ctx)
     HIPM_HIPQ(hipq_conv2d_run(c->plan, in_ptr(op, 0), ym->dev, nullptr, op_stream(op)));
 }
 
+bool eltwise_is_plain_sum(const op_t *op); // two inputs, SUM, unit coefficients: computes what add computes
+
 // 1: the only reader of the convolution's output is an add or a relu of this workspace that can take over the launch
 bool sole_reader_fuses(op_t *op)
 {
@@ -182,8 +184,8 @@ bool sole_reader_fuses(op_t *op)
     if (r->entry->tp == &op_relu_tp)
         return true; // any plan runs with the ReLU clamp (hipq_conv2d_run_relu)
     // hipq_conv2d_run_add exists for the MFMA plans
-    return r->entry->tp == &op_add_tp && r->input_size == 2 && r->input_tensors[0]->mem != r->input_tensors[1]->mem
-        && strncmp(hipq_conv2d_plan_kernel(c->plan), "conv_mfma", 9) == 0;
+    return (r->entry->tp == &op_add_tp || eltwise_is_plain_sum(r)) && r->input_size == 2
+        && r->input_tensors[0]->mem != r->input_tensors[1]->mem && strncmp(hipq_conv2d_plan_kernel(c->plan), "conv_mfma", 9) == 0;
 }
 
 void conv_run(op_t *op)
@@ -326,7 +328,18 @@ void add_config(op_t *op)
     HIPM_CHECK(e->qi.n >= 2);
 }
 
-void add_run(op_t *op)
+// A two-input SUM with unit coefficients gives add's bytes on the same inputs (eltwise.c:137-271 against add.c:83-148:
+// the oracle's two restatements, both pinned against the reference, agree on every case tried), so it takes the same
+// fused path.
+bool eltwise_is_plain_sum(const op_t *op)
+{
+    const ew_op_t *e = reinterpret_cast<const ew_op_t *>(op);
+    return op->entry->tp == &op_eltwise_tp && op->input_size == 2 && e->operation == SETTING_ELTWISE_OP_SUM && e->coeff != nullptr
+        && e->coeff[0] == 1.0f && e->coeff[1] == 1.0f;
+}
+
+// the add (or plain two-input SUM) `op` as the epilogue of the convolution that left it its launch; false: run it plainly
+bool run_fused_into_convolution(op_t *op)
 {
     ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
     for (int i = 0; i < 2; ++i) {
@@ -345,10 +358,18 @@ void add_run(op_t *op)
         if (hipq_conv2d_run_add(c->plan, x, res, o == 0, e->qi.alpha[o], e->qi.zp[o], e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0],
                                 out_ptr(op), op_stream(op)) == 0) {
             ++g_fused_adds;
-            return; // the convolution's own output stays unwritten; its hook stays for whoever asks
+            return true; // the convolution's own output stays unwritten; its hook stays for whoever asks
         }
-        break;      // parameters outside the fused kernel's range: the plain path below settles the hook
+        break; // parameters outside the fused kernel's range: the caller's plain path settles the hook
     }
+    return false;
+}
+
+void add_run(op_t *op)
+{
+    ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    if (run_fused_into_convolution(op))
+        return;
     HIPM_HIPQ(hipq_add_u8(in_ptr(op, 0), in_ptr(op, 1), out_ptr(op), e->bytes, e->qi.alpha[0], e->qi.zp[0], e->qi.alpha[1],
                           e->qi.zp[1], e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0], op_stream(op)));
 }
@@ -382,6 +403,8 @@ void eltwise_config(op_t *op)
 void eltwise_run(op_t *op)
 {
     ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    if (eltwise_is_plain_sum(op) && run_fused_into_convolution(op))
+        return;
     const void *ins[HIPQ_MAX_ELTWISE_INPUTS];
     for (size_t i = 0; i < op->input_size; ++i)
         ins[i] = in_ptr(op, (int)i);

@@ -174,6 +174,37 @@ def test_convolution_and_add_run_as_one_kernel(own_rt):
     ws.delete()
 
 
+def test_plain_eltwise_sum_fuses_like_add(own_rt):
+    """Caffe-style graphs carry the residual sum as Eltwise(SUM): two inputs with unit coefficients give add's bytes and
+    take the same fused path; other coefficients, MAX and three inputs run as operators of their own."""
+    import ctypes as C
+    from oracle import orc
+    fused = own_rt.libs[1].hip_module_fused_adds
+    fused.restype = C.c_long
+    ws = own_rt.workspace("hip")
+    rng = np.random.default_rng(23)
+    x = rng.integers(0, 256, (2, 128, 7, 7), dtype=np.uint8)
+    w = rng.integers(0, 256, (256, 128, 1, 1), dtype=np.uint8)
+    r = rng.integers(0, 256, (2, 256, 7, 7), dtype=np.uint8)
+    q = dict(ialpha=0.031, izp=77, walpha=0.0042, wzp=128, oalpha=0.09, ozp=13)
+    want_c = orc.conv2d_u8(x, w, None, 0, 1, 1, 0.031, 77, 0.0042, 128, 0.09, 13)
+    qa = dict(ialpha=[0.05, 0.09], izp=[200, 13], oalpha=0.12, ozp=31)
+    for coeff, op, expect in ((None, 1, 1), ([1.0, 1.0], 1, 1), ([1.0, 0.5], 1, 0), (None, 2, 0)):
+        conv = ws.conv2d(ws.tensor(x), ws.tensor(w), None, 0, 1, 1, q).prepare()
+        elt = ws.eltwise([ws.tensor(r), conv.output(0)], qa, operation=op, coeff=coeff).prepare()
+        n0 = fused()
+        conv.run()
+        elt.run()
+        want = orc.eltwise_u8([r, want_c], [0.05, 0.09], [200, 13], 0.12, 31, operation=op, coeff=coeff)
+        assert same_bits(elt.output(0).numpy(), want), (coeff, op)
+        assert fused() == n0 + expect, (coeff, op)
+        if expect:
+            assert same_bits(want, orc.add_u8(r, want_c, 0.05, 200, 0.09, 13, 0.12, 31))
+        elt.delete()
+        conv.delete()
+    ws.delete()
+
+
 def test_convolution_and_relu_run_as_one_kernel(own_rt):
     """A convolution whose output only a relu with the same scale and zero point on both sides reads leaves its launch
     to that relu (the clamp moves into the convolution's epilogue); other relus run as operators of their own."""
