@@ -1504,7 +1504,7 @@ extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t
         }
         pad_off = wbuf.size();
         wbuf.resize(pad_off + 64, (uint8_t)pad_byte); // source of out-of-image taps
-        static const bool no_halo = getenv("HIPQ_NO_HALO") != nullptr; // for A/B measurements
+        static const bool no_halo = getenv("HIPQ_NO_SPECIAL_KERNELS") != nullptr; // A/B measurements: tile kernels only
         p->special = no_halo ? 0 : 1;
         set_mfma_name(p, smallc);
     } else if (!sgn && d.group == d.C && d.K == d.C && d.in_cs == d.out_cs && d.R == 3 && d.S == 3 && d.stride_h == d.stride_w
