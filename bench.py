@@ -103,6 +103,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--no-fuse", action="store_true", help="run every residual add as its own kernel")
+    ap.add_argument("--no-branches", action="store_true",
+                    help="skip the extra measurement of the pass as two half-batch branches of one HIP graph")
     ap.add_argument("--layers", action="store_true", help="print a per-layer table to stderr")
     ap.add_argument("--tune", action="store_true",
                     help="before timing, let the executor search tile shape / load stages per convolution inside the network "
@@ -193,6 +195,21 @@ def main():
             print("%-12s %-28s %-22s %8.1f us %s %8.1f GB/s" % (s["label"], s["kernel"], shape, t * 1e3, tp,
                                                                  s["bytes"] / (t * 1e-3) / 1e9), file=sys.stderr)
 
+    # ---- the same pass as two half-batch branches of one graph (reported beside `value`, never as `value`: the
+    # roofline below is that of kernels launched one at a time at the full batch) --------------------------------
+    branched = None
+    if not args.no_branches and not args.no_graph and args.batch >= 2:
+        from nart_amd.runner import BranchedExecutor
+        out_t = ex.buf[case.output.name]
+        whole = out_t.clone()
+        br = BranchedExecutor(ex, build, 2)
+        out_t.zero_()
+        br.capture()
+        bms, _ = time_steps(br.replay, args.steps, args.warmup)
+        branched = {"branches": 2, "ms_per_step": round(bms, 4), "value": round(args.batch / (bms * 1e-3), 1),
+                    "output_equals_single_branch": bool(torch.equal(out_t, whole))}
+        del br
+
     unit = "images/s"
     value = args.batch / (ms * 1e-3)
     res = {"metric": "ResNet-50-int8 images/sec @bs64; int8 conv TOPS (% of MFMA i8 peak)" if args.workload == "resnet50"
@@ -205,6 +222,8 @@ def main():
                       "conv_fc_gop_per_step": round(case.conv_ops() / 1e9, 2)},
            "conv_tops_whole_step": round(case.conv_ops() / (ms * 1e-3) / 1e12, 2),
            "roofline": roof, "kernel_families": families}
+    if branched is not None:
+        res["two_branch_graph"] = branched
     if not args.no_cpu:
         i0 = {"x": x[:1], "y": y[:1]}
         res["cpu_baseline"] = cpu_baseline(build, i0)

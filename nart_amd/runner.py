@@ -15,8 +15,12 @@ class HipqExecutor:
     """fuse_add: a convolution whose only consumer is a two-input add is launched with the add fused into its
     epilogue (hipq_conv2d_run_add); the convolution's own output tensor is then never materialised."""
 
-    def __init__(self, case, fuse_add=False):
+    def __init__(self, case, fuse_add=False, share=None):
+        """share = (parent, first): every tensor of this executor is the batch slice [first, first + N) of the
+        parent executor's tensor of the same name (the batch is the outermost dimension of both layouts, so the
+        slice is contiguous).  The parent runs the same network at a larger batch; nothing is allocated here."""
         self.case = case
+        self.share = share
         self.fused = {}      # conv output name -> the add node that absorbs it
         if fuse_add:
             uses = {}
@@ -36,19 +40,12 @@ class HipqExecutor:
         self.graph = None
         T = case.tensors
         inp = case.input
-        if inp.dtype == "f32":
-            self.buf[inp.name] = torch.zeros(inp.shape, dtype=torch.float32, device="cuda")
-        else:
-            N, C, H, W = inp.shape
-            self.buf[inp.name] = torch.zeros((N, H, W, hipq.channel_stride(C)), dtype=torch.uint8, device="cuda")
+        self.buf[inp.name] = self._tensor(inp)
         for node in case.nodes:
             y = T[node.output]
             xs = [T[i] for i in node.inputs]
             N, C, H, W = y.shape
-            if y.dtype == "f32":
-                out = torch.zeros(y.shape, dtype=torch.float32, device="cuda")
-            else:
-                out = torch.zeros((N, H, W, hipq.channel_stride(C)), dtype=torch.uint8, device="cuda")
+            out = self._tensor(y)
             self.buf[y.name] = out
             ins = [self.buf.get(i) for i in node.inputs]
             a = node.attrs
@@ -71,9 +68,11 @@ class HipqExecutor:
                     res_first = add.inputs[0] == other
                     ot, st = T[other], T[add.output]
                     self._pending[id(add)] = (plan, ins[0], other, res_first, ot, st, nbytes + int(np.prod(y.shape)))
-                    del self.buf[y.name]  # never materialised
+                    self.buf.pop(y.name, None)  # never materialised
                     continue
                 self.fused.pop(node.output, None)
+                if out is None:
+                    raise RuntimeError("shared executor: %s is fused away in the parent but not here" % y.name)
                 fn = (lambda p=plan, i=ins[0], o=out: p(i, o))
                 self._add(node, plan.kernel, fn, plan.ops, nbytes)
                 self.steps[-1]["plan"] = plan
@@ -111,6 +110,16 @@ class HipqExecutor:
                 self._add(node, "add_u8_kernel", fn, 0, 3 * int(np.prod(y.shape)))
             else:
                 raise ValueError("unknown node kind " + node.kind)
+
+    def _tensor(self, t):
+        N, C, H, W = t.shape
+        if self.share is not None:
+            parent, first = self.share
+            whole = parent.buf.get(t.name)
+            return None if whole is None else whole[first:first + N]  # None: fused away in the parent as well
+        if t.dtype == "f32":
+            return torch.zeros(t.shape, dtype=torch.float32, device="cuda")
+        return torch.zeros((N, H, W, hipq.channel_stride(C)), dtype=torch.uint8, device="cuda")
 
     def _add(self, node, kernel, fn, ops, nbytes):
         self.steps.append({"label": node.output, "kind": node.kind, "kernel": kernel, "fn": fn, "ops": ops,
@@ -197,6 +206,56 @@ class HipqExecutor:
 
     def capture(self):
         """Record one pass into a HIP graph (kernel nodes only: no memsets, no allocations)."""
+        self.run()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            self.run()
+        self.graph = g
+        return g
+
+    def replay(self):
+        self.graph.replay()
+
+
+class BranchedExecutor:
+    """One pass over a batch run as `branches` part-batches side by side, each on a stream of its own.
+
+    Every operator of the path treats the images of a batch independently, and the batch is the outermost dimension
+    of every device tensor, so a part-batch is a contiguous slice of the whole batch's tensors: the part executors
+    share the parent's buffers (HipqExecutor(share=...)) and the parent's input / output stay the interface.
+    Two chains of kernels that do not depend on each other let the GPU start one chain's next kernel while the other
+    chain's current kernel drains its last work-groups, and the chains drift apart so that kernels bound by
+    different units (HBM, LDS, matrix cores) overlap; the arithmetic, and so every output byte, is unchanged.
+    The reference has no counterpart: its parade is one sequential op list (art/src/parade.c:184-197)."""
+
+    def __init__(self, parent, build, branches=2):
+        N = parent.case.input.shape[0]
+        if branches < 2 or N < branches:
+            raise ValueError("branches must be between 2 and the batch size")
+        self.parent = parent
+        bounds = [N * b // branches for b in range(branches + 1)]
+        self.parts = [HipqExecutor(build(hi - lo), fuse_add=bool(parent.fused), share=(parent, lo))
+                      for lo, hi in zip(bounds[:-1], bounds[1:])]
+        for p in self.parts:
+            if [s["label"] for s in p.steps] != [s["label"] for s in parent.steps]:
+                raise RuntimeError("part-batch executor launches a different operator list than its parent")
+        self.side = [torch.cuda.Stream() for _ in self.parts[1:]]  # default priority
+        self.graph = None
+
+    def run(self):
+        cur = torch.cuda.current_stream()
+        for s in self.side:
+            s.wait_stream(cur)
+        self.parts[0].run()
+        for s, p in zip(self.side, self.parts[1:]):
+            with torch.cuda.stream(s):
+                p.run()
+        for s in self.side:
+            cur.wait_stream(s)
+
+    def capture(self):
+        """One HIP graph with a branch per part-batch (kernel nodes and the fork / join dependencies only)."""
         self.run()
         torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()

@@ -8,7 +8,7 @@ pytestmark = pytest.mark.gpu
 torch = pytest.importorskip("torch")
 
 from nart_amd import cases  # noqa: E402
-from nart_amd.runner import HipqExecutor  # noqa: E402
+from nart_amd.runner import BranchedExecutor, HipqExecutor  # noqa: E402
 
 from oracle import casecpu as case_oracle  # noqa: E402
 
@@ -78,6 +78,29 @@ def test_graph_replay_matches_eager():
         for n in case.nodes:
             got = ex.fetch(n.output)
             assert np.array_equal(got.view(np.uint8), eager[n.output].view(np.uint8)), (seed, n.output)
+
+
+@pytest.mark.parametrize("build,batch,branches", [(lambda n: cases.resnet50(N=n, hw=64), 5, 2),
+                                                   (lambda n: cases.mobilenet_v2(N=n, hw=96), 4, 3)],
+                         ids=["resnet50_n5_two", "mobilenetv2_n4_three"])
+def test_part_batches_on_streams_match_the_oracle(build, batch, branches):
+    """The batch run as concurrent part-batches (slices of the same buffers, one stream each, eagerly and as one
+    HIP graph with a branch per part) must leave exactly the oracle's bytes in every tensor, replay after replay."""
+    case = build(batch)
+    ex = HipqExecutor(case, fuse_add=True)
+    br = BranchedExecutor(ex, build, branches)
+    assert [p.case.input.shape[0] for p in br.parts] == ([2, 3] if branches == 2 else [1, 1, 2])
+    br.capture()
+    for seed, how in ((5, br.run), (6, br.replay), (7, br.replay)):
+        x = case_oracle.random_input(case, seed=seed)
+        vals = case_oracle.run_case(case, x)
+        for t in ex.buf.values():
+            t.zero_()
+        ex.set_input(x)
+        torch.cuda.synchronize()
+        how()
+        torch.cuda.synchronize()
+        compare_all(case, ex, vals)
 
 
 def test_batch64_properties_resnet50_stage():
