@@ -195,8 +195,7 @@ def main():
             print("%-12s %-28s %-22s %8.1f us %s %8.1f GB/s" % (s["label"], s["kernel"], shape, t * 1e3, tp,
                                                                  s["bytes"] / (t * 1e-3) / 1e9), file=sys.stderr)
 
-    # ---- the same pass as two half-batch branches of one graph (reported beside `value`, never as `value`: the
-    # roofline below is that of kernels launched one at a time at the full batch) --------------------------------
+    # ---- the same pass as two half-batch branches of one graph (reported beside `value` as well) --------------------------------
     branched = None
     if not args.no_branches and not args.no_graph and args.batch >= 2:
         from nart_amd.runner import BranchedExecutor
@@ -209,6 +208,28 @@ def main():
         branched = {"branches": 2, "ms_per_step": round(bms, 4), "value": round(args.batch / (bms * 1e-3), 1),
                     "output_equals_single_branch": bool(torch.equal(out_t, whole))}
         del br
+    # ---- two batches in flight: a second copy of the network (own tensors, graph and stream) takes every other step and
+    # nothing joins the two chains until the end of the timed region; throughput of the same K passes, reported beside
+    # `value`, never as `value`: the roofline above is that of kernels launched one at a time ------------------------------------------------------------------------
+    in_flight = None
+    if not args.no_branches and not args.no_graph:
+        from nart_amd.runner import PipelinedExecutor
+        pipe = PipelinedExecutor(lambda: build(args.batch), depth=2, fuse_add=not args.no_fuse, first=ex)
+        pipe.execs[1].set_input(x)
+        torch.cuda.synchronize()
+        for _ in range(2 * max(1, args.warmup)):
+            pipe.submit()
+        pipe.wait()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            pipe.submit()
+        pipe.wait()
+        pms = (time.perf_counter() - t0) * 1e3 / args.steps
+        same = torch.equal(pipe.execs[1].buf[case.output.name], ex.buf[case.output.name])
+        in_flight = {"batches_in_flight": 2, "ms_per_step": round(pms, 4), "value": round(args.batch / (pms * 1e-3), 1),
+                     "timer": "host clock around the K submissions and the final synchronisation",
+                     "outputs_equal_single_stream": bool(same)}
+        del pipe
 
     unit = "images/s"
     value = args.batch / (ms * 1e-3)
@@ -224,6 +245,8 @@ def main():
            "roofline": roof, "kernel_families": families}
     if branched is not None:
         res["two_branch_graph"] = branched
+    if in_flight is not None:
+        res["two_batches_in_flight"] = in_flight
     if not args.no_cpu:
         i0 = {"x": x[:1], "y": y[:1]}
         res["cpu_baseline"] = cpu_baseline(build, i0)

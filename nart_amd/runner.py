@@ -5,6 +5,8 @@ This is the Python-side counterpart of the reference's parade: a flat list of pr
 pass into a HIP graph so that a launch-bound step replays without per-kernel host overhead.
 All device tensors are channels-last with padded channel stride (see include/hipq.h).
 """
+import time
+
 import numpy as np
 import torch
 
@@ -266,3 +268,60 @@ class BranchedExecutor:
 
     def replay(self):
         self.graph.replay()
+
+
+class PipelinedExecutor:
+    """`depth` independent copies of one network (own tensors, own HIP graph, own stream each) that take consecutive
+    batches in turn, so that `depth` batches are in flight at once: `submit()` replays the next copy's graph and returns
+    its executor without waiting; the caller synchronises (`wait()`) before it reads a copy's output or refills its
+    input.  One chain of dependent kernels leaves the GPU partly idle while each kernel ramps up and drains; a second,
+    unrelated chain fills those gaps, and because the chains are never joined they drift into complementary phases
+    (an HBM-bound layer of one batch beside a latency-bound layer of the other).  More than two chains add nothing.
+    The reference has no counterpart inside one parade; its equivalent is two parades on two workspaces, which
+    nart_promark -p 2 drives the same way through the `hip` module."""
+
+    def __init__(self, build, depth=2, fuse_add=True, first=None):
+        if depth < 1:
+            raise ValueError("depth must be at least 1")
+        self.execs = [first if (k == 0 and first is not None) else HipqExecutor(build(), fuse_add=fuse_add)
+                      for k in range(depth)]
+        self.turn = 0
+        cur = torch.cuda.current_stream()
+        for ex in self.execs:
+            if ex.graph is None:
+                ex.capture()
+        # The runtime multiplexes HIP streams over a few hardware queues (4 by default), and two streams that share a
+        # queue run their kernels one after the other.  Which queue a new stream gets depends on how many streams the
+        # process created before, so with two copies a few candidate partners are timed and the best one is kept.
+        cands = [torch.cuda.Stream() for _ in range(depth if depth != 2 else 4)]  # default priority
+        for st in cands:
+            st.wait_stream(cur)
+        self.streams = cands[:depth]
+        if depth == 2:
+            best = None
+            for partner in cands[1:]:
+                self.streams = [cands[0], partner]
+                self._burst(4)
+                t0 = time.perf_counter()
+                self._burst(8)
+                t = time.perf_counter() - t0
+                if best is None or t < best[0]:
+                    best = (t, partner)
+            self.streams = [cands[0], best[1]]
+            self.turn = 0
+
+    def _burst(self, n):
+        for _ in range(n):
+            self.submit()
+        self.wait()
+
+    def submit(self):
+        k = self.turn
+        self.turn = (k + 1) % len(self.execs)
+        with torch.cuda.stream(self.streams[k]):
+            self.execs[k].replay()
+        return self.execs[k]
+
+    def wait(self):
+        for st in self.streams:
+            st.synchronize()

@@ -8,7 +8,7 @@ pytestmark = pytest.mark.gpu
 torch = pytest.importorskip("torch")
 
 from nart_amd import cases  # noqa: E402
-from nart_amd.runner import BranchedExecutor, HipqExecutor  # noqa: E402
+from nart_amd.runner import BranchedExecutor, HipqExecutor, PipelinedExecutor  # noqa: E402
 
 from oracle import casecpu as case_oracle  # noqa: E402
 
@@ -101,6 +101,30 @@ def test_part_batches_on_streams_match_the_oracle(build, batch, branches):
         how()
         torch.cuda.synchronize()
         compare_all(case, ex, vals)
+
+
+def test_two_batches_in_flight_match_the_oracle():
+    """Two copies of the network on two streams take consecutive batches without waiting for each other; every
+    batch's output must equal the oracle's, whichever copy and whichever overlap it ran under."""
+    build = lambda: cases.resnet18(N=3, hw=96)  # noqa: E731
+    pipe = PipelinedExecutor(build, depth=2)
+    case = pipe.execs[0].case
+    xs = [case_oracle.random_input(case, seed=s) for s in (11, 12, 13, 14)]
+    want = [case_oracle.run_case(case, x)[case.output.name] for x in xs]
+    for lo in (0, 2):  # two rounds: the second one re-uses both copies
+        used = []
+        for j, x in enumerate(xs[lo:lo + 2]):
+            ex = pipe.execs[(pipe.turn + j) % 2]
+            ex.buf[case.output.name].zero_()
+            ex.set_input(x)
+            torch.cuda.synchronize()  # inputs are written on the current stream, the copies run on their own
+            used.append(ex)
+        for _ in used:
+            pipe.submit()
+        pipe.wait()
+        for ex, w in zip(used, want[lo:lo + 2]):
+            got = ex.output()
+            assert np.array_equal(got.view(np.uint8), w.view(np.uint8))
 
 
 def test_batch64_properties_resnet50_stage():
