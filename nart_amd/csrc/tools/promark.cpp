@@ -13,6 +13,9 @@
 //   -y  time the host<->device copies of inputs and outputs as well
 //   -s  after timing: load the -i files into the inputs (in order), run once, write every output tensor to
 //       nart-out-<tensor name with '/' -> '_'>.bin
+//   -p  (not in the reference) after the timed runs, load the engine p - 1 more times, every copy into workspaces of its
+//       own, and time run_times passes handed to the copies in turn without waiting in between: p batches in flight.
+//       A GPU workspace owns a stream, so the copies' kernels overlap; the line printed is the time per batch.
 //
 // Difference from the reference, on purpose: GPU modules run asynchronously, and the reference's timed region
 // (promark.cpp:467-476) only waits for the device when -y makes it read an output.  This runner also looks for an
@@ -336,7 +339,7 @@ double now_ms()
 
 int usage(const char *argv0)
 {
-    fprintf(stderr, "Usage: \n%s -m model [-c config] [-n run_times] [{-i blob.bin}] [-s] [-d] [-b batch_size] [-r name:d0,d1,...] [-y]\n",
+    fprintf(stderr, "Usage: \n%s -m model [-c config] [-n run_times] [{-i blob.bin}] [-s] [-d] [-b batch_size] [-r name:d0,d1,...] [-y] [-p parades_in_flight]\n",
             argv0);
     return 1;
 }
@@ -348,12 +351,12 @@ int main(int argc, char *argv[])
     if (argc == 1)
         return usage(argv[0]);
     std::string model_file, config_file;
-    int run_times = 10, batch_size = -1;
+    int run_times = 10, batch_size = -1, in_flight = 1;
     std::vector<std::string> inputs;
     bool save_flag = false, randomized = false, with_copies = false;
     std::map<std::string, std::vector<int>> shape_by_name;
     int ch;
-    while ((ch = getopt(argc, argv, "i:sm:c:n:b:r:dy")) != -1) {
+    while ((ch = getopt(argc, argv, "i:sm:c:n:b:r:dyp:")) != -1) {
         switch (ch) {
         case 'm': model_file = optarg; break;
         case 'c': config_file = optarg; break;
@@ -363,6 +366,7 @@ int main(int argc, char *argv[])
         case 's': save_flag = true; break;
         case 'd': randomized = true; break;
         case 'y': with_copies = true; break;
+        case 'p': in_flight = atoi(optarg); break;
         case 'r': {
             const std::string arg(optarg);
             const size_t pos = arg.find(':');
@@ -384,7 +388,7 @@ int main(int argc, char *argv[])
         default: return usage(argv[0]);
         }
     }
-    if (model_file.empty() || run_times < 0)
+    if (model_file.empty() || run_times < 0 || in_flight < 1 || in_flight > 8)
         return usage(argv[0]);
     printf("parse args ...\n  modelfile  : %s\n  config_file: %s\n  run_time   : %d\n\n", model_file.c_str(), config_file.c_str(),
            run_times);
@@ -418,27 +422,30 @@ int main(int argc, char *argv[])
         return 1;
     }
 
-    if (batch_size > 0) {
-        for (size_t i = 0; i < input_cnt; i++)
-            in_t[i]->shape.dim[in_t[i]->shape.batch_axis] = (uint32_t)batch_size;
-        if (!parade_apply_reshape(parade)) {
-            fprintf(stderr, "Reshape parade failed\n");
-            return 1;
+    auto reshape = [&](parade_t *pa, size_t n_in, tensor_array_t tin) {
+        if (batch_size > 0) {
+            for (size_t i = 0; i < n_in; i++)
+                tin[i]->shape.dim[tin[i]->shape.batch_axis] = (uint32_t)batch_size;
+            if (!parade_apply_reshape(pa))
+                return false;
         }
-    }
-    if (!shape_by_name.empty()) {
-        for (size_t i = 0; i < input_cnt; i++) {
-            auto it = in_t[i]->name ? shape_by_name.find(in_t[i]->name) : shape_by_name.end();
-            if (it == shape_by_name.end())
-                continue;
-            in_t[i]->shape.dim_size = (int32_t)it->second.size();
-            for (size_t d = 0; d < it->second.size() && d < 8; d++)
-                in_t[i]->shape.dim[d] = (uint32_t)it->second[d];
+        if (!shape_by_name.empty()) {
+            for (size_t i = 0; i < n_in; i++) {
+                auto it = tin[i]->name ? shape_by_name.find(tin[i]->name) : shape_by_name.end();
+                if (it == shape_by_name.end())
+                    continue;
+                tin[i]->shape.dim_size = (int32_t)it->second.size();
+                for (size_t d = 0; d < it->second.size() && d < 8; d++)
+                    tin[i]->shape.dim[d] = (uint32_t)it->second[d];
+            }
+            if (!parade_apply_reshape(pa))
+                return false;
         }
-        if (!parade_apply_reshape(parade)) {
-            fprintf(stderr, "Reshape parade failed\n");
-            return 1;
-        }
+        return true;
+    };
+    if (!reshape(parade, input_cnt, in_t)) {
+        fprintf(stderr, "Reshape parade failed\n");
+        return 1;
     }
     print_tensors("input tensors", input_cnt, in_t);
     print_tensors("output tensors", output_cnt, out_t);
@@ -491,6 +498,46 @@ int main(int argc, char *argv[])
     if (run_times > 0)
         printf("\nTest finised, average cost: %gms\n\n", total / run_times);
 
+    // ---- -p: several parades in flight -----------------------------------------------------------------------
+    std::vector<Context> more_ctx((size_t)in_flight - 1);
+    std::vector<parade_t *> parades(1, parade);
+    for (int k = 1; k < in_flight; k++) {
+        Context &c = more_ctx[(size_t)k - 1];
+        parade_t *pa = init_modules(config, c) ? load_model(model_file.c_str(), c) : nullptr;
+        size_t n_in = 0;
+        tensor_array_t tin = nullptr;
+        if (pa == nullptr || !parade_get_input_tensors(pa, &n_in, &tin) || !reshape(pa, n_in, tin)) {
+            fprintf(stderr, "loading copy %d of the engine failed\n", k);
+            return 1;
+        }
+        for (size_t i = 0; i < n_in; i++) {
+            memset(mem_cpu_data(tin[i]->mem), 0, tensor_bytes(tin[i]));
+            (void)mem_data(tin[i]->mem); // upload outside the timed region
+        }
+        parade_run(pa);
+        parades.push_back(pa);
+    }
+    if (in_flight > 1 && run_times > 0) {
+        auto sync_every = [&]() {
+            sync_all();
+            for (Context &c : more_ctx)
+                for (size_t i = 0; i + 1 < c.ws.size(); i++)
+                    if (c.sync[i])
+                        c.sync[i](c.ws[i]);
+        };
+        for (size_t j = 0; j < input_cnt; j++)
+            (void)mem_data(in_t[j]->mem);
+        for (int it = 0; it < 2 * in_flight; it++)
+            parade_run(parades[(size_t)(it % in_flight)]);
+        sync_every();
+        const double t0 = now_ms();
+        for (int it = 0; it < run_times; it++)
+            parade_run(parades[(size_t)(it % in_flight)]);
+        sync_every();
+        printf("%d parades in flight, %d passes: average cost per batch: %gms\n\n", in_flight, run_times,
+               (now_ms() - t0) / run_times);
+    }
+
     int rc = 0;
     if (save_flag) {
         if (inputs.size() != input_cnt) {
@@ -510,8 +557,12 @@ int main(int argc, char *argv[])
                 rc = 1;
         }
     }
-    parade_delete(parade);
+    for (parade_t *pa : parades)
+        parade_delete(pa);
     for (size_t i = 0; i + 1 < ctx.ws.size(); i++)
         workspace_delete(ctx.ws[i]);
+    for (Context &c : more_ctx)
+        for (size_t i = 0; i + 1 < c.ws.size(); i++)
+            workspace_delete(c.ws[i]);
     return rc;
 }

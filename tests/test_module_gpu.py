@@ -298,11 +298,12 @@ def test_command_line_runner(tmp_path):
     npdt = {"u8": np.uint8, "f32": np.float32}
     np.ascontiguousarray(x, npdt[big.input.dtype]).tofile(tmp_path / "in.bin")
     shown = {"u8": "UINT8", "f32": "FLOAT32"}[big.input.dtype] + " " + ", ".join(str(d) for d in big.input.shape)
-    for extra in ([], ["-y"], ["-d"]):
+    for extra in ([], ["-y"], ["-d"], ["-p", "2"]):
         r = subprocess.run([tool, "-m", "engine.bin", "-c", "cfg.json", "-n", "3", "-b", "3", "-i", "in.bin", "-s"] + extra,
                            cwd=tmp_path, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, timeout=300)
         assert r.returncode == 0, r.stderr[-2000:]
         assert "average cost" in r.stdout and "Process 2 : cost" in r.stdout and shown in r.stdout, r.stdout
+        assert ("2 parades in flight, 3 passes: average cost per batch" in r.stdout) == (extra == ["-p", "2"]), r.stdout
         name = "nart-out-" + case.output.name.replace("/", "_") + ".bin"
         got = np.fromfile(tmp_path / name, dtype=npdt[big.output.dtype]).reshape(big.output.shape)
         want = casecpu.run_case(big, x)[big.output.name]
