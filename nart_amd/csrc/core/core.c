@@ -731,9 +731,12 @@ static void rd_setting(op_t *op, buffer_t *b)
         }
         return;
     }
-    size_t count = (size_t)rd_i32(b);
+    int32_t count32 = rd_i32(b);
+    ART_CHECK(count32 >= 0);
+    size_t count = (size_t)count32;
     if (dtype == dtSTR) {
         char **strs = (char **)calloc(count ? count : 1, sizeof(char *));
+        ART_CHECK(strs != NULL);
         for (size_t i = 0; i < count; ++i)
             strs[i] = rd_string(b);
         ART_CHECK(op_setting_array_set(op, item, dtype, count, strs));
@@ -805,6 +808,7 @@ static parade_t *read_parade(buffer_t *b, const deserialize_param_t *param, uint
     size_t cur = 0;
 
     int32_t n_in = rd_i32(b);
+    ART_CHECK(n_in >= 0 && n_in <= n_tensors); /* every count below comes from the file: none may outrun the table */
     p->input_tensors = (tensor_t **)calloc((size_t)n_in + 1, sizeof(tensor_t *));
     for (int32_t i = 0; i < n_in; ++i) {
         tensor_t *t = rd_tensor_decl(b, param->input_mem_tp);
@@ -814,6 +818,7 @@ static parade_t *read_parade(buffer_t *b, const deserialize_param_t *param, uint
     }
 
     int32_t n_w = rd_i32(b);
+    ART_CHECK(n_w >= 0 && n_w <= n_tensors - n_in);
     p->weight_tensors = (tensor_t **)calloc((size_t)n_w + 1, sizeof(tensor_t *));
     for (int32_t i = 0; i < n_w; ++i) { /* weights carry their data inline; it is written through the host view */
         tensor_t *t = rd_tensor_decl(b, param->input_mem_tp);
@@ -827,6 +832,7 @@ static parade_t *read_parade(buffer_t *b, const deserialize_param_t *param, uint
     int32_t n_ops = rd_i32(b);
     for (int32_t i = 0; i < n_ops; ++i) {
         int32_t op_in = rd_i32(b), op_out = rd_i32(b);
+        ART_CHECK(op_in >= 0 && op_in <= 255 && op_out >= 0); /* workspace_new_op takes the input count as a byte */
         uint64_t code = rd_u64(b);
         tensor_t **ins = (tensor_t **)calloc((size_t)op_in + 1, sizeof(tensor_t *));
         for (int32_t j = 0; j < op_in; ++j) {
@@ -853,6 +859,7 @@ static parade_t *read_parade(buffer_t *b, const deserialize_param_t *param, uint
     }
 
     int32_t n_out = rd_i32(b);
+    ART_CHECK(n_out >= 0 && n_out <= n_tensors);
     p->output_tensors = (tensor_t **)calloc((size_t)n_out + 1, sizeof(tensor_t *));
     for (int32_t i = 0; i < n_out; ++i) {
         int32_t idx = rd_i32(b);

@@ -203,3 +203,52 @@ def test_workspace_creation_fails_loudly_without_gpu():
     rt = art.Runtime(os.path.join(LIB, "libart.so"), [os.path.join(LIB, "libart_module_hip.so")])
     with pytest.raises(AssertionError, match="workspace_new failed"):
         rt.workspace("hip")
+
+
+_MALFORMED_LOADER = r"""
+import ctypes as C, os, struct, sys
+sys.path.insert(0, sys.argv[1])
+from nart_amd import art, cases, engine
+rt = art.Runtime(os.path.join(sys.argv[1], "nart_amd", "lib", "libart.so"))
+data = bytearray(engine.write_engine(cases.single_fc(M=2, K=64, Nout=16)))
+off = 4 + 4 + struct.unpack_from("<i", data, 4)[0]   # version, name -> tensor_count
+n_tensors, n_in = struct.unpack_from("<ii", data, off)
+how = sys.argv[2]
+if how == "inputs_outrun_table":
+    struct.pack_into("<i", data, off, 0)             # a table of no tensors, one input declared
+elif how == "negative_inputs":
+    struct.pack_into("<i", data, off + 4, -3)
+elif how == "truncated":
+    del data[len(data) // 2:]
+pos = [0]
+READ = C.CFUNCTYPE(C.c_size_t, C.c_size_t, C.c_void_p, C.c_void_p)
+def read(sz, dst, _):
+    chunk = bytes(data[pos[0]:pos[0] + sz]); C.memmove(dst, chunk, len(chunk)); pos[0] += len(chunk); return len(chunk)
+cb = READ(read)
+class Param(C.Structure):
+    _fields_ = [("workspaces", C.POINTER(C.POINTER(art.workspace_t))), ("input_mem_tp", C.POINTER(art.mem_tp))]
+core = rt.core
+core.nart_buffer_new.restype = C.c_void_p; core.nart_buffer_new.argtypes = [C.c_size_t]
+core.buffer_set_buffer_read_func.argtypes = [C.c_void_p, READ, C.c_void_p]
+core.deserialize_parade.restype = C.c_void_p; core.deserialize_parade.argtypes = [C.c_void_p, C.POINTER(Param)]
+buf = core.nart_buffer_new(1 << 16)
+core.buffer_set_buffer_read_func(buf, cb, None)
+ws = (C.POINTER(art.workspace_t) * 1)(None)
+print("loading", how, flush=True)
+core.deserialize_parade(buf, C.byref(Param(ws, rt.cpu_mem_tp)))
+print("returned", flush=True)
+"""
+
+
+@pytest.mark.parametrize("how", ["inputs_outrun_table", "negative_inputs", "truncated"])
+def test_malformed_engine_file_aborts_instead_of_overrunning(how, tmp_path):
+    """Counts in an engine file are checked against the tensor table before anything is written through them; a file
+    that lies about them ends in the runtime's CHECK failure (abort, the reference's error behaviour:
+    art/include/art/log.h CHECK), never in a write past the table."""
+    import signal
+    import sys
+    script = tmp_path / "load.py"
+    script.write_text(_MALFORMED_LOADER)
+    r = subprocess.run([sys.executable, str(script), ROOT, how], stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=120)
+    assert b"loading" in r.stdout and b"returned" not in r.stdout
+    assert r.returncode == -signal.SIGABRT, (r.returncode, r.stderr[-500:])
