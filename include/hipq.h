@@ -102,15 +102,18 @@ const char *hipq_conv2d_plan_kernel(const hipq_conv2d_plan *plan);
  */
 int hipq_conv2d_plan_select(hipq_conv2d_plan *plan, int tile, int stages);
 /*
- * Tuning hook (no counterpart in the reference) for the two specialised MFMA kernels.  Halo-tile kernel (name
+ * Tuning hook (no counterpart in the reference) for the specialised MFMA kernels.  Halo-tile kernel (name
  * "..._halo"): 3x3 / stride 1 / pad 1 convolutions whose input channel stride is a multiple of 64 load each input tile with
  * its halo once and form the nine taps from LDS instead of streaming every tap from memory.  Pointwise kernel (name
  * "..._pointwise"): 1x1 / stride 1 convolutions with at most 64 input and 256 output channels (weight zero point 128)
  * feed the MFMA from global memory wave by wave, without LDS staging or barriers (hipq_conv2d_run only: the fused add
- * of hipq_conv2d_run_add and accumulator dumps take the tile kernel).
+ * of hipq_conv2d_run_add and accumulator dumps take the tile kernel).  Two-group kernel (name "..._k2"): the tile
+ * kernel with 512 threads, two groups of four waves that each reduce every other 64-byte slab of k and add their partial
+ * accumulators through LDS (plain convolutions with an even number of at least 8 slabs; not with an explicit stage count).
  * mode 1 (the default) uses them where they measured faster: the halo kernel for 64-channel inputs up to 63 pixels
- * wide, the pointwise kernel wherever it applies; mode 2 the halo kernel also for 128, 256 and 512 channels (128-channel
- * tiles, images up to 31 pixels wide); mode 0 neither.  Identical results in every mode.  Plans that do not run the MFMA
+ * wide, the pointwise kernel wherever it applies, the two-group kernel for layers with at most one tile per CU (256);
+ * mode 2 the halo kernel also for 128, 256 and 512 channels (128-channel tiles, images up to 31 pixels wide) and the
+ * two-group kernel whatever the number of tiles; mode 0 none of them.  Identical results in every mode.  Plans that do not run the MFMA
  * kernel return an error.
  */
 int hipq_conv2d_plan_special(hipq_conv2d_plan *plan, int mode);

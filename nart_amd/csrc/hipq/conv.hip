@@ -741,6 +741,238 @@ __global__ __launch_bounds__(256) void conv_mfma_dma_kernel(const ConvArgs a)
 }
 
 // ------------------------------------------------------------------------------------------------
+// The same tile with the reduction shared by TWO groups of four waves (512 threads): group g streams and multiplies the
+// slabs g, g + 2, g + 4, ... through NS stages of its own, and the two partial accumulators are added through LDS before
+// the epilogue.  A layer with few tiles (a 14x14 or 7x7 image at a moderate batch) leaves most CUs with a single
+// work-group, i.e. one wave per SIMD, whose load issue, fragment reads and multiplies then run strictly one after the
+// other; a second wave per SIMD working on the other half of the reduction overlaps them without adding a byte of
+// global traffic (unlike smaller tiles) and without a reduction through memory (unlike a split across work-groups).
+// Aligned addressing, weight zero point 128 (or int8), an even number of slabs, no fused residual: the host checks.
+template <int BM, int BN, int WM, int WN, int NS>
+__global__ __launch_bounds__(512) void conv_mfma_dma_k2_kernel(const ConvArgs a)
+{
+    constexpr bool HAS_WZP = false;
+    constexpr int TM = BM / WM / 32, TN = BN / WN / 32;
+    constexpr int NPB = BM / 64, NPA = BN / 64, LPS = NPA + NPB; // loads per thread and stage
+    constexpr int STAGE = (BM + BN) * 64;
+    constexpr int OSTR = BN + 16;
+    constexpr int GROUP_BYTES = NS * STAGE; // the stages of one group
+    constexpr int LDS_BYTES = 2 * GROUP_BYTES;
+    static_assert(LDS_BYTES >= BM * BN * 4 && LDS_BYTES >= BM * OSTR, "the stages double as reduction and staging buffers");
+    static_assert(WM * WN == 4 && TM >= 1 && TN >= 1 && NPB >= 1 && NPA >= 1 && NS >= 2, "tile shape");
+    static_assert((NS - 2) * LPS <= 63, "vmcnt range");
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[LDS_BYTES];
+
+    const int grp = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 8); // wave-uniform
+    const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;  // position inside the group
+    const int wm = wave % WM, wn = wave / WM;
+    uint8_t *const glds = lds + grp * GROUP_BYTES;
+    const int ng = a.nslab >> 1; // slabs per group
+    const int nblk = a.nbm * a.nbn;
+    const int L = (int)(blockIdx.x % 8) * (int)(gridDim.x / 8) + (int)(blockIdx.x / 8);
+    if (L >= nblk)
+        return;
+    const int bm = L / a.nbn, bn = L % a.nbn;
+
+    // ---- activation source: LDS slot tid (+256 j) = phys chunk (tid & 3) of row (tid >> 2) + 64 j holds the
+    // logical chunk (tid & 3) ^ ((row >> 2) & 3) of that pixel's 64-byte k slab
+    int lp_pix[NPB], lp_ih0[NPB], lp_iw0[NPB];
+    bool lp_ok[NPB];
+    const int ohw = a.OH * a.OW;
+#pragma unroll
+    for (int j = 0; j < NPB; j++) {
+        const int m = bm * BM + (tid >> 2) + 64 * j;
+        lp_ok[j] = m < a.P;
+        const int mm = lp_ok[j] ? m : 0;
+        const int n = fast_div(mm, ohw, a.inv_ohw), rem = mm - n * ohw;
+        const int oh = fast_div(rem, a.OW, a.inv_ow), ow = rem - oh * a.OW;
+        lp_ih0[j] = oh * a.stride_h - a.pad_h;
+        lp_iw0[j] = ow * a.stride_w - a.pad_w;
+        lp_pix[j] = n * a.H * a.W;
+    }
+    const int chunk16 = ((tid & 3) ^ ((tid >> 4) & 3)) * 16;
+    // per-pixel base pointers (possibly outside the tensor for border pixels: never dereferenced
+    // unless the tap is inside the image) + a uniform byte offset of the current (tap, channel slab)
+    const uint8_t *lp_ptr[NPB];
+    bool lp_in[NPB];
+    int tap_r = 0, tap_s = 0, tap_c = 0, tap_off = 0;
+    auto set_tap = [&]() {
+#pragma unroll
+        for (int j = 0; j < NPB; j++)
+            lp_in[j] = lp_ok[j] && (unsigned)(lp_ih0[j] + tap_r) < (unsigned)a.H && (unsigned)(lp_iw0[j] + tap_s) < (unsigned)a.W;
+        tap_off = (tap_r * a.W + tap_s) * a.in_cs;
+    };
+#pragma unroll
+    for (int j = 0; j < NPB; j++)
+        lp_ptr[j] = a.x + (ptrdiff_t)(lp_pix[j] + lp_ih0[j] * a.W + lp_iw0[j]) * a.in_cs + chunk16;
+    set_tap();
+    const uint8_t *wsrc = a.wpack + (size_t)bn * BN * 64 + tid * 16;
+    const int wave_off = __builtin_amdgcn_readfirstlane(wave) * 1024;
+    const size_t wslab = (size_t)a.kout_pad * 64;
+    const bool pad_last = chunk16 + 64 * (a.nslab - 1) >= a.in_cs * a.R * a.S; // only ever true for 1x1 kernels
+
+    auto advance = [&]() { // step the (tap, channel slab) position by one slab
+        tap_c += 64;
+        if (tap_c == a.in_cs) {
+            tap_c = 0;
+            if (++tap_s == a.S) {
+                tap_s = 0;
+                ++tap_r;
+            }
+            set_tap();
+        }
+    };
+    if (grp)
+        advance(); // group 1 starts at slab 1
+    int st_issue = 0; // stage the next issue() fills; stages are used round-robin
+    auto issue = [&](int slab) { // slab: index in the whole reduction
+        uint8_t *st = glds + st_issue * STAGE + wave_off;
+        st_issue = st_issue + 1 == NS ? 0 : st_issue + 1;
+        const uint8_t *ws = wsrc + slab * wslab;
+#pragma unroll
+        for (int j = 0; j < NPA; j++)
+            __builtin_amdgcn_global_load_lds((gptr_t)(ws + j * 4096), (lptr_t)(st + j * 4096), 16, 0, 0);
+        const int off = tap_off + tap_c;
+        // 1x1 kernels whose channel stride is not a multiple of 64: the chunks of the last slab that lie beyond the
+        // pixel's own bytes (their weights are pad slots) come from the pad buffer, not from the next pixel
+        const bool skip = pad_last && slab == a.nslab - 1;
+#pragma unroll
+        for (int j = 0; j < NPB; j++) {
+            const uint8_t *src = lp_in[j] && !skip ? lp_ptr[j] + off : a.padbuf;
+            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(st + BN * 64 + j * 4096), 16, 0, 0);
+        }
+        advance();
+        advance(); // the slab in between belongs to the other group
+    };
+
+    const int swz = (lane >> 2) & 3, half = lane >> 5;
+    const int foff0 = (lane & 31) * 64 + (((0 + half) ^ swz) << 4);
+    const int foff1 = (lane & 31) * 64 + (((2 + half) ^ swz) << 4);
+    const int arow = wn * (TN * 32) * 64, brow = BN * 64 + wm * (TM * 32) * 64;
+
+    // first the stage loads, then the (ordinary) loads of the folded bias (see conv_mfma_dma_kernel)
+    for (int s = 0; s < NS - 1 && s < ng; s++)
+        issue(2 * s + grp);
+
+    const int ch0 = bn * BN + wn * (TN * 32);
+    v16i acc[TN][TM];
+#pragma unroll
+    for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const v4i bias = *reinterpret_cast<const v4i *>(a.bias2 + ch0 + tn * 32 + g * 8 + (lane >> 5) * 4);
+#pragma unroll
+            for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    acc[tn][tm][g * 4 + e] = grp ? 0 : bias[e];
+        }
+    int colsum[TM];
+#pragma unroll
+    for (int tm = 0; tm < TM; tm++)
+        colsum[tm] = 0;
+
+
+    // Fragment reads run one k-step (32 bytes of k) ahead of the MFMAs that consume them, so the LDS latency
+    // hides behind the matrix pipe.  make_ready(i) = slab i has landed for every wave, and every wave's reads of the
+    // stage that slab i+NS-1 will occupy (the stage of slab i-1) have returned their data.
+    int st_comp = 0;
+    auto make_ready = [&](int i) {
+        if (i + NS - 2 <= ng - 1)
+            wait_vmcnt<(NS - 2) * LPS>(); // this group's slabs i+1 .. i+NS-2 may still be in flight
+        else
+            wait_vmcnt<0>();
+        // This wave's fragment reads of slab i-1 must have RETURNED, not merely been issued, before the barrier lets any
+        // wave refill that stage: the load unit's LDS writes are not ordered against another wave's pending ds_reads.
+        // (The reads were issued a whole multiply() ago, so the wait is normally free.)
+        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0), vmcnt / expcnt untouched
+        __builtin_amdgcn_s_barrier();
+        if (i + NS - 1 < ng)
+            issue(2 * (i + NS - 1) + grp);
+    };
+    auto read_frags = [&](v4i(&af)[TN], v4i(&bf)[TM], const uint8_t *buf, int fo) {
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++)
+            af[tn] = *reinterpret_cast<const v4i *>(buf + arow + tn * 2048 + fo);
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+            bf[tm] = *reinterpret_cast<const v4i *>(buf + brow + tm * 2048 + fo);
+    };
+    auto multiply = [&](v4i(&af)[TN], v4i(&bf)[TM]) {
+#pragma unroll
+        for (int tm = 0; tm < TM; tm++)
+            bf[tm] ^= (int)a.xmask;
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+            for (int tm = 0; tm < TM; tm++)
+                acc[tn][tm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[tn], bf[tm], acc[tn][tm], 0, 0, 0);
+        if (HAS_WZP) {
+#pragma unroll
+            for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    colsum[tm] = __builtin_amdgcn_sdot4(bf[tm][e], 0x01010101, colsum[tm], false);
+        }
+    };
+
+    v4i af0[TN], bf0[TM], af1[TN], bf1[TM];
+    make_ready(0);
+    read_frags(af0, bf0, glds, foff0);
+    for (int i = 0; i + 1 < ng; i++) { // the last slab is peeled off: no conditional reads inside the loop
+        const uint8_t *buf = glds + st_comp * STAGE;
+        st_comp = st_comp + 1 == NS ? 0 : st_comp + 1;
+        read_frags(af1, bf1, buf, foff1);
+        multiply(af0, bf0);
+        make_ready(i + 1);
+        read_frags(af0, bf0, glds + st_comp * STAGE, foff0);
+        multiply(af1, bf1);
+    }
+    read_frags(af1, bf1, glds + st_comp * STAGE, foff1);
+    multiply(af0, bf0);
+    multiply(af1, bf1);
+
+    // ---- the two partial sums meet in LDS, then group 0 runs the usual epilogue ---------------------------------
+    __syncthreads(); // every wave has finished reading the last stages; no load is in flight any more
+    int32_t *red = reinterpret_cast<int32_t *>(lds) + wave * (TN * TM * 16 * 64) + lane; // [wave][register][lane]
+    if (grp) {
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+            for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    red[((tn * TM + tm) * 16 + r) * 64] = acc[tn][tm][r];
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    if (!grp) {
+#pragma unroll
+        for (int tn = 0; tn < TN; tn++)
+#pragma unroll
+            for (int tm = 0; tm < TM; tm++)
+#pragma unroll
+                for (int r = 0; r < 16; r++)
+                    acc[tn][tm][r] = (int32_t)((uint32_t)acc[tn][tm][r] + (uint32_t)red[((tn * TM + tm) * 16 + r) * 64]);
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F); // the sums are in registers before the staging tile overwrites the buffer
+    __builtin_amdgcn_s_barrier();
+    if (grp) {
+        // group 1 only keeps the barrier count of conv_epilogue's staged path (one barrier; the plain path has none)
+        if (!(a.acc_out != nullptr || (a.out_cs & 15))) {
+            __builtin_amdgcn_s_barrier();
+        }
+        return;
+    }
+    if (a.fastq && a.lo == 0 && a.q.hi == 255)
+        conv_epilogue<BM, BN, WM, WN, HAS_WZP, true, true, TM, TN>(a, acc, colsum, lds, bm, bn, wm, wn);
+    else if (a.fastq)
+        conv_epilogue<BM, BN, WM, WN, HAS_WZP, true, false, TM, TN>(a, acc, colsum, lds, bm, bn, wm, wn);
+    else
+        conv_epilogue<BM, BN, WM, WN, HAS_WZP, false, false, TM, TN>(a, acc, colsum, lds, bm, bn, wm, wn);
+}
+
+// ------------------------------------------------------------------------------------------------
 // 3x3, stride 1, pad 1 convolutions (in_cs a multiple of 64).  The nine taps of an output pixel read nine shifted copies
 // of the same input bytes, so instead of streaming one 64-byte slab per pixel and tap, the work-group loads, per
 // 64-channel slab, the pixels [m0 - W - 1, m0 + BM + W] of the flattened (n, h, w) index space ONCE (a "halo tile" of
@@ -1360,6 +1592,8 @@ static bool pointwise_applies(const hipq_conv2d_plan *p)
         && p->args.fastq;
 }
 
+static bool k2_applies(const hipq_conv2d_plan *p);
+
 static void set_mfma_name(hipq_conv2d_plan *p, bool smallc)
 {
     char nm[96];
@@ -1367,7 +1601,8 @@ static void set_mfma_name(hipq_conv2d_plan *p, bool smallc)
         snprintf(nm, sizeof nm, "conv_mfma_i8_pointwise%s", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
     else
         snprintf(nm, sizeof nm, "conv_mfma_i8_%dx%d%s%s%s%s", kTiles[p->tile].bm, kTiles[p->tile].bn, smallc ? "_c4" : "",
-                 p->has_wzp ? "_wzp" : "", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "", halo_applies(p) ? "_halo" : "");
+                 p->has_wzp ? "_wzp" : "", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "",
+                 halo_applies(p) ? "_halo" : (!smallc && k2_applies(p)) ? "_k2" : ""); // _k2: unless a residual add is fused
     p->name = nm;
 }
 
@@ -1594,9 +1829,9 @@ extern "C" int hipq_conv2d_plan_select(hipq_conv2d_plan *p, int tile, int stages
         p->tile = tile;
         p->args.nbm = (p->args.P + kTiles[tile].bm - 1) / kTiles[tile].bm;
         p->args.nbn = (p->d.out_cs + kTiles[tile].bn - 1) / kTiles[tile].bn;
-        set_mfma_name(p, false);
     }
     p->stages = stages;
+    set_mfma_name(p, false);
     return 0;
 }
 
@@ -1674,6 +1909,38 @@ static bool launch_halo(const hipq_conv2d_plan *p, const ConvArgs &a, const dim3
     }
 }
 
+// conv_mfma_dma_k2_kernel (the reduction shared by two groups of four waves): plain convolutions (no fused residual)
+// with aligned addressing, an even number of at least 8 slabs, a tile of at most 128 + 64 or 64 + 128 rows per stage
+// pair, and - by the built-in rule - no more tiles than the chip has CUs, i.e. layers that would otherwise run one wave
+// per SIMD.  Measured inside the ResNet-50 pass the 7x7 layers gain 20 %; layers with one to two tiles per CU gain
+// nothing (two four-wave work-groups already share their CUs) and 128x128 tiles lose.  An explicit stage count
+// (hipq_conv2d_plan_select) keeps the four-wave kernel.
+constexpr int kCUs = 256;
+static bool k2_applies(const hipq_conv2d_plan *p)
+{
+    const ConvArgs &a = p->args;
+    const bool aligned = a.in_cs % 64 == 0 || (a.R == 1 && a.S == 1 && a.in_cs % 16 == 0);
+    if (!(p->special && p->stages == 0 && p->variant == kMfma && !p->has_wzp && aligned && (a.nslab & 1) == 0 && a.nslab >= 8))
+        return false;
+    if (kTiles[p->tile].bm + kTiles[p->tile].bn > 256)
+        return false;
+    return p->special == 2 || a.nbm * a.nbn <= kCUs;
+}
+
+template <int BM, int BN, int WM, int WN>
+static bool launch_k2(const hipq_conv2d_plan *p, const ConvArgs &a, const dim3 grid, hipStream_t st)
+{
+    if constexpr (BM + BN > 256) {
+        return false;
+    } else {
+        if (!k2_applies(p) || a.res != nullptr)
+            return false;
+        // one work-group per CU: LDS is no constraint, so the deepest stream the stages allow
+        hipLaunchKernelGGL((conv_mfma_dma_k2_kernel<BM, BN, WM, WN, (BM + BN <= 192 ? 4 : 3)>), grid, dim3(512), 0, st, a);
+        return true;
+    }
+}
+
 template <int BM, int BN, int WM, int WN>
 static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_t st)
 {
@@ -1711,6 +1978,8 @@ static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_
             launch_dma_aligned<BM, BN, WM, WN, 3, true>(grid, a, st);
         else
             launch_dma_aligned<BM, BN, WM, WN, 2, true>(grid, a, st);
+    } else if (aligned && launch_k2<BM, BN, WM, WN>(p, a, grid, st)) {
+        // the reduction shared by two groups of waves
     } else if (aligned) {
         // Few tiles, long reduction (fully-connected layers at small batch): the weights stream from HBM through a
         // handful of CUs, and only the bytes each of them keeps in flight cover the memory latency: eight stages.

@@ -167,8 +167,8 @@ class Conv2d:
         return self
 
     def special(self, mode=1):
-        """Tuning hook: the halo-tile (3x3 stride 1) and pointwise (small 1x1) kernels: 0 never, 1 built-in rule,
-        2 wherever they apply (include/hipq.h)."""
+        """Tuning hook: the halo-tile (3x3 stride 1), pointwise (small 1x1) and two-group (few tiles, long reduction)
+        kernels: 0 never, 1 built-in rule, 2 wherever they apply (include/hipq.h)."""
         check(lib().hipq_conv2d_plan_special(self.handle, int(mode)))
         self.kernel = lib().hipq_conv2d_plan_kernel(self.handle).decode()
         return self

@@ -555,3 +555,55 @@ def test_golden_int8_outputs_on_gpu():
             hipq.dequantize_i8(hipq.to_device_nhwc(ins[0]), fd, a["q"][0])
             got = fd.cpu().numpy()
         assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), name
+
+
+def test_two_group_kernel_matches_the_oracle():
+    """Layers with a long reduction and few tiles run the tile kernel with two groups of waves that reduce every other
+    slab each and add their partial sums through LDS: 3x3 and 1x1 kernels, stride 2, a partial last slab (1x1 with a
+    channel stride that is no multiple of 64), ragged pixel and channel tiles, accumulator dumps, int8 tensors, every tile
+    shape; an odd number of slabs, an explicit stage count or mode 0 keep the four-wave kernel."""
+    rng = np.random.default_rng(47)
+    #         N   C    H   W   K   R  pad stride
+    shapes = [(2, 256, 14, 14, 256, 3, 1, 1), (3, 512, 7, 7, 200, 3, 1, 1), (5, 512, 9, 9, 96, 1, 0, 1), (2, 1000, 3, 5, 130, 1, 0, 1),
+              (1, 128, 17, 17, 64, 3, 1, 2), (64, 2048, 1, 1, 1000, 1, 0, 1), (1, 64, 12, 12, 32, 3, 0, 1)]
+    for N, C, H, W, K, R, pad, stride in shapes:
+        print("two-group case", N, C, H, W, K, R, pad, stride, flush=True)
+        x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+        w = rng.integers(0, 256, (K, C, R, R), dtype=np.uint8)
+        b = rng.integers(-30000, 30000, K).astype(np.int32)
+        q = (rand_q(rng), int(rng.integers(0, 256)), rand_q(rng), 128, rand_q(rng, 1e-2, 1.0), int(rng.integers(0, 256)))
+        want, want_acc = orc.conv2d_u8(x, w, b, pad, stride, 1, *q, return_acc=True)
+        plan = hipq.Conv2d(x.shape, w, b, pad, stride, 1, *q)
+        nslab = (R * R * plan.desc.in_cs + 63) // 64
+        eligible = nslab % 2 == 0 and nslab >= 8
+        assert plan.kernel.endswith("_k2") == eligible, (plan.kernel, nslab)  # every case here has at most 256 tiles
+        xd = hipq.to_device_nhwc(x)
+        assert np.array_equal(hipq.from_device_nhwc(plan(xd), K), want), (x.shape, K, plan.kernel)
+        plan.special(2)
+        for tile in (0, 2, 3, 4):
+            plan.select(tile, 0)
+            # on request the halo kernel takes the 3x3 / stride 1 / pad 1 layers it can (128-channel tiles, narrow images)
+            halo = R == 3 and pad == 1 and stride == 1 and C in (128, 256, 512) and tile in (0, 3) and W <= 31
+            assert plan.kernel.endswith("_halo") == halo and plan.kernel.endswith("_k2") == (eligible and not halo), (plan.kernel, tile)
+            assert np.array_equal(hipq.from_device_nhwc(plan(xd), K), want), (x.shape, K, tile, plan.kernel)
+            acc = torch.empty((N, plan.OH, plan.OW, plan.desc.out_cs), dtype=torch.int32, device="cuda")
+            plan(xd, acc=acc)
+            assert np.array_equal(acc.cpu().numpy()[..., :K].transpose(0, 3, 1, 2), want_acc), (x.shape, tile)
+        plan.select(1, 0)  # the 256-pixel tile has no two-group variant
+        assert not plan.kernel.endswith("_k2")
+        plan.select(3, 3)  # an explicit stage count means the four-wave kernel
+        assert not plan.kernel.endswith("_k2")
+        assert np.array_equal(hipq.from_device_nhwc(plan(xd), K), want)
+        plan.select(3, 0).special(0)
+        assert not plan.kernel.endswith("_k2")
+        assert np.array_equal(hipq.from_device_nhwc(plan(xd), K), want)
+        xs, ws = x.view(np.int8), w.view(np.int8)
+        want8 = orc.conv2d_i8(xs, ws, b, pad, stride, 1, q[0], q[2], q[4], 7)
+        p8 = hipq.Conv2d(x.shape, ws, b, pad, stride, 1, q[0], 0, q[2], 0, q[4], 0, obits=7, dtype=hipq.DTYPE_I8)
+        assert p8.kernel.endswith("_k2") == eligible, p8.kernel
+        assert np.array_equal(hipq.from_device_nhwc(p8(hipq.to_device_nhwc(xs)), K).view(np.int8), want8), (x.shape, K)
+    # asymmetric weights keep the generic kernel
+    x = rng.integers(0, 256, (1, 256, 8, 8), dtype=np.uint8)
+    w = rng.integers(0, 256, (64, 256, 3, 3), dtype=np.uint8)
+    plan = hipq.Conv2d(x.shape, w, None, 1, 1, 1, 0.02, 7, 0.005, 100, 0.05, 3)
+    assert not plan.kernel.endswith("_k2"), plan.kernel
