@@ -1935,8 +1935,13 @@ static bool launch_k2(const hipq_conv2d_plan *p, const ConvArgs &a, const dim3 g
     } else {
         if (!k2_applies(p) || a.res != nullptr)
             return false;
-        // one work-group per CU: LDS is no constraint, so the deepest stream the stages allow
-        hipLaunchKernelGGL((conv_mfma_dma_k2_kernel<BM, BN, WM, WN, (BM + BN <= 192 ? 4 : 3)>), grid, dim3(512), 0, st, a);
+        if (a.nbm * a.nbn <= kCUs || BM + BN > 192) {
+            // one work-group per CU: LDS is no constraint, so the deepest stream the stages allow
+            hipLaunchKernelGGL((conv_mfma_dma_k2_kernel<BM, BN, WM, WN, (BM + BN <= 192 ? 4 : 3)>), grid, dim3(512), 0, st, a);
+        } else {
+            // more tiles than CUs (on request only): three stages per group, so that two work-groups still share a CU
+            hipLaunchKernelGGL((conv_mfma_dma_k2_kernel<BM, BN, WM, WN, 3>), grid, dim3(512), 0, st, a);
+        }
         return true;
     }
 }

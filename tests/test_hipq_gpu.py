@@ -565,7 +565,8 @@ def test_two_group_kernel_matches_the_oracle():
     rng = np.random.default_rng(47)
     #         N   C    H   W   K   R  pad stride
     shapes = [(2, 256, 14, 14, 256, 3, 1, 1), (3, 512, 7, 7, 200, 3, 1, 1), (5, 512, 9, 9, 96, 1, 0, 1), (2, 1000, 3, 5, 130, 1, 0, 1),
-              (1, 128, 17, 17, 64, 3, 1, 2), (64, 2048, 1, 1, 1000, 1, 0, 1), (1, 64, 12, 12, 32, 3, 0, 1)]
+              (1, 128, 17, 17, 64, 3, 1, 2), (64, 2048, 1, 1, 1000, 1, 0, 1), (1, 64, 12, 12, 32, 3, 0, 1),
+              (16, 512, 14, 14, 512, 1, 0, 1)]  # the last one: more tiles than CUs with the small tiles (on request only)
     for N, C, H, W, K, R, pad, stride in shapes:
         print("two-group case", N, C, H, W, K, R, pad, stride, flush=True)
         x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
@@ -576,7 +577,7 @@ def test_two_group_kernel_matches_the_oracle():
         plan = hipq.Conv2d(x.shape, w, b, pad, stride, 1, *q)
         nslab = (R * R * plan.desc.in_cs + 63) // 64
         eligible = nslab % 2 == 0 and nslab >= 8
-        assert plan.kernel.endswith("_k2") == eligible, (plan.kernel, nslab)  # every case here has at most 256 tiles
+        assert plan.kernel.endswith("_k2") == eligible, (plan.kernel, nslab)  # every case has at most 256 tiles of the rule's own tile
         xd = hipq.to_device_nhwc(x)
         assert np.array_equal(hipq.from_device_nhwc(plan(xd), K), want), (x.shape, K, plan.kernel)
         plan.special(2)
