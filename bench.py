@@ -227,6 +227,7 @@ def main():
         pms = (time.perf_counter() - t0) * 1e3 / args.steps
         same = torch.equal(pipe.execs[1].buf[case.output.name], ex.buf[case.output.name])
         in_flight = {"batches_in_flight": 2, "ms_per_step": round(pms, 4), "value": round(args.batch / (pms * 1e-3), 1),
+                     "conv_tops_whole_step": round(case.conv_ops() / (pms * 1e-3) / 1e12, 2),
                      "timer": "host clock around the K submissions and the final synchronisation",
                      "outputs_equal_single_stream": bool(same)}
         del pipe
