@@ -1449,7 +1449,10 @@ __global__ __launch_bounds__(256) void conv_depthwise3x3_kernel(const ConvArgs a
     const int per_row = nstrip * cq;
     const int total = a.N * ohp * per_row; // the host guarantees it fits in 31 bits
     const int qmode = a.fastq ? (a.lo == 0 && a.q.hi == 255 ? 2 : 1) : 0;
-    for (int idx = blockIdx.x * 256 + threadIdx.x; idx < total; idx += gridDim.x * 256) {
+    // work-groups go to the 8 XCDs in turn: renumbered so that each XCD works on one contiguous eighth of the (image-major)
+    // index space, the eighth whose pixels its convolution tiles read and write (the grid is a multiple of 8)
+    const int L = (int)(blockIdx.x & 7) * (int)(gridDim.x >> 3) + (int)(blockIdx.x >> 3);
+    for (int idx = L * 256 + threadIdx.x; idx < total; idx += gridDim.x * 256) {
         if (a.acc_out != nullptr)
             depthwise3x3_body<STRIDE, HAS_WZP, 0, true>(a, idx, per_row, cq, ohp); // test path: exactness only
         else if (qmode == 2)
@@ -2066,7 +2069,7 @@ static int run_conv(const hipq_conv2d_plan *p, ConvArgs &a, hipStream_t st)
         break;
     case kDepthwise3x3: {
         const size_t total = (size_t)a.N * ((a.OH + 1) / 2) * ((a.OW + 3) / 4) * (a.in_cs / 4);
-        const dim3 grid((unsigned)std::min<size_t>((total + 255) / 256, 256 * 64)), block(256);
+        const dim3 grid((unsigned)((std::min<size_t>((total + 255) / 256, 256 * 64) + 7) / 8 * 8)), block(256); // a multiple of 8
         if (p->d.stride_h == 1) {
             if (p->has_wzp)
                 hipLaunchKernelGGL((conv_depthwise3x3_kernel<1, true>), grid, block, 0, st, a);
