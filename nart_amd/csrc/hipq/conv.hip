@@ -1206,7 +1206,10 @@ __device__ static inline void pointwise_strips(const ConvArgs &a, const uint8_t 
     const int nb = (a.out_cs + 31) >> 5, nstrips = (a.P + 31) >> 5;
     const int prow = 16 * ((p >> 2) & 1) + 4 * (p >> 3) + (p & 3); // the channel (within a block) MFMA row p stands for
     const int32_t *lbias = reinterpret_cast<const int32_t *>(lds + 256 * 64);
-    for (int strip = blockIdx.x * 4 + wave; strip < nstrips; strip += gridDim.x * 4) {
+    // work-groups go to the 8 XCDs in turn: XCD x takes the x-th contiguous eighth of the strips (the pixels its tile
+    // kernels read and write), its work-groups interleaved inside that eighth (the grid is a multiple of 8)
+    const int xcd = blockIdx.x & 7, s8 = (nstrips + 7) >> 3, s_end = min((xcd + 1) * s8, nstrips);
+    for (int strip = xcd * s8 + (int)(blockIdx.x >> 3) * 4 + wave; strip < s_end; strip += (int)(gridDim.x >> 3) * 4) {
         const int m = strip * 32 + p;
         const bool ok = m < a.P;
         v4i bf[NKS];
@@ -1959,7 +1962,7 @@ static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_
     if (pointwise_applies(p) && a.acc_out == nullptr && a.res == nullptr) {
         // persistent work-groups (four waves, a strip of 32 pixels each per turn), five to a CU
         const int nstrips = (a.P + 31) / 32, want = (nstrips + 3) / 4;
-        const dim3 pgrid(want < 1280 ? want : 1280);
+        const dim3 pgrid(((want < 1280 ? want : 1280) + 7) / 8 * 8);
         if (a.in_cs <= 32)
             hipLaunchKernelGGL(conv_mfma_pointwise_kernel<1>, pgrid, block, 0, st, a);
         else

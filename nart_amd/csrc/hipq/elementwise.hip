@@ -261,7 +261,10 @@ __global__ __launch_bounds__(256) void pool_max16_u8_kernel(const PoolArgs p, do
     const int c16n = p.cs >> 4;
     const int total = p.N * p.OH * p.OW * c16n; // the host guarantees 31 bits
     const int radd = (1 << (p.shift - 1)) + (p.oz << p.shift);
-    for (int idx = blockIdx.x * 256 + threadIdx.x; idx < total; idx += gridDim.x * 256) {
+    // work-groups go to the 8 XCDs in turn: renumbered so that each XCD works on a contiguous eighth of the (image-major)
+    // index space, the eighth whose pixels its convolution tiles read (the grid is a multiple of 8)
+    const int L = (int)(blockIdx.x & 7) * (int)(gridDim.x >> 3) + (int)(blockIdx.x >> 3);
+    for (int idx = L * 256 + threadIdx.x; idx < total; idx += gridDim.x * 256) {
         const int m = (int)((double)idx * inv_c16);
         const int mm = m - (m * c16n > idx) + ((m + 1) * c16n <= idx), c0 = (idx - mm * c16n) * 16;
         int row = (int)((double)mm * inv_ow);
@@ -755,7 +758,7 @@ extern "C" int hipq_pool_u8(const void *x, void *y, int N, int C, int H, int W, 
         && (long long)N * H * W * cs < (1ll << 31) && (reinterpret_cast<uintptr_t>(x) & 15) == 0
         && (reinterpret_cast<uintptr_t>(y) & 15) == 0) {
         const size_t total16 = (size_t)N * OH * OW * (cs / 16);
-        hipLaunchKernelGGL(pool_max16_u8_kernel, dim3(grid_for(total16)), dim3(256), 0, static_cast<hipStream_t>(stream), p,
+        hipLaunchKernelGGL(pool_max16_u8_kernel, dim3((grid_for(total16) + 7) / 8 * 8), dim3(256), 0, static_cast<hipStream_t>(stream), p,
                            1.0 / (cs / 16), 1.0 / OW, 1.0 / OH);
         return launch_status("pool_max16_u8_kernel");
     }
