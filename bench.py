@@ -97,7 +97,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--batch", type=int, default=64)
+    ap.add_argument("--batch", type=int, default=None, help="images per step (fc: rows M); default 64, for --workload fc 128 (BASELINE configs[1])")
     ap.add_argument("--workload", default="resnet50", choices=["resnet50", "resnet18", "mobilenetv2", "conv", "fc"])
     ap.add_argument("--kernel-reps", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -113,6 +113,8 @@ def main():
                     help="also launch a plain 256 MiB device copy (copy_bytes_kernel): the known-size reference that a "
                          "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE run of this command is scaled by")
     args = ap.parse_args()
+    if args.batch is None:
+        args.batch = 128 if args.workload == "fc" else 64
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU's share of the batch: this build runs on a single GPU only "
                  "(--gpus %d refused; batch-sharded inference needs no collectives)." % args.gpus)

@@ -117,6 +117,17 @@ int hipq_conv2d_plan_select(hipq_conv2d_plan *plan, int tile, int stages);
  * kernel return an error.
  */
 int hipq_conv2d_plan_special(hipq_conv2d_plan *plan, int mode);
+/*
+ * Tuning hook (no counterpart in the reference) for the streaming kernel (name "..._stream_<rows>x<cols>"): 1x1 / stride 1
+ * layers over at most 256 pixels whose input rows are multiples of 128 bytes (weight zero point 128, or int8) - in
+ * practice the fully-connected layers, op_quant_ip_u8xu8_run (src/op/ip.cpp:133-209), whose pixels are the batch.  They
+ * are bound by the weight stream, so the output is cut into strips of 16 or 32 channels, one work-group each, whose waves
+ * split the reduction and feed the 16x16x64 MFMA straight from global memory.  rows: pixel rows per work-group (16, 32, 64
+ * or 128), cols: 16 or 32, waves: 4 or 8 (not every combination exists); 0, 0, 0 returns to the built-in rule (one strip
+ * of 16 channels over every pixel row up to 128, four waves).  hipq_conv2d_plan_special(plan, 0) switches the kernel off.
+ * Identical results for every choice.  Plans that the kernel does not serve return an error.
+ */
+int hipq_conv2d_plan_stream(hipq_conv2d_plan *plan, int rows, int cols, int waves);
 
 /*
  * Run: op_conv_2d_u8xu8_run — src/op/conv_2d_uint8_impl.c:39-165 (im2col src/utils/im2col.cpp:487,

@@ -1284,6 +1284,126 @@ __global__ __launch_bounds__(256) void conv_mfma_pointwise_kernel(const ConvArgs
 }
 
 // ------------------------------------------------------------------------------------------------
+// Fully-connected layers and other 1x1 / stride 1 layers over a few hundred pixels at most (op_quant_ip_u8xu8_run,
+// art/modules/quant/src/op/ip.cpp:133-209, with the batch as the pixels).  Such a layer is a weight stream: every weight
+// byte is used once per pixel row and the weights are many times larger than the activations, so the time is the time
+// it takes to pull the weights out of HBM, and that takes every CU.  The tile kernels cannot give every CU a share (a
+// 128-row by 4096-column problem has 32 of their tiles); this kernel cuts the output into narrow column strips instead:
+//   * a work-group owns 16*NB output channels of 16*MB pixel rows and the whole reduction;
+//   * nothing is staged in LDS: with v_mfma_i32_16x16x64_i8 lane (r, q) of the weight operand holds bytes [16q, 16q + 16)
+//     of weight row r of a 64-byte slab - 16 contiguous bytes of the packed weights - and lane (p, q) of the pixel
+//     operand the same bytes of pixel row p, so both operands are plain 128-bit global loads; a weight fragment is
+//     used by MB multiplies, a pixel fragment by NB, all of this wave;
+//   * the NW waves of the work-group split the reduction (pairs of slabs, so that a wave reads whole 128-byte lines) and
+//     keep four slabs of loads in flight each; their partial sums meet once, in LDS, and the waves share the epilogue.
+// Requires in_cs % 128 == 0, weight zero point 128 (or int8), no fused residual: the host checks.
+template <int MB, int NB, int NW>
+__global__ __launch_bounds__(NW * 64) void conv_mfma_stream_kernel(const ConvArgs a, const int mtiles)
+{
+    constexpr int NT = MB * NB;  // 16x16 accumulator tiles per wave
+    constexpr int RING = 4;      // slabs of loads in flight per wave
+    __shared__ __attribute__((aligned(16))) int32_t red[NW * NT * 4 * 64]; // [wave][tile][register][lane]
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, q = lane >> 4;
+    // Work-groups go to the 8 XCDs in turn; the m-tiles of one column strip get consecutive numbers inside one XCD, so
+    // that the second reader of a strip's weights finds them in that XCD's L2.
+    const int per_xcd = (int)gridDim.x >> 3, idx = (int)blockIdx.x >> 3;
+    const int nt = (idx / mtiles) * 8 + ((int)blockIdx.x & 7), mt = idx % mtiles;
+    (void)per_xcd;
+    const int n0 = nt * (16 * NB), m0 = mt * (16 * MB);
+    if (n0 >= a.out_cs)
+        return;
+
+    const int nch = a.nslab >> 1;                                   // chunks of two slabs
+    const int cnt = wave < nch ? 2 * ((nch - wave + NW - 1) / NW) : 0; // slabs of this wave
+    const uint8_t *wp = a.wpack + (size_t)(n0 + r) * 64 + ((q ^ ((r >> 2) & 3)) << 4);
+    const size_t wslab = (size_t)a.kout_pad * 64;
+    const uint8_t *xp[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++) {
+        const int m = min(m0 + mb * 16 + r, a.P - 1); // rows beyond the last pixel repeat it; their results are dropped
+        xp[mb] = a.x + (size_t)m * a.in_cs + q * 16;
+    }
+
+    v4i acc[MB][NB];
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+            acc[mb][nb] = v4i{0, 0, 0, 0};
+
+    if (cnt > 0) {
+        v4i wf[RING][NB], xf[RING][MB];
+        auto load = [&](int slot, int t) {
+            const int tt = min(t, cnt - 1); // past the end: the last slab once more (loaded, never multiplied)
+            const int slab = 2 * (wave + NW * (tt >> 1)) + (tt & 1);
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++)
+                wf[slot][nb] = __builtin_nontemporal_load(reinterpret_cast<const v4i *>(wp + slab * wslab + nb * 1024));
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++)
+                xf[slot][mb] = *reinterpret_cast<const v4i *>(xp[mb] + slab * 64);
+        };
+#pragma unroll
+        for (int u = 0; u < RING - 1; u++)
+            load(u, u);
+        for (int t = 0; t < cnt; t += RING) {
+#pragma unroll
+            for (int u = 0; u < RING; u++) {
+                load((u + RING - 1) % RING, t + u + RING - 1);
+                if (t + u < cnt) {
+#pragma unroll
+                    for (int mb = 0; mb < MB; mb++) {
+                        const v4i xs = xf[u][mb] ^ (int)a.xmask;
+#pragma unroll
+                        for (int nb = 0; nb < NB; nb++)
+                            acc[mb][nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[u][nb], xs, acc[mb][nb], 0, 0, 0);
+                    }
+                }
+            }
+        }
+    }
+
+    // ---- the waves' partial sums meet in LDS; wave w finishes the tiles w, w + NW, ...
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int nb = 0; nb < NB; nb++)
+#pragma unroll
+            for (int v = 0; v < 4; v++)
+                red[((wave * NT + mb * NB + nb) * 4 + v) * 64 + lane] = acc[mb][nb][v];
+    __syncthreads();
+#pragma unroll
+    for (int tl = 0; tl < (NT + NW - 1) / NW; tl++) {
+        const int tile = wave + tl * NW;
+        if (tile >= NT)
+            break;
+        const int mb = tile / NB, nb = tile % NB;
+        const int m = m0 + mb * 16 + r, ko = n0 + nb * 16 + 4 * q; // this lane: 4 consecutive channels of one pixel
+        const v4i bias = *reinterpret_cast<const v4i *>(a.bias2 + ko);
+        int32_t v[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            uint32_t s = (uint32_t)bias[e];
+#pragma unroll
+            for (int w = 0; w < NW; w++)
+                s += (uint32_t)red[((w * NT + tile) * 4 + e) * 64 + lane];
+            v[e] = (int32_t)s;
+        }
+        if (m >= a.P || ko >= a.out_cs)
+            continue;
+        if (a.acc_out != nullptr)
+            *reinterpret_cast<v4i *>(a.acc_out + (size_t)m * a.out_cs + ko) = v4i{v[0], v[1], v[2], v[3]};
+        int32_t rq[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+            rq[e] = a.fastq ? conv_requant<true>(a, v[e]) : conv_requant<false>(a, v[e]);
+        *reinterpret_cast<uint32_t *>(a.y + (size_t)m * a.out_cs + ko) = pack_low_bytes(rq[0], rq[1], rq[2], rq[3]);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // Depthwise 3x3 (group == C == K, stride 1 or 2): HBM-bound on paper (16 bytes in, 16 bytes out per output pixel and
 // 16 channels), in practice bounded by vector ALU work, so the kernel is written for instruction count.
 // One thread owns 4 channels (one dword of the channels-last tensors) of a strip of 4 output pixels along W; a
@@ -1560,6 +1680,11 @@ struct TileShape {
 static const TileShape kTiles[] = {{128, 128}, {256, 64}, {128, 64}, {64, 128}, {64, 64}};
 constexpr int kNumTiles = sizeof(kTiles) / sizeof(kTiles[0]);
 
+// conv_mfma_stream_kernel: a work-group's share is 16 * mb pixel rows by 16 * nb output channels, nw waves
+struct StreamShape {
+    int mb, nb, nw;
+};
+
 struct hipq_conv2d_plan {
     hipq_conv2d_desc d;
     ConvArgs args;
@@ -1567,6 +1692,7 @@ struct hipq_conv2d_plan {
     int tile;       // index into kTiles
     int stages = 0; // load stages of the DMA kernel; 0 = the built-in rule
     int special = 1; // the halo-tile and pointwise kernels: 0 never, 1 built-in rule, 2 wherever they apply
+    StreamShape stream = {0, 0, 0}; // explicit shape of the streaming kernel (hipq_conv2d_plan_stream); mb = 0: built-in rule
     bool has_wzp;
     void *d_w = nullptr, *d_bias = nullptr;
     std::string name;
@@ -1600,10 +1726,32 @@ static bool pointwise_applies(const hipq_conv2d_plan *p)
 
 static bool k2_applies(const hipq_conv2d_plan *p);
 
+// conv_mfma_stream_kernel: 1x1 / stride 1 layers over at most 256 pixels (fully-connected layers: the pixels are the
+// batch) whose rows are whole 128-byte lines, weight zero point 128 (or int8).  Shape of a work-group's share: 16 * mb
+// pixel rows by 16 * nb output channels.  A strip that holds every pixel row reads each weight byte once; two m-tiles
+// per strip halve the pixel bytes a CU pulls through its L1 (what bounds the kernel once the weights stream at full
+// rate) and read the weights twice, the second time from L2.
+static bool stream_applies(const hipq_conv2d_plan *p, StreamShape *shape = nullptr)
+{
+    const hipq_conv2d_desc &d = p->d;
+    const ConvArgs &a = p->args;
+    if (!(p->special && p->variant == kMfma && !p->has_wzp && d.R == 1 && d.S == 1 && d.stride_h == 1 && d.stride_w == 1
+          && d.pad_h == 0 && d.pad_w == 0 && d.in_cs % 128 == 0 && a.P <= 256))
+        return false;
+    if (shape) {
+        const int rows = (a.P + 15) / 16;
+        *shape = p->stream.mb ? p->stream : StreamShape{rows > 4 ? 8 : rows > 2 ? 4 : rows > 1 ? 2 : 1, 1, 4};
+    }
+    return true;
+}
+
 static void set_mfma_name(hipq_conv2d_plan *p, bool smallc)
 {
     char nm[96];
-    if (pointwise_applies(p))
+    StreamShape ss;
+    if (!smallc && stream_applies(p, &ss))
+        snprintf(nm, sizeof nm, "conv_mfma_i8_stream_%dx%d%s", 16 * ss.mb, 16 * ss.nb, p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
+    else if (pointwise_applies(p))
         snprintf(nm, sizeof nm, "conv_mfma_i8_pointwise%s", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
     else
         snprintf(nm, sizeof nm, "conv_mfma_i8_%dx%d%s%s%s%s", kTiles[p->tile].bm, kTiles[p->tile].bn, smallc ? "_c4" : "",
@@ -1713,7 +1861,9 @@ extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t
         a.rowb = smallc ? 4 * ((d.S + 3) / 4 * 4) : d.in_cs;
         a.Ktot = smallc ? d.R * a.rowb : d.R * d.S * d.in_cs;
         a.nslab = (a.Ktot + 63) / 64;
-        a.kout_pad = (d.K + 127) / 128 * 128;
+        // every tile kernel indexes weight rows and folded constants by output-channel TILE, i.e. up to out_cs rounded up
+        // to its tile width: the padding covers the output stride, not just K (a caller may write into a wider buffer)
+        a.kout_pad = (std::max(d.K, d.out_cs) + 127) / 128 * 128;
         p->has_wzp = boff != 0;
         // weights: [slab][kout_pad][64 bytes]; chunk c of row ko is stored at chunk c ^ ((ko >> 2) & 3),
         // the order the kernel keeps in LDS.  Rows of pad output channels stay zero (their outputs are
@@ -1853,6 +2003,29 @@ extern "C" int hipq_conv2d_plan_special(hipq_conv2d_plan *p, int mode)
     return 0;
 }
 
+extern "C" int hipq_conv2d_plan_stream(hipq_conv2d_plan *p, int rows, int cols, int waves)
+{
+    clear_error();
+    HIPQ_REQUIRE(p, "hipq_conv2d_plan_stream: null plan");
+    HIPQ_REQUIRE(stream_applies(p), "hipq_conv2d_plan_stream: this plan does not run the streaming kernel (it runs %s)", p->name.c_str());
+    if (rows == 0 && cols == 0 && waves == 0) {
+        p->stream = {0, 0, 0};
+    } else {
+        const int key = rows / 16 * 100 + cols / 16 * 10 + waves;
+        static const int ok[] = {814, 818, 424, 428, 414, 418, 214, 224, 114, 124};
+        bool found = rows % 16 == 0 && cols % 16 == 0;
+        if (found) {
+            found = false;
+            for (int k : ok)
+                found = found || k == key;
+        }
+        HIPQ_REQUIRE(found, "hipq_conv2d_plan_stream: no instantiation for %d rows x %d columns with %d waves", rows, cols, waves);
+        p->stream = {rows / 16, cols / 16, waves};
+    }
+    set_mfma_name(p, false);
+    return 0;
+}
+
 // Load stages.  Short reductions (few slabs) run with two stages: the smaller LDS footprint lets four work-groups
 // share a CU and overlap their load, multiply and store phases.  Long reductions (3x3 layers, wide 1x1 layers) run
 // with four (three for the largest tile): measured inside the whole network, where a layer's input comes from HBM
@@ -1959,6 +2132,30 @@ static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_
     const dim3 grid((nblk + 7) / 8 * 8), block(256);
     if (p->variant == kMfma && launch_halo<BM, BN, WM, WN>(p, a, grid, st))
         return;
+    StreamShape ss;
+    if (a.res == nullptr && stream_applies(p, &ss)) {
+        const int mtiles = (a.P + 16 * ss.mb - 1) / (16 * ss.mb), ntiles = (a.out_cs + 16 * ss.nb - 1) / (16 * ss.nb);
+        const dim3 sgrid((ntiles + 7) / 8 * 8 * mtiles);
+        const int key = ss.mb * 100 + ss.nb * 10 + ss.nw;
+        switch (key) {
+#define HIPQ_STREAM_CASE(MB_, NB_, NW_)                                                                                  \
+    case MB_ * 100 + NB_ * 10 + NW_:                                                                                    \
+        hipLaunchKernelGGL((conv_mfma_stream_kernel<MB_, NB_, NW_>), sgrid, dim3(NW_ * 64), 0, st, a, mtiles);          \
+        return;
+            HIPQ_STREAM_CASE(8, 1, 4)
+            HIPQ_STREAM_CASE(8, 1, 8)
+            HIPQ_STREAM_CASE(4, 2, 4)
+            HIPQ_STREAM_CASE(4, 2, 8)
+            HIPQ_STREAM_CASE(4, 1, 4)
+            HIPQ_STREAM_CASE(4, 1, 8)
+            HIPQ_STREAM_CASE(2, 1, 4)
+            HIPQ_STREAM_CASE(2, 2, 4)
+            HIPQ_STREAM_CASE(1, 1, 4)
+            HIPQ_STREAM_CASE(1, 2, 4)
+#undef HIPQ_STREAM_CASE
+        default: break; // an unknown forced shape: the tile kernels below
+        }
+    }
     if (pointwise_applies(p) && a.acc_out == nullptr && a.res == nullptr) {
         // persistent work-groups (four waves, a strip of 32 pixels each per turn), five to a CU
         const int nstrips = (a.P + 31) / 32, want = (nstrips + 3) / 4;

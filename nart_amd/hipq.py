@@ -43,6 +43,7 @@ _SIGS = {
     "hipq_conv2d_plan_kernel": (C.c_char_p, [C.c_void_p]),
     "hipq_conv2d_plan_select": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
     "hipq_conv2d_plan_special": (C.c_int, [C.c_void_p, C.c_int]),
+    "hipq_conv2d_plan_stream": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int]),
     "hipq_conv2d_run_relu": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "hipq_conv2d_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "hipq_conv2d_run_add": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_float, C.c_int,
@@ -170,6 +171,12 @@ class Conv2d:
         """Tuning hook: the halo-tile (3x3 stride 1), pointwise (small 1x1) and two-group (few tiles, long reduction)
         kernels: 0 never, 1 built-in rule, 2 wherever they apply (include/hipq.h)."""
         check(lib().hipq_conv2d_plan_special(self.handle, int(mode)))
+        self.kernel = lib().hipq_conv2d_plan_kernel(self.handle).decode()
+        return self
+
+    def stream(self, rows=0, cols=0, waves=0):
+        """Tuning hook: shape of the streaming (fully-connected) kernel's work-groups (include/hipq.h)."""
+        check(lib().hipq_conv2d_plan_stream(self.handle, rows, cols, waves))
         self.kernel = lib().hipq_conv2d_plan_kernel(self.handle).decode()
         return self
 

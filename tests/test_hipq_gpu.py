@@ -184,6 +184,77 @@ def test_ip_as_1x1():
     assert np.array_equal(yd.cpu().numpy().reshape(M, -1)[:, :No], want)
 
 
+def test_fc_streaming_kernel():
+    """Fully-connected layers (op_quant_ip_u8xu8_run, ip.cpp:133-209) on the streaming kernel: BASELINE configs[1] at
+    its stated shape (M=128, K=4096, N=4096, full-range values, log-uniform scales) and the shapes around it, accumulators
+    and bytes against the oracle; every work-group shape the kernel is instantiated for gives the same bytes."""
+    rng = np.random.default_rng(141)
+    shapes = [(128, 4096, 4096, False), (1, 512, 1000, False), (64, 2048, 1000, True), (5, 128, 37, False),
+              (17, 256, 16, True), (130, 384, 100, False), (256, 1024, 48, False), (33, 1280, 1000, False)]
+    for M, Kd, No, relu in shapes:
+        print("fc case", M, Kd, No, relu, flush=True)
+        x = rng.integers(0, 256, (M, Kd), dtype=np.uint8)
+        w = rng.integers(0, 256, (No, Kd), dtype=np.uint8)
+        b = rng.integers(-50000, 50000, No).astype(np.int32)
+        ia, wa = rand_q(rng), rand_q(rng)
+        # the output scale follows the spread of the sums (about 74 * 74 * sqrt(K) in input units), so that the bytes
+        # are not all saturated; the accumulators are compared whatever the scales
+        oa = float(np.float32(ia * wa * np.sqrt(Kd) * 60.0))
+        q = (ia, 128 if M == 128 else int(rng.integers(0, 256)), wa, 128, oa, int(rng.integers(0, 256)))
+        want_y, want_acc = orc.ip_u8(x, w, b, *q, return_acc=True)
+        if relu:
+            want_y = np.maximum(want_y, q[5]).astype(np.uint8)
+        plan = hipq.Conv2d((M, Kd, 1, 1), w.reshape(No, Kd, 1, 1), b, 0, 1, 1, *q, relu=relu)
+        assert "_stream_" in plan.kernel, plan.kernel
+        xd = hipq.to_device_nhwc(x.reshape(M, Kd, 1, 1))
+        acc = torch.zeros((M, 1, 1, plan.desc.out_cs), dtype=torch.int32, device="cuda")
+        yd = plan(xd, acc=acc)
+        torch.cuda.synchronize()
+        got_acc = acc.cpu().numpy().reshape(M, -1)[:, :No]
+        assert np.array_equal(got_acc, want_acc), (M, Kd, No, plan.kernel, int((got_acc != want_acc).sum()))
+        first = yd.cpu().numpy().reshape(M, -1)
+        assert np.array_equal(first[:, :No], want_y), (M, Kd, No, plan.kernel)
+        assert len(np.unique(want_y)) > 8 or M < 8, "degenerate case: the scales saturate the outputs"
+        for rows, cols, waves in ((128, 16, 4), (128, 16, 8), (64, 32, 4), (64, 32, 8), (64, 16, 4), (64, 16, 8), (32, 16, 4),
+                                  (32, 32, 4), (16, 16, 4), (16, 32, 4)):
+            plan.stream(rows, cols, waves)
+            assert plan.kernel.endswith("_stream_%dx%d" % (rows, cols)), plan.kernel
+            y2 = plan(xd).cpu().numpy().reshape(M, -1)
+            assert np.array_equal(y2[:, :No], want_y), (M, Kd, No, rows, cols, waves)
+        plan.stream()
+        # the tile kernels serve the same plan when the streaming kernel is switched off, with the same bytes
+        plan.special(0)
+        assert "_stream_" not in plan.kernel
+        y3 = plan(xd).cpu().numpy().reshape(M, -1)
+        assert np.array_equal(y3[:, :No], want_y), (M, Kd, No, plan.kernel)
+        plan.close()
+    with pytest.raises(hipq.HipqError):  # not a streaming plan
+        hipq.Conv2d((1, 64, 8, 8), np.zeros((64, 64, 3, 3), np.uint8), None, 1, 1, 1, 0.1, 0, 0.1, 128, 0.1, 0).stream(64, 16, 4)
+    with pytest.raises(hipq.HipqError):  # no such instantiation
+        hipq.Conv2d((4, 128, 1, 1), np.zeros((16, 128, 1, 1), np.uint8), None, 0, 1, 1, 0.1, 0, 0.1, 128, 0.1, 0).stream(128, 32, 4)
+
+
+def test_output_stride_wider_than_the_channels():
+    """A caller may write a convolution's output into a buffer with a wider channel stride than the layout rule gives
+    (hipq_conv2d_desc.out_cs): the packed weights and folded constants cover every output-channel tile of that stride."""
+    rng = np.random.default_rng(142)
+    N, C, H, W, K = 2, 64, 9, 9, 64
+    x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+    w = rng.integers(0, 256, (K, C, 3, 3), dtype=np.uint8)
+    b = rng.integers(-1000, 1000, K).astype(np.int32)
+    q = (0.02, 120, 0.005, 128, 0.05, 3)
+    want = orc.conv2d_u8(x, w, b, 1, 1, 1, *q)
+    for out_cs in (256, 384):
+        plan = hipq.Conv2d(x.shape, w, b, 1, 1, 1, *q, out_cs=out_cs)
+        for tile in (-1, 0, 2, 3, 4):
+            if tile >= 0:
+                plan.special(0).select(tile)
+            yd = plan(hipq.to_device_nhwc(x))
+            torch.cuda.synchronize()
+            got = yd.cpu().numpy()[..., :K].transpose(0, 3, 1, 2)
+            assert np.array_equal(got, want), (out_cs, plan.kernel)
+
+
 def test_elementwise():
     rng = np.random.default_rng(15)
     for n in (1, 15, 16, 4099, 64 * 56 * 56 * 16 + 3):
