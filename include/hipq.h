@@ -122,9 +122,10 @@ int hipq_conv2d_plan_special(hipq_conv2d_plan *plan, int mode);
  * layers over at most 256 pixels whose input rows are multiples of 128 bytes (weight zero point 128, or int8) - in
  * practice the fully-connected layers, op_quant_ip_u8xu8_run (src/op/ip.cpp:133-209), whose pixels are the batch.  They
  * are bound by the weight stream, so the output is cut into strips of 16 or 32 channels, one work-group each, whose waves
- * split the reduction and feed the 16x16x64 MFMA straight from global memory.  rows: pixel rows per work-group (16, 32, 64
- * or 128), cols: 16 or 32, waves: 4 or 8 (not every combination exists); 0, 0, 0 returns to the built-in rule (one strip
- * of 16 channels over every pixel row up to 128, four waves).  hipq_conv2d_plan_special(plan, 0) switches the kernel off.
+ * split the reduction and stream their shares through LDS stages of their own into the 16x16x64 MFMA.  rows: pixel rows
+ * per work-group (16, 32, 64 or 128), cols: 16 or 32 (128 x 32 does not exist), waves: 4; 0, 0, 0 returns to the built-in rule (one strip
+ * shape that minimises what a CU pulls through its L1).  hipq_conv2d_plan_special(plan, 0) switches the kernel off, and so
+ * does naming a tile with hipq_conv2d_plan_select.
  * Identical results for every choice.  Plans that the kernel does not serve return an error.
  */
 int hipq_conv2d_plan_stream(hipq_conv2d_plan *plan, int rows, int cols, int waves);

@@ -1289,42 +1289,82 @@ __global__ __launch_bounds__(256) void conv_mfma_pointwise_kernel(const ConvArgs
 // byte is used once per pixel row and the weights are many times larger than the activations, so the time is the time
 // it takes to pull the weights out of HBM, and that takes every CU.  The tile kernels cannot give every CU a share (a
 // 128-row by 4096-column problem has 32 of their tiles); this kernel cuts the output into narrow column strips instead:
-//   * a work-group owns 16*NB output channels of 16*MB pixel rows and the whole reduction;
-//   * nothing is staged in LDS: with v_mfma_i32_16x16x64_i8 lane (r, q) of the weight operand holds bytes [16q, 16q + 16)
-//     of weight row r of a 64-byte slab - 16 contiguous bytes of the packed weights - and lane (p, q) of the pixel
-//     operand the same bytes of pixel row p, so both operands are plain 128-bit global loads; a weight fragment is
-//     used by MB multiplies, a pixel fragment by NB, all of this wave;
-//   * the NW waves of the work-group split the reduction (pairs of slabs, so that a wave reads whole 128-byte lines) and
-//     keep four slabs of loads in flight each; their partial sums meet once, in LDS, and the waves share the epilogue.
+//   * a work-group owns 16*NB output channels of 16*MB pixel rows and the whole reduction, on v_mfma_i32_16x16x64_i8:
+//     a weight fragment (16 rows of a 64-byte slab, 1 KB of the packed weights) is used by MB multiplies, a pixel
+//     fragment by NB, all of one wave;
+//   * the NW waves split the reduction in chunks of 128 bytes of k (two slabs: whole cache lines of the pixel rows), and
+//     each wave streams ITS chunks through LDS stages of its own, R deep, with the load unit (global_load_lds_dwordx4,
+//     eight lanes per 128-byte line: loading the MFMA operand straight into registers would make neighbouring lanes ask
+//     for 16 bytes of sixteen different rows, a quarter of the L1 rate).  No barrier in the loop: a wave waits for its
+//     own loads (vmcnt) and refills a stage once its own reads of it have returned (lgkmcnt);
+//   * 16-byte piece c of pixel row r sits at piece c ^ (r & 7) of its 128-byte LDS row, the blocks of eight rows are
+//     spaced so that rows r and r + 8 start in different halves of the banks, the weights keep their packed order: the
+//     fragment reads are free of bank conflicts;
+//   * the waves' partial sums meet once, in LDS, and the waves share the epilogue.
 // Requires in_cs % 128 == 0, weight zero point 128 (or int8), no fused residual: the host checks.
-template <int MB, int NB, int NW>
-__global__ __launch_bounds__(NW * 64) void conv_mfma_stream_kernel(const ConvArgs a, const int mtiles)
+template <int MB, int NB>
+struct StreamCfg {
+    static constexpr int ROWS = 16 * MB;
+    static constexpr int XI = ROWS / 8;            // pixel loads per chunk: 8 rows of 128 bytes each
+    static constexpr int PER = XI + 2 * NB;        // loads per chunk
+    // block j of 8 pixel rows sits at j * 1024 + ((j + 1) >> 1) * 128: the two blocks of a 16-row fragment start in
+    // different halves of the banks
+    static constexpr int XBYTES = XI * 1024 + (XI / 2 + 1) * 128;
+    static constexpr int STAGE = XBYTES + 2 * NB * 1024;
+    static constexpr int R0 = (160 * 1024) / (4 * STAGE);
+    static constexpr int R = R0 > 4 ? 4 : R0;      // stages per wave (four waves)
+    static_assert(R >= 2 && (R - 1) * PER <= 63, "stage count / vmcnt range");
+};
+
+template <int MB, int NB>
+__global__ __launch_bounds__(256) void conv_mfma_stream_kernel(const ConvArgs a, const int mtiles)
 {
-    constexpr int NT = MB * NB;  // 16x16 accumulator tiles per wave
-    constexpr int RING = 4;      // slabs of loads in flight per wave
-    __shared__ __attribute__((aligned(16))) int32_t red[NW * NT * 4 * 64]; // [wave][tile][register][lane]
+    using Cfg = StreamCfg<MB, NB>;
+    constexpr int NW = 4, NT = MB * NB, R = Cfg::R, STAGE = Cfg::STAGE, PER = Cfg::PER, XI = Cfg::XI;
+    constexpr int WOFF = Cfg::XBYTES; // the weight slabs follow the pixel rows in a stage
+    static_assert(NW * R * STAGE >= NW * NT * 1024, "the stages double as the reduction buffer");
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[NW * R * STAGE];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int r = lane & 15, q = lane >> 4;
     // Work-groups go to the 8 XCDs in turn; the m-tiles of one column strip get consecutive numbers inside one XCD, so
     // that the second reader of a strip's weights finds them in that XCD's L2.
-    const int per_xcd = (int)gridDim.x >> 3, idx = (int)blockIdx.x >> 3;
+    const int idx = (int)blockIdx.x >> 3;
     const int nt = (idx / mtiles) * 8 + ((int)blockIdx.x & 7), mt = idx % mtiles;
-    (void)per_xcd;
     const int n0 = nt * (16 * NB), m0 = mt * (16 * MB);
     if (n0 >= a.out_cs)
         return;
 
-    const int nch = a.nslab >> 1;                                   // chunks of two slabs
-    const int cnt = wave < nch ? 2 * ((nch - wave + NW - 1) / NW) : 0; // slabs of this wave
-    const uint8_t *wp = a.wpack + (size_t)(n0 + r) * 64 + ((q ^ ((r >> 2) & 3)) << 4);
+    const int nch = a.nslab >> 1;                                // chunks of two slabs
+    const int cnt = wave < nch ? (nch - wave + NW - 1) / NW : 0; // chunks of this wave
+    // Every work-group reads the same pixel rows: each starts the reduction at a different chunk, so that they do not
+    // all ask for the same lines at the same time (the order of an exact integer sum is free).
+    const int rot = (nt * 7 + mt * 3) % nch;
+    auto chunk_of = [&](int t) {
+        int c = wave + NW * t + rot;
+        return c >= nch ? c - nch : c;
+    };
+    uint8_t *const wl = lds + wave * (R * STAGE);
+    // load lane l of pixel instruction j: row 8 j + (l >> 3), LDS piece l & 7 = logical piece (l & 7) ^ (row & 7)
+    const int xrow = lane >> 3, xoff = ((lane & 7) ^ xrow) << 4;
+    const uint8_t *wsrc = a.wpack + (size_t)n0 * 64 + lane * 16;
     const size_t wslab = (size_t)a.kout_pad * 64;
-    const uint8_t *xp[MB];
+    auto issue = [&](int t) {
+        const int chunk = chunk_of(t);
+        uint8_t *st = wl + (t % R) * STAGE;
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++) {
-        const int m = min(m0 + mb * 16 + r, a.P - 1); // rows beyond the last pixel repeat it; their results are dropped
-        xp[mb] = a.x + (size_t)m * a.in_cs + q * 16;
-    }
+        for (int j = 0; j < XI; j++) {
+            const int m = min(m0 + 8 * j + xrow, a.P - 1); // rows beyond the last pixel repeat it; their results are dropped
+            const uint8_t *src = a.x + (uint32_t)(m * a.in_cs + chunk * 128 + xoff);
+            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(st + j * 1024 + ((j + 1) >> 1) * 128), 16, 0, 0);
+        }
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+            for (int nb = 0; nb < NB; nb++)
+                __builtin_amdgcn_global_load_lds((gptr_t)(wsrc + (size_t)(2 * chunk + h) * wslab + nb * 1024),
+                                                 (lptr_t)(st + WOFF + (h * NB + nb) * 1024), 16, 0, 0);
+    };
 
     v4i acc[MB][NB];
 #pragma unroll
@@ -1333,39 +1373,47 @@ __global__ __launch_bounds__(NW * 64) void conv_mfma_stream_kernel(const ConvArg
         for (int nb = 0; nb < NB; nb++)
             acc[mb][nb] = v4i{0, 0, 0, 0};
 
-    if (cnt > 0) {
-        v4i wf[RING][NB], xf[RING][MB];
-        auto load = [&](int slot, int t) {
-            const int tt = min(t, cnt - 1); // past the end: the last slab once more (loaded, never multiplied)
-            const int slab = 2 * (wave + NW * (tt >> 1)) + (tt & 1);
+    for (int u = 0; u < R - 1 && u < cnt; u++)
+        issue(u);
+    // fragment addresses inside a stage: weights in packed order; pixel row 16 mb + r lives in block 2 mb + (r >> 3)
+    // (rows r and r + 8 fall into different halves of the banks), piece (4 h + q) of the row at piece ^ (r & 7)
+    const int wfo = WOFF + r * 64 + ((q ^ ((r >> 2) & 3)) << 4);
+    const int xfo = (r >> 3) * 1152 + (r & 7) * 128; // + 2176 per 16-row fragment
+    for (int t = 0; t < cnt; t++) {
+        // this wave's fragment reads of chunk t - 1 have returned (the load unit's LDS writes are not ordered against
+        // pending reads), then its stage is refilled
+        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
+        if (t + R - 1 < cnt)
+            issue(t + R - 1);
+        const int ahead = min(R - 1, cnt - 1 - t); // chunks younger than t in flight
+        if (ahead >= 3)
+            wait_vmcnt<3 * PER>();
+        else if (ahead == 2)
+            wait_vmcnt<(R > 2 ? 2 : 0) * PER>();
+        else if (ahead == 1)
+            wait_vmcnt<PER>();
+        else
+            wait_vmcnt<0>();
+        const uint8_t *st = wl + (t % R) * STAGE;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            v4i wf[NB];
 #pragma unroll
             for (int nb = 0; nb < NB; nb++)
-                wf[slot][nb] = __builtin_nontemporal_load(reinterpret_cast<const v4i *>(wp + slab * wslab + nb * 1024));
+                wf[nb] = *reinterpret_cast<const v4i *>(st + wfo + (h * NB + nb) * 1024);
 #pragma unroll
-            for (int mb = 0; mb < MB; mb++)
-                xf[slot][mb] = *reinterpret_cast<const v4i *>(xp[mb] + slab * 64);
-        };
+            for (int mb = 0; mb < MB; mb++) {
+                const v4i xs = *reinterpret_cast<const v4i *>(st + mb * 2176 + xfo + (((4 * h + q) ^ (r & 7)) << 4)) ^ (int)a.xmask;
 #pragma unroll
-        for (int u = 0; u < RING - 1; u++)
-            load(u, u);
-        for (int t = 0; t < cnt; t += RING) {
-#pragma unroll
-            for (int u = 0; u < RING; u++) {
-                load((u + RING - 1) % RING, t + u + RING - 1);
-                if (t + u < cnt) {
-#pragma unroll
-                    for (int mb = 0; mb < MB; mb++) {
-                        const v4i xs = xf[u][mb] ^ (int)a.xmask;
-#pragma unroll
-                        for (int nb = 0; nb < NB; nb++)
-                            acc[mb][nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[u][nb], xs, acc[mb][nb], 0, 0, 0);
-                    }
-                }
+                for (int nb = 0; nb < NB; nb++)
+                    acc[mb][nb] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[nb], xs, acc[mb][nb], 0, 0, 0);
             }
         }
     }
 
     // ---- the waves' partial sums meet in LDS; wave w finishes the tiles w, w + NW, ...
+    __syncthreads(); // every wave is done with its stages; no load is in flight any more
+    int32_t *red = reinterpret_cast<int32_t *>(lds); // [wave][tile][register][lane]
 #pragma unroll
     for (int mb = 0; mb < MB; mb++)
 #pragma unroll
@@ -1692,6 +1740,7 @@ struct hipq_conv2d_plan {
     int tile;       // index into kTiles
     int stages = 0; // load stages of the DMA kernel; 0 = the built-in rule
     int special = 1; // the halo-tile and pointwise kernels: 0 never, 1 built-in rule, 2 wherever they apply
+    bool tile_selected = false;     // hipq_conv2d_plan_select named a tile: the tile kernels, not the streaming kernel
     StreamShape stream = {0, 0, 0}; // explicit shape of the streaming kernel (hipq_conv2d_plan_stream); mb = 0: built-in rule
     bool has_wzp;
     void *d_w = nullptr, *d_bias = nullptr;
@@ -1724,6 +1773,7 @@ static bool pointwise_applies(const hipq_conv2d_plan *p)
         && p->args.fastq;
 }
 
+constexpr int kCUs = 256;
 static bool k2_applies(const hipq_conv2d_plan *p);
 
 // conv_mfma_stream_kernel: 1x1 / stride 1 layers over at most 256 pixels (fully-connected layers: the pixels are the
@@ -1735,12 +1785,29 @@ static bool stream_applies(const hipq_conv2d_plan *p, StreamShape *shape = nullp
 {
     const hipq_conv2d_desc &d = p->d;
     const ConvArgs &a = p->args;
-    if (!(p->special && p->variant == kMfma && !p->has_wzp && d.R == 1 && d.S == 1 && d.stride_h == 1 && d.stride_w == 1
-          && d.pad_h == 0 && d.pad_w == 0 && d.in_cs % 128 == 0 && a.P <= 256))
+    if (!(p->special && !p->tile_selected && p->variant == kMfma && !p->has_wzp && d.R == 1 && d.S == 1 && d.stride_h == 1
+          && d.stride_w == 1 && d.pad_h == 0 && d.pad_w == 0 && d.in_cs % 128 == 0 && a.P <= 256))
         return false;
     if (shape) {
+        if (p->stream.mb) {
+            *shape = p->stream;
+            return true;
+        }
+        // What a CU pulls through its L1 bounds the kernel once the weights stream at full rate: per work-group
+        // (16 mb + 16 nb) rows of k bytes, times the rounds of work-groups the chip needs.  The smallest product wins,
+        // more work-groups on a tie (measured: 128 x 4096 x 4096 takes 8.6 us as 64 x 32, 11.3 as 128 x 16, 10.1 as
+        // 32 x 32; 64 x 2048 x 1000 takes 3.5 us as 16 x 16, 4.7 as 64 x 16).
+        static const StreamShape cand[] = {{8, 1, 4}, {4, 2, 4}, {4, 1, 4}, {2, 2, 4}, {2, 1, 4}, {1, 2, 4}, {1, 1, 4}};
         const int rows = (a.P + 15) / 16;
-        *shape = p->stream.mb ? p->stream : StreamShape{rows > 4 ? 8 : rows > 2 ? 4 : rows > 1 ? 2 : 1, 1, 4};
+        long long best = -1, best_wgs = 0;
+        for (const StreamShape &c : cand) {
+            if (c.mb > 1 && c.mb / 2 >= rows)
+                continue; // half of the rows would be padding
+            const long long wgs = (long long)((rows + c.mb - 1) / c.mb) * ((a.out_cs + 16 * c.nb - 1) / (16 * c.nb));
+            const long long cost = ((wgs + kCUs - 1) / kCUs) * (c.mb + c.nb);
+            if (best < 0 || cost < best || (cost == best && wgs > best_wgs))
+                best = cost, best_wgs = wgs, *shape = c;
+        }
     }
     return true;
 }
@@ -1982,6 +2049,7 @@ extern "C" int hipq_conv2d_plan_select(hipq_conv2d_plan *p, int tile, int stages
     HIPQ_REQUIRE(tile >= -1 && tile < kNumTiles && (stages == 0 || (stages >= 2 && stages <= 4) || stages == 8),
                  "hipq_conv2d_plan_select: tile must be -1 (keep) or 0..%d, stages 0 (built-in rule), 2..4 or 8", kNumTiles - 1);
     if (tile >= 0) {
+        p->tile_selected = true;
         p->tile = tile;
         p->args.nbm = (p->args.P + kTiles[tile].bm - 1) / kTiles[tile].bm;
         p->args.nbn = (p->d.out_cs + kTiles[tile].bn - 1) / kTiles[tile].bn;
@@ -2012,7 +2080,7 @@ extern "C" int hipq_conv2d_plan_stream(hipq_conv2d_plan *p, int rows, int cols, 
         p->stream = {0, 0, 0};
     } else {
         const int key = rows / 16 * 100 + cols / 16 * 10 + waves;
-        static const int ok[] = {814, 818, 424, 428, 414, 418, 214, 224, 114, 124};
+        static const int ok[] = {814, 424, 414, 224, 214, 124, 114};
         bool found = rows % 16 == 0 && cols % 16 == 0;
         if (found) {
             found = false;
@@ -2094,7 +2162,6 @@ static bool launch_halo(const hipq_conv2d_plan *p, const ConvArgs &a, const dim3
 // per SIMD.  Measured inside the ResNet-50 pass the 7x7 layers gain 20 %; layers with one to two tiles per CU gain
 // nothing (two four-wave work-groups already share their CUs) and 128x128 tiles lose.  An explicit stage count
 // (hipq_conv2d_plan_select) keeps the four-wave kernel.
-constexpr int kCUs = 256;
 static bool k2_applies(const hipq_conv2d_plan *p)
 {
     const ConvArgs &a = p->args;
@@ -2138,20 +2205,17 @@ static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_
         const dim3 sgrid((ntiles + 7) / 8 * 8 * mtiles);
         const int key = ss.mb * 100 + ss.nb * 10 + ss.nw;
         switch (key) {
-#define HIPQ_STREAM_CASE(MB_, NB_, NW_)                                                                                  \
-    case MB_ * 100 + NB_ * 10 + NW_:                                                                                    \
-        hipLaunchKernelGGL((conv_mfma_stream_kernel<MB_, NB_, NW_>), sgrid, dim3(NW_ * 64), 0, st, a, mtiles);          \
+#define HIPQ_STREAM_CASE(MB_, NB_)                                                                                       \
+    case MB_ * 100 + NB_ * 10 + 4:                                                                                      \
+        hipLaunchKernelGGL((conv_mfma_stream_kernel<MB_, NB_>), sgrid, dim3(256), 0, st, a, mtiles);                    \
         return;
-            HIPQ_STREAM_CASE(8, 1, 4)
-            HIPQ_STREAM_CASE(8, 1, 8)
-            HIPQ_STREAM_CASE(4, 2, 4)
-            HIPQ_STREAM_CASE(4, 2, 8)
-            HIPQ_STREAM_CASE(4, 1, 4)
-            HIPQ_STREAM_CASE(4, 1, 8)
-            HIPQ_STREAM_CASE(2, 1, 4)
-            HIPQ_STREAM_CASE(2, 2, 4)
-            HIPQ_STREAM_CASE(1, 1, 4)
-            HIPQ_STREAM_CASE(1, 2, 4)
+            HIPQ_STREAM_CASE(8, 1)
+            HIPQ_STREAM_CASE(4, 2)
+            HIPQ_STREAM_CASE(4, 1)
+            HIPQ_STREAM_CASE(2, 2)
+            HIPQ_STREAM_CASE(2, 1)
+            HIPQ_STREAM_CASE(1, 2)
+            HIPQ_STREAM_CASE(1, 1)
 #undef HIPQ_STREAM_CASE
         default: break; // an unknown forced shape: the tile kernels below
         }
