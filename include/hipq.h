@@ -90,6 +90,17 @@ typedef struct hipq_conv2d_plan hipq_conv2d_plan;
  */
 int hipq_conv2d_plan_create(const hipq_conv2d_desc *desc, const uint8_t *w, const int32_t *bias,
                             hipq_conv2d_plan **plan_out);
+/*
+ * The same with one weight scale per output channel: walpha is a host array of K floats that replaces desc->walpha, and
+ * channel k is requantised with (mult, shift) = get_quant_scale_int32(ialpha * walpha[k] / oalpha)
+ * (quant_helper.h:60-118) - the arithmetic of op_conv_2d_u8xu8_run (src/op/conv_2d_uint8_impl.c:57-66, 127-143) with
+ * the pair chosen per channel.  The reference CPU module reads walpha[0] only; a per-channel array is what its CUDA
+ * sibling accepts (art/modules/cuda_quant/src/op/conv_2d_quant.cu:751-764).  With K equal scales the result is
+ * bit-identical to hipq_conv2d_plan_create.  Zero points, output scale, bias and clamps stay per tensor.  Every run entry
+ * point works on such a plan (kernel name suffix "_perchannel").
+ */
+int hipq_conv2d_plan_create_per_channel(const hipq_conv2d_desc *desc, const uint8_t *w, const int32_t *bias,
+                                        const float *walpha, hipq_conv2d_plan **plan_out);
 void hipq_conv2d_plan_destroy(hipq_conv2d_plan *plan);
 /* Name of the kernel variant the plan dispatches to (for logs and tests). */
 const char *hipq_conv2d_plan_kernel(const hipq_conv2d_plan *plan);

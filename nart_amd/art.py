@@ -200,7 +200,8 @@ class Op:
             self.set_array(SETTING_QUANT_IZERO_POINT, dtUINT8, np.atleast_1d(izp))
             self.set_array(SETTING_QUANT_IBITS, dtUINT8, [bits] * ia.size)
         if walpha is not None:
-            self.set_array(SETTING_QUANT_WALPHA, dtFLOAT32, [walpha])
+            # one entry = a per-tensor scale; one entry per output channel = per-channel scales
+            self.set_array(SETTING_QUANT_WALPHA, dtFLOAT32, np.atleast_1d(np.asarray(walpha, dtype=np.float32)))
             self.set_array(SETTING_QUANT_WZERO_POINT, dtUINT8, [wzp])
             self.set_array(SETTING_QUANT_WBITS, dtUINT8, [bits])
         if oalpha is not None:

@@ -86,6 +86,10 @@ struct ConvArgs {
     int qadd;  // 2^(qt-1) + zp * 2^qt
     double inv_ohw, inv_ow; // 1 / (OH*OW), 1 / OW (depthwise 3x3: 1 / work items per row, 1 / channel quads)
     double inv_oh;          // 1 / OH
+    // per-output-channel requantisation (a weight scale per channel): multipliers and shifts, padded like bias2;
+    // nullptr = the per-tensor pair in q.  Such plans requantise with the 64-bit form, channel by channel.
+    const uint32_t *qmult;
+    const int32_t *qshift;
     const uint8_t *res; // fused residual add: the other operand (same layout as y), or nullptr
     int res_first;      // 1: the residual is input 0 of the add, the convolution's output input 1
     AddParams addq;
@@ -120,6 +124,16 @@ __device__ static inline int32_t conv_requant(const ConvArgs &a, int32_t v)
     return out;
 }
 
+// Per-channel form: channel ch has its own (mult, shift); zero point and clamps are the tensor's.
+__device__ static inline int32_t conv_requant_ch(const ConvArgs &a, int32_t v, int ch)
+{
+    const int32_t r = (int32_t)(rshift_rn((int64_t)v * (int64_t)a.qmult[ch], a.qshift[ch]) + a.q.zp);
+    return r < a.lo ? a.lo : (r > a.q.hi ? a.q.hi : r);
+}
+
+// The element-wise epilogue (no LDS transpose): accumulator dumps, outputs too narrow for 128-bit rows, per-channel scales.
+__host__ __device__ static inline bool plain_epilogue(const ConvArgs &a) { return a.acc_out != nullptr || (a.out_cs & 15) || a.qmult != nullptr; }
+
 // Pack the low bytes of four values into a dword (three v_perm_b32 / v_or_b32; works for negative values, whose
 // low byte is their two's complement int8).
 __device__ static inline uint32_t pack_low_bytes(int32_t r0, int32_t r1, int32_t r2, int32_t r3)
@@ -135,8 +149,8 @@ __device__ static inline void conv_epilogue(const ConvArgs &a, v16i (&acc)[TN][T
     const int tid = threadIdx.x, lane = tid & 63, half = lane >> 5;
     const int ch0 = bn * BN + wn * (TN * 32);
     const int m0 = bm * BM; // first pixel of the tile
-    if (a.acc_out != nullptr || (a.out_cs & 15)) {
-        // plain path: accumulator dump requested, or an output too narrow for 128-bit rows
+    if (plain_epilogue(a)) {
+        // plain path: accumulator dump requested, an output too narrow for 128-bit rows, or per-channel scales
 #pragma unroll
         for (int tm = 0; tm < TM; tm++) {
             const int m = m0 + wm * (TM * 32) + tm * 32 + (lane & 31);
@@ -155,7 +169,7 @@ __device__ static inline void conv_epilogue(const ConvArgs &a, v16i (&acc)[TN][T
                         const int32_t v = (int32_t)((uint32_t)acc[tn][tm][g * 4 + e] + (HAS_WZP ? (uint32_t)colsum[tm] : 0u));
                         if (a.acc_out)
                             a.acc_out[(size_t)m * a.out_cs + ko + e] = v;
-                        rq[e] = conv_requant<FAST>(a, v);
+                        rq[e] = a.qmult ? conv_requant_ch(a, v, ko + e) : conv_requant<FAST>(a, v);
                     }
                     uint32_t packed = pack_low_bytes(rq[0], rq[1], rq[2], rq[3]);
                     if (a.res) {
@@ -959,7 +973,7 @@ __global__ __launch_bounds__(512) void conv_mfma_dma_k2_kernel(const ConvArgs a)
     __builtin_amdgcn_s_barrier();
     if (grp) {
         // group 1 only keeps the barrier count of conv_epilogue's staged path (one barrier; the plain path has none)
-        if (!(a.acc_out != nullptr || (a.out_cs & 15))) {
+        if (!plain_epilogue(a)) {
             __builtin_amdgcn_s_barrier();
         }
         return;
@@ -1446,7 +1460,7 @@ __global__ __launch_bounds__(256) void conv_mfma_stream_kernel(const ConvArgs a,
         int32_t rq[4];
 #pragma unroll
         for (int e = 0; e < 4; e++)
-            rq[e] = a.fastq ? conv_requant<true>(a, v[e]) : conv_requant<false>(a, v[e]);
+            rq[e] = a.qmult ? conv_requant_ch(a, v[e], ko + e) : a.fastq ? conv_requant<true>(a, v[e]) : conv_requant<false>(a, v[e]);
         *reinterpret_cast<uint32_t *>(a.y + (size_t)m * a.out_cs + ko) = pack_low_bytes(rq[0], rq[1], rq[2], rq[3]);
     }
 }
@@ -1606,7 +1620,7 @@ __device__ static inline void depthwise3x3_body(const ConvArgs &a, int idx, int 
             } else {
 #pragma unroll
                 for (int c = 0; c < 4; c++)
-                    packed |= (uint32_t)conv_requant<QMODE == 1>(a, v[c]) << (8 * c);
+                    packed |= (uint32_t)((QMODE == 0 && a.qmult) ? conv_requant_ch(a, v[c], c0 + c) : conv_requant<QMODE == 1>(a, v[c])) << (8 * c);
             }
             *reinterpret_cast<uint32_t *>(a.y + (obase + (uint32_t)(o * a.out_cs))) = packed;
         }
@@ -1619,7 +1633,7 @@ __global__ __launch_bounds__(256) void conv_depthwise3x3_kernel(const ConvArgs a
     const int cq = a.in_cs >> 2, nstrip = (a.OW + 3) >> 2, ohp = (a.OH + 1) >> 1;
     const int per_row = nstrip * cq;
     const int total = a.N * ohp * per_row; // the host guarantees it fits in 31 bits
-    const int qmode = a.fastq ? (a.lo == 0 && a.q.hi == 255 ? 2 : 1) : 0;
+    const int qmode = (a.fastq && a.qmult == nullptr) ? (a.lo == 0 && a.q.hi == 255 ? 2 : 1) : 0;
     // work-groups go to the 8 XCDs in turn: renumbered so that each XCD works on one contiguous eighth of the (image-major)
     // index space, the eighth whose pixels its convolution tiles read and write (the grid is a multiple of 8)
     const int L = (int)(blockIdx.x & 7) * (int)(gridDim.x >> 3) + (int)(blockIdx.x >> 3);
@@ -1673,7 +1687,7 @@ __global__ __launch_bounds__(256) void conv_depthwise_kernel(const ConvArgs a)
         for (int e = 0; e < 4; e++) {
             if (a.acc_out)
                 a.acc_out[(size_t)m * a.out_cs + c0 + e] = acc[e];
-            packed |= (uint32_t)(conv_requant<false>(a, acc[e]) & 255) << (8 * e);
+            packed |= (uint32_t)((a.qmult ? conv_requant_ch(a, acc[e], c0 + e) : conv_requant<false>(a, acc[e])) & 255) << (8 * e);
         }
         *reinterpret_cast<uint32_t *>(a.y + (size_t)m * a.out_cs + c0) = packed;
     }
@@ -1709,7 +1723,7 @@ __global__ __launch_bounds__(256) void conv_direct_kernel(const ConvArgs a)
         }
         if (a.acc_out)
             a.acc_out[(size_t)m * a.out_cs + k] = (int32_t)acc;
-        a.y[(size_t)m * a.out_cs + k] = (uint8_t)conv_requant<false>(a, (int32_t)acc);
+        a.y[(size_t)m * a.out_cs + k] = (uint8_t)(a.qmult ? conv_requant_ch(a, (int32_t)acc, k) : conv_requant<false>(a, (int32_t)acc));
     }
 }
 
@@ -1743,7 +1757,7 @@ struct hipq_conv2d_plan {
     bool tile_selected = false;     // hipq_conv2d_plan_select named a tile: the tile kernels, not the streaming kernel
     StreamShape stream = {0, 0, 0}; // explicit shape of the streaming kernel (hipq_conv2d_plan_stream); mb = 0: built-in rule
     bool has_wzp;
-    void *d_w = nullptr, *d_bias = nullptr;
+    void *d_w = nullptr, *d_bias = nullptr, *d_q = nullptr;
     std::string name;
 };
 
@@ -1770,7 +1784,7 @@ static bool pointwise_applies(const hipq_conv2d_plan *p)
     const hipq_conv2d_desc &d = p->d;
     return p->special && p->variant == kMfma && !p->has_wzp && d.R == 1 && d.S == 1 && d.stride_h == 1 && d.stride_w == 1
         && d.pad_h == 0 && d.pad_w == 0 && d.in_cs % 16 == 0 && d.in_cs <= 64 && d.out_cs % 16 == 0 && p->args.kout_pad <= 256
-        && p->args.fastq;
+        && p->args.fastq && p->args.qmult == nullptr;
 }
 
 constexpr int kCUs = 256;
@@ -1825,6 +1839,8 @@ static void set_mfma_name(hipq_conv2d_plan *p, bool smallc)
                  p->has_wzp ? "_wzp" : "", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "",
                  halo_applies(p) ? "_halo" : (!smallc && k2_applies(p)) ? "_k2" : ""); // _k2: unless a residual add is fused
     p->name = nm;
+    if (p->d_q)
+        p->name += "_perchannel";
 }
 
 static int conv_out_dim(int in, int pad, int k, int stride)
@@ -1852,8 +1868,9 @@ static int choose_tile(long long P, int out_cs, bool expand)
     return count(0) >= 200 ? 0 : 3;      // 128x128, or 64x128 when that leaves most CUs idle
 }
 
-extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t *w, const int32_t *bias,
-                                       hipq_conv2d_plan **plan_out)
+// walpha_pc: nullptr, or K weight scales (one per output channel), which replace desc.walpha
+static int plan_create(const hipq_conv2d_desc *dp, const uint8_t *w, const int32_t *bias, const float *walpha_pc,
+                       hipq_conv2d_plan **plan_out)
 {
     clear_error();
     HIPQ_REQUIRE(dp && w && plan_out, "hipq_conv2d_plan_create: null argument");
@@ -1891,7 +1908,25 @@ extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t
         return fail("conv: tensor too large for 32-bit indexing (or empty output)");
     }
     a.P = (int)P;
-    hipq_quant_scale(d.ialpha * d.walpha / d.oalpha, 32, &a.q.mult, &a.q.shift);
+    // per-channel weight scales: one (mult, shift) per output channel, derived exactly like the tensor's pair; the
+    // tensor's own pair is that of channel 0 (what the reference CPU module, which reads walpha[0] only, would use)
+    std::vector<uint32_t> qbuf;
+    if (walpha_pc != nullptr) {
+        const size_t npad = ((size_t)std::max(d.K, d.out_cs) + 127) / 128 * 128;
+        qbuf.assign(2 * npad, 0);
+        for (size_t k = 0; k < npad; k++) {
+            uint32_t m;
+            int sh;
+            hipq_quant_scale(d.ialpha * walpha_pc[k < (size_t)d.K ? k : 0] / d.oalpha, 32, &m, &sh);
+            if (!valid_shift(sh)) {
+                delete p;
+                return fail("conv: requantisation shift %d of channel %zu outside 1..62 (scale %g)", sh, k,
+                            (double)(d.ialpha * walpha_pc[k < (size_t)d.K ? k : 0] / d.oalpha));
+            }
+            qbuf[k] = m, qbuf[npad + k] = (uint32_t)sh;
+        }
+    }
+    hipq_quant_scale(d.ialpha * (walpha_pc ? walpha_pc[0] : d.walpha) / d.oalpha, 32, &a.q.mult, &a.q.shift);
     a.q.zp = sgn ? 0 : d.ozp;
     a.q.hi = (1 << d.obits) - 1;
     // fused ReLU: max(y, ozp); a zero point beyond the saturation value (obits < 8) leaves only that value, as the
@@ -2012,6 +2047,11 @@ extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t
     hipError_t e = hipMalloc(&p->d_w, wbuf.size());
     if (e == hipSuccess)
         e = hipMalloc(&p->d_bias, bbuf.size() * sizeof(int32_t));
+    if (e == hipSuccess && !qbuf.empty()) {
+        e = hipMalloc(&p->d_q, qbuf.size() * sizeof(uint32_t));
+        if (e == hipSuccess)
+            e = hipMemcpy(p->d_q, qbuf.data(), qbuf.size() * sizeof(uint32_t), hipMemcpyHostToDevice);
+    }
     if (e == hipSuccess)
         e = hipMemcpy(p->d_w, wbuf.data(), wbuf.size(), hipMemcpyHostToDevice);
     if (e == hipSuccess)
@@ -2023,8 +2063,30 @@ extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t
     a.wpack = static_cast<const uint8_t *>(p->d_w);
     a.bias2 = static_cast<const int32_t *>(p->d_bias);
     a.padbuf = a.wpack + pad_off;
+    if (p->d_q) {
+        a.qmult = static_cast<const uint32_t *>(p->d_q);
+        a.qshift = reinterpret_cast<const int32_t *>(a.qmult + qbuf.size() / 2);
+        if (p->variant == kMfma || p->variant == kMfmaSmallC)
+            set_mfma_name(p, p->variant == kMfmaSmallC); // the pointwise kernel does not serve per-channel scales
+        else
+            p->name += "_perchannel";
+    }
     *plan_out = p;
     return 0;
+}
+
+extern "C" int hipq_conv2d_plan_create(const hipq_conv2d_desc *dp, const uint8_t *w, const int32_t *bias,
+                                       hipq_conv2d_plan **plan_out)
+{
+    return plan_create(dp, w, bias, nullptr, plan_out);
+}
+
+extern "C" int hipq_conv2d_plan_create_per_channel(const hipq_conv2d_desc *dp, const uint8_t *w, const int32_t *bias,
+                                                   const float *walpha, hipq_conv2d_plan **plan_out)
+{
+    clear_error();
+    HIPQ_REQUIRE(walpha, "hipq_conv2d_plan_create_per_channel: null walpha");
+    return plan_create(dp, w, bias, walpha, plan_out);
 }
 
 extern "C" void hipq_conv2d_plan_destroy(hipq_conv2d_plan *p)
@@ -2035,6 +2097,8 @@ extern "C" void hipq_conv2d_plan_destroy(hipq_conv2d_plan *p)
         (void)hipFree(p->d_w);
     if (p->d_bias)
         (void)hipFree(p->d_bias);
+    if (p->d_q)
+        (void)hipFree(p->d_q);
     delete p;
 }
 
@@ -2241,7 +2305,7 @@ static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_
             hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, false, true>), grid, block, 0, st, a);
     } else if (p->has_wzp) { // rare (asymmetric weights): generic addressing only
         hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, kStages, true, false>), grid, block, 0, st, a);
-    } else if (aligned && a.res != nullptr && a.fastq && a.addq.fast && a.acc_out == nullptr && (a.out_cs & 15) == 0) {
+    } else if (aligned && a.res != nullptr && a.fastq && a.addq.fast && !plain_epilogue(a)) {
         // residual add in the accumulator layout, residual tile prefetched into LDS
         const int ns = p->stages ? p->stages : (a.nslab >= kDeepFrom ? 3 : kStages);
         if (ns >= 4)

@@ -21,6 +21,7 @@ struct QSet {
     uint8_t *zp = nullptr;
     uint8_t *bits = nullptr;
     size_t n = 0;
+    size_t n_alpha = 0; // length of the alpha array alone (a weight scale per output channel has K entries)
 };
 
 void read_qset(op_t *op, uint32_t ia, uint32_t iz, uint32_t ib, QSet *q)
@@ -31,6 +32,7 @@ void read_qset(op_t *op, uint32_t ia, uint32_t iz, uint32_t ib, QSet *q)
     HIPM_CHECK(op_setting_array_get(op, ib, dtUINT8, &n3, &q->bits));
     HIPM_CHECK(q->alpha && q->zp && q->bits && n1 >= 1 && n2 >= 1 && n3 >= 1);
     q->n = n1 < n2 ? n1 : n2;
+    q->n_alpha = n1;
 }
 #define READ_I(op, q) read_qset(op, SETTING_QUANT_IALPHA, SETTING_QUANT_IZERO_POINT, SETTING_QUANT_IBITS, q)
 #define READ_W(op, q) read_qset(op, SETTING_QUANT_WALPHA, SETTING_QUANT_WZERO_POINT, SETTING_QUANT_WBITS, q)
@@ -110,6 +112,7 @@ struct conv_op_t {
     hipq_conv2d_plan *plan;
     hipq_conv2d_desc desc; // what the plan was built for (re-used when prepare is called again unchanged)
     const void *w_seen;    // identity of the weights the plan was packed from
+    uint64_t pc_seen;      // checksum of the per-channel weight scales the plan was built with (0: per tensor)
     int defer;             // 0 undecided, 1 leave the launch to the add / relu that reads the output, -1 launch at run()
 };
 
@@ -203,11 +206,27 @@ void conv_run(op_t *op)
     HIPM_HIPQ(hipq_conv2d_run(c->plan, in_ptr(op, 0), out_ptr(op), nullptr, op_stream(op)));
 }
 
+// A walpha array with one entry per output channel (and more than one channel) selects per-channel requantisation, the
+// convention of the reference's CUDA sibling (cuda_quant/src/op/conv_2d_quant.cu:751-764); a single entry is the
+// per-tensor scale the reference CPU module reads (conv_2d_uint8_impl.c:57-66).
+const float *per_channel_walpha(const conv_op_t *c)
+{
+    return c->num_output > 1 && c->qw.n_alpha == c->num_output ? c->qw.alpha : nullptr;
+}
+
 void build_plan(op_t *op, const hipq_conv2d_desc &d, const uint8_t *w, const void *w_id)
 {
     conv_op_t *c = reinterpret_cast<conv_op_t *>(op);
     c->defer = 0; // decided at the next run, when every operator of the pass has been prepared
-    if (c->plan && memcmp(&c->desc, &d, sizeof d) == 0 && c->w_seen == w_id)
+    const float *wa_pc = per_channel_walpha(c);
+    uint64_t pc_id = 0;
+    if (wa_pc) {
+        pc_id = 1469598103934665603ull;
+        for (size_t i = 0; i < c->num_output * sizeof(float); ++i)
+            pc_id = (pc_id ^ reinterpret_cast<const uint8_t *>(wa_pc)[i]) * 1099511628211ull;
+        pc_id |= 1;
+    }
+    if (c->plan && memcmp(&c->desc, &d, sizeof d) == 0 && c->w_seen == w_id && c->pc_seen == pc_id)
         return; // prepare is called again after a reshape (art/src/parade.c:199-215): nothing changed
     hipq_conv2d_plan_destroy(c->plan);
     c->plan = nullptr;
@@ -218,9 +237,13 @@ void build_plan(op_t *op, const hipq_conv2d_desc &d, const uint8_t *w, const voi
                                                 ? hip_mem_host_in(op->input_tensors[2]->mem)
                                                 : mem_cpu_data(op->input_tensors[2]->mem));
     } // without a bias the accumulator starts at zero (the reference reads an unset buffer there)
-    HIPM_HIPQ(hipq_conv2d_plan_create(&d, w, bias, &c->plan));
+    if (wa_pc)
+        HIPM_HIPQ(hipq_conv2d_plan_create_per_channel(&d, w, bias, wa_pc, &c->plan));
+    else
+        HIPM_HIPQ(hipq_conv2d_plan_create(&d, w, bias, &c->plan));
     c->desc = d;
     c->w_seen = w_id;
+    c->pc_seen = pc_id;
     op->run_func = conv_run;
 }
 

@@ -39,6 +39,8 @@ _SIGS = {
     "hipq_nchw_to_nhwc_u8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_void_p]),
     "hipq_nhwc_to_nchw_u8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_void_p]),
     "hipq_conv2d_plan_create": (C.c_int, [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p)]),
+    "hipq_conv2d_plan_create_per_channel": (C.c_int, [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.c_void_p,
+                                                      C.POINTER(C.c_void_p)]),
     "hipq_conv2d_plan_destroy": (None, [C.c_void_p]),
     "hipq_conv2d_plan_kernel": (C.c_char_p, [C.c_void_p]),
     "hipq_conv2d_plan_select": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
@@ -139,8 +141,14 @@ class Conv2d:
 
     def __init__(self, x_shape, w, bias, pad, stride, group, ialpha, izp, walpha, wzp, oalpha, ozp, obits=8,
                  relu=False, in_cs=None, out_cs=None, dtype=DTYPE_U8):
-        """dtype=DTYPE_I8: int8 symmetric tensors (w is an int8 array, zero points are ignored)."""
+        """dtype=DTYPE_I8: int8 symmetric tensors (w is an int8 array, zero points are ignored).
+        walpha: a float, or an array of K floats = one weight scale per output channel."""
         N, Cc, H, W = x_shape
+        wa_pc = None
+        if not np.isscalar(walpha):
+            wa_pc = np.ascontiguousarray(walpha, np.float32).reshape(-1)
+            assert wa_pc.size == np.asarray(w).shape[0], "one weight scale per output channel"
+            walpha = float(wa_pc[0])
         w = np.ascontiguousarray(w, np.int8 if dtype == DTYPE_I8 else np.uint8)
         K, _, R, S = w.shape
         ph, pw = (pad, pad) if np.isscalar(pad) else pad
@@ -153,8 +161,12 @@ class Conv2d:
         self.OH, self.OW = conv_out_dim(H, ph, R, sh), conv_out_dim(W, pw, S, sw)
         b = None if bias is None else np.ascontiguousarray(bias, np.int32)
         h = C.c_void_p()
-        check(lib().hipq_conv2d_plan_create(C.byref(d), C.c_void_p(w.ctypes.data),
-                                            C.c_void_p(b.ctypes.data) if b is not None else None, C.byref(h)))
+        bp = C.c_void_p(b.ctypes.data) if b is not None else None
+        if wa_pc is None:
+            check(lib().hipq_conv2d_plan_create(C.byref(d), C.c_void_p(w.ctypes.data), bp, C.byref(h)))
+        else:
+            check(lib().hipq_conv2d_plan_create_per_channel(C.byref(d), C.c_void_p(w.ctypes.data), bp,
+                                                            C.c_void_p(wa_pc.ctypes.data), C.byref(h)))
         self.handle = h
         self.kernel = lib().hipq_conv2d_plan_kernel(h).decode()
         m = re.match(r"conv_mfma_i8_(\d+x\d+)", self.kernel)

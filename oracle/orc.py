@@ -33,6 +33,10 @@ def lib():
         L.orc_fnv1a64.restype = C.c_uint64
         L.orc_fnv1a64.argtypes = [C.c_void_p, C.c_size_t]
         L.orc_quant_scale.argtypes = [C.c_float, C.c_int, C.POINTER(C.c_uint32), C.POINTER(C.c_int)]
+        L.orc_requant_per_channel_u8.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_float,
+                                                 C.c_void_p, C.c_float, C.c_int, C.c_int]
+        L.orc_requant_per_channel_i8.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_float,
+                                                 C.c_void_p, C.c_float, C.c_int]
         _LIB = L
     return _LIB
 
@@ -239,6 +243,36 @@ def dequantize_i8(x, ialpha):
     y = np.empty(x.shape, np.float32)
     lib().orc_dequantize_i8(_p(x), _p(y), C.c_size_t(x.size), _f(ialpha))
     return y
+
+
+def requant_per_channel_u8(acc, ialpha, walpha, oalpha, ozp, obits=8):
+    """acc: int32 [N, K, ...] (or [M, K]); walpha: K floats.  See quant_oracle.h."""
+    acc = np.ascontiguousarray(acc, np.int32)
+    wa = np.ascontiguousarray(walpha, np.float32).reshape(-1)
+    outer, K = acc.shape[0], acc.shape[1]
+    assert wa.size == K
+    inner = int(np.prod(acc.shape[2:])) if acc.ndim > 2 else 1
+    y = np.empty(acc.shape, np.uint8)
+    lib().orc_requant_per_channel_u8(_p(acc), _p(y), outer, K, inner, _f(ialpha), _p(wa), _f(oalpha), int(ozp), int(obits))
+    return y
+
+
+def requant_per_channel_i8(acc, ialpha, walpha, oalpha, obits=8):
+    acc = np.ascontiguousarray(acc, np.int32)
+    wa = np.ascontiguousarray(walpha, np.float32).reshape(-1)
+    outer, K = acc.shape[0], acc.shape[1]
+    assert wa.size == K
+    inner = int(np.prod(acc.shape[2:])) if acc.ndim > 2 else 1
+    y = np.empty(acc.shape, np.int8)
+    lib().orc_requant_per_channel_i8(_p(acc), _p(y), outer, K, inner, _f(ialpha), _p(wa), _f(oalpha), int(obits))
+    return y
+
+
+def conv2d_u8_per_channel(x, w, bias, pad, stride, group, ialpha, izp, walpha, wzp, oalpha, ozp, obits=8):
+    """walpha: K floats.  The accumulators do not depend on the scales."""
+    _, acc = conv2d_u8(x, w, bias, pad, stride, group, ialpha, izp, float(np.float32(walpha[0])), wzp, oalpha, ozp, obits,
+                       return_acc=True)
+    return requant_per_channel_u8(acc, ialpha, walpha, oalpha, ozp, obits)
 
 
 class XorShift:

@@ -452,6 +452,37 @@ static inline int8_t requant_acc_i8(int32_t acc, uint32_t mult, int shift, int o
     return orc_ssat_bits((int32_t)orc_rshift_rn((int64_t)acc * (int64_t)mult, shift), obits);
 }
 
+/* per-channel weight scales: the epilogues above with (mult, shift) = get_quant_scale_int32(ialpha * walpha[k] / oalpha) */
+void orc_requant_per_channel_u8(const int32_t *acc, uint8_t *y, size_t outer, size_t K, size_t inner, float ialpha,
+                                const float *walpha, float oalpha, int ozp, int obits)
+{
+    for (size_t k = 0; k < K; k++) {
+        uint32_t mult;
+        int shift;
+        orc_quant_scale(ialpha * walpha[k] / oalpha, 32, &mult, &shift);
+        for (size_t o = 0; o < outer; o++)
+            for (size_t i = 0; i < inner; i++) {
+                const size_t at = (o * K + k) * inner + i;
+                y[at] = requant_acc(acc[at], mult, shift, ozp, obits);
+            }
+    }
+}
+
+void orc_requant_per_channel_i8(const int32_t *acc, int8_t *y, size_t outer, size_t K, size_t inner, float ialpha,
+                                const float *walpha, float oalpha, int obits)
+{
+    for (size_t k = 0; k < K; k++) {
+        uint32_t mult;
+        int shift;
+        orc_quant_scale(ialpha * walpha[k] / oalpha, 32, &mult, &shift);
+        for (size_t o = 0; o < outer; o++)
+            for (size_t i = 0; i < inner; i++) {
+                const size_t at = (o * K + k) * inner + i;
+                y[at] = requant_acc_i8(acc[at], mult, shift, obits);
+            }
+    }
+}
+
 /* op_conv_2d_i8xi8_run — conv_2d_int8_impl.c:34-174 with im2col_i8 (utils/im2col.cpp:22-116: out-of-image taps
  * are 0) and the portable branch of gemm_i8xi8 (gemm/default/gemm.c:257-303: int32 += int8 * int8). */
 void orc_conv2d_i8(const int8_t *x, const int8_t *w, const int32_t *bias, int8_t *y, int32_t *acc_out, int N,

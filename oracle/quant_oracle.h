@@ -116,6 +116,17 @@ void orc_quantize_i8(const float *x, int8_t *y, size_t count, float oalpha, int 
 /* op_dequantize_run_i8 — dequantize.c:125-136. */
 void orc_dequantize_i8(const int8_t *x, float *y, size_t count, float ialpha);
 
+/* Per-channel weight scales.  The reference CPU module reads walpha[0] only (conv_2d_uint8_impl.c:57-66); its CUDA
+ * sibling forms one scale ialpha * walpha[k] / oalpha per output channel (cuda_quant/src/op/conv_2d_quant.cu:751-764).
+ * This is the CPU module's epilogue (conv_2d_uint8_impl.c:159-164 / conv_2d_int8_impl.c:148-172) with its (mult, shift)
+ * pair derived per channel by get_quant_scale_int32: acc is [outer, K, inner] int32 (NCHW accumulators: outer = N,
+ * inner = OH*OW; inner-product accumulators: outer = M, inner = 1).  Pinned by tests/test_oracle.py: equal scales give
+ * the per-tensor functions' bytes, and exact rational rounding per channel. */
+void orc_requant_per_channel_u8(const int32_t *acc, uint8_t *y, size_t outer, size_t K, size_t inner, float ialpha,
+                                const float *walpha, float oalpha, int ozp, int obits);
+void orc_requant_per_channel_i8(const int32_t *acc, int8_t *y, size_t outer, size_t K, size_t inner, float ialpha,
+                                const float *walpha, float oalpha, int obits);
+
 /* FNV-1a-64 over a byte buffer (the checksum the recorded known answers use). */
 uint64_t orc_fnv1a64(const uint8_t *p, size_t n);
 

@@ -254,6 +254,62 @@ def test_output_stride_wider_than_the_channels():
             assert np.array_equal(got, want), (out_cs, plan.kernel)
 
 
+def test_per_channel_weight_scales():
+    """One weight scale per output channel (hipq_conv2d_plan_create_per_channel): every kernel family against the
+    oracle's per-channel requantisation; K equal scales give the per-tensor plan's bytes; the fused add, the run-time
+    ReLU, accumulator dumps, int8 tensors and the fully-connected kernel work on such plans."""
+    rng = np.random.default_rng(143)
+    #        N   C    H   W   K   R  pad st group
+    cases = [(2, 64, 14, 14, 64, 3, 1, 1, 1), (1, 3, 33, 33, 24, 7, 3, 2, 1), (3, 32, 9, 9, 96, 1, 0, 1, 1),
+             (2, 256, 7, 7, 128, 1, 0, 1, 1), (2, 32, 12, 12, 32, 3, 1, 1, 32), (1, 48, 11, 11, 48, 3, 1, 2, 48),
+             (1, 24, 7, 7, 24, 5, 2, 1, 24), (1, 16, 8, 8, 32, 3, 1, 1, 4), (40, 256, 1, 1, 100, 1, 0, 1, 1)]
+    kerns = set()
+    for N, C, H, W, K, R, pad, st, grp in cases:
+        print("per-channel case", N, C, H, W, K, R, pad, st, grp, flush=True)
+        x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+        w = rng.integers(0, 256, (K, C // grp, R, R), dtype=np.uint8)
+        b = rng.integers(-3000, 3000, K).astype(np.int32)
+        ia, izp, wzp, ozp = rand_q(rng), int(rng.integers(0, 256)), 128, int(rng.integers(0, 256))
+        wa = np.exp(rng.uniform(np.log(1e-3), np.log(3e-2), K)).astype(np.float32)
+        oa = float(np.float32(ia * 5e-3 * np.sqrt(C // grp * R * R) * 60.0))
+        want = orc.conv2d_u8_per_channel(x, w, b, pad, st, grp, ia, izp, wa, wzp, oa, ozp)
+        _, want_acc = orc.conv2d_u8(x, w, b, pad, st, grp, ia, izp, float(wa[0]), wzp, oa, ozp, return_acc=True)
+        plan = hipq.Conv2d(x.shape, w, b, pad, st, grp, ia, izp, wa, wzp, oa, ozp)
+        assert plan.kernel.endswith("_perchannel"), plan.kernel
+        kerns.add(plan.kernel)
+        xd = hipq.to_device_nhwc(x)
+        acc = torch.zeros((N, plan.OH, plan.OW, plan.desc.out_cs), dtype=torch.int32, device="cuda")
+        got = hipq.from_device_nhwc(plan(xd, acc=acc), K)
+        assert np.array_equal(acc.cpu().numpy()[..., :K].transpose(0, 3, 1, 2), want_acc), plan.kernel
+        assert np.array_equal(got, want), (plan.kernel, int((got != want).sum()))
+        assert np.array_equal(hipq.from_device_nhwc(plan(xd), K), want), plan.kernel  # without the dump
+        assert len(np.unique(want)) > 8
+        # run-time ReLU
+        assert np.array_equal(hipq.from_device_nhwc(plan.run_relu(xd), K), np.maximum(want, ozp)), plan.kernel
+        # K equal scales == the per-tensor plan
+        same = np.full(K, wa[0], np.float32)
+        p_same = hipq.Conv2d(x.shape, w, b, pad, st, grp, ia, izp, same, wzp, oa, ozp)
+        p_tensor = hipq.Conv2d(x.shape, w, b, pad, st, grp, ia, izp, float(wa[0]), wzp, oa, ozp)
+        assert torch.equal(p_same(xd)[..., :K], p_tensor(xd)[..., :K]), plan.kernel
+        if grp == 1:  # fused residual add on a per-channel plan
+            res = rng.integers(0, 256, want.shape, dtype=np.uint8)
+            ra, rz, sa, sz = rand_q(rng, 1e-2, 1e-1), int(rng.integers(0, 256)), rand_q(rng, 3e-2, 3e-1), int(rng.integers(0, 256))
+            yd = plan.run_add(xd, hipq.to_device_nhwc(res), False, ra, rz, sa, sz, plan.empty_output())
+            assert np.array_equal(hipq.from_device_nhwc(yd, K), orc.add_u8(want, res, oa, ozp, ra, rz, sa, sz)), plan.kernel
+    assert any("stream" in k for k in kerns) and any("depthwise3x3" in k for k in kerns) and any("_c4" in k for k in kerns), kerns
+    assert "conv_depthwise_u8_perchannel" in kerns and "conv_direct_u8_perchannel" in kerns, kerns
+    # int8 symmetric tensors
+    x = rng.integers(-128, 128, (2, 64, 9, 9), dtype=np.int8)
+    w = rng.integers(-128, 128, (80, 64, 3, 3), dtype=np.int8)
+    b = rng.integers(-3000, 3000, 80).astype(np.int32)
+    wa = np.exp(rng.uniform(np.log(1e-3), np.log(3e-2), 80)).astype(np.float32)
+    _, acc8 = orc.conv2d_i8(x, w, b, 1, 1, 1, 0.02, float(wa[0]), 9.0, 7, return_acc=True)
+    want8 = orc.requant_per_channel_i8(acc8, 0.02, wa, 9.0, 7)
+    p8 = hipq.Conv2d(x.shape, w, b, 1, 1, 1, 0.02, 0, wa, 0, 9.0, 0, obits=7, dtype=hipq.DTYPE_I8)
+    assert np.array_equal(hipq.from_device_nhwc(p8(hipq.to_device_nhwc(x)), 80).view(np.int8), want8), p8.kernel
+    assert len(np.unique(want8)) > 8
+
+
 def test_elementwise():
     rng = np.random.default_rng(15)
     for n in (1, 15, 16, 4099, 64 * 56 * 56 * 16 + 3):

@@ -124,6 +124,35 @@ def test_single_ops_through_the_op_api(own_rt):
     ws.delete()
 
 
+def test_per_channel_weight_scales_through_the_op_api(own_rt):
+    """A walpha array with one entry per output channel selects per-channel requantisation (the convention of the
+    reference's CUDA module, cuda_quant/src/op/conv_2d_quant.cu:751-764); one entry stays per tensor.  conv_2d and ip."""
+    from oracle import orc
+    ws = own_rt.workspace("hip")
+    rng = np.random.default_rng(12)
+    x = rng.integers(0, 256, (2, 24, 9, 11), dtype=np.uint8)
+    w = rng.integers(0, 256, (40, 24, 3, 3), dtype=np.uint8)
+    b = rng.integers(-5000, 5000, 40).astype(np.int32)
+    wa = np.exp(rng.uniform(np.log(1e-3), np.log(2e-2), 40)).astype(np.float32)
+    q = dict(ialpha=0.031, izp=77, walpha=wa, wzp=128, oalpha=0.9, ozp=13)
+    tx, tw, tb = ws.tensor(x), ws.tensor(w), ws.tensor(b)
+    conv = ws.conv2d(tx, tw, tb, 1, 2, 1, q).prepare().run()
+    want = orc.conv2d_u8_per_channel(x, w, b, 1, 2, 1, 0.031, 77, wa, 128, 0.9, 13)
+    assert same_bits(conv.output(0).numpy(), want) and len(np.unique(want)) > 8
+    conv.prepare().run()  # prepared again with the same scales: the plan is kept
+    assert same_bits(conv.output(0).numpy(), want)
+    xf = rng.integers(0, 256, (6, 256), dtype=np.uint8)
+    wf = rng.integers(0, 256, (37, 256), dtype=np.uint8)
+    waf = np.exp(rng.uniform(np.log(1e-3), np.log(2e-2), 37)).astype(np.float32)
+    ip = ws.ip(ws.tensor(xf), ws.tensor(wf), None, dict(ialpha=0.02, izp=128, walpha=waf, wzp=128, oalpha=2.5, ozp=100)).prepare().run()
+    _, acc = orc.ip_u8(xf, wf, None, 0.02, 128, float(waf[0]), 128, 2.5, 100, return_acc=True)
+    want_ip = orc.requant_per_channel_u8(acc, 0.02, waf, 2.5, 100)
+    assert same_bits(ip.output(0).numpy().reshape(6, 37), want_ip) and len(np.unique(want_ip)) > 8
+    for o in (ip, conv):
+        o.delete()
+    ws.delete()
+
+
 def test_convolution_and_add_run_as_one_kernel(own_rt):
     """A convolution whose output only an add reads leaves its launch to that add (one fused kernel, the convolution's
     output is never written); whoever asks for the elided tensor afterwards gets it computed on demand.  Results are

@@ -475,3 +475,34 @@ def test_concat_and_softmax_closed_forms():
     # along another axis the same numbers appear with the axes swapped
     xt = np.ascontiguousarray(x.transpose(0, 2, 1, 3))
     assert np.array_equal(orc.softmax_u8(xt, 2, 0.05, 128, 1.0 / 255, 0).transpose(0, 2, 1, 3), y)
+
+
+def test_per_channel_requantisation_is_pinned():
+    """Per-channel weight scales (no counterpart in the reference CPU module, which reads walpha[0]): (a) with K equal
+    scales the bytes are those of the per-tensor functions, which the compiled reference pins; (b) every channel equals
+    exact rational rounding with ITS scale ialpha * walpha[k] / oalpha (fp32 operations in that order)."""
+    rng = np.random.default_rng(77)
+    N, C, H, W, K = 2, 6, 7, 5, 9
+    x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+    w = rng.integers(0, 256, (K, C, 3, 3), dtype=np.uint8)
+    b = rng.integers(-3000, 3000, K).astype(np.int32)
+    ia, izp, wzp, oa, ozp = 0.021, 117, 131, 0.37, 11
+    same = np.full(K, 0.0043, np.float32)
+    y_t, acc = orc.conv2d_u8(x, w, b, 1, 1, 1, ia, izp, float(same[0]), wzp, oa, ozp, return_acc=True)
+    assert np.array_equal(orc.conv2d_u8_per_channel(x, w, b, 1, 1, 1, ia, izp, same, wzp, oa, ozp), y_t)
+    wa = np.exp(rng.uniform(np.log(5e-4), np.log(5e-2), K)).astype(np.float32)
+    y = orc.conv2d_u8_per_channel(x, w, b, 1, 1, 1, ia, izp, wa, wzp, oa, ozp)
+    assert len(np.unique(y)) > 20
+    for k in range(K):
+        scale = np.float32(np.float32(ia) * wa[k]) / np.float32(oa)
+        assert np.array_equal(y[:, k], _requant(acc[:, k], scale, ozp)), k
+        # and each channel alone is the per-tensor function with that channel's scale
+        y_k = orc.conv2d_u8(x, w, b, 1, 1, 1, ia, izp, float(wa[k]), wzp, oa, ozp)
+        assert np.array_equal(y[:, k], y_k[:, k]), k
+    # int8 symmetric
+    xs, ws = x.view(np.int8), w.view(np.int8)
+    y8_t, acc8 = orc.conv2d_i8(xs, ws, b, 1, 1, 1, ia, float(same[0]), oa, 7, return_acc=True)
+    assert np.array_equal(orc.requant_per_channel_i8(acc8, ia, same, oa, 7), y8_t)
+    y8 = orc.requant_per_channel_i8(acc8, ia, wa, oa, 7)
+    for k in range(K):
+        assert np.array_equal(y8[:, k], orc.conv2d_i8(xs, ws, b, 1, 1, 1, ia, float(wa[k]), oa, 7)[:, k]), k
