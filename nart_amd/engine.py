@@ -152,7 +152,7 @@ class Parade:
     class _Param(C.Structure):
         _fields_ = [("workspaces", C.POINTER(C.POINTER(art.workspace_t))), ("input_mem_tp", C.POINTER(art.mem_tp))]
 
-    def __init__(self, rt, data, workspaces, input_workspace=None):
+    def __init__(self, rt, data, workspaces, input_workspace=None, prepare=True):
         core = rt.core
         self.rt, self.workspaces = rt, list(workspaces)
         pos = [0]
@@ -184,7 +184,8 @@ class Parade:
         self.ptr = core.deserialize_parade(buf, C.byref(param))
         core.nart_buffer_delete(buf)
         assert self.ptr, "deserialize_parade failed"
-        core.parade_prepare(self.ptr)
+        if prepare:
+            core.parade_prepare(self.ptr)
 
     def transform_param(self):
         """(operators, means, stds, paddings) of input 0's pre-processing block (parade_get_transfrom_param, parade.c:128-138;

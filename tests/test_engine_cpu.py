@@ -252,3 +252,23 @@ def test_malformed_engine_file_aborts_instead_of_overrunning(how, tmp_path):
     r = subprocess.run([sys.executable, str(script), ROOT, how], stdout=subprocess.PIPE, stderr=subprocess.PIPE, timeout=120)
     assert b"loading" in r.stdout and b"returned" not in r.stdout
     assert r.returncode == -signal.SIGABRT, (r.returncode, r.stderr[-500:])
+
+
+def test_art_compat_surface_without_a_gpu():
+    """nart_amd.art_compat offers the names of the reference's `nart.art` package (python/nart/art/__init__.py:31-73);
+    without a GPU the `hip` module cannot make a workspace, which is reported like any module that fails to load."""
+    from nart_amd import art_compat
+    for name in ("RuntimeContext", "Parade", "create_context_from_json", "create_context_for_target", "load_parade",
+                 "get_empty_io", "set_package_dir"):
+        assert hasattr(art_compat, name), name
+    for name in ("run", "forward", "reshape", "input_shapes", "output_shapes", "input_dtypes", "output_dtypes",
+                 "get_tensor_shape", "get_tensor_dtype", "get_input_names", "get_output_names", "get_raw_tensor_data"):
+        assert callable(getattr(art_compat.Parade, name)), name
+    try:
+        import torch
+        if torch.cuda.is_available():
+            return
+    except ImportError:
+        pass
+    with pytest.raises(RuntimeError, match="none of the modules"):
+        art_compat.RuntimeContext(["no_such_module"], "no_such_module")
