@@ -10,7 +10,7 @@
  *     not installed (the GPU test box).
  * Everything here is ABI: field order, field types, enum values, symbol names.  The reference builds
  * with ART_CONSTRAINT_WITH_NAME (top-level CMakeLists.txt:19), so setting_constraint_t carries `name`.
- * tests/test_art_abi.py compiles a probe against BOTH header sets and compares every size and offset.
+ * tests/test_engine_cpu.py compiles a probe against BOTH header sets and compares every size and offset.
  */
 #ifndef NART_HIP_ART_H
 #define NART_HIP_ART_H

@@ -37,6 +37,7 @@ static void hm_free(mem_t *mm)
     m->host = m->dev = m->stage = nullptr;
     m->host_cap = m->dev_cap = m->stage_cap = m->size = 0;
     m->host_valid = m->dev_valid = false;
+    m->up_pending = false;
     m->pending = nullptr;
 }
 
@@ -65,6 +66,10 @@ static void ensure_host(hip_mem_t *m)
     HIPM_HIP(hipHostMalloc(&p, m->size ? m->size : 1, hipHostMallocDefault));
     memset(p, 0, m->size);
     if (m->host) {
+        if (m->up_pending) { // an upload may still read the old mirror
+            HIPM_HIP(hipStreamSynchronize(m->up_stream));
+            m->up_pending = false;
+        }
         memcpy(p, m->host, m->host_cap);
         HIPM_HIP(hipHostFree(m->host));
     }
@@ -97,6 +102,17 @@ static void upload(hip_mem_t *m, hipStream_t st)
         HIPM_HIP(hipMemcpyAsync(m->dev, m->host, m->size, hipMemcpyHostToDevice, st));
     }
     m->dev_valid = true;
+    m->up_pending = true; // the copy still reads the mirror
+    m->up_stream = st;
+}
+
+// the mirror is about to be handed out for writing: an upload that still reads it must finish first
+static void finish_upload(hip_mem_t *m)
+{
+    if (m->up_pending) {
+        HIPM_HIP(hipStreamSynchronize(m->up_stream));
+        m->up_pending = false;
+    }
 }
 
 // mem_cpu_data(): the caller may read or WRITE through the pointer (the runtime fills inputs and weights this
@@ -110,6 +126,7 @@ static void *hm_cpu_data(const mem_t *mm)
         download(m);
     }
     ensure_host(m);
+    finish_upload(m);
     m->host_valid = true;
     m->dev_valid = false;
     return m->host;
@@ -155,7 +172,10 @@ static void *hm_data(const mem_t *mm)
 {
     mem_t *m = const_cast<mem_t *>(mm);
     const void *p = hip_mem_dev_in(m, nullptr);
-    HIPM_HIP(hipStreamSynchronize(nullptr));
+    // the caller is foreign code with streams of its own: every producer of this memory (kernels on a workspace
+    // stream, a settled convolution, the upload on the null stream) must have finished
+    HIPM_HIP(hipDeviceSynchronize());
+    as_hip(m)->up_pending = false;
     as_hip(m)->host_valid = false;
     return const_cast<void *>(p);
 }
@@ -200,8 +220,10 @@ void hip_mem_tag(tensor_t *t)
             m->pending = nullptr;
             m->dev_valid = false;
         }
-        if (m->dev_valid && !m->host_valid && m->dev)
+        if (m->dev_valid && !m->host_valid && m->dev) {
+            HIPM_HIP(hipDeviceSynchronize()); // the producing kernels run on a workspace stream
             download(m);
+        }
         m->dev_valid = false;
         m->layout = layout;
         m->N = N, m->C = C, m->H = H, m->W = W;

@@ -83,6 +83,10 @@ struct hip_mem_t {
     hip_layout_t layout;
     int N, C, H, W, cs; // geometry for HIP_LAYOUT_NHWC_U8
     bool host_valid, dev_valid;
+    // An upload reads the pinned mirror asynchronously on `up_stream`: the mirror may only be handed out for writing
+    // once that copy has finished.
+    bool up_pending;
+    hipStream_t up_stream;
     // Deferred producer.  A convolution whose only reader is an add does not launch at its own run(): it leaves this
     // hook, and the add runs both as one fused kernel (hip_ops.cpp).  Whoever else asks for the contents first - the
     // host, another workspace, a re-run - makes the hook launch the plain convolution into `dev` (hip_mem_settle).

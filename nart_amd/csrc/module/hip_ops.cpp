@@ -38,6 +38,24 @@ void read_qset(op_t *op, uint32_t ia, uint32_t iz, uint32_t ib, QSet *q)
 #define READ_W(op, q) read_qset(op, SETTING_QUANT_WALPHA, SETTING_QUANT_WZERO_POINT, SETTING_QUANT_WBITS, q)
 #define READ_O(op, q) read_qset(op, SETTING_QUANT_OALPHA, SETTING_QUANT_OZERO_POINT, SETTING_QUANT_OBITS, q)
 
+// The device geometry of a tensor's memory is its producer's (a reshape that keeps the element count does not move
+// bytes, hip_mem_tag).  An operator that takes N/C/H/W from the tensor's SHAPE but strides from the memory must see
+// the two agree: a reshape that regroups channels and pixels (channel shuffle, space-to-depth) in front of it would
+// otherwise compute on the wrong layout; like every unsupported case, it aborts.
+void same_shape_and_geometry(const op_t *op, const tensor_t *t)
+{
+    const hip_mem_t *m = as_hip(t->mem);
+    const shape_t &s = t->shape;
+    const bool ok = m->layout == HIP_LAYOUT_NHWC_U8 && s.dim_size == 4 && m->N == (int)s.dim[0] && m->C == (int)s.dim[1]
+        && m->H == (int)s.dim[2] && m->W == (int)s.dim[3];
+    if (!ok) {
+        fprintf(stderr, "[hip module] %s: tensor %s has shape [%u, %u, %u, %u] but its memory holds [%d, %d, %d, %d]: a "
+                        "reshape that regroups channels and pixels in front of this operator is not implemented\n",
+                op->entry->tp->name, t->name ? t->name : "?", s.dim[0], s.dim[1], s.dim[2], s.dim[3], m->N, m->C, m->H, m->W);
+        abort();
+    }
+}
+
 void alloc_and_tag(op_t *op)
 {
     for (size_t i = 0; i < op->input_size; ++i) {
@@ -267,6 +285,7 @@ void conv_prepare(op_t *op)
     const shape_t &xs = op->input_tensors[0]->shape;
     const hip_mem_t *xm = as_hip(op->input_tensors[0]->mem), *ym = as_hip(op->output_tensors[0].mem);
     HIPM_CHECK(xs.dim_size == 4 && xm->layout == HIP_LAYOUT_NHWC_U8 && ym->layout == HIP_LAYOUT_NHWC_U8);
+    same_shape_and_geometry(op, op->input_tensors[0]);
     hipq_conv2d_desc d;
     memset(&d, 0, sizeof d);
     d.N = (int)xs.dim[0], d.C = (int)xs.dim[1], d.H = (int)xs.dim[2], d.W = (int)xs.dim[3];
@@ -531,6 +550,8 @@ void concat_prepare(op_t *op)
     for (size_t i = 0; i < op->input_size; ++i) {
         const hip_mem_t *x = as_hip(op->input_tensors[i]->mem);
         HIPM_CHECK(x->layout == HIP_LAYOUT_NHWC_U8 && x->N == y->N && x->H == y->H && x->W == y->W);
+        if (op->input_tensors[i]->shape.dim_size == 4)
+            same_shape_and_geometry(op, op->input_tensors[i]);
     }
     op->run_func = concat_run;
 }
@@ -562,6 +583,8 @@ void softmax_prepare(op_t *op)
         abort();
     }
     HIPM_CHECK(as_hip(op->input_tensors[0]->mem)->layout == HIP_LAYOUT_NHWC_U8);
+    if (op->input_tensors[0]->shape.dim_size == 4)
+        same_shape_and_geometry(op, op->input_tensors[0]);
     op->run_func = softmax_run;
 }
 
@@ -603,6 +626,7 @@ void pool_prepare(op_t *op)
     require_hip_u8(op, 1);
     alloc_and_tag(op);
     HIPM_CHECK(op->input_tensors[0]->shape.dim_size == 4);
+    same_shape_and_geometry(op, op->input_tensors[0]);
     op->run_func = pool_run;
 }
 

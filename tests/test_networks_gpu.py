@@ -202,3 +202,25 @@ def test_full_size_reruns_are_identical(build):
         ex.replay()
         torch.cuda.synchronize()
         assert torch.equal(first[case.output.name], ex.buf[case.output.name]), "graph replay %d" % it
+
+
+@pytest.mark.parametrize("name,build,batch", [("resnet18", cases.resnet18, 32), ("mobilenetv2", cases.mobilenet_v2, 64)],
+                         ids=["resnet18_n32", "mobilenetv2_n64"])
+def test_full_size_batches_against_the_oracle(name, build, batch):
+    """BASELINE configs[2] at its batch of 32 and configs[3] at its batch of 64, 224x224: the first and the last image
+    of the batch carry the oracle's values in every tensor (the reference convolution runs one image at a time anyway,
+    conv_2d_uint8_impl.c:104)."""
+    case = build(N=batch)
+    ex = HipqExecutor(case, fuse_add=True)
+    x = case_oracle.random_input(case, seed=12)
+    ex.set_input(x)
+    ex.run()
+    torch.cuda.synchronize()
+    case1 = build(N=1)
+    for i in (0, batch - 1):
+        vals = case_oracle.run_case(case1, x[i:i + 1])
+        for node in case.nodes:
+            if node.output in ex.fused:
+                continue
+            got, want = ex.fetch(node.output)[i:i + 1], vals[node.output]
+            assert np.array_equal(np.ascontiguousarray(got).view(np.uint8), want.view(np.uint8)), (name, i, node.kind, node.output)
