@@ -51,14 +51,54 @@ def build_hipq(force=False):
     if not force and _newer(out, deps):
         return out
     os.makedirs(LIB, exist_ok=True)
-    objs = []
+    objs, usage = [], {}
     for s in srcs:
         o = os.path.join(LIB, "obj_hipq_" + os.path.basename(s) + ".o")
         lang = ["-x", "hip"] if s.endswith(".hip") else []
-        _run([HIPCC] + HIP_FLAGS + ["-I" + INC, "-I" + os.path.join(CSRC, "hipq"), "-c"] + lang + [s, "-o", o])
+        cmd = [HIPCC] + HIP_FLAGS + ["-I" + INC, "-I" + os.path.join(CSRC, "hipq"), "-c"] + lang + [s, "-o", o]
+        if s.endswith(".hip"):
+            usage.update(_compile_with_usage(cmd))
+        else:
+            _run(cmd)
         objs.append(o)
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + objs)
+    import json
+    with open(os.path.join(LIB, "kernel_resources.json"), "w") as f:
+        json.dump(usage, f, indent=0, sort_keys=True)
     return out
+
+
+def _compile_with_usage(cmd):
+    """Compile one HIP source with the compiler's per-kernel resource remarks switched on and return
+    {mangled kernel name: {"vgprs", "scratch", "lds", "occupancy"}}.  A kernel that uses scratch memory (a register
+    array that the optimiser could not keep in registers, or spills) fails the build: every kernel here is written to
+    live in registers, and one careless edit of a shared epilogue has cost the largest tiles a factor of three."""
+    import re
+    cmd = cmd + ["-Rpass-analysis=kernel-resource-usage"]
+    print(" ".join(cmd), flush=True)
+    p = subprocess.run(cmd, stderr=subprocess.PIPE, text=True)
+    keep = [ln for ln in p.stderr.splitlines() if "-Rpass-analysis=kernel-resource-usage" not in ln
+            and "not a recognized feature" not in ln]
+    if keep:
+        print("\n".join(keep), file=sys.stderr, flush=True)
+    if p.returncode != 0:
+        raise subprocess.CalledProcessError(p.returncode, cmd)
+    usage, cur = {}, None
+    keys = {"VGPRs": "vgprs", "ScratchSize [bytes/lane]": "scratch", "LDS Size [bytes/block]": "lds",
+            "Occupancy [waves/SIMD]": "occupancy"}
+    for ln in p.stderr.splitlines():
+        m = re.search(r"remark:\s+Function Name: (\S+)", ln)
+        if m:
+            cur = usage.setdefault(m.group(1), {})
+            continue
+        m = re.search(r"remark:\s+([A-Za-z /\[\]]+): (\d+)", ln)
+        if m and cur is not None and m.group(1).strip() in keys:
+            cur[keys[m.group(1).strip()]] = int(m.group(2))
+    bad = sorted(k for k, v in usage.items() if v.get("scratch", 0) > 0)
+    if bad:
+        raise RuntimeError("kernels that use scratch memory (bytes per lane): "
+                           + ", ".join("%s=%d" % (k, usage[k]["scratch"]) for k in bad))
+    return usage
 
 
 def build_art(force=False):

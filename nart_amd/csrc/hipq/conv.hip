@@ -163,13 +163,18 @@ __device__ static inline void conv_epilogue(const ConvArgs &a, v16i (&acc)[TN][T
                     const int ko = ch0 + tn * 32 + g * 8 + half * 4;
                     if (ko >= a.out_cs)
                         continue;
+                    // one requantisation form for this path (it is never the fast one): the 64-bit product with the
+                    // channel's own multiplier and shift where the plan has them, the tensor's otherwise
                     int32_t rq[4];
 #pragma unroll
                     for (int e = 0; e < 4; e++) {
                         const int32_t v = (int32_t)((uint32_t)acc[tn][tm][g * 4 + e] + (HAS_WZP ? (uint32_t)colsum[tm] : 0u));
                         if (a.acc_out)
                             a.acc_out[(size_t)m * a.out_cs + ko + e] = v;
-                        rq[e] = a.qmult ? conv_requant_ch(a, v, ko + e) : conv_requant<FAST>(a, v);
+                        const uint32_t qm = a.qmult ? a.qmult[ko + e] : a.q.mult;
+                        const int qs = a.qmult ? a.qshift[ko + e] : a.q.shift;
+                        const int32_t r = (int32_t)(rshift_rn((int64_t)v * (int64_t)qm, qs) + a.q.zp);
+                        rq[e] = r < a.lo ? a.lo : (r > a.q.hi ? a.q.hi : r);
                     }
                     uint32_t packed = pack_low_bytes(rq[0], rq[1], rq[2], rq[3]);
                     if (a.res) {

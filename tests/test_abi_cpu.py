@@ -58,3 +58,17 @@ def test_compute_entry_points_fail_loudly_without_gpu():
         pass
     with pytest.raises(hipq.HipqError):
         hipq.Conv2d((1, 16, 4, 4), np.zeros((16, 16, 1, 1), np.uint8), None, 0, 1, 1, 0.1, 0, 0.1, 0, 0.1, 0)
+
+
+def test_no_kernel_uses_scratch_memory():
+    """The build records every kernel's register, LDS and scratch use (nart_amd/lib/kernel_resources.json) and refuses
+    kernels with scratch memory; the record must be there and clean, and the MFMA tile kernels must fit the register
+    budget their occupancy assumes."""
+    import json
+    path = os.path.join(ROOT, "nart_amd", "lib", "kernel_resources.json")
+    assert os.path.exists(path), "run `python -m nart_amd.build` (it writes the record)"
+    usage = json.load(open(path))
+    assert len(usage) > 50
+    assert all(v["scratch"] == 0 for v in usage.values())
+    tiles = {k: v for k, v in usage.items() if "conv_mfma_dma_kernel" in k}
+    assert tiles and all(v["vgprs"] <= 168 for v in tiles.values())  # three waves per SIMD at least
