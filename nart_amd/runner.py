@@ -206,13 +206,15 @@ class HipqExecutor:
                 print("tune %-12s %-28s window %.1f -> %.1f us  choice %s" % (s["label"], plan.kernel, base, best_t, best), flush=True)
         return chosen
 
-    def capture(self):
-        """Record one pass into a HIP graph (kernel nodes only: no memsets, no allocations)."""
+    def capture(self, passes=1):
+        """Record `passes` passes into a HIP graph (kernel nodes only: no memsets, no allocations).  A network of one or
+        two kernels is shorter than a graph launch: its callers record several passes per graph."""
         self.run()
         torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
-            self.run()
+            for _ in range(passes):
+                self.run()
         self.graph = g
         return g
 
