@@ -52,15 +52,20 @@ def build_hipq(force=False):
         return out
     os.makedirs(LIB, exist_ok=True)
     objs, usage = [], {}
-    for s in srcs:
+
+    def compile_one(s):
         o = os.path.join(LIB, "obj_hipq_" + os.path.basename(s) + ".o")
         lang = ["-x", "hip"] if s.endswith(".hip") else []
         cmd = [HIPCC] + HIP_FLAGS + ["-I" + INC, "-I" + os.path.join(CSRC, "hipq"), "-c"] + lang + [s, "-o", o]
         if s.endswith(".hip"):
-            usage.update(_compile_with_usage(cmd))
-        else:
-            _run(cmd)
-        objs.append(o)
+            return o, _compile_with_usage(cmd)
+        _run(cmd)
+        return o, {}
+    from concurrent.futures import ThreadPoolExecutor
+    with ThreadPoolExecutor(max_workers=4) as pool:  # the translation units are independent; the largest takes minutes
+        for o, u in pool.map(compile_one, srcs):
+            objs.append(o)
+            usage.update(u)
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", out] + objs)
     import json
     with open(os.path.join(LIB, "kernel_resources.json"), "w") as f:
