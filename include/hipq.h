@@ -171,6 +171,21 @@ int hipq_conv2d_run_relu(const hipq_conv2d_plan *plan, const void *x, void *y, v
 int hipq_conv2d_run_add(const hipq_conv2d_plan *plan, const void *x, const void *residual, int residual_is_input0,
                         float res_alpha, int res_zp, float oalpha, int ozp, int obits, void *y, void *stream);
 
+/*
+ * Convolution with the max pooling that follows it in one kernel: y = maxpool3x3/2/1(conv(x)), bit-identical to
+ * hipq_conv2d_run followed by hipq_pool_u8(HIPQ_POOL_MAX, kernel 3, stride 2, pad 1) whose input and output scale and
+ * zero point both equal the convolution's output parameters (op_conv_2d_u8xu8_run, then op_quant_pool_max_run -
+ * src/op/pool.c:96-160: with equal scales the pooling's rescale is the identity).  Serves the stem of a residual
+ * network: uint8 tensors, an input with at most 4 channels (channel stride 4), stride 2, at most 64 output channels,
+ * convolution rows of at most 128 pixels, weight zero point 128, a per-tensor weight scale.  The convolution's own output
+ * never travels to memory.  hipq_conv2d_maxpool_fusable answers (1 / 0) whether a plan and a pooling operator -
+ * described by its settings and its output size OH x OW, as inferred by art/src/op.c:903-967 - can run this way;
+ * hipq_conv2d_run_maxpool fails with an error otherwise (run the two operators separately).  y: NHWC [N, OH, OW, 64].
+ */
+int hipq_conv2d_maxpool_fusable(const hipq_conv2d_plan *plan, int OH, int OW, int kernel, int stride, int pad, float ialpha,
+                                int izp, float oalpha, int ozp, int obits);
+int hipq_conv2d_run_maxpool(const hipq_conv2d_plan *plan, const void *x, void *y, int OH, int OW, void *stream);
+
 /* ---- inner product: op_quant_ip_u8xu8_run — src/op/ip.cpp:133-209.
  * Expressed as a 1x1 convolution over M "pixels": desc {N=M, C=Kdim, H=W=1, K=Nout, R=S=1}.
  * When the reference's input is [M, C, H, W] with H*W > 1, pass the weights re-ordered from

@@ -122,6 +122,17 @@ __device__ static inline u32x4 add_16(u32x4 a, u32x4 b, const AddParams &p)
     return y;
 }
 
+// byte-wise unsigned maximum of two packed dwords
+__device__ static inline uint32_t max_u8x4(uint32_t a, uint32_t b)
+{
+    // per byte: a >= b ? a : b, from the borrow of (a | 0x80) - (b & 0x7f) combined with the top bits
+    const uint32_t H = 0x80808080u;
+    const uint32_t d = (a | H) - (b & ~H);       // no borrow across bytes
+    const uint32_t ge = ((a & ~b) | (~(a ^ b) & d)) & H; // top bit set where a >= b
+    const uint32_t m = (ge >> 7) * 0xffu;        // 0xff in those bytes
+    return (a & m) | (b & ~m);
+}
+
 // Fills *p from the operator's settings; returns false if a scale is outside the fixed-point range.
 bool make_add_params(float ia0, int iz0, float ia1, int iz1, float oa, int oz, int obits, AddParams *p);
 

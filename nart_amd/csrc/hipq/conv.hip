@@ -52,6 +52,7 @@
 
 #include "common.h"
 #include "conv_shared.h"
+#include "conv_stem.h"
 
 namespace hipq {
 
@@ -2112,6 +2113,36 @@ extern "C" int hipq_conv2d_run_add(const hipq_conv2d_plan *p, const void *x, con
         : make_add_params(p->d.oalpha, p->d.ozp, res_alpha, res_zp, oalpha, ozp, obits, &a.addq);
     HIPQ_REQUIRE(ok, "hipq_conv2d_run_add: scales out of the fixed-point range");
     return run_conv(p, a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int hipq_conv2d_maxpool_fusable(const hipq_conv2d_plan *p, int OH, int OW, int kernel, int stride, int pad,
+                                           float ialpha, int izp, float oalpha, int ozp, int obits)
+{
+    if (!p || p->variant != kMfmaSmallC || p->has_wzp || p->d.dtype != HIPQ_DTYPE_U8 || p->d.obits != 8 || obits != 8)
+        return 0;
+    const ConvArgs &a = p->args;
+    // the pooling's rescale must be the identity (equal scale and zero point on both sides, which are the convolution's
+    // output parameters), and its geometry the one the kernel implements
+    if (kernel != 3 || stride != 2 || pad != 1 || ialpha != oalpha || izp != ozp || ialpha != p->d.oalpha || izp != p->d.ozp)
+        return 0;
+    if (OH != (a.OH - 1) / 2 + 1 || OW != (a.OW - 1) / 2 + 1)
+        return 0;
+    return conv_stem_maxpool_applies(a, a.rowb) ? 1 : 0;
+}
+
+extern "C" int hipq_conv2d_run_maxpool(const hipq_conv2d_plan *p, const void *x, void *y, int OH, int OW, void *stream)
+{
+    clear_error();
+    HIPQ_REQUIRE(p && x && y, "hipq_conv2d_run_maxpool: null argument");
+    HIPQ_REQUIRE(hipq_conv2d_maxpool_fusable(p, OH, OW, 3, 2, 1, p->d.oalpha, p->d.ozp, p->d.oalpha, p->d.ozp, 8),
+                 "hipq_conv2d_run_maxpool: this plan (%s) does not fuse with a 3x3 / stride 2 / pad 1 max pooling to %d x %d: run "
+                 "the two operators separately", p->name.c_str(), OH, OW);
+    ConvArgs a = p->args;
+    a.x = static_cast<const uint8_t *>(x);
+    a.y = nullptr;
+    a.acc_out = nullptr;
+    launch_conv_stem_maxpool(a, static_cast<uint8_t *>(y), OH, OW, static_cast<hipStream_t>(stream));
+    return launch_status("conv_stem_maxpool_kernel");
 }
 
 static int run_conv(const hipq_conv2d_plan *p, ConvArgs &a, hipStream_t st)

@@ -246,16 +246,6 @@ __global__ __launch_bounds__(256) void pool_u8_kernel(const PoolArgs p)
 
 // Max pooling with a channel stride that is a multiple of 16: a thread owns 16 channels of one output pixel (128-bit
 // loads, one 128-bit store), 32-bit index arithmetic.  The byte-wise maxima are taken on the packed dwords.
-__device__ static inline uint32_t max_u8x4(uint32_t a, uint32_t b)
-{
-    // per byte: a >= b ? a : b, from the borrow of (a | 0x80) - (b & 0x7f) combined with the top bits
-    const uint32_t H = 0x80808080u;
-    const uint32_t d = (a | H) - (b & ~H);       // no borrow across bytes
-    const uint32_t ge = ((a & ~b) | (~(a ^ b) & d)) & H; // top bit set where a >= b
-    const uint32_t m = (ge >> 7) * 0xffu;        // 0xff in those bytes
-    return (a & m) | (b & ~m);
-}
-
 __global__ __launch_bounds__(256) void pool_max16_u8_kernel(const PoolArgs p, double inv_c16, double inv_ow, double inv_oh)
 {
     const int c16n = p.cs >> 4;

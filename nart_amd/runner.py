@@ -35,6 +35,7 @@ class HipqExecutor:
                         and u[0].kind == "add" and u[0].inputs[0] != u[0].inputs[1] and node.output != case.output.name
                         and not any(a is u[0] for a in self.fused.values())):  # one convolution per add
                     self.fused[node.output] = u[0]  # launched at the add's position: both operands exist by then
+        self.pooled = {}     # conv output name -> the max-pooling node computed inside the convolution's kernel
         self._pending = {}   # id(add node) -> the deferred convolution
         self.buf = {}        # tensor name -> device tensor
         self.steps = []      # (label, kernel name, callable, algorithmic ops, compulsory bytes)
@@ -64,6 +65,18 @@ class HipqExecutor:
                                    a["group"], x.alpha, x.zp, a["walpha"], a["wzp"], y.alpha, y.zp, relu=a["relu"])
                 self.plans.append(plan)
                 nbytes = int(np.prod(x.shape)) + int(np.prod(y.shape)) + case.weights[a["w"]].size + 4 * a["K"]
+                u = [nd for nd in case.nodes if node.output in nd.inputs]
+                if (fuse_add and len(u) == 1 and u[0].kind == "pool" and u[0].attrs["method"] == 0
+                        and node.output != case.output.name):
+                    # the stem: a 3x3 / stride 2 / pad 1 max pooling with the convolution's own scale runs inside the
+                    # convolution's kernel (hipq_conv2d_run_maxpool); the convolution's output is never materialised
+                    pa, pt = u[0].attrs, T[u[0].output]
+                    if plan.maxpool_fusable(pt.shape[2], pt.shape[3], pa["k"], pa["stride"], pa["pad"], y.alpha, y.zp,
+                                            pt.alpha, pt.zp):
+                        self.pooled[node.output] = u[0]
+                        self._pending[id(u[0])] = (plan, ins[0], nbytes - int(np.prod(y.shape)) + int(np.prod(pt.shape)))
+                        self.buf.pop(y.name, None)
+                        continue
                 if node.output in self.fused and plan.kernel.startswith("conv_mfma"):
                     add = self.fused[node.output]
                     other = [i for i in add.inputs if i != node.output][0]
@@ -95,6 +108,11 @@ class HipqExecutor:
                 fn = (lambda p=plan, i=ins[0], o=out: p(i, o))
                 self._add(node, plan.kernel, fn, 2 * Nn * a["K"] * Cc * Hh * Ww,
                           Nn * Cc * Hh * Ww + Nn * a["K"] + a["K"] * Cc * Hh * Ww + 4 * a["K"])
+            elif node.kind == "pool" and id(node) in self._pending:
+                plan, xin, nbytes = self._pending.pop(id(node))
+                fn = (lambda p=plan, i=xin, o=out: p.run_maxpool(i, o))
+                self.steps.append({"label": node.output, "kind": "conv+pool", "kernel": "conv_mfma_i8_stem+maxpool", "fn": fn,
+                                   "ops": plan.ops, "bytes": nbytes, "plan": plan})
             elif node.kind == "pool":
                 x = xs[0]
                 fn = (lambda i=ins[0], o=out, x=x, y=y, a=a: hipq.pool_u8(i, o, x.shape[1], a["k"], a["pad"], a["stride"],
@@ -128,6 +146,11 @@ class HipqExecutor:
                            "bytes": nbytes})
 
     # ---- data in / out ---------------------------------------------------------------------------
+    @property
+    def elided(self):
+        """Names of the tensors that are never materialised (absorbed into a fused kernel)."""
+        return set(self.fused) | set(self.pooled)
+
     def set_input(self, x):
         inp = self.case.input
         if inp.dtype == "f32":

@@ -310,6 +310,53 @@ def test_per_channel_weight_scales():
     assert len(np.unique(want8)) > 8
 
 
+def test_stem_convolution_with_fused_max_pooling():
+    """hipq_conv2d_run_maxpool: the stem convolution (at most 4 input channels, stride 2) and the 3x3 / stride 2 / pad 1
+    max pooling behind it in one kernel, against the oracle's convolution followed by the oracle's pooling: odd and even
+    image sizes (ragged last row block, rows of fewer than 128 pixels), 7x7 / 6x6 / 5x5 kernels (a kernel row of 5 to 8 taps is one 32-byte k-step), 1 to 4 input channels,
+    fewer than 64 output channels, ReLU folded into the convolution, shifts inside and outside the one-multiply form."""
+    rng = np.random.default_rng(151)
+    #        N  C   H    W   K  R pad relu
+    cases = [(2, 3, 224, 224, 64, 7, 3, True), (3, 3, 64, 64, 64, 7, 3, False), (1, 4, 50, 36, 52, 5, 2, True),
+             (2, 1, 37, 52, 64, 5, 1, False), (1, 3, 18, 20, 49, 7, 3, True), (1, 2, 9, 12, 64, 6, 0, False)]
+    for N, C, H, W, K, R, pad, relu in cases:
+        print("stem case", N, C, H, W, K, R, pad, relu, flush=True)
+        x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+        w = rng.integers(0, 256, (K, C, R, R), dtype=np.uint8)
+        b = rng.integers(-20000, 20000, K).astype(np.int32)
+        ia, izp, wa = rand_q(rng), int(rng.integers(0, 256)), rand_q(rng)
+        ozp = 0 if relu else int(rng.integers(0, 256))
+        for oa in (float(np.float32(ia * wa * np.sqrt(C * R * R) * 60.0)), float(np.float32(ia * wa * 40.0))):
+            q = (ia, izp, wa, 128, oa, ozp)
+            conv = orc.conv2d_u8(x, w, b, pad, 2, 1, *q)
+            if relu:
+                conv = np.maximum(conv, ozp).astype(np.uint8)
+            want = orc.pool_u8(conv, 3, 1, 2, 0, False, oa, ozp, oa, ozp)
+            plan = hipq.Conv2d(x.shape, w, b, pad, 2, 1, *q, relu=relu)
+            POH, POW = want.shape[2], want.shape[3]
+            assert plan.maxpool_fusable(POH, POW, 3, 2, 1, oa, ozp, oa, ozp), plan.kernel
+            assert not plan.maxpool_fusable(POH, POW, 3, 2, 1, oa, ozp, float(np.float32(oa * 1.5)), ozp)  # a real rescale
+            assert not plan.maxpool_fusable(POH, POW, 2, 2, 0, oa, ozp, oa, ozp)                            # another window
+            assert not plan.maxpool_fusable(POH + 1, POW, 3, 2, 1, oa, ozp, oa, ozp)                        # ceil_mode sizes
+            yd = torch.full((N, POH, POW, 64), 7, dtype=torch.uint8, device="cuda")
+            plan.run_maxpool(hipq.to_device_nhwc(x), yd)
+            torch.cuda.synchronize()
+            got = yd.cpu().numpy()[..., :K].transpose(0, 3, 1, 2)
+            assert np.array_equal(got, want), (N, C, H, W, K, R, pad, relu, oa, int((got != want).sum()))
+            # and the two operators run separately give the same bytes
+            yc = plan(hipq.to_device_nhwc(x))
+            yp = torch.empty((N, POH, POW, 64), dtype=torch.uint8, device="cuda")
+            hipq.pool_u8(yc, yp, K, 3, 1, 2, 0, oa, ozp, oa, ozp)
+            assert torch.equal(yp[..., :K], yd[..., :K])
+    # plans the kernel does not serve refuse
+    p64 = hipq.Conv2d((1, 64, 8, 8), np.zeros((64, 64, 3, 3), np.uint8), None, 1, 2, 1, 0.1, 0, 0.1, 128, 0.1, 0)
+    assert not p64.maxpool_fusable(2, 2, 3, 2, 1, 0.1, 0, 0.1, 0)
+    with pytest.raises(hipq.HipqError):
+        p64.run_maxpool(torch.zeros((1, 8, 8, 64), dtype=torch.uint8, device="cuda"), torch.zeros((1, 2, 2, 64), dtype=torch.uint8, device="cuda"))
+    s1 = hipq.Conv2d((1, 3, 16, 16), np.zeros((64, 3, 3, 3), np.uint8), None, 1, 1, 1, 0.1, 0, 0.1, 128, 0.1, 0)  # stride 1
+    assert not s1.maxpool_fusable(8, 8, 3, 2, 1, 0.1, 0, 0.1, 0)
+
+
 def test_elementwise():
     rng = np.random.default_rng(15)
     for n in (1, 15, 16, 4099, 64 * 56 * 56 * 16 + 3):
