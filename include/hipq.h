@@ -104,6 +104,9 @@ int hipq_conv2d_plan_create_per_channel(const hipq_conv2d_desc *desc, const uint
 void hipq_conv2d_plan_destroy(hipq_conv2d_plan *plan);
 /* Name of the kernel variant the plan dispatches to (for logs and tests). */
 const char *hipq_conv2d_plan_kernel(const hipq_conv2d_plan *plan);
+/* Name of the kernel variant that hipq_conv2d_run_add dispatches to for this plan, assuming the 32-bit form of the add
+ * ("" for a plan that cannot fuse the add).  The string is valid until the calling thread's next call. */
+const char *hipq_conv2d_plan_kernel_add(const hipq_conv2d_plan *plan);
 
 /*
  * Tuning hook (no counterpart in the reference): choose the work-group tile (index: 0 128x128, 1 256x64, 2 128x64,
@@ -121,11 +124,16 @@ int hipq_conv2d_plan_select(hipq_conv2d_plan *plan, int tile, int stages);
  * of hipq_conv2d_run_add and accumulator dumps take the tile kernel).  Two-group kernel (name "..._k2"): the tile
  * kernel with 512 threads, two groups of four waves that each reduce every other 64-byte slab of k and add their partial
  * accumulators through LDS (plain convolutions with an even number of at least 8 slabs; not with an explicit stage count).
+ * Widening kernel (name "..._expand"): 1x1 convolutions without padding from 64, 128 or 256 input channels (stride) to
+ * at least twice as many and 256 to 1024 output channels over at least 1024 pixels (weight zero point 128) keep a wave's
+ * pixel operands in registers while a work-group walks a contiguous range of 128-pixel x 64-channel output tiles, with
+ * the residual add of hipq_conv2d_run_add applied in place on a prefetched residual tile.
  * mode 1 (the default) uses them where they measured faster: the halo kernel for 64-channel inputs up to 63 pixels
- * wide, the pointwise kernel wherever it applies, the two-group kernel for layers with at most one tile per CU (256);
- * mode 2 the halo kernel also for 128, 256 and 512 channels (128-channel tiles, images up to 31 pixels wide) and the
- * two-group kernel whatever the number of tiles; mode 0 none of them.  Identical results in every mode.  Plans that do not run the MFMA
- * kernel return an error.
+ * wide, the pointwise kernel wherever it applies, the two-group kernel for layers with at most one tile per CU (256),
+ * the widening kernel with the add at 64 input channels and without it at 256;
+ * mode 2 the halo kernel also for 128, 256 and 512 channels (128-channel tiles, images up to 31 pixels wide), the
+ * two-group kernel whatever the number of tiles and the widening kernel wherever it applies; mode 0 none of them.
+ * Identical results in every mode.  Plans that do not run the MFMA kernel return an error.
  */
 int hipq_conv2d_plan_special(hipq_conv2d_plan *plan, int mode);
 /*

@@ -53,14 +53,25 @@ def build_hipq(force=False):
     os.makedirs(LIB, exist_ok=True)
     objs, usage = [], {}
 
+    headers = [d for d in deps if d.endswith(".h")]
+
     def compile_one(s):
+        import json
         o = os.path.join(LIB, "obj_hipq_" + os.path.basename(s) + ".o")
+        u = o + ".usage.json"  # the resource remarks of this translation unit, kept beside its object
+        if not force and _newer(o, [s] + headers) and os.path.exists(u):
+            with open(u) as f:
+                return o, json.load(f)
         lang = ["-x", "hip"] if s.endswith(".hip") else []
         cmd = [HIPCC] + HIP_FLAGS + ["-I" + INC, "-I" + os.path.join(CSRC, "hipq"), "-c"] + lang + [s, "-o", o]
+        usage = {}
         if s.endswith(".hip"):
-            return o, _compile_with_usage(cmd)
-        _run(cmd)
-        return o, {}
+            usage = _compile_with_usage(cmd)
+        else:
+            _run(cmd)
+        with open(u, "w") as f:
+            json.dump(usage, f)
+        return o, usage
     from concurrent.futures import ThreadPoolExecutor
     with ThreadPoolExecutor(max_workers=4) as pool:  # the translation units are independent; the largest takes minutes
         for o, u in pool.map(compile_one, srcs):

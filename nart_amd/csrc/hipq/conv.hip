@@ -53,6 +53,7 @@
 #include "common.h"
 #include "conv_shared.h"
 #include "conv_stem.h"
+#include "conv_expand.h"
 
 namespace hipq {
 
@@ -1559,12 +1560,21 @@ static bool stream_applies(const hipq_conv2d_plan *p, StreamShape *shape = nullp
     return true;
 }
 
+// conv_mfma_expand_kernel (conv_expand.hip): a 1x1 layer that widens the channels, for this launch's arguments (with a
+// residual to add or without)
+static bool expand_applies(const hipq_conv2d_plan *p, const ConvArgs &a)
+{
+    return p->variant == kMfma && p->special && !p->tile_selected && !p->has_wzp && conv_expand_applies(a, p->special == 2);
+}
+
 static void set_mfma_name(hipq_conv2d_plan *p, bool smallc)
 {
     char nm[96];
     StreamShape ss;
     if (!smallc && stream_applies(p, &ss))
         snprintf(nm, sizeof nm, "conv_mfma_i8_stream_%dx%d%s", 16 * ss.mb, 16 * ss.nb, p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
+    else if (!smallc && expand_applies(p, p->args))
+        snprintf(nm, sizeof nm, "conv_mfma_i8_expand%s", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
     else if (pointwise_applies(p))
         snprintf(nm, sizeof nm, "conv_mfma_i8_pointwise%s", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
     else
@@ -1836,6 +1846,26 @@ extern "C" void hipq_conv2d_plan_destroy(hipq_conv2d_plan *p)
 }
 
 extern "C" const char *hipq_conv2d_plan_kernel(const hipq_conv2d_plan *p) { return p ? p->name.c_str() : ""; }
+
+extern "C" const char *hipq_conv2d_plan_kernel_add(const hipq_conv2d_plan *p)
+{
+    if (!p || (p->variant != kMfma && p->variant != kMfmaSmallC))
+        return "";
+    static thread_local std::string nm;
+    ConvArgs a = p->args;
+    a.res = a.padbuf; // any non-null pointer: the question is which kernel a launch with a residual goes to
+    a.addq.fast = 1;  // the 32-bit form of the add, which ordinary scale ratios allow
+    char buf[96];
+    if (expand_applies(p, a))
+        snprintf(buf, sizeof buf, "conv_mfma_i8_expand%s+add", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
+    else
+        snprintf(buf, sizeof buf, "conv_mfma_i8_%dx%d%s%s%s+add", kTiles[p->tile].bm, kTiles[p->tile].bn,
+                 p->variant == kMfmaSmallC ? "_c4" : "", p->has_wzp ? "_wzp" : "", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
+    nm = buf;
+    if (p->d_q)
+        nm += "_perchannel";
+    return nm.c_str();
+}
 
 extern "C" int hipq_conv2d_plan_select(hipq_conv2d_plan *p, int tile, int stages)
 {
@@ -2150,6 +2180,10 @@ static int run_conv(const hipq_conv2d_plan *p, ConvArgs &a, hipStream_t st)
     switch (p->variant) {
     case kMfma:
     case kMfmaSmallC:
+        if (expand_applies(p, a)) {
+            launch_conv_expand(a, st); // a channel-widening 1x1 layer: pixel operands in registers, channel tiles in a loop
+            break;
+        }
         switch (p->tile) {
         case 0: launch_mfma<128, 128, 2, 2>(p, a, st); break;
         case 1: launch_mfma<256, 64, 4, 1>(p, a, st); break;

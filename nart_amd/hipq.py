@@ -43,6 +43,7 @@ _SIGS = {
                                                       C.POINTER(C.c_void_p)]),
     "hipq_conv2d_plan_destroy": (None, [C.c_void_p]),
     "hipq_conv2d_plan_kernel": (C.c_char_p, [C.c_void_p]),
+    "hipq_conv2d_plan_kernel_add": (C.c_char_p, [C.c_void_p]),
     "hipq_conv2d_plan_select": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
     "hipq_conv2d_plan_special": (C.c_int, [C.c_void_p, C.c_int]),
     "hipq_conv2d_plan_stream": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int]),
@@ -174,6 +175,11 @@ class Conv2d:
         m = re.match(r"conv_mfma_i8_(\d+x\d+)", self.kernel)
         self._tile0 = TILE_INDEX.get(m.group(1), -1) if m else -1  # the built-in choice, for the tuner to return to
         self.ops = 2 * N * K * self.OH * self.OW * (Cc // group) * R * S
+
+    @property
+    def kernel_add(self):
+        """Name of the kernel run_add dispatches to ("" when the plan cannot fuse the add)."""
+        return lib().hipq_conv2d_plan_kernel_add(self.handle).decode()
 
     def select(self, tile=-1, stages=0):
         """Tuning hook: work-group tile index and load stages of the MFMA kernel (include/hipq.h)."""

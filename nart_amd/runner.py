@@ -122,7 +122,7 @@ class HipqExecutor:
                 plan, xin, other, res_first, ot, st, nbytes = self._pending.pop(id(node))
                 fn = (lambda p=plan, i=xin, r=self.buf[other], rf=res_first, ot=ot, st=st, o=out:
                       p.run_add(i, r, rf, ot.alpha, ot.zp, st.alpha, st.zp, o))
-                self.steps.append({"label": node.output, "kind": "conv+add", "kernel": plan.kernel + "+add", "fn": fn,
+                self.steps.append({"label": node.output, "kind": "conv+add", "kernel": plan.kernel_add or plan.kernel + "+add", "fn": fn,
                                    "ops": plan.ops, "bytes": nbytes, "plan": plan})
             elif node.kind == "add":
                 fn = (lambda i=ins, o=out, xs=xs, y=y: hipq.add_u8(i[0], i[1], o, xs[0].alpha, xs[0].zp, xs[1].alpha,
@@ -210,6 +210,8 @@ class HipqExecutor:
                 continue  # the generic-addressing kernel has a single variant
             if plan.kernel.endswith("pointwise") and s["kind"] != "conv+add":
                 continue  # the pointwise kernel has no tile or stages (the fused add runs a tile kernel)
+            if "expand" in s["kernel"] or "_stream_" in s["kernel"]:
+                continue  # neither have these two; naming a tile would take the layer away from them for good
             lo, hi = max(0, k - before), min(len(self.steps), k + 1 + after)
             base = self._time_window(lo, hi, reps)
             best, best_t = (-1, 0), base
@@ -223,7 +225,7 @@ class HipqExecutor:
                 plan.select(*best)
             else:  # back to the built-in choice
                 plan.select(plan._tile0, 0)
-            s["kernel"] = plan.kernel + ("+add" if s["kind"] == "conv+add" else "")
+            s["kernel"] = (plan.kernel_add or plan.kernel + "+add") if s["kind"] == "conv+add" else plan.kernel
             chosen[s["label"]] = (best, round(base, 2), round(best_t, 2))
             if verbose:
                 print("tune %-12s %-28s window %.1f -> %.1f us  choice %s" % (s["label"], plan.kernel, base, best_t, best), flush=True)

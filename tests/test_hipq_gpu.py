@@ -144,6 +144,70 @@ def test_conv_with_fused_residual_add():
         plan.run_add(hipq.to_device_nhwc(xdw), hipq.to_device_nhwc(xdw), False, 0.05, 0, 0.07, 0, plan.empty_output())
 
 
+def test_channel_widening_1x1_layers():
+    """conv_mfma_expand_kernel (1x1, 64 / 128 / 256 input channels, at least four times 64 output channels, 1024 pixels
+    or more): alone against the oracle's convolution (accumulator dump through the tile kernels aside, outputs only), with
+    ReLU, and with the residual add fused in, both operand orders; ragged pixel counts, an output width that is not a
+    multiple of 64, strides, int8 tensors.  special(0) runs the same plans on the tile kernels: identical bytes."""
+    rng = np.random.default_rng(77)
+    shapes = [  # N, C, H, W, K, stride
+        (2, 64, 28, 28, 256, 1), (1, 128, 40, 30, 512, 1), (8, 256, 28, 28, 1024, 2), (1, 64, 33, 37, 272, 1),
+        (3, 128, 21, 19, 300, 1), (4, 256, 47, 30, 520, 2),
+    ]
+    seen = set()
+    for i, (N, C, H, W, K, st) in enumerate(shapes):
+        x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+        w = rng.integers(0, 256, (K, C, 1, 1), dtype=np.uint8)
+        b = rng.integers(-30000, 30000, K).astype(np.int32)
+        for relu in (False, True):
+            q = (rand_q(rng), int(rng.integers(0, 256)), rand_q(rng), 128, rand_q(rng, 1e-2, 1.0), int(rng.integers(0, 256)))
+            plan = hipq.Conv2d(x.shape, w, b, 0, st, 1, *q, relu=relu)
+            # built-in rule: without the add at 256 input channels only; special(2): wherever the kernel applies
+            assert (plan.kernel == "conv_mfma_i8_expand") == (C == 256), plan.kernel
+            plan.special(2)
+            print("widening case", i, x.shape, w.shape, st, relu, plan.kernel, flush=True)
+            assert plan.kernel == "conv_mfma_i8_expand", plan.kernel
+            seen.add(plan.kernel)
+            want = orc.conv2d_u8(x, w, b, 0, st, 1, *q)
+            if relu:
+                want = orc.relu_u8(want, q[4], q[5], q[4], q[5])
+            xd = hipq.to_device_nhwc(x)
+            got = hipq.from_device_nhwc(plan(xd), K)
+            assert np.array_equal(got, want), (i, relu, int((got != want).sum()))
+            plan.special(0)
+            assert np.array_equal(hipq.from_device_nhwc(plan(xd), K), want), (i, relu, plan.kernel)
+        for res_first, ratio, obits in ((False, 1.0, 8), (True, 1.7, 8), (False, 0.6, 7)):
+            q = (rand_q(rng), int(rng.integers(0, 256)), rand_q(rng), 128, rand_q(rng, 1e-2, 1.0), int(rng.integers(0, 256)))
+            plan = hipq.Conv2d(x.shape, w, b, 0, st, 1, *q)
+            assert (plan.kernel_add == "conv_mfma_i8_expand+add") == (C == 64), plan.kernel_add  # built-in rule
+            plan.special(2)
+            assert plan.kernel_add == "conv_mfma_i8_expand+add", plan.kernel_add
+            conv = orc.conv2d_u8(x, w, b, 0, st, 1, *q)
+            res = rng.integers(0, 256, conv.shape, dtype=np.uint8)
+            ra, rz = float(np.float32(q[4] * ratio)), int(rng.integers(0, 256))
+            oa, oz = float(np.float32(max(q[4], ra) * 1.3)), int(rng.integers(0, 1 << obits))
+            print("widening case with add", i, res_first, ratio, obits, plan.kernel_add, flush=True)
+            want = (orc.add_u8(res, conv, ra, rz, q[4], q[5], oa, oz, obits) if res_first
+                    else orc.add_u8(conv, res, q[4], q[5], ra, rz, oa, oz, obits))
+            xd, rd = hipq.to_device_nhwc(x), hipq.to_device_nhwc(res)
+            for mode in (2, 0):
+                plan.special(mode)
+                y = plan.empty_output()
+                plan.run_add(xd, rd, res_first, ra, rz, oa, oz, y, obits=obits)
+                torch.cuda.synchronize()
+                got = hipq.from_device_nhwc(y, K)
+                assert np.array_equal(got, want), (i, res_first, ratio, obits, mode, int((got != want).sum()))
+    # int8 tensors through the same kernel
+    x = rng.integers(-128, 128, (2, 64, 24, 24), dtype=np.int8)
+    w = rng.integers(-127, 128, (256, 64, 1, 1), dtype=np.int8)
+    b = rng.integers(-30000, 30000, 256).astype(np.int32)
+    for obits in (8, 7):
+        plan = hipq.Conv2d(x.shape, w, b, 0, 1, 1, 0.02, 0, 0.004, 0, 0.09, 0, obits=obits, dtype=hipq.DTYPE_I8).special(2)
+        assert plan.kernel == "conv_mfma_i8_expand_signed", plan.kernel
+        got = hipq.from_device_nhwc(plan(hipq.to_device_nhwc(x)), 256).view(np.int8)
+        assert np.array_equal(got, orc.conv2d_i8(x, w, b, 0, 1, 1, 0.02, 0.004, 0.09, obits=obits)), obits
+
+
 def test_conv_grouped_and_depthwise():
     rng = np.random.default_rng(13)
     kerns = set()
