@@ -34,7 +34,9 @@
 extern "C" {
 #endif
 
-#define HIPQ_ABI_VERSION 2
+/* 3: per-channel weight scales, the fused stem (convolution + max pooling), the streaming and channel-widening kernels'
+ * hooks, hipq_conv2d_plan_kernel_add.  Every entry point of version 2 is unchanged. */
+#define HIPQ_ABI_VERSION 3
 
 #define HIPQ_ELTWISE_SUM 1 /* SETTING_ELTWISE_OP_SUM */
 #define HIPQ_ELTWISE_MAX 2 /* SETTING_ELTWISE_OP_MAX */
@@ -189,10 +191,12 @@ int hipq_conv2d_run_add(const hipq_conv2d_plan *plan, const void *x, const void 
  * never travels to memory.  hipq_conv2d_maxpool_fusable answers (1 / 0) whether a plan and a pooling operator -
  * described by its settings and its output size OH x OW, as inferred by art/src/op.c:903-967 - can run this way;
  * hipq_conv2d_run_maxpool fails with an error otherwise (run the two operators separately).  y: NHWC [N, OH, OW, 64].
+ * relu != 0 also applies the ReLU clamp of hipq_conv2d_run_relu between the two (conv, relu, pool as three operators
+ * with equal scales: op_quant_relu_run is then max(x, zero point)).
  */
 int hipq_conv2d_maxpool_fusable(const hipq_conv2d_plan *plan, int OH, int OW, int kernel, int stride, int pad, float ialpha,
                                 int izp, float oalpha, int ozp, int obits);
-int hipq_conv2d_run_maxpool(const hipq_conv2d_plan *plan, const void *x, void *y, int OH, int OW, void *stream);
+int hipq_conv2d_run_maxpool(const hipq_conv2d_plan *plan, const void *x, void *y, int OH, int OW, int relu, void *stream);
 
 /* ---- inner product: op_quant_ip_u8xu8_run — src/op/ip.cpp:133-209.
  * Expressed as a 1x1 convolution over M "pixels": desc {N=M, C=Kdim, H=W=1, K=Nout, R=S=1}.

@@ -2160,7 +2160,7 @@ extern "C" int hipq_conv2d_maxpool_fusable(const hipq_conv2d_plan *p, int OH, in
     return conv_stem_maxpool_applies(a, a.rowb) ? 1 : 0;
 }
 
-extern "C" int hipq_conv2d_run_maxpool(const hipq_conv2d_plan *p, const void *x, void *y, int OH, int OW, void *stream)
+extern "C" int hipq_conv2d_run_maxpool(const hipq_conv2d_plan *p, const void *x, void *y, int OH, int OW, int relu, void *stream)
 {
     clear_error();
     HIPQ_REQUIRE(p && x && y, "hipq_conv2d_run_maxpool: null argument");
@@ -2171,6 +2171,8 @@ extern "C" int hipq_conv2d_run_maxpool(const hipq_conv2d_plan *p, const void *x,
     a.x = static_cast<const uint8_t *>(x);
     a.y = nullptr;
     a.acc_out = nullptr;
+    if (relu)
+        a.lo = std::min(p->d.ozp, a.q.hi); // the ReLU clamp, as in hipq_conv2d_run_relu
     launch_conv_stem_maxpool(a, static_cast<uint8_t *>(y), OH, OW, static_cast<hipStream_t>(stream));
     return launch_status("conv_stem_maxpool_kernel");
 }

@@ -93,7 +93,7 @@ typedef std::map<const mem_t *, std::set<const op_t *>> reader_map;
 
 // keyed by workspace (the runtime is single-threaded, art/include/art/workspace.h has no locking either)
 std::map<const workspace_t *, reader_map> g_readers;
-long g_fused_adds = 0, g_fused_relus = 0; // fused launches so far (hip_module_fused_adds / _relus)
+long g_fused_adds = 0, g_fused_relus = 0, g_fused_pools = 0; // fused launches so far (hip_module_fused_adds / _relus / _pools)
 
 reader_map &readers_of(op_t *op) { return g_readers[op->workspace]; }
 
@@ -187,6 +187,8 @@ void conv_launch_plain(void *ctx)
 }
 
 bool eltwise_is_plain_sum(const op_t *op); // two inputs, SUM, unit coefficients: computes what add computes
+// a max pooling that the stem convolution's kernel can compute as well (hipq_conv2d_maxpool_fusable)
+bool pool_fuses_with(const op_t *pool_op, const hipq_conv2d_plan *plan);
 
 // 1: the only reader of the convolution's output is an add or a relu of this workspace that can take over the launch
 bool sole_reader_fuses(op_t *op)
@@ -204,6 +206,8 @@ bool sole_reader_fuses(op_t *op)
         return false;
     if (r->entry->tp == &op_relu_tp)
         return true; // any plan runs with the ReLU clamp (hipq_conv2d_run_relu)
+    if (r->entry->tp == &op_pool_tp)
+        return pool_fuses_with(r, c->plan);
     // hipq_conv2d_run_add exists for the MFMA plans
     return (r->entry->tp == &op_add_tp || eltwise_is_plain_sum(r)) && r->input_size == 2
         && r->input_tensors[0]->mem != r->input_tensors[1]->mem && strncmp(hipq_conv2d_plan_kernel(c->plan), "conv_mfma", 9) == 0;
@@ -342,6 +346,7 @@ struct ew_op_t {
     uint32_t operation;
     float *coeff;
     size_t bytes; // device bytes to process (pad channels included)
+    int defer;    // relu: 0 undecided, 1 leave the (fused) launch to the max pooling that reads the output, -1 launch at run()
 };
 
 size_t device_bytes_of(const tensor_t *t)
@@ -473,24 +478,80 @@ void relu_config(op_t *op)
     READ_O(op, &e->qo);
 }
 
+// the relu `op` whose input is a convolution that left it its launch (conv_run): with equal scales and zero points on
+// both sides the relu is max(x, zp), the convolution's lower clamp
+bool relu_is_clamp_of(const ew_op_t *e, const conv_op_t *c)
+{
+    return e->qi.alpha[0] == c->desc.oalpha && e->qi.zp[0] == c->desc.ozp && e->qo.alpha[0] == c->desc.oalpha
+        && e->qo.zp[0] == c->desc.ozp && e->qo.bits[0] == c->desc.obits;
+}
+
+// convolution + relu as one launch into the relu's output memory `y`; false: not possible, run the relu plainly
+bool relu_launch_into(op_t *op, void *y)
+{
+    ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    hip_mem_t *m = as_hip(op->input_tensors[0]->mem);
+    if (m->pending != conv_launch_plain)
+        return false;
+    op_t *cop = static_cast<op_t *>(m->pending_ctx);
+    conv_op_t *c = reinterpret_cast<conv_op_t *>(cop);
+    if (!relu_is_clamp_of(e, c) || hipq_conv2d_run_relu(c->plan, in_ptr(cop, 0), y, op_stream(op)) != 0)
+        return false;
+    ++g_fused_relus;
+    return true;
+}
+
+// the hook a relu leaves on its output when a max pooling will take over (relu_run): whoever else asks first gets the
+// convolution and the relu as one launch, or as two
+void relu_launch_deferred(void *ctx)
+{
+    op_t *op = static_cast<op_t *>(ctx);
+    ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    void *y = as_hip(op->output_tensors[0].mem)->dev;
+    if (!relu_launch_into(op, y))
+        HIPM_HIPQ(hipq_relu_u8(in_ptr(op, 0), y, e->bytes, e->qi.alpha[0], e->qi.zp[0], e->qo.alpha[0], e->qo.zp[0],
+                               e->qo.bits[0], op_stream(op)));
+}
+
 void relu_run(op_t *op)
 {
     ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
     hip_mem_t *m = as_hip(op->input_tensors[0]->mem);
-    if (m->pending == conv_launch_plain) {
-        // the input is a convolution that left its launch to this relu (conv_run).  With equal scales and zero points
-        // on both sides the relu is max(x, zp): the convolution's lower clamp.
-        op_t *cop = static_cast<op_t *>(m->pending_ctx);
-        conv_op_t *c = reinterpret_cast<conv_op_t *>(cop);
-        if (e->qi.alpha[0] == c->desc.oalpha && e->qi.zp[0] == c->desc.ozp && e->qo.alpha[0] == c->desc.oalpha
-            && e->qo.zp[0] == c->desc.ozp && e->qo.bits[0] == c->desc.obits
-            && hipq_conv2d_run_relu(c->plan, in_ptr(cop, 0), out_ptr(op), op_stream(op)) == 0) {
-            ++g_fused_relus;
+    if (m->pending == conv_launch_plain && relu_is_clamp_of(e, reinterpret_cast<conv_op_t *>(m->pending_ctx))) {
+        // conv -> relu -> max pooling (the stem of a residual network): if the pooling is this relu's only reader and can
+        // run inside the convolution's kernel, the relu passes the launch on to it
+        if (e->defer == 0) {
+            static const bool off = getenv("NART_HIP_NO_FUSION") != nullptr;
+            e->defer = -1;
+            const reader_map &rm = readers_of(op);
+            const auto it = rm.find(op->output_tensors[0].mem);
+            if (!off && it != rm.end() && it->second.size() == 1) {
+                const op_t *r = *it->second.begin();
+                if (r->workspace == op->workspace && r->entry->tp == &op_pool_tp
+                    && pool_fuses_with(r, reinterpret_cast<conv_op_t *>(m->pending_ctx)->plan))
+                    e->defer = 1;
+            }
+        }
+        if (e->defer == 1) {
+            hip_mem_t *ym = as_hip(op->output_tensors[0].mem);
+            (void)out_ptr(op); // the buffer exists and the device side is the current one - once the hook has run
+            ym->pending = relu_launch_deferred;
+            ym->pending_ctx = op;
             return;
         }
     }
+    if (relu_launch_into(op, out_ptr(op)))
+        return;
     HIPM_HIPQ(hipq_relu_u8(in_ptr(op, 0), out_ptr(op), e->bytes, e->qi.alpha[0], e->qi.zp[0], e->qo.alpha[0], e->qo.zp[0],
                            e->qo.bits[0], op_stream(op)));
+}
+
+void relu_destroy(op_t *op)
+{
+    // a launch left to a pooling (relu_run) must not outlive the operator
+    if (op->output_size > 0 && op->output_tensors != nullptr && op->output_tensors[0].mem != nullptr
+        && is_hip_mem(op->output_tensors[0].mem) && as_hip(op->output_tensors[0].mem)->pending_ctx == op)
+        as_hip(op->output_tensors[0].mem)->pending = nullptr;
 }
 
 void relu_prepare(op_t *op)
@@ -500,6 +561,7 @@ void relu_prepare(op_t *op)
     alloc_and_tag(op);
     same_geometry(op);
     e->bytes = device_bytes_of(&op->output_tensors[0]);
+    e->defer = 0;
     op->run_func = relu_run;
 }
 
@@ -611,9 +673,51 @@ void pool_config(op_t *op)
     READ_O(op, &p->qo);
 }
 
+bool pool_fuses_with(const op_t *op, const hipq_conv2d_plan *plan)
+{
+    const pool_op_t *p = reinterpret_cast<const pool_op_t *>(op);
+    if (p->method != SETTING_POOL_MAX || p->kernel_h != p->kernel_w || p->stride_h != p->stride_w || p->pad_h != p->pad_w
+        || op->output_tensors[0].mem == nullptr || !is_hip_mem(op->output_tensors[0].mem))
+        return false;
+    const hip_mem_t *y = as_hip(op->output_tensors[0].mem);
+    return hipq_conv2d_maxpool_fusable(plan, y->H, y->W, (int)p->kernel_h, (int)p->stride_h, (int)p->pad_h, p->qi.alpha[0],
+                                       p->qi.zp[0], p->qo.alpha[0], p->qo.zp[0], p->qo.bits[0]) != 0;
+}
+
+// the pooling `op` inside the kernel of the convolution that left it its launch, directly (conv_run) or through a relu
+// (relu_run); false: run it plainly
+bool pool_run_fused(op_t *op)
+{
+    hip_mem_t *x = as_hip(op->input_tensors[0]->mem);
+    op_t *cop = nullptr;
+    int relu = 0;
+    if (x->pending == conv_launch_plain) {
+        cop = static_cast<op_t *>(x->pending_ctx);
+    } else if (x->pending == relu_launch_deferred) {
+        hip_mem_t *cm = as_hip(static_cast<op_t *>(x->pending_ctx)->input_tensors[0]->mem);
+        if (cm->pending != conv_launch_plain)
+            return false; // someone asked for the convolution's own output in between: it has run
+        cop = static_cast<op_t *>(cm->pending_ctx);
+        relu = 1;
+    } else {
+        return false;
+    }
+    conv_op_t *c = reinterpret_cast<conv_op_t *>(cop);
+    if (!pool_fuses_with(op, c->plan))
+        return false;
+    const hip_mem_t *y = as_hip(op->output_tensors[0].mem);
+    const void *xin = in_ptr(cop, 0);
+    if (hipq_conv2d_run_maxpool(c->plan, xin, out_ptr(op), y->H, y->W, relu, op_stream(op)) != 0)
+        return false;
+    ++g_fused_pools;
+    return true; // the hooks stay for whoever asks for the intermediate tensors
+}
+
 void pool_run(op_t *op)
 {
     pool_op_t *p = reinterpret_cast<pool_op_t *>(op);
+    if (pool_run_fused(op))
+        return;
     const hip_mem_t *x = as_hip(op->input_tensors[0]->mem), *y = as_hip(op->output_tensors[0].mem);
     HIPM_HIPQ(hipq_pool_u8(in_ptr(op, 0), out_ptr(op), x->N, x->C, x->H, x->W, y->H, y->W, x->cs, (int)p->kernel_h,
                            (int)p->kernel_w, (int)p->pad_h, (int)p->pad_w, (int)p->stride_h, (int)p->stride_w,
@@ -786,6 +890,7 @@ static workspace_t *ws_new(const setting_entry_t *settings)
 // How many add operators have run fused into the convolution that produces one of their inputs (diagnostics, tests).
 ART_PUBLIC long hip_module_fused_adds(void) { return g_fused_adds; }
 ART_PUBLIC long hip_module_fused_relus(void) { return g_fused_relus; }
+ART_PUBLIC long hip_module_fused_pools(void) { return g_fused_pools; }
 
 ART_PUBLIC void *hip_workspace_stream(workspace_t *w) { return reinterpret_cast<hip_workspace_t *>(w)->stream; }
 
@@ -812,7 +917,7 @@ ART_PUBLIC op_tp_entry_t hip_op_table[] = {
     HIP_ENTRY(op_hip_dequantize_tp, qdq_op_t, dequantize_config, destroy_nothing, dequantize_prepare),
     HIP_ENTRY(op_conv_2d_tp, conv_op_t, conv_config, conv_destroy, conv_prepare),
     HIP_ENTRY(op_ip_tp, conv_op_t, ip_config, conv_destroy, ip_prepare),
-    HIP_ENTRY(op_relu_tp, ew_op_t, relu_config, destroy_nothing, relu_prepare),
+    HIP_ENTRY(op_relu_tp, ew_op_t, relu_config, relu_destroy, relu_prepare),
     HIP_ENTRY(op_add_tp, ew_op_t, add_config, destroy_nothing, add_prepare),
     HIP_ENTRY(op_eltwise_tp, ew_op_t, eltwise_config, destroy_nothing, eltwise_prepare),
     HIP_ENTRY(op_pool_tp, pool_op_t, pool_config, destroy_nothing, pool_prepare),

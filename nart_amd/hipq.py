@@ -52,7 +52,7 @@ _SIGS = {
     "hipq_conv2d_run_add": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_float, C.c_int,
                                       C.c_int, C.c_void_p, C.c_void_p]),
     "hipq_conv2d_maxpool_fusable": (C.c_int, [C.c_void_p] + [C.c_int] * 5 + [C.c_float, C.c_int, C.c_float, C.c_int, C.c_int]),
-    "hipq_conv2d_run_maxpool": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
+    "hipq_conv2d_run_maxpool": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
     "hipq_ip_reorder_weights": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 6),
     "hipq_add_u8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_float, C.c_int, C.c_float,
                               C.c_int, C.c_float, C.c_int, C.c_int, C.c_void_p]),
@@ -228,9 +228,10 @@ class Conv2d:
         """Can the 3x3 / stride 2 / pad 1 max pooling that follows run inside this convolution's kernel (include/hipq.h)?"""
         return bool(lib().hipq_conv2d_maxpool_fusable(self.handle, OH, OW, kernel, stride, pad, ialpha, izp, oalpha, ozp, obits))
 
-    def run_maxpool(self, x, y):
-        """y = maxpool3x3/2/1(conv(x)) in one launch; y: [N, OH, OW, 64] (include/hipq.h: hipq_conv2d_run_maxpool)."""
-        check(lib().hipq_conv2d_run_maxpool(self.handle, _ptr(x), _ptr(y), y.shape[1], y.shape[2], _stream()))
+    def run_maxpool(self, x, y, relu=False):
+        """y = maxpool3x3/2/1(conv(x)) in one launch, with the ReLU clamp in between if relu; y: [N, OH, OW, 64]
+        (include/hipq.h: hipq_conv2d_run_maxpool)."""
+        check(lib().hipq_conv2d_run_maxpool(self.handle, _ptr(x), _ptr(y), y.shape[1], y.shape[2], int(bool(relu)), _stream()))
         return y
 
     def close(self):

@@ -412,6 +412,11 @@ def test_stem_convolution_with_fused_max_pooling():
             yp = torch.empty((N, POH, POW, 64), dtype=torch.uint8, device="cuda")
             hipq.pool_u8(yc, yp, K, 3, 1, 2, 0, oa, ozp, oa, ozp)
             assert torch.equal(yp[..., :K], yd[..., :K])
+            if not relu:  # the ReLU clamp asked for at run time (conv, relu, pool as three operators with equal scales)
+                want_r = orc.pool_u8(orc.relu_u8(conv, oa, ozp, oa, ozp), 3, 1, 2, 0, False, oa, ozp, oa, ozp)
+                plan.run_maxpool(hipq.to_device_nhwc(x), yd, relu=True)
+                torch.cuda.synchronize()
+                assert np.array_equal(yd.cpu().numpy()[..., :K].transpose(0, 3, 1, 2), want_r), (N, C, H, W, K, R, "relu at run time")
     # plans the kernel does not serve refuse
     p64 = hipq.Conv2d((1, 64, 8, 8), np.zeros((64, 64, 3, 3), np.uint8), None, 1, 2, 1, 0.1, 0, 0.1, 128, 0.1, 0)
     assert not p64.maxpool_fusable(2, 2, 3, 2, 1, 0.1, 0, 0.1, 0)

@@ -264,6 +264,50 @@ def test_convolution_and_relu_run_as_one_kernel(own_rt):
     ws.delete()
 
 
+def test_stem_convolution_relu_and_max_pooling_run_as_one_kernel(own_rt):
+    """conv_2d (3 channels, 7x7, stride 2) -> relu -> max pooling 3x3 / 2 / 1 with equal scales: the relu passes the
+    convolution's launch on to the pooling, which runs all three in the convolution's kernel (no relu in between: the
+    pooling takes the launch directly).  A pooling the kernel does not implement (2x2), a relu that rescales, or a
+    host that asks for an intermediate tensor get the operators one by one, with the same bytes."""
+    import ctypes as C
+    from oracle import orc
+    from nart_amd import art
+    pools = own_rt.libs[1].hip_module_fused_pools
+    pools.restype = C.c_long
+    ws = own_rt.workspace("hip")
+    rng = np.random.default_rng(23)
+    x = rng.integers(0, 256, (2, 3, 64, 48), dtype=np.uint8)
+    w = rng.integers(0, 256, (64, 3, 7, 7), dtype=np.uint8)
+    b = rng.integers(-5000, 5000, 64).astype(np.int32)
+    q = dict(ialpha=0.031, izp=77, walpha=0.0042, wzp=128, oalpha=0.09, ozp=60)
+    want_c = orc.conv2d_u8(x, w, b, 3, 2, 1, 0.031, 77, 0.0042, 128, 0.09, 60)
+    want_r = orc.relu_u8(want_c, 0.09, 60, 0.09, 60)
+    qs = dict(ialpha=0.09, izp=60, oalpha=0.09, ozp=60)
+    for with_relu, kernel, pad, peek, expect in ((True, 3, 1, False, 1), (False, 3, 1, False, 1), (True, 2, 0, False, 0),
+                                                 (True, 3, 1, True, 0)):
+        conv = ws.conv2d(ws.tensor(x), ws.tensor(w), ws.tensor(b), 3, 2, 1, q).prepare()
+        relu = ws.relu(conv.output(0), qs).prepare() if with_relu else None
+        src = relu if with_relu else conv
+        pool = ws.pool(src.output(0), kernel, pad, 2, 0, False, qs).prepare()  # method 0: max
+        n0 = pools()
+        conv.run()
+        if relu:
+            relu.run()
+        if peek:  # the host reads the relu's output before the pooling runs: the deferred launch happens here
+            assert same_bits(relu.output(0).numpy(), want_r)
+        pool.run()
+        want = orc.pool_u8(want_r if with_relu else want_c, kernel, pad, 2, 0, False, 0.09, 60, 0.09, 60)
+        assert same_bits(pool.output(0).numpy(), want), (with_relu, kernel, peek)
+        assert pools() == n0 + expect, (with_relu, kernel, peek)
+        # the intermediate tensors are still there for whoever asks
+        assert same_bits(src.output(0).numpy(), want_r if with_relu else want_c)
+        pool.delete()
+        if relu:
+            relu.delete()
+        conv.delete()
+    ws.delete()
+
+
 def test_concat_softmax_through_the_op_api(own_rt):
     import refrun
     from oracle import orc
