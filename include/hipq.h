@@ -182,6 +182,23 @@ int hipq_conv2d_run_add(const hipq_conv2d_plan *plan, const void *x, const void 
                         float res_alpha, int res_zp, float oalpha, int ozp, int obits, void *y, void *stream);
 
 /*
+ * hipq_conv2d_run_add followed, in the same kernel, by the 1x1 convolution `next` that reads the sum (the last layer of
+ * one bottleneck block, its residual add, and the first layer of the next block): y = add(conv(x), residual) and
+ * y_next = next(y), bit-identical to hipq_conv2d_run_add followed by hipq_conv2d_run(next, y, y_next).  The sum is
+ * written once and never read back.  Serves uint8 plans where `plan` is a 1x1 convolution from 64 or 128 to a multiple
+ * of 64 (at most 1024) channels over at least 1024 pixels that the widening kernel computes, and `next` a 1x1 / stride 1
+ * convolution of the same pixels to 64 or 128 channels (channel stride equal to that) whose input scale and zero point
+ * are the sum's oalpha / ozp, obits 8, weight zero points 128, per-tensor weight scales.
+ * hipq_conv2d_add_conv_fusable answers (1 / 0) whether two plans and an add can run this way;
+ * hipq_conv2d_run_add_conv fails with an error otherwise.  A ReLU that `next` was created with applies to y_next.
+ */
+int hipq_conv2d_add_conv_fusable(const hipq_conv2d_plan *plan, int residual_is_input0, float res_alpha, int res_zp,
+                                 float oalpha, int ozp, int obits, const hipq_conv2d_plan *next);
+int hipq_conv2d_run_add_conv(const hipq_conv2d_plan *plan, const void *x, const void *residual, int residual_is_input0,
+                             float res_alpha, int res_zp, float oalpha, int ozp, int obits, void *y,
+                             const hipq_conv2d_plan *next, void *y_next, void *stream);
+
+/*
  * Convolution with the max pooling that follows it in one kernel: y = maxpool3x3/2/1(conv(x)), bit-identical to
  * hipq_conv2d_run followed by hipq_pool_u8(HIPQ_POOL_MAX, kernel 3, stride 2, pad 1) whose input and output scale and
  * zero point both equal the convolution's output parameters (op_conv_2d_u8xu8_run, then op_quant_pool_max_run -

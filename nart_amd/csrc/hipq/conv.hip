@@ -2145,6 +2145,56 @@ extern "C" int hipq_conv2d_run_add(const hipq_conv2d_plan *p, const void *x, con
     return run_conv(p, a, static_cast<hipStream_t>(stream));
 }
 
+// the launch arguments of hipq_conv2d_run_add for plan p (everything but the tensors)
+static bool add_args(const hipq_conv2d_plan *p, int residual_is_input0, float res_alpha, int res_zp, float oalpha, int ozp,
+                     int obits, ConvArgs *a)
+{
+    *a = p->args;
+    a->res = a->padbuf; // any non-null pointer; the caller sets the real one
+    a->res_first = residual_is_input0 ? 1 : 0;
+    return residual_is_input0 ? make_add_params(res_alpha, res_zp, p->d.oalpha, p->d.ozp, oalpha, ozp, obits, &a->addq)
+                              : make_add_params(p->d.oalpha, p->d.ozp, res_alpha, res_zp, oalpha, ozp, obits, &a->addq);
+}
+
+extern "C" int hipq_conv2d_add_conv_fusable(const hipq_conv2d_plan *p, int residual_is_input0, float res_alpha, int res_zp,
+                                            float oalpha, int ozp, int obits, const hipq_conv2d_plan *next)
+{
+    if (!p || !next || p->variant != kMfma || next->variant != kMfma || !p->special || p->tile_selected || p->has_wzp
+        || next->has_wzp || p->d.dtype != HIPQ_DTYPE_U8 || next->d.dtype != HIPQ_DTYPE_U8 || obits != 8)
+        return 0;
+    if (res_zp < 0 || res_zp > 255 || ozp < 0 || ozp > 255)
+        return 0;
+    // the next layer must read the sum with the scale and zero point it is written with
+    if (next->d.ialpha != oalpha || next->d.izp != ozp)
+        return 0;
+    ConvArgs a;
+    if (!add_args(p, residual_is_input0, res_alpha, res_zp, oalpha, ozp, obits, &a))
+        return 0;
+    return conv_expand_chain_applies(a, next->args) ? 1 : 0;
+}
+
+extern "C" int hipq_conv2d_run_add_conv(const hipq_conv2d_plan *p, const void *x, const void *residual, int residual_is_input0,
+                                        float res_alpha, int res_zp, float oalpha, int ozp, int obits, void *y,
+                                        const hipq_conv2d_plan *next, void *y_next, void *stream)
+{
+    clear_error();
+    HIPQ_REQUIRE(p && next && x && y && residual && y_next, "hipq_conv2d_run_add_conv: null argument");
+    HIPQ_REQUIRE(hipq_conv2d_add_conv_fusable(p, residual_is_input0, res_alpha, res_zp, oalpha, ozp, obits, next),
+                 "hipq_conv2d_run_add_conv: these two plans (%s, then %s) do not run as one kernel: run hipq_conv2d_run_add and "
+                 "hipq_conv2d_run", p->name.c_str(), next->name.c_str());
+    ConvArgs a, a2 = next->args;
+    add_args(p, residual_is_input0, res_alpha, res_zp, oalpha, ozp, obits, &a);
+    a.x = static_cast<const uint8_t *>(x);
+    a.y = static_cast<uint8_t *>(y);
+    a.res = static_cast<const uint8_t *>(residual);
+    a.acc_out = nullptr;
+    a2.x = nullptr;
+    a2.y = static_cast<uint8_t *>(y_next);
+    a2.acc_out = nullptr;
+    launch_conv_expand_chain(a, a2, static_cast<hipStream_t>(stream));
+    return launch_status("conv_mfma_expand_kernel (chained)");
+}
+
 extern "C" int hipq_conv2d_maxpool_fusable(const hipq_conv2d_plan *p, int OH, int OW, int kernel, int stride, int pad,
                                            float ialpha, int izp, float oalpha, int ozp, int obits)
 {

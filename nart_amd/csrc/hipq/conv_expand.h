@@ -9,5 +9,9 @@ namespace hipq {
 // layer the kernel can compute, not only those where it measured faster than the kernels it replaces
 bool conv_expand_applies(const ConvArgs &a, bool wherever);
 void launch_conv_expand(const ConvArgs &a, hipStream_t st);
+// chained form: a (with its residual add) followed, in the same kernel, by the 1x1 convolution a2 that reads the sum
+// (a2.x is not used: the sum's bytes never come back from memory; a2.y receives a2's output)
+bool conv_expand_chain_applies(const ConvArgs &a, const ConvArgs &a2);
+void launch_conv_expand_chain(const ConvArgs &a, const ConvArgs &a2, hipStream_t st);
 
 } // namespace hipq

@@ -23,6 +23,13 @@
 //     16-byte pieces then leave as 128-bit stores; without a residual they go to a staging tile.  Those stores are issued
 //     one tile late, after the next tile's multiplies, so that the wait for the next tile's operands - vmcnt counts loads
 //     and stores alike - never waits for a store that was issued a moment ago.
+//   * chained form: the 1x1 convolution that READS the sum (the first layer of the next bottleneck block: 256 -> 64,
+//     512 -> 128) runs in the same kernel.  A wave owns all 64 channels of its 32 pixels in every tile, so the bytes it has
+//     just written to LDS are, for those pixels, one 64-byte slab of the next convolution's reduction: after each tile
+//     it multiplies them with that slab of the next layer's weights (fetched beside the tile's own) into a second set of
+//     accumulators, and after the last tile it requantises those and stores the next layer's output.  The sum is still
+//     written (the next block's add reads it), but never read back: a launch, and one pass over the largest tensors
+//     of the network, disappear.  A work-group then takes whole rows of tiles (all channels of 128 pixels).
 // Requirements (checked by the host): 1x1 kernel, no padding, one group, input channel stride 64, 128 or 256, at most
 // 1024 output channels (their folded biases sit in LDS), weight zero point 128 (or int8), one-multiply requantisation,
 // 32-bit form of the add, output rows of whole 16-byte pieces.
@@ -36,11 +43,12 @@ constexpr int kBM = 128, kBN = 64, kOSTR = kBN + 16; // pixels and channels of a
 constexpr int kMaxTiles = 16;                        // channel tiles, at most (their folded biases sit in LDS)
 
 // The wave's 32 x 64 accumulators -> bytes in the staging tile (row = pixel of the work-group, 80-byte rows).
-template <bool PLAIN_SAT>
-__device__ inline void plain_to_staging(const ConvArgs &a, const v16i (&acc)[2], uint8_t *stg, int pl, int half)
+template <bool PLAIN_SAT, int TN = 2>
+__device__ inline void plain_to_staging(const ConvArgs &a, const v16i (&acc)[TN], uint8_t *stg, int pl, int half)
 {
+    constexpr int kOSTR = TN * 32 + 16; // shadows the tile's: rows of TN * 32 channels
 #pragma unroll
-    for (int tn = 0; tn < 2; tn++)
+    for (int tn = 0; tn < TN; tn++)
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             uint32_t packed;
@@ -120,23 +128,35 @@ __device__ inline void fused_in_place(const ConvArgs &a, const v16i (&acc)[2], u
 
 } // namespace
 
-template <int NSLAB, bool FUSED, bool SAT>
-__global__ __launch_bounds__(256) void conv_mfma_expand_kernel(const ConvArgs a, const int ntiles, const int total)
+// MID: 0, or the output channels (64 / 128) of the chained 1x1 convolution a2, whose output goes to a2.y
+template <int NSLAB, bool FUSED, bool SAT, int MID>
+__global__ __launch_bounds__(256) void conv_mfma_expand_kernel(const ConvArgs a, const ConvArgs a2, const int ntiles, const int total)
 {
     constexpr int WBYTES = NSLAB * 4096;         // one channel tile of weights: NSLAB slabs of 64 rows x 64 bytes
     constexpr int RBYTES = kBM * kBN;            // one residual tile
     constexpr int R_OFF = 2 * WBYTES;            // fused: two residual tiles; plain: one staging tile
     constexpr int B_OFF = R_OFF + (FUSED ? 2 * RBYTES : kBM * kOSTR);
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[B_OFF + kMaxTiles * kBN * 4];
+    constexpr int W2BYTES = MID * 64;            // chained: one slab of the next layer's weights (MID rows x 64 bytes)
+    constexpr int W2_OFF = B_OFF + kMaxTiles * kBN * 4, S2_OFF = W2_OFF + 2 * W2BYTES; // then its output staging tile
+    constexpr int TN2 = MID / 32;
+    static_assert(MID == 0 || (FUSED && SAT && (MID == 64 || MID == 128)), "the chained form follows a fused add to uint8");
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[S2_OFF + (MID ? kBM * (MID + 16) : 0)];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int half = lane >> 5, p = lane & 31, swz = (lane >> 2) & 3;
     // work-groups go to the 8 XCDs in turn: XCD x takes the x-th contiguous eighth of the tile list (the grid is a
     // multiple of 8), so neighbours in the list - which share pixels or weights - share an L2
     const int g = (int)(blockIdx.x % 8) * (int)(gridDim.x / 8) + (int)(blockIdx.x / 8);
-    const int t0 = (int)((long long)total * g / (int)gridDim.x), t1 = (int)((long long)total * (g + 1) / (int)gridDim.x);
-    if (t0 >= t1)
-        return;
+    int t0, t1;
+    if (MID) { // whole rows of tiles: work-group g takes the 128 pixels of row g
+        t0 = g * ntiles, t1 = t0 + ntiles;
+        if (t0 >= total)
+            return;
+    } else {
+        t0 = (int)((long long)total * g / (int)gridDim.x), t1 = (int)((long long)total * (g + 1) / (int)gridDim.x);
+        if (t0 >= t1)
+            return;
+    }
 
     // ---- tile t -> LDS buffer (t - t0) & 1: its weights, and its residual tile when fused ----
     const size_t wslab = (size_t)a.kout_pad * 64;
@@ -157,6 +177,12 @@ __global__ __launch_bounds__(256) void conv_mfma_expand_kernel(const ConvArgs a,
                 const uint8_t *src = m < a.P && ch < a.out_cs ? a.res + (size_t)m * a.out_cs + ch : a.padbuf;
                 __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(rb + jj * 4096), 16, 0, 0);
             }
+        }
+        if (MID) { // slab nt of the next layer's weights: its input channels 64 nt .. 64 nt + 63 are this tile's outputs
+            const uint8_t *w2 = a2.wpack + (size_t)nt * a2.kout_pad * 64 + tid * 16;
+#pragma unroll
+            for (int jj = 0; jj < W2BYTES / 4096; jj++)
+                __builtin_amdgcn_global_load_lds((gptr_t)(w2 + jj * 4096), (lptr_t)(lds + W2_OFF + buf * W2BYTES + wave_off + jj * 4096), 16, 0, 0);
         }
     };
     int mt = t0 / ntiles, nt = t0 - mt * ntiles; // the current tile; the list is walked without further divisions
@@ -186,6 +212,18 @@ __global__ __launch_bounds__(256) void conv_mfma_expand_kernel(const ConvArgs a,
                 bf[s][k] = ldg128(xrow + s * 64 + k * 32 + half * 16) ^ (int)a.xmask;
     };
     load_pixels(mt);
+    v16i acc2[MID ? TN2 : 1]; // chained: 32 pixels x MID channels of the next layer, from its folded bias
+    if (MID) {
+#pragma unroll
+        for (int tn = 0; tn < TN2; tn++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const v4i bv = *reinterpret_cast<const v4i *>(a2.bias2 + tn * 32 + q * 8 + half * 4);
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    acc2[tn][q * 4 + e] = bv[e];
+            }
+    }
     const int foff[2] = {p * 64 + (((0 + half) ^ swz) << 4), p * 64 + (((2 + half) ^ swz) << 4)};
 
     // the finished tile's 16-byte pieces: four lanes per pixel row, two passes of 64 rows
@@ -254,6 +292,21 @@ __global__ __launch_bounds__(256) void conv_mfma_expand_kernel(const ConvArgs a,
             fused_in_place<SAT>(a, acc, lds + R_OFF + buf * RBYTES, pl, half);
         else
             plain_to_staging<SAT>(a, acc, lds + R_OFF, pl, half);
+        if (MID) {
+            // the 64 bytes this wave has just written for each of its pixels are slab nt of the next layer's reduction
+            __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): own writes
+            const uint8_t *row = lds + R_OFF + buf * RBYTES + pl * kBN, *w2b = lds + W2_OFF + buf * W2BYTES;
+            const int rsw = (pl >> 1) & 3;
+#pragma unroll
+            for (int k = 0; k < 2; k++) {
+                const v4i b2 = *reinterpret_cast<const v4i *>(row + (((2 * k + half) ^ rsw) << 4)) ^ (int)a2.xmask;
+#pragma unroll
+                for (int tn = 0; tn < TN2; tn++) {
+                    const v4i af = *reinterpret_cast<const v4i *>(w2b + tn * 2048 + foff[k]);
+                    acc2[tn] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, b2, acc2[tn], 0, 0, 0);
+                }
+            }
+        }
         pmt = mt, pnt = nt;
         mt = nmt, nt = nnt;
     }
@@ -262,6 +315,24 @@ __global__ __launch_bounds__(256) void conv_mfma_expand_kernel(const ConvArgs a,
     v4i staged[2];
     read_staged((t1 - 1 - t0) & 1, staged);
     store_tile(pmt, pnt, staged);
+    if (MID) {
+        // the next layer's 128 pixels x MID channels: requantise, transpose through LDS, 128-bit stores
+        uint8_t *stg2 = lds + S2_OFF;
+        if (a2.lo == 0 && a2.q.hi == 255)
+            plain_to_staging<true, MID ? TN2 : 1>(a2, acc2, stg2, pl, half);
+        else
+            plain_to_staging<false, MID ? TN2 : 1>(a2, acc2, stg2, pl, half);
+        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
+        __builtin_amdgcn_s_barrier();
+        constexpr int LPR = (MID ? MID : 64) / 16, RPP = 256 / LPR; // lanes per pixel row, rows per pass
+        const int c16 = (tid % LPR) * 16;
+#pragma unroll
+        for (int r = tid / LPR; r < kBM; r += RPP) {
+            const int m = pmt * kBM + r;
+            if (m < a2.P && c16 < a2.out_cs)
+                *reinterpret_cast<v4i *>(a2.y + (size_t)m * a2.out_cs + c16) = *reinterpret_cast<const v4i *>(stg2 + r * (MID + 16) + c16);
+        }
+    }
 }
 
 bool conv_expand_applies(const ConvArgs &a, bool wherever)
@@ -276,11 +347,16 @@ bool conv_expand_applies(const ConvArgs &a, bool wherever)
         && (wherever || (a.res != nullptr ? a.in_cs == 64 : a.in_cs == 256));
 }
 
-template <int NSLAB>
-static void launch_expand_n(const ConvArgs &a, hipStream_t st)
+template <int NSLAB, int MID>
+static void launch_expand_n(const ConvArgs &a, const ConvArgs &a2, hipStream_t st)
 {
     const bool fused = a.res != nullptr;
     const int mtiles = (a.P + kBM - 1) / kBM, ntiles = (a.out_cs + kBN - 1) / kBN, total = mtiles * ntiles;
+    if (MID) {
+        const dim3 grid((unsigned)((mtiles + 7) / 8 * 8)), block(256);
+        hipLaunchKernelGGL((conv_mfma_expand_kernel<NSLAB, true, true, MID>), grid, block, 0, st, a, a2, ntiles, total);
+        return;
+    }
     // three work-groups per CU (measured: two leave the vector units idle while a work-group waits for its tile, four slow
     // every work-group's arithmetic down by more than they hide), fewer where their LDS does not fit; at least two tiles each
     const int lds = 2 * NSLAB * 4096 + (fused ? 2 * kBM * kBN : kBM * kOSTR) + kMaxTiles * kBN * 4;
@@ -289,22 +365,46 @@ static void launch_expand_n(const ConvArgs &a, hipStream_t st)
     const dim3 grid((unsigned)wgs), block(256);
     if (fused) {
         if (a.addq.hi == 255)
-            hipLaunchKernelGGL((conv_mfma_expand_kernel<NSLAB, true, true>), grid, block, 0, st, a, ntiles, total);
+            hipLaunchKernelGGL((conv_mfma_expand_kernel<NSLAB, true, true, 0>), grid, block, 0, st, a, a2, ntiles, total);
         else
-            hipLaunchKernelGGL((conv_mfma_expand_kernel<NSLAB, true, false>), grid, block, 0, st, a, ntiles, total);
+            hipLaunchKernelGGL((conv_mfma_expand_kernel<NSLAB, true, false, 0>), grid, block, 0, st, a, a2, ntiles, total);
     } else if (a.lo == 0 && a.q.hi == 255) {
-        hipLaunchKernelGGL((conv_mfma_expand_kernel<NSLAB, false, true>), grid, block, 0, st, a, ntiles, total);
+        hipLaunchKernelGGL((conv_mfma_expand_kernel<NSLAB, false, true, 0>), grid, block, 0, st, a, a2, ntiles, total);
     } else {
-        hipLaunchKernelGGL((conv_mfma_expand_kernel<NSLAB, false, false>), grid, block, 0, st, a, ntiles, total);
+        hipLaunchKernelGGL((conv_mfma_expand_kernel<NSLAB, false, false, 0>), grid, block, 0, st, a, a2, ntiles, total);
     }
 }
 
 void launch_conv_expand(const ConvArgs &a, hipStream_t st)
 {
     switch (a.nslab) {
-    case 1: launch_expand_n<1>(a, st); break;
-    case 2: launch_expand_n<2>(a, st); break;
-    default: launch_expand_n<4>(a, st); break; // conv_expand_applies: in_cs is 64, 128 or 256
+    case 1: launch_expand_n<1, 0>(a, a, st); break;
+    case 2: launch_expand_n<2, 0>(a, a, st); break;
+    default: launch_expand_n<4, 0>(a, a, st); break; // conv_expand_applies: in_cs is 64, 128 or 256
+    }
+}
+
+bool conv_expand_chain_applies(const ConvArgs &a, const ConvArgs &a2)
+{
+    return a.res != nullptr && conv_expand_applies(a, true) && a.in_cs <= 128 && a.out_cs % kBN == 0 && a.addq.hi == 255
+        && a2.R == 1 && a2.S == 1 && a2.pad_h == 0 && a2.pad_w == 0 && a2.stride_h == 1 && a2.stride_w == 1 && a2.group == 1
+        && a2.bwz == 0 && a2.xmask != 0 && a2.N == a.N && a2.H == a.OH && a2.W == a.OW && a2.in_cs == a.out_cs && a2.P == a.P
+        && a2.nslab == a.out_cs / kBN && (a2.out_cs == 64 || a2.out_cs == 128) && a2.kout_pad >= a2.out_cs && a2.fastq
+        && !plain_epilogue(a2) && a2.res == nullptr;
+}
+
+void launch_conv_expand_chain(const ConvArgs &a, const ConvArgs &a2, hipStream_t st)
+{
+    if (a2.out_cs == 64) {
+        if (a.nslab == 1)
+            launch_expand_n<1, 64>(a, a2, st);
+        else
+            launch_expand_n<2, 64>(a, a2, st);
+    } else {
+        if (a.nslab == 1)
+            launch_expand_n<1, 128>(a, a2, st);
+        else
+            launch_expand_n<2, 128>(a, a2, st);
     }
 }
 

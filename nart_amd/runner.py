@@ -36,6 +36,8 @@ class HipqExecutor:
                         and not any(a is u[0] for a in self.fused.values())):  # one convolution per add
                     self.fused[node.output] = u[0]  # launched at the add's position: both operands exist by then
         self.pooled = {}     # conv output name -> the max-pooling node computed inside the convolution's kernel
+        self.chained = {}    # add output name -> the 1x1 convolution node computed inside the fused add's kernel
+        self._early = {}     # id(conv node) -> its plan, created ahead of its turn (when an add looked at it)
         self._pending = {}   # id(add node) -> the deferred convolution
         self.buf = {}        # tensor name -> device tensor
         self.steps = []      # (label, kernel name, callable, algorithmic ops, compulsory bytes)
@@ -44,7 +46,19 @@ class HipqExecutor:
         T = case.tensors
         inp = case.input
         self.buf[inp.name] = self._tensor(inp)
+        def conv_plan(node):
+            a, x, y = node.attrs, T[node.inputs[0]], T[node.output]
+            plan = self._early.pop(id(node), None)
+            if plan is None:
+                plan = hipq.Conv2d(x.shape, case.weights[a["w"]], case.weights[a["b"]], a["pad"], a["stride"],
+                                   a["group"], x.alpha, x.zp, a["walpha"], a["wzp"], y.alpha, y.zp, relu=a["relu"])
+            nbytes = int(np.prod(x.shape)) + int(np.prod(y.shape)) + case.weights[a["w"]].size + 4 * a["K"]
+            return plan, nbytes
+
+        done = set()  # nodes computed inside an earlier node's kernel
         for node in case.nodes:
+            if id(node) in done:
+                continue
             y = T[node.output]
             xs = [T[i] for i in node.inputs]
             N, C, H, W = y.shape
@@ -61,10 +75,8 @@ class HipqExecutor:
                 self._add(node, "dequantize_u8_kernel", fn, 0, 5 * int(np.prod(y.shape)))
             elif node.kind == "conv":
                 x = xs[0]
-                plan = hipq.Conv2d(x.shape, case.weights[a["w"]], case.weights[a["b"]], a["pad"], a["stride"],
-                                   a["group"], x.alpha, x.zp, a["walpha"], a["wzp"], y.alpha, y.zp, relu=a["relu"])
+                plan, nbytes = conv_plan(node)
                 self.plans.append(plan)
-                nbytes = int(np.prod(x.shape)) + int(np.prod(y.shape)) + case.weights[a["w"]].size + 4 * a["K"]
                 u = [nd for nd in case.nodes if node.output in nd.inputs]
                 if (fuse_add and len(u) == 1 and u[0].kind == "pool" and u[0].attrs["method"] == 0
                         and node.output != case.output.name):
@@ -120,6 +132,32 @@ class HipqExecutor:
                 self._add(node, "pool_u8_kernel", fn, 0, int(np.prod(x.shape)) + int(np.prod(y.shape)))
             elif node.kind == "add" and id(node) in self._pending:
                 plan, xin, other, res_first, ot, st, nbytes = self._pending.pop(id(node))
+                # the 1x1 convolution that reads the sum (the first layer of the next block) in the same kernel
+                nxt = None
+                for nd in case.nodes:
+                    na = nd.attrs
+                    if (nd.kind == "conv" and nd.inputs[0] == node.output and na["k"] == 1 and na["stride"] == 1
+                            and na["pad"] == 0 and na["group"] == 1 and nd.output != case.output.name):
+                        p2, nb2 = conv_plan(nd)
+                        if plan.add_conv_fusable(res_first, ot.alpha, ot.zp, st.alpha, st.zp, p2):
+                            nxt = (nd, p2, nb2)
+                            break
+                        self._early[id(nd)] = p2
+                if nxt is not None:
+                    nd, p2, nb2 = nxt
+                    y2 = self._tensor(T[nd.output])
+                    if y2 is None:
+                        raise RuntimeError("shared executor: %s is fused away in the parent but not here" % nd.output)
+                    self.buf[nd.output] = y2
+                    self.plans.append(p2)
+                    self.chained[node.output] = nd
+                    done.add(id(nd))
+                    fn = (lambda p=plan, i=xin, r=self.buf[other], rf=res_first, ot=ot, st=st, o=out, p2=p2, y2=y2:
+                          p.run_add_conv(i, r, rf, ot.alpha, ot.zp, st.alpha, st.zp, o, p2, y2))
+                    self.steps.append({"label": node.output, "kind": "conv+add+conv", "kernel": "conv_mfma_i8_expand+add+conv",
+                                       "fn": fn, "ops": plan.ops + p2.ops, "bytes": nbytes + nb2 - int(np.prod(st.shape)),
+                                       "plan": plan})
+                    continue
                 fn = (lambda p=plan, i=xin, r=self.buf[other], rf=res_first, ot=ot, st=st, o=out:
                       p.run_add(i, r, rf, ot.alpha, ot.zp, st.alpha, st.zp, o))
                 self.steps.append({"label": node.output, "kind": "conv+add", "kernel": plan.kernel_add or plan.kernel + "+add", "fn": fn,
@@ -267,8 +305,10 @@ class BranchedExecutor:
         self.parts = [HipqExecutor(build(hi - lo), fuse_add=bool(parent.fused), share=(parent, lo))
                       for lo, hi in zip(bounds[:-1], bounds[1:])]
         for p in self.parts:
-            if [s["label"] for s in p.steps] != [s["label"] for s in parent.steps]:
-                raise RuntimeError("part-batch executor launches a different operator list than its parent")
+            # a part may cut its launches differently (a kernel that serves two operators at the parent's size need not
+            # at the part's), but it must materialise exactly the parent's tensors: they are slices of the same buffers
+            if p.elided != parent.elided or set(p.buf) != set(parent.buf):
+                raise RuntimeError("part-batch executor materialises other tensors than its parent")
         self.side = [torch.cuda.Stream() for _ in self.parts[1:]]  # default priority
         self.graph = None
 

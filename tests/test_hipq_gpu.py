@@ -208,6 +208,60 @@ def test_channel_widening_1x1_layers():
         assert np.array_equal(got, orc.conv2d_i8(x, w, b, 0, 1, 1, 0.02, 0.004, 0.09, obits=obits)), obits
 
 
+def test_fused_add_chained_with_the_next_1x1_convolution():
+    """hipq_conv2d_run_add_conv: the widening 1x1 convolution of a bottleneck block, its residual add and the first 1x1
+    convolution of the next block in one kernel, against the oracle's three operators: both operand orders of the add,
+    64 and 128 channels out of the second convolution, with and without its ReLU, ragged pixel counts, five channel tiles.
+    The sum itself is written as well.  Pairs the kernel does not serve are refused."""
+    rng = np.random.default_rng(78)
+    shapes = [  # N, C, H, W, K, mid, relu
+        (2, 64, 28, 28, 256, 64, True), (1, 128, 40, 30, 512, 128, True), (1, 64, 33, 37, 256, 128, False),
+        (3, 128, 21, 19, 320, 64, True),
+    ]
+    for i, (N, C, H, W, K, mid, relu) in enumerate(shapes):
+        x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+        w = rng.integers(0, 256, (K, C, 1, 1), dtype=np.uint8)
+        b = rng.integers(-30000, 30000, K).astype(np.int32)
+        w2 = rng.integers(0, 256, (mid, K, 1, 1), dtype=np.uint8)
+        b2 = rng.integers(-30000, 30000, mid).astype(np.int32)
+        for res_first, ratio in ((False, 1.0), (True, 1.7)):
+            # output scales of the order of the accumulators' spread: the requantisation shifts then lie inside the range of
+            # the one-multiply form, which the kernel requires (as the scales of a calibrated network do)
+            ia, wa = rand_q(rng), rand_q(rng)
+            q = (ia, int(rng.integers(0, 256)), wa, 128, float(np.float32(ia * wa * np.sqrt(C) * 40.0)), int(rng.integers(0, 256)))
+            plan = hipq.Conv2d(x.shape, w, b, 0, 1, 1, *q)
+            conv = orc.conv2d_u8(x, w, b, 0, 1, 1, *q)
+            res = rng.integers(0, 256, conv.shape, dtype=np.uint8)
+            ra, rz = float(np.float32(q[4] * ratio)), int(rng.integers(0, 256))
+            oa, oz = float(np.float32(max(q[4], ra) * 1.3)), int(rng.integers(0, 256))
+            want = orc.add_u8(res, conv, ra, rz, q[4], q[5], oa, oz) if res_first else orc.add_u8(conv, res, q[4], q[5], ra, rz, oa, oz)
+            wa2 = rand_q(rng)
+            q2 = (oa, oz, wa2, 128, float(np.float32(oa * wa2 * np.sqrt(K) * 40.0)), int(rng.integers(0, 256)))
+            nxt = hipq.Conv2d(want.shape, w2, b2, 0, 1, 1, *q2, relu=relu)
+            want2 = orc.conv2d_u8(want, w2, b2, 0, 1, 1, *q2)
+            if relu:
+                want2 = orc.relu_u8(want2, q2[4], q2[5], q2[4], q2[5])
+            print("chained case", i, x.shape, K, mid, relu, res_first, flush=True)
+            assert plan.add_conv_fusable(res_first, ra, rz, oa, oz, nxt)
+            y, y2 = plan.empty_output(), nxt.empty_output()
+            y.fill_(3), y2.fill_(5)
+            plan.run_add_conv(hipq.to_device_nhwc(x), hipq.to_device_nhwc(res), res_first, ra, rz, oa, oz, y, nxt, y2)
+            torch.cuda.synchronize()
+            got, got2 = hipq.from_device_nhwc(y, K), hipq.from_device_nhwc(y2, mid)
+            assert np.array_equal(got, want), (i, res_first, "sum", int((got != want).sum()))
+            assert np.array_equal(got2, want2), (i, res_first, "next layer", int((got2 != want2).sum()))
+            # refusals: another input scale of the second convolution, a 3x3 second convolution, an explicit tile
+            other = hipq.Conv2d(want.shape, w2, b2, 0, 1, 1, float(np.float32(oa * 1.01)), oz, *q2[2:])
+            assert not plan.add_conv_fusable(res_first, ra, rz, oa, oz, other)
+            if i == 0:
+                k3 = hipq.Conv2d(want.shape, rng.integers(0, 256, (mid, K, 3, 3), dtype=np.uint8), b2, 1, 1, 1, *q2)
+                assert not plan.add_conv_fusable(res_first, ra, rz, oa, oz, k3)
+                with pytest.raises(hipq.HipqError, match="do not run as one kernel"):
+                    plan.run_add_conv(hipq.to_device_nhwc(x), hipq.to_device_nhwc(res), res_first, ra, rz, oa, oz, y, k3, k3.empty_output())
+                plan.select(4, 0)
+                assert not plan.add_conv_fusable(res_first, ra, rz, oa, oz, nxt)
+
+
 def test_conv_grouped_and_depthwise():
     rng = np.random.default_rng(13)
     kerns = set()
