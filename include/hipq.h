@@ -190,13 +190,14 @@ int hipq_conv2d_run_add(const hipq_conv2d_plan *plan, const void *x, const void 
  * convolution of the same pixels to 64 or 128 channels (channel stride equal to that) whose input scale and zero point
  * are the sum's oalpha / ozp, obits 8, weight zero points 128, per-tensor weight scales.
  * hipq_conv2d_add_conv_fusable answers (1 / 0) whether two plans and an add can run this way;
- * hipq_conv2d_run_add_conv fails with an error otherwise.  A ReLU that `next` was created with applies to y_next.
+ * hipq_conv2d_run_add_conv fails with an error otherwise.  A ReLU that `next` was created with applies to y_next;
+ * next_relu != 0 applies the ReLU clamp of hipq_conv2d_run_relu to y_next whatever `next` was created with.
  */
 int hipq_conv2d_add_conv_fusable(const hipq_conv2d_plan *plan, int residual_is_input0, float res_alpha, int res_zp,
                                  float oalpha, int ozp, int obits, const hipq_conv2d_plan *next);
 int hipq_conv2d_run_add_conv(const hipq_conv2d_plan *plan, const void *x, const void *residual, int residual_is_input0,
                              float res_alpha, int res_zp, float oalpha, int ozp, int obits, void *y,
-                             const hipq_conv2d_plan *next, void *y_next, void *stream);
+                             const hipq_conv2d_plan *next, int next_relu, void *y_next, void *stream);
 
 /*
  * Convolution with the max pooling that follows it in one kernel: y = maxpool3x3/2/1(conv(x)), bit-identical to

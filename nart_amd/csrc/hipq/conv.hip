@@ -2175,7 +2175,7 @@ extern "C" int hipq_conv2d_add_conv_fusable(const hipq_conv2d_plan *p, int resid
 
 extern "C" int hipq_conv2d_run_add_conv(const hipq_conv2d_plan *p, const void *x, const void *residual, int residual_is_input0,
                                         float res_alpha, int res_zp, float oalpha, int ozp, int obits, void *y,
-                                        const hipq_conv2d_plan *next, void *y_next, void *stream)
+                                        const hipq_conv2d_plan *next, int next_relu, void *y_next, void *stream)
 {
     clear_error();
     HIPQ_REQUIRE(p && next && x && y && residual && y_next, "hipq_conv2d_run_add_conv: null argument");
@@ -2191,6 +2191,8 @@ extern "C" int hipq_conv2d_run_add_conv(const hipq_conv2d_plan *p, const void *x
     a2.x = nullptr;
     a2.y = static_cast<uint8_t *>(y_next);
     a2.acc_out = nullptr;
+    if (next_relu)
+        a2.lo = std::min(next->d.ozp, a2.q.hi); // the ReLU clamp, as in hipq_conv2d_run_relu
     launch_conv_expand_chain(a, a2, static_cast<hipStream_t>(stream));
     return launch_status("conv_mfma_expand_kernel (chained)");
 }

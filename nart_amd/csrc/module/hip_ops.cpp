@@ -93,7 +93,7 @@ typedef std::map<const mem_t *, std::set<const op_t *>> reader_map;
 
 // keyed by workspace (the runtime is single-threaded, art/include/art/workspace.h has no locking either)
 std::map<const workspace_t *, reader_map> g_readers;
-long g_fused_adds = 0, g_fused_relus = 0, g_fused_pools = 0; // fused launches so far (hip_module_fused_adds / _relus / _pools)
+long g_fused_adds = 0, g_fused_relus = 0, g_fused_pools = 0, g_chained_convs = 0; // fused launches so far (hip_module_fused_*)
 
 reader_map &readers_of(op_t *op) { return g_readers[op->workspace]; }
 
@@ -189,6 +189,9 @@ void conv_launch_plain(void *ctx)
 bool eltwise_is_plain_sum(const op_t *op); // two inputs, SUM, unit coefficients: computes what add computes
 // a max pooling that the stem convolution's kernel can compute as well (hipq_conv2d_maxpool_fusable)
 bool pool_fuses_with(const op_t *pool_op, const hipq_conv2d_plan *plan);
+// the convolution `op` as the tail of the kernel that computes the add it reads (hipq_conv2d_run_add_conv); y: where its
+// output goes, relu: with the ReLU clamp.  false: not possible, run it plainly
+bool conv_run_chained(op_t *op, void *y, int relu);
 
 // 1: the only reader of the convolution's output is an add or a relu of this workspace that can take over the launch
 bool sole_reader_fuses(op_t *op)
@@ -225,6 +228,8 @@ void conv_run(op_t *op)
         ym->pending_ctx = op;
         return;
     }
+    if (conv_run_chained(op, out_ptr(op), 0))
+        return;
     HIPM_HIPQ(hipq_conv2d_run(c->plan, in_ptr(op, 0), out_ptr(op), nullptr, op_stream(op)));
 }
 
@@ -346,7 +351,8 @@ struct ew_op_t {
     uint32_t operation;
     float *coeff;
     size_t bytes; // device bytes to process (pad channels included)
-    int defer;    // relu: 0 undecided, 1 leave the (fused) launch to the max pooling that reads the output, -1 launch at run()
+    int defer;    // 0 undecided, 1 leave the (fused) launch to a reader of the output (relu: a max pooling; add: a 1x1
+                  // convolution), -1 launch at run()
 };
 
 size_t device_bytes_of(const tensor_t *t)
@@ -385,40 +391,145 @@ bool eltwise_is_plain_sum(const op_t *op)
         && e->coeff[0] == 1.0f && e->coeff[1] == 1.0f;
 }
 
-// the add (or plain two-input SUM) `op` as the epilogue of the convolution that left it its launch; false: run it plainly
-bool run_fused_into_convolution(op_t *op)
+// which input of the add (or plain two-input SUM) `op` is a convolution that left it its launch (conv_run) and whose
+// output the add reads with the scale it was written with; -1: none
+int deferred_conv_input(op_t *op)
 {
-    ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    const ew_op_t *e = reinterpret_cast<const ew_op_t *>(op);
     for (int i = 0; i < 2; ++i) {
         hip_mem_t *m = as_hip(op->input_tensors[i]->mem);
         if (m->pending != conv_launch_plain)
             continue;
-        // input i is a convolution that left its launch to this add (conv_run): run both as one kernel, provided the
-        // add reads the convolution's output with the scale it was written with
-        op_t *cop = static_cast<op_t *>(m->pending_ctx);
-        conv_op_t *c = reinterpret_cast<conv_op_t *>(cop);
-        const int o = 1 - i;
-        if (e->qi.alpha[i] != c->desc.oalpha || e->qi.zp[i] != c->desc.ozp)
-            break;
-        const void *res = in_ptr(op, o); // settles the other input if it is deferred as well
-        const void *x = in_ptr(cop, 0);
-        if (hipq_conv2d_run_add(c->plan, x, res, o == 0, e->qi.alpha[o], e->qi.zp[o], e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0],
-                                out_ptr(op), op_stream(op)) == 0) {
-            ++g_fused_adds;
-            return true; // the convolution's own output stays unwritten; its hook stays for whoever asks
-        }
-        break; // parameters outside the fused kernel's range: the caller's plain path settles the hook
+        const conv_op_t *c = reinterpret_cast<const conv_op_t *>(static_cast<op_t *>(m->pending_ctx));
+        return e->qi.alpha[i] == c->desc.oalpha && e->qi.zp[i] == c->desc.ozp ? i : -1;
     }
-    return false;
+    return -1;
+}
+
+// the add `op` as the epilogue of the convolution that left it its launch, into y; false: run it plainly
+bool run_fused_into_convolution(op_t *op, void *y)
+{
+    ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    const int i = deferred_conv_input(op);
+    if (i < 0)
+        return false;
+    op_t *cop = static_cast<op_t *>(as_hip(op->input_tensors[i]->mem)->pending_ctx);
+    conv_op_t *c = reinterpret_cast<conv_op_t *>(cop);
+    const int o = 1 - i;
+    const void *res = in_ptr(op, o); // settles the other input if it is deferred as well
+    const void *x = in_ptr(cop, 0);
+    if (hipq_conv2d_run_add(c->plan, x, res, o == 0, e->qi.alpha[o], e->qi.zp[o], e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0], y,
+                            op_stream(op)) != 0)
+        return false; // parameters outside the fused kernel's range: the caller's plain path settles the hook
+    ++g_fused_adds;
+    return true; // the convolution's own output stays unwritten; its hook stays for whoever asks
+}
+
+void add_plain_into(op_t *op, void *y)
+{
+    ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    if (op->entry->tp == &op_add_tp) {
+        HIPM_HIPQ(hipq_add_u8(in_ptr(op, 0), in_ptr(op, 1), y, e->bytes, e->qi.alpha[0], e->qi.zp[0], e->qi.alpha[1], e->qi.zp[1],
+                              e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0], op_stream(op)));
+        return;
+    }
+    const void *ins[HIPQ_MAX_ELTWISE_INPUTS];
+    for (size_t i = 0; i < op->input_size; ++i)
+        ins[i] = in_ptr(op, (int)i);
+    HIPM_HIPQ(hipq_eltwise_u8(ins, (int)op->input_size, e->coeff, e->qi.alpha, e->qi.zp, y, e->bytes, (int)e->operation,
+                              e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0], op_stream(op)));
+}
+
+// The hook an add leaves on its output when a 1x1 convolution that reads the sum can run in the same kernel
+// (add_defers): that convolution's run() launches hipq_conv2d_run_add_conv; whoever else asks for the sum first gets
+// the convolution + add launch (or the plain add).
+void add_launch_deferred(void *ctx)
+{
+    op_t *op = static_cast<op_t *>(ctx);
+    void *y = as_hip(op->output_tensors[0].mem)->dev;
+    if (!run_fused_into_convolution(op, y))
+        add_plain_into(op, y);
+}
+
+// Does the add leave its launch to a reader?  Decided once per prepare: a convolution was deferred into this add, and a
+// 1x1 convolution of this workspace reads the sum and can run as the tail of the same kernel.
+bool add_defers(op_t *op)
+{
+    ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    const int i = deferred_conv_input(op);
+    if (i < 0)
+        return false;
+    if (e->defer == 0) {
+        static const bool off = getenv("NART_HIP_NO_FUSION") != nullptr;
+        e->defer = -1;
+        const conv_op_t *c = reinterpret_cast<const conv_op_t *>(static_cast<op_t *>(as_hip(op->input_tensors[i]->mem)->pending_ctx));
+        const int o = 1 - i;
+        const reader_map &rm = readers_of(op);
+        const auto it = rm.find(op->output_tensors[0].mem);
+        if (!off && it != rm.end())
+            for (const op_t *r : it->second) {
+                if (r->workspace != op->workspace || r->entry->tp != &op_conv_2d_tp)
+                    continue;
+                const conv_op_t *rc = reinterpret_cast<const conv_op_t *>(r);
+                if (rc->plan != nullptr && r->input_tensors[0]->mem == op->output_tensors[0].mem
+                    && hipq_conv2d_add_conv_fusable(c->plan, o == 0, e->qi.alpha[o], e->qi.zp[o], e->qo.alpha[0], e->qo.zp[0],
+                                                    e->qo.bits[0], rc->plan)) {
+                    e->defer = 1;
+                    break;
+                }
+            }
+    }
+    return e->defer == 1;
+}
+
+bool add_or_sum_run_fused(op_t *op)
+{
+    if (add_defers(op)) {
+        hip_mem_t *ym = as_hip(op->output_tensors[0].mem);
+        (void)out_ptr(op); // the buffer exists and the device side is the current one - once the hook has run
+        ym->pending = add_launch_deferred;
+        ym->pending_ctx = op;
+        return true;
+    }
+    return run_fused_into_convolution(op, out_ptr(op));
+}
+
+bool conv_run_chained(op_t *op, void *y, int relu)
+{
+    hip_mem_t *sm = as_hip(op->input_tensors[0]->mem); // the sum
+    if (sm->pending != add_launch_deferred)
+        return false;
+    op_t *aop = static_cast<op_t *>(sm->pending_ctx);
+    ew_op_t *e = reinterpret_cast<ew_op_t *>(aop);
+    const int i = deferred_conv_input(aop);
+    if (i < 0)
+        return false; // somebody asked for the first convolution's own output in between: it has run
+    op_t *cop = static_cast<op_t *>(as_hip(aop->input_tensors[i]->mem)->pending_ctx);
+    conv_op_t *c = reinterpret_cast<conv_op_t *>(cop), *c2 = reinterpret_cast<conv_op_t *>(op);
+    const int o = 1 - i;
+    if (!hipq_conv2d_add_conv_fusable(c->plan, o == 0, e->qi.alpha[o], e->qi.zp[o], e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0],
+                                      c2->plan))
+        return false;
+    const void *res = in_ptr(aop, o);
+    const void *x = in_ptr(cop, 0);
+    if (sm->pending != add_launch_deferred)
+        return false; // settling the residual reached the sum (it cannot: the sum is not its own input), be safe
+    sm->pending = nullptr; // the sum is written by the launch below
+    if (hipq_conv2d_run_add_conv(c->plan, x, res, o == 0, e->qi.alpha[o], e->qi.zp[o], e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0],
+                                 sm->dev, c2->plan, relu, y, op_stream(op)) != 0) {
+        add_launch_deferred(aop); // cannot happen after the check above; keep the sum correct anyway
+        return false;
+    }
+    ++g_fused_adds;
+    ++g_chained_convs;
+    return true;
 }
 
 void add_run(op_t *op)
 {
-    ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
-    if (run_fused_into_convolution(op))
+    if (add_or_sum_run_fused(op))
         return;
-    HIPM_HIPQ(hipq_add_u8(in_ptr(op, 0), in_ptr(op, 1), out_ptr(op), e->bytes, e->qi.alpha[0], e->qi.zp[0], e->qi.alpha[1],
-                          e->qi.zp[1], e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0], op_stream(op)));
+    add_plain_into(op, out_ptr(op));
 }
 
 void add_prepare(op_t *op)
@@ -428,6 +539,7 @@ void add_prepare(op_t *op)
     alloc_and_tag(op);
     same_geometry(op); // broadcasting adds are not implemented (the reference's loop has none either, add.c:135)
     e->bytes = device_bytes_of(&op->output_tensors[0]);
+    e->defer = 0;
     op->run_func = add_run;
 }
 
@@ -450,7 +562,7 @@ void eltwise_config(op_t *op)
 void eltwise_run(op_t *op)
 {
     ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
-    if (eltwise_is_plain_sum(op) && run_fused_into_convolution(op))
+    if (eltwise_is_plain_sum(op) && add_or_sum_run_fused(op))
         return;
     const void *ins[HIPQ_MAX_ELTWISE_INPUTS];
     for (size_t i = 0; i < op->input_size; ++i)
@@ -468,6 +580,7 @@ void eltwise_prepare(op_t *op)
     alloc_and_tag(op);
     same_geometry(op);
     e->bytes = device_bytes_of(&op->output_tensors[0]);
+    e->defer = 0;
     op->run_func = eltwise_run;
 }
 
@@ -495,7 +608,9 @@ bool relu_launch_into(op_t *op, void *y)
         return false;
     op_t *cop = static_cast<op_t *>(m->pending_ctx);
     conv_op_t *c = reinterpret_cast<conv_op_t *>(cop);
-    if (!relu_is_clamp_of(e, c) || hipq_conv2d_run_relu(c->plan, in_ptr(cop, 0), y, op_stream(op)) != 0)
+    if (!relu_is_clamp_of(e, c))
+        return false;
+    if (!conv_run_chained(cop, y, 1) && hipq_conv2d_run_relu(c->plan, in_ptr(cop, 0), y, op_stream(op)) != 0)
         return false;
     ++g_fused_relus;
     return true;
@@ -546,9 +661,9 @@ void relu_run(op_t *op)
                            e->qo.bits[0], op_stream(op)));
 }
 
-void relu_destroy(op_t *op)
+void deferred_launch_destroy(op_t *op)
 {
-    // a launch left to a pooling (relu_run) must not outlive the operator
+    // a launch left to a reader (relu_run, add_or_sum_run_fused) must not outlive the operator
     if (op->output_size > 0 && op->output_tensors != nullptr && op->output_tensors[0].mem != nullptr
         && is_hip_mem(op->output_tensors[0].mem) && as_hip(op->output_tensors[0].mem)->pending_ctx == op)
         as_hip(op->output_tensors[0].mem)->pending = nullptr;
@@ -891,6 +1006,7 @@ static workspace_t *ws_new(const setting_entry_t *settings)
 ART_PUBLIC long hip_module_fused_adds(void) { return g_fused_adds; }
 ART_PUBLIC long hip_module_fused_relus(void) { return g_fused_relus; }
 ART_PUBLIC long hip_module_fused_pools(void) { return g_fused_pools; }
+ART_PUBLIC long hip_module_chained_convs(void) { return g_chained_convs; }
 
 ART_PUBLIC void *hip_workspace_stream(workspace_t *w) { return reinterpret_cast<hip_workspace_t *>(w)->stream; }
 
@@ -917,9 +1033,9 @@ ART_PUBLIC op_tp_entry_t hip_op_table[] = {
     HIP_ENTRY(op_hip_dequantize_tp, qdq_op_t, dequantize_config, destroy_nothing, dequantize_prepare),
     HIP_ENTRY(op_conv_2d_tp, conv_op_t, conv_config, conv_destroy, conv_prepare),
     HIP_ENTRY(op_ip_tp, conv_op_t, ip_config, conv_destroy, ip_prepare),
-    HIP_ENTRY(op_relu_tp, ew_op_t, relu_config, relu_destroy, relu_prepare),
-    HIP_ENTRY(op_add_tp, ew_op_t, add_config, destroy_nothing, add_prepare),
-    HIP_ENTRY(op_eltwise_tp, ew_op_t, eltwise_config, destroy_nothing, eltwise_prepare),
+    HIP_ENTRY(op_relu_tp, ew_op_t, relu_config, deferred_launch_destroy, relu_prepare),
+    HIP_ENTRY(op_add_tp, ew_op_t, add_config, deferred_launch_destroy, add_prepare),
+    HIP_ENTRY(op_eltwise_tp, ew_op_t, eltwise_config, deferred_launch_destroy, eltwise_prepare),
     HIP_ENTRY(op_pool_tp, pool_op_t, pool_config, destroy_nothing, pool_prepare),
     HIP_ENTRY(op_reshape_tp, ew_op_t, reshape_config, destroy_nothing, reshape_prepare),
     HIP_ENTRY(op_concat_tp, axis_op_t, concat_config, destroy_nothing, concat_prepare),

@@ -53,7 +53,7 @@ _SIGS = {
                                       C.c_int, C.c_void_p, C.c_void_p]),
     "hipq_conv2d_add_conv_fusable": (C.c_int, [C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_float, C.c_int, C.c_int, C.c_void_p]),
     "hipq_conv2d_run_add_conv": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_float, C.c_int,
-                                           C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
+                                           C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
     "hipq_conv2d_maxpool_fusable": (C.c_int, [C.c_void_p] + [C.c_int] * 5 + [C.c_float, C.c_int, C.c_float, C.c_int, C.c_int]),
     "hipq_conv2d_run_maxpool": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
     "hipq_ip_reorder_weights": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 6),
@@ -232,10 +232,10 @@ class Conv2d:
         return bool(lib().hipq_conv2d_add_conv_fusable(self.handle, int(bool(residual_first)), res_alpha, res_zp, oalpha, ozp,
                                                        obits, nxt.handle))
 
-    def run_add_conv(self, x, residual, residual_first, res_alpha, res_zp, oalpha, ozp, y, nxt, y_next, obits=8):
+    def run_add_conv(self, x, residual, residual_first, res_alpha, res_zp, oalpha, ozp, y, nxt, y_next, obits=8, next_relu=False):
         """y = add(conv(x), residual) and y_next = nxt(y) in one launch (include/hipq.h: hipq_conv2d_run_add_conv)."""
         check(lib().hipq_conv2d_run_add_conv(self.handle, _ptr(x), _ptr(residual), int(bool(residual_first)), res_alpha, res_zp,
-                                             oalpha, ozp, obits, _ptr(y), nxt.handle, _ptr(y_next), _stream()))
+                                             oalpha, ozp, obits, _ptr(y), nxt.handle, int(bool(next_relu)), _ptr(y_next), _stream()))
         return y, y_next
 
     def maxpool_fusable(self, OH, OW, kernel, stride, pad, ialpha, izp, oalpha, ozp, obits=8):

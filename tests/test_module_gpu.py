@@ -234,6 +234,55 @@ def test_plain_eltwise_sum_fuses_like_add(own_rt):
     ws.delete()
 
 
+def test_add_and_the_next_1x1_convolution_run_as_one_kernel(own_rt):
+    """conv_2d (64 -> 256, 1x1) -> add -> conv_2d (256 -> 64, 1x1) [-> relu]: the first convolution defers to the add, the
+    add defers to the convolution that reads the sum, and that convolution (or the relu behind it) launches all of it as
+    one kernel; the sum is written as well, for its other readers.  A host that reads the sum before the second
+    convolution runs gets convolution + add as one kernel and the second convolution on its own.  Same bytes as the
+    operators run one by one, pass after pass."""
+    import ctypes as C
+    from oracle import orc
+    chained = own_rt.libs[1].hip_module_chained_convs
+    chained.restype = C.c_long
+    ws = own_rt.workspace("hip")
+    rng = np.random.default_rng(24)
+    x = rng.integers(0, 256, (2, 64, 24, 24), dtype=np.uint8)
+    w = rng.integers(0, 256, (256, 64, 1, 1), dtype=np.uint8)
+    b = rng.integers(-5000, 5000, 256).astype(np.int32)
+    r = rng.integers(0, 256, (2, 256, 24, 24), dtype=np.uint8)
+    w2 = rng.integers(0, 256, (64, 256, 1, 1), dtype=np.uint8)
+    b2 = rng.integers(-5000, 5000, 64).astype(np.int32)
+    q = dict(ialpha=0.031, izp=77, walpha=0.0042, wzp=128, oalpha=0.09, ozp=13)
+    q2 = dict(ialpha=0.12, izp=31, walpha=0.003, wzp=128, oalpha=0.4, ozp=40)
+    want_c = orc.conv2d_u8(x, w, b, 0, 1, 1, 0.031, 77, 0.0042, 128, 0.09, 13)
+    want_a = orc.add_u8(r, want_c, 0.05, 200, 0.09, 13, 0.12, 31)
+    want_2 = orc.conv2d_u8(want_a, w2, b2, 0, 1, 1, 0.12, 31, 0.003, 128, 0.4, 40)
+    want_r = orc.relu_u8(want_2, 0.4, 40, 0.4, 40)
+    for with_relu, peek, expect in ((True, False, 1), (False, False, 1), (True, True, 0)):
+        conv = ws.conv2d(ws.tensor(x), ws.tensor(w), ws.tensor(b), 0, 1, 1, q).prepare()
+        add = ws.add(ws.tensor(r), conv.output(0), dict(ialpha=[0.05, 0.09], izp=[200, 13], oalpha=0.12, ozp=31)).prepare()
+        conv2 = ws.conv2d(add.output(0), ws.tensor(w2), ws.tensor(b2), 0, 1, 1, q2).prepare()
+        relu = ws.relu(conv2.output(0), dict(ialpha=0.4, izp=40, oalpha=0.4, ozp=40)).prepare() if with_relu else None
+        for rep in range(2):
+            n0 = chained()
+            conv.run()
+            add.run()
+            if peek:
+                assert same_bits(add.output(0).numpy(), want_a)
+            conv2.run()
+            if relu:
+                relu.run()
+            last = relu if relu else conv2
+            assert same_bits(last.output(0).numpy(), want_r if relu else want_2), (with_relu, peek, rep)
+            assert chained() == n0 + expect, (with_relu, peek, rep)
+            assert same_bits(add.output(0).numpy(), want_a), (with_relu, peek, rep)
+        assert same_bits(conv2.output(0).numpy(), want_2)  # elided behind the relu: computed on demand
+        assert same_bits(conv.output(0).numpy(), want_c)
+        for o in ([relu] if relu else []) + [conv2, add, conv]:
+            o.delete()
+    ws.delete()
+
+
 def test_convolution_and_relu_run_as_one_kernel(own_rt):
     """A convolution whose output only a relu with the same scale and zero point on both sides reads leaves its launch
     to that relu (the clamp moves into the convolution's epilogue); other relus run as operators of their own."""
