@@ -54,6 +54,7 @@
 #include "conv_shared.h"
 #include "conv_stem.h"
 #include "conv_expand.h"
+#include "conv_rows.h"
 
 namespace hipq {
 
@@ -1567,12 +1568,20 @@ static bool expand_applies(const hipq_conv2d_plan *p, const ConvArgs &a)
     return p->variant == kMfma && p->special && !p->tile_selected && !p->has_wzp && conv_expand_applies(a, p->special == 2);
 }
 
+// conv3x3_c64_rows_kernel (conv_rows.hip): 3x3 / stride 1 / pad 1 with 64 channels in and out, rows resident in LDS
+static bool rows_applies(const hipq_conv2d_plan *p, const ConvArgs &a)
+{
+    return p->variant == kMfma && p->special == 1 && !p->tile_selected && !p->has_wzp && conv_rows_applies(a);
+}
+
 static void set_mfma_name(hipq_conv2d_plan *p, bool smallc)
 {
     char nm[96];
     StreamShape ss;
     if (!smallc && stream_applies(p, &ss))
         snprintf(nm, sizeof nm, "conv_mfma_i8_stream_%dx%d%s", 16 * ss.mb, 16 * ss.nb, p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
+    else if (!smallc && rows_applies(p, p->args))
+        snprintf(nm, sizeof nm, "conv_mfma_i8_rows3x3%s", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
     else if (!smallc && expand_applies(p, p->args))
         snprintf(nm, sizeof nm, "conv_mfma_i8_expand%s", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
     else if (pointwise_applies(p))
@@ -2234,6 +2243,10 @@ static int run_conv(const hipq_conv2d_plan *p, ConvArgs &a, hipStream_t st)
     switch (p->variant) {
     case kMfma:
     case kMfmaSmallC:
+        if (rows_applies(p, a)) {
+            launch_conv_rows(a, st); // 3x3 with 64 channels: the input rows stay in LDS, the weights in registers
+            break;
+        }
         if (expand_applies(p, a)) {
             launch_conv_expand(a, st); // a channel-widening 1x1 layer: pixel operands in registers, channel tiles in a loop
             break;

@@ -1,0 +1,205 @@
+// 3x3 / stride 1 / pad 1 convolutions with 64 input and at most 64 output channels on images up to 64 pixels wide (the
+// middle layer of ResNet-50's first bottleneck stage, every layer of ResNet-18's first stage, the single-layer case of
+// the benchmark configurations).  gfx950 only.
+//
+// Reproduces op_conv_2d_u8xu8_run (art/modules/quant/src/op/conv_2d_uint8_impl.c:39-165) bit for bit, like the tile
+// kernels of conv.hip; int8 tensors (conv_2d_int8_impl.c:34-174) through the same code with xmask = 0.
+//
+// The tile kernels stream, for every output tile, nine weight slabs and nine shifted copies of the input through LDS,
+// with a barrier per slab; such a layer then takes 18 us for 3 us of matrix work.  With 64 channels the whole weight
+// tensor is 36 KB - 144 registers per lane as MFMA operands - and an image row is a few KB, so:
+//   * a work-group owns `rb` output rows of one image (the host picks rb so that the grid fills the chip in whole
+//     rounds); the rb + 2 input rows go into LDS ONCE with the load unit, 1 KB per instruction, beside a pad pixel left
+//     and right of every row and pad rows above / below the image that hold the byte izp;
+//   * the weights of all nine taps (both k-steps, both halves of the 64 output channels) are loaded into registers once
+//     and stay there;
+//   * a wave computes 32 pixels of an output row x 64 channels at a time: per tap and k-step its pixel operand - lane
+//     (p, h): bytes [32 s + 16 h, +16) of pixel (row + dr, col + ds) - is one 128-bit LDS read, closed-form addressing,
+//     no border tests, no barrier anywhere in the loop;
+//   * the 32 x 64 result bytes are transposed through a 2 KB LDS patch private to the wave (no barrier either) and leave
+//     as two 128-bit stores per lane, 2 KB contiguous in memory.
+// Requirements (checked by the host): 3x3, stride 1, pad 1, one group, input and output channel stride 64, image rows
+// of at most 64 pixels, weight zero point 128 (or int8), one-multiply requantisation, per-tensor weight scale.
+#include "conv_rows.h"
+
+namespace hipq {
+
+namespace {
+constexpr int kMaxRB = 8;                   // output rows per work-group, at most
+constexpr int kRowPitch = 64 + 5 * 1024;    // bytes of an input row in LDS: the left pad pixel, then up to 5 loads of 1 KB
+                                            // (64 pixels and the pad pixel to their right)
+constexpr int kPatch = 32 * 64;             // a wave's output staging: 32 pixels x 64 channels
+}
+
+template <bool PLAIN_SAT>
+__global__ __launch_bounds__(256, 2) void conv3x3_c64_rows_kernel(const ConvArgs a, const int nrb, const int rb)
+{
+    constexpr int P_OFF = (kMaxRB + 2) * kRowPitch;
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[P_OFF + 4 * kPatch];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int half = lane >> 5, p = lane & 31, swz = (lane >> 2) & 3;
+    const int n = (int)blockIdx.x / nrb, r0 = ((int)blockIdx.x % nrb) * rb;
+    const int nrows = min(rb, a.H - r0);      // output rows of this work-group
+    const int nin = nrows + 2;                // input rows r0 - 1 .. r0 + nrows
+
+    // ---- this lane's weight operands for the whole kernel: [tap][k-step][channel half]; issued before the rows, so that
+    // a wait that leaves the LAST loads outstanding (below) covers them ----
+    v4i wreg[9][2][2];
+#pragma unroll
+    for (int t = 0; t < 9; t++)
+#pragma unroll
+        for (int s = 0; s < 2; s++)
+#pragma unroll
+            for (int tn = 0; tn < 2; tn++)
+                wreg[t][s][tn] = ldg128(a.wpack + (size_t)t * a.kout_pad * 64 + (tn * 32 + p) * 64 + (((2 * s + half) ^ swz) << 4));
+    v16i bias[2];
+#pragma unroll
+    for (int tn = 0; tn < 2; tn++)
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const v4i b = *reinterpret_cast<const v4i *>(a.bias2 + tn * 32 + g * 8 + half * 4);
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                bias[tn][g * 4 + e] = b[e];
+        }
+
+    // ---- the input rows, once: row j of the patch = image row r0 - 1 + j; beyond the image: the byte izp.  Item
+    // i = (row j, 1 KB block) goes to wave i % 4, rows ascending: of the first four rows every wave loads nblk items ----
+    const int nblk = (a.W * 64 + 64 + 1023) >> 10; // 1 KB loads per row: its pixels and the pad pixel to their right
+    const int items = nin * nblk;
+    for (int i = wave; i < items; i += 4) {
+        const int j = i / nblk, blk = i - j * nblk, ir = r0 - 1 + j;
+        const int off = blk * 1024 + lane * 16;
+        const bool ok = (unsigned)ir < (unsigned)a.H && off < a.W * 64;
+        // the lanes of a row's loads that lie beyond its pixels read the pad source: that is the pad pixel to the right
+        const uint8_t *src = ok ? a.x + ((size_t)(n * a.H + ir) * a.W) * 64 + off : a.padbuf;
+        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(lds + j * kRowPitch + 64 + blk * 1024), 16, 0, 0);
+    }
+    if (tid < nin * 4) { // the pad pixel left of every row
+        const uint32_t pw = a.padword;
+        *reinterpret_cast<u32x4 *>(lds + (tid >> 2) * kRowPitch + (tid & 3) * 16) = u32x4{pw, pw, pw, pw};
+    }
+    // The first two output rows need the first four input rows only: wait for those (this wave's loads beyond them may
+    // stay in flight), compute, and take the rest of the rows when they have had that long to arrive.
+    const int mine = (items - wave + 3) >> 2, later = mine > nblk ? mine - nblk : 0;
+    switch (later) {
+    case 0: wait_vmcnt<0>(); break;
+    case 1: wait_vmcnt<1>(); break;
+    case 2: wait_vmcnt<2>(); break;
+    case 3: wait_vmcnt<3>(); break;
+    case 4: wait_vmcnt<4>(); break;
+    case 5: wait_vmcnt<5>(); break;
+    case 6: wait_vmcnt<6>(); break;
+    case 7: wait_vmcnt<7>(); break;
+    case 8: wait_vmcnt<8>(); break;
+    case 9: wait_vmcnt<9>(); break;
+    case 10: wait_vmcnt<10>(); break;
+    default: wait_vmcnt<0>(); break; // more than that cannot be outstanding with 10 rows of 5 blocks over 4 waves... be safe
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+
+    const int nseg = (a.W + 31) >> 5;         // 32-pixel segments of a row
+    uint8_t *patch = lds + P_OFF + wave * kPatch;
+    // one unit: 32 pixels of an output row x 64 channels
+    auto compute = [&](int u) {
+        const int row = u / nseg, seg = u - row * nseg;
+        const int col = min(seg * 32 + p, a.W - 1); // lanes beyond the row compute a copy that is never stored
+        // pixel (row + dr, col + ds) of the patch, ds = -1 .. 1: patch row row + dr, pixel slot col + ds + 1
+        const uint8_t *base = lds + row * kRowPitch + col * 64 + half * 16;
+        v16i acc[2] = {bias[0], bias[1]};
+#pragma unroll
+        for (int dr = 0; dr < 3; dr++)
+#pragma unroll
+            for (int ds = 0; ds < 3; ds++)
+#pragma unroll
+                for (int s = 0; s < 2; s++) {
+                    const v4i bf = *reinterpret_cast<const v4i *>(base + dr * kRowPitch + ds * 64 + s * 32) ^ (int)a.xmask;
+                    acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[dr * 3 + ds][s][0], bf, acc[0], 0, 0, 0);
+                    acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[dr * 3 + ds][s][1], bf, acc[1], 0, 0, 0);
+                }
+        // requantise, transpose through the wave's own patch (16-byte piece c of pixel q at piece c ^ (q & 3)), store
+#pragma unroll
+        for (int tn = 0; tn < 2; tn++)
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                uint32_t packed;
+                if (PLAIN_SAT) {
+                    int32_t r[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        r[e] = (__mulhi(acc[tn][g * 4 + e], (int)a.q.mult) + a.qadd) >> a.qt;
+                    uint32_t p01, p23, b01, b23;
+                    asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p01) : "v"(r[0]), "v"(r[1]));
+                    asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(r[2]), "v"(r[3]));
+                    asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
+                    asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
+                    packed = (b01 & 0xffffu) | (b23 << 16);
+                } else {
+                    int32_t rq[4];
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        rq[e] = conv_requant<true>(a, acc[tn][g * 4 + e]);
+                    packed = pack_low_bytes(rq[0], rq[1], rq[2], rq[3]);
+                }
+                const int ch = tn * 32 + g * 8 + half * 4;
+                *reinterpret_cast<uint32_t *>(patch + p * 64 + (((ch >> 4) ^ (p & 3)) << 4) + (ch & 15)) = packed;
+            }
+        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): the wave's own writes
+        uint8_t *yrow = a.y + ((size_t)(n * a.H + r0 + row) * a.W + seg * 32) * 64;
+#pragma unroll
+        for (int k = 0; k < 2; k++) {
+            const int q = (lane >> 2) + 16 * k, c = lane & 3; // pixel of the segment, 16-byte piece
+            const v4i v = *reinterpret_cast<const v4i *>(patch + q * 64 + ((c ^ (q & 3)) << 4));
+            if (seg * 32 + q < a.W)
+                *reinterpret_cast<v4i *>(yrow + q * 64 + c * 16) = v;
+        }
+        __builtin_amdgcn_s_waitcnt(0xC07F); // the patch is read before the next unit overwrites it
+    };
+    const int units = nrows * nseg, early = min(2 * nseg, units); // (row, segment) pairs; those of the first two rows
+    int u = wave;
+    for (; u < early; u += 4)
+        compute(u);
+    wait_vmcnt<0>(); // this wave's remaining loads have landed (its stores so far as well), then everybody's
+    __builtin_amdgcn_s_barrier();
+    for (; u < units; u += 4)
+        compute(u);
+}
+
+bool conv_rows_applies(const ConvArgs &a)
+{
+    return a.R == 3 && a.S == 3 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 1 && a.pad_w == 1 && a.group == 1
+        && a.in_cs == 64 && a.out_cs == 64 && a.K <= 64 && a.nslab == 9 && a.W <= 64 && a.W >= 1 && a.OH == a.H && a.OW == a.W
+        && a.bwz == 0 && a.fastq && !plain_epilogue(a) && a.res == nullptr;
+}
+
+// Output rows per work-group: two work-groups fit a CU (their registers), so the grid runs in rounds of 512; the cost of
+// a choice is its number of rounds times the rows a work-group loads and computes.
+static int rows_per_wg(int N, int H)
+{
+    int best = 1;
+    long best_cost = 0;
+    for (int rb = 1; rb <= kMaxRB; rb++) {
+        const long wgs = (long)N * ((H + rb - 1) / rb);
+        const long cost = ((wgs + 511) / 512) * (rb + 2 + 2); // + 2 input rows, + 2: the fixed part (weights, first loads)
+        if (rb == 1 || cost < best_cost) {
+            best = rb;
+            best_cost = cost;
+        }
+    }
+    return best;
+}
+
+void launch_conv_rows(const ConvArgs &a, hipStream_t st)
+{
+    static const int rb_env = getenv("HIPQ_ROWS_RB") ? atoi(getenv("HIPQ_ROWS_RB")) : 0;
+    const int rb = rb_env ? rb_env : rows_per_wg(a.N, a.H), nrb = (a.H + rb - 1) / rb;
+    const dim3 grid(a.N * nrb), block(256);
+    if (a.lo == 0 && a.q.hi == 255)
+        hipLaunchKernelGGL(conv3x3_c64_rows_kernel<true>, grid, block, 0, st, a, nrb, rb);
+    else
+        hipLaunchKernelGGL(conv3x3_c64_rows_kernel<false>, grid, block, 0, st, a, nrb, rb);
+}
+
+} // namespace hipq

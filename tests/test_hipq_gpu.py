@@ -639,7 +639,7 @@ def test_relu_decided_at_run_time():
     rng = np.random.default_rng(47)
     kerns = set()
     #         N, C,  H,  W,  K,  R, pad, stride, group
-    shapes = [(2, 64, 12, 12, 64, 3, 1, 1, 1), (1, 32, 9, 9, 96, 1, 0, 1, 1), (2, 256, 7, 7, 128, 1, 0, 1, 1), (1, 3, 20, 20, 32, 3, 1, 2, 1),
+    shapes = [(2, 64, 12, 12, 64, 3, 1, 1, 1), (1, 64, 9, 9, 48, 3, 1, 1, 1), (1, 32, 9, 9, 96, 1, 0, 1, 1), (2, 256, 7, 7, 128, 1, 0, 1, 1), (1, 3, 20, 20, 32, 3, 1, 2, 1),
               (2, 48, 10, 10, 48, 3, 1, 1, 48), (1, 32, 9, 9, 32, 3, 1, 2, 32), (1, 24, 7, 7, 24, 5, 2, 1, 24), (1, 16, 8, 8, 32, 3, 1, 1, 4)]
     for N, C, H, W, K, R, pad, st, g in shapes:
         x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
@@ -662,6 +662,43 @@ def test_relu_decided_at_run_time():
         p8.run_relu(hipq.to_device_nhwc(np.zeros((1, 16, 4, 4), np.int8)))
 
 
+def test_conv3x3_rows_kernel():
+    """conv3x3_c64_rows_kernel (3x3 / stride 1 / pad 1, 64 channels in, 49 to 64 out, images up to 64 pixels wide; input
+    rows resident in LDS, weights in registers) against the oracle and against the tile kernels: widths that are and
+    are not multiples of 16 and 32 (the pad pixel right of a row comes with the row's loads), one-pixel and one-row
+    images, row blocks that do not divide the height, several images, ReLU, fewer output bits, int8 tensors."""
+    rng = np.random.default_rng(47)
+    shapes = [(2, 56, 56, 64), (1, 9, 64, 64), (3, 17, 63, 52), (1, 1, 1, 64), (2, 5, 32, 49), (1, 30, 16, 64), (4, 3, 33, 60),
+              (1, 64, 48, 64), (64, 8, 8, 64)]
+    for i, (N, H, W, K) in enumerate(shapes):
+        print("rows case", N, H, W, K, flush=True)
+        x = rng.integers(0, 256, (N, 64, H, W), dtype=np.uint8)
+        w = rng.integers(0, 256, (K, 64, 3, 3), dtype=np.uint8)
+        b = rng.integers(-30000, 30000, K).astype(np.int32)
+        ia, wa = rand_q(rng), rand_q(rng)
+        relu, obits = bool(i & 1), (8, 8, 7)[i % 3]
+        q = (ia, int(rng.integers(0, 256)), wa, 128, float(np.float32(ia * wa * 24.0 * 40.0)), int(rng.integers(0, 1 << obits)))
+        want = orc.conv2d_u8(x, w, b, 1, 1, 1, *q, obits=obits)
+        if relu:
+            want = orc.relu_u8(want, q[4], q[5], q[4], q[5], obits)
+        plan = hipq.Conv2d(x.shape, w, b, 1, 1, 1, *q, relu=relu, obits=obits)
+        assert plan.kernel == "conv_mfma_i8_rows3x3", plan.kernel
+        xd = hipq.to_device_nhwc(x)
+        got = hipq.from_device_nhwc(plan(xd), K)
+        assert np.array_equal(got, want), (N, H, W, K, relu, obits, int((got != want).sum()))
+        plan.special(0)
+        assert "rows3x3" not in plan.kernel
+        assert np.array_equal(hipq.from_device_nhwc(plan(xd), K), want)
+    x = rng.integers(-128, 128, (2, 64, 20, 24), dtype=np.int8)
+    w = rng.integers(-127, 128, (64, 64, 3, 3), dtype=np.int8)
+    b = rng.integers(-30000, 30000, 64).astype(np.int32)
+    for obits in (8, 7):
+        plan = hipq.Conv2d(x.shape, w, b, 1, 1, 1, 0.02, 0, 0.004, 0, 2.0, 0, obits=obits, dtype=hipq.DTYPE_I8)
+        assert plan.kernel == "conv_mfma_i8_rows3x3_signed", plan.kernel
+        got = hipq.from_device_nhwc(plan(hipq.to_device_nhwc(x)), 64).view(np.int8)
+        assert np.array_equal(got, orc.conv2d_i8(x, w, b, 1, 1, 1, 0.02, 0.004, 2.0, obits=obits)), obits
+
+
 def test_conv3x3_halo_kernel_matches_the_streaming_kernel_and_the_oracle():
     """3x3 / stride 1 / pad 1 layers load a pixel tile with its halo once and read the nine taps from LDS: every tile
     shape, one and several channel slabs, images narrower and wider than a tile, several images per tile (taps must
@@ -677,7 +714,8 @@ def test_conv3x3_halo_kernel_matches_the_streaming_kernel_and_the_oracle():
         q = (rand_q(rng), int(rng.integers(0, 256)), rand_q(rng), 128, rand_q(rng, 1e-2, 1.0), int(rng.integers(0, 256)))
         want, want_acc = orc.conv2d_u8(x, w, b, 1, 1, 1, *q, return_acc=True)
         plan = hipq.Conv2d(x.shape, w, b, 1, 1, 1, *q)
-        assert plan.kernel.endswith("_halo") == (C == 64), plan.kernel  # the built-in rule: single channel slab only
+        # the built-in rule: single channel slab only (64 output channels with a one-multiply requantisation: the rows kernel)
+        assert (plan.kernel.endswith("_halo") or "rows3x3" in plan.kernel) == (C == 64), plan.kernel
         plan.special(2)
         xd = hipq.to_device_nhwc(x)
         for tile in (0, 2, 3, 4):
