@@ -11,6 +11,8 @@ Prints ONE JSON line:
                         their measured durations, against the chip's dense int8 MFMA peak
   kernel_families       every family's time, TOP/s and GB/s (launch-by-launch timing, see per_kernel_times)
   sustained             the same replay loop kept running for at least two seconds
+  library_int8_gemm     a yardstick: the vendor library's plain int8 GEMM (int32 output) on every layer's GEMM shape, summed,
+                        beside the sum of this build's convolution-family launches
   module_path           the same network as an engine file run by nart_promark on the `hip` workspace (the drop-in path),
                         a child process
   other_workloads       BASELINE configs[0..3] at their stated sizes: time, rate, fraction of the roof that bounds them,
@@ -211,6 +213,61 @@ def measure_workload(build, batch, inner, kernel_reps, check_rows):
     return res
 
 
+def library_gemm(case, ex, kt):
+    """The vendor library's plain int8 GEMM (`torch._int_mm`: int8 x int8 -> int32, hipBLASLt) on the GEMM shape of
+    every dense convolution and fully-connected layer of the case - M = N*OH*OW pixels, K = C*R*S, N = output channels,
+    operands already laid out (no patch gathering, no requantisation, no residual add, an int32 result) - summed over
+    the layers, beside the sum of this build's launches that do the whole of that work.  A yardstick for what the
+    matrix pipes deliver on these shapes, not a code path of the library."""
+    import numpy as np
+    import torch
+    shapes = []
+    for n in case.nodes:
+        y, x = case.tensors[n.output], case.tensors[n.inputs[0]]
+        if n.kind == "conv" and n.attrs["group"] == 1:
+            shapes.append((int(np.prod(y.shape)) // y.shape[1], x.shape[1] * n.attrs["k"] ** 2, y.shape[1]))
+        elif n.kind == "ip":
+            shapes.append((y.shape[0], int(np.prod(x.shape[1:])), y.shape[1]))
+    times, skipped = {}, 0
+    for s in set(shapes):
+        M, K, N = s
+        K8 = (K + 7) // 8 * 8          # the library wants multiples of 8: the stem's 147 is padded with zeros
+        if M <= 16 or N % 8:
+            continue
+        a = torch.randint(-128, 128, (M, K8), dtype=torch.int8, device="cuda")
+        b = torch.randint(-128, 128, (N, K8), dtype=torch.int8, device="cuda").t()   # k contiguous, as the packed weights
+        try:
+            for _ in range(2):
+                torch._int_mm(a, b)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                for _ in range(10):
+                    torch._int_mm(a, b)
+            g.replay()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            times[s] = e0.elapsed_time(e1) / 10
+        except RuntimeError:
+            pass
+        del a, b
+    done = [s for s in shapes if s in times]
+    skipped = len(shapes) - len(done)
+    lib_ms = sum(times[s] for s in done)
+    ops = sum(2.0 * s[0] * s[1] * s[2] for s in done)
+    ours_ms = sum(t for s, t in zip(ex.steps, kt) if s["kernel"].startswith("conv_mfma") and s["ops"])
+    ours_ops = sum(s["ops"] for s in ex.steps if s["kernel"].startswith("conv_mfma") and s["ops"])
+    return {"layers": len(done), "layers_skipped": skipped, "library_ms": round(lib_ms, 4),
+            "library_TOPs": round(ops / (lib_ms * 1e-3) / 1e12, 1) if lib_ms else None,
+            "this_build_ms": round(ours_ms, 4),
+            "this_build_TOPs": round(ours_ops / (ours_ms * 1e-3) / 1e12, 1) if ours_ms else None,
+            "note": "library: torch._int_mm per layer shape, int32 output, no im2col / requantisation / add / pooling; "
+                    "this build: its convolution-family launches, which include all of those"}
+
+
 def module_path(build, batch, steps):
     """The drop-in path: the network as an engine file, run by nart_promark (the counterpart of the reference's
     tools/promark.cpp) on the `hip` workspace through hip_module_tp, every operator launched by the module's run
@@ -406,6 +463,9 @@ def main():
         if args.batch >= 2:
             extra("two_branch_graph", two_branch)
         extra("two_batches_in_flight", in_flight)
+
+    if not args.no_extras and not args.no_graph:
+        extra("library_int8_gemm", lambda: library_gemm(case, ex, kt))
 
     if not args.no_extras and args.workload == "resnet50":
         extra("module_path", lambda: module_path(build, args.batch, 50))
