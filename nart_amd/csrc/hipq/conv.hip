@@ -54,6 +54,7 @@
 #include "conv_shared.h"
 #include "conv_stem.h"
 #include "conv_expand.h"
+#include "conv_dw.h"
 #include "conv_rows.h"
 
 namespace hipq {
@@ -2260,6 +2261,10 @@ static int run_conv(const hipq_conv2d_plan *p, ConvArgs &a, hipStream_t st)
         }
         break;
     case kDepthwise3x3: {
+        if (!p->has_wzp && conv_dw_slide_applies(a)) {
+            launch_conv_dw_slide(a, st); // a thread walks down the image: every input row loaded and transposed once
+            break;
+        }
         const size_t total = (size_t)a.N * ((a.OH + 1) / 2) * ((a.OW + 3) / 4) * (a.in_cs / 4);
         const dim3 grid((unsigned)((std::min<size_t>((total + 255) / 256, 256 * 64) + 7) / 8 * 8)), block(256); // a multiple of 8
         if (p->d.stride_h == 1) {

@@ -277,6 +277,41 @@ def test_conv_grouped_and_depthwise():
     assert "conv_depthwise_u8" in kerns and "conv_direct_u8" in kerns
 
 
+def test_depthwise3x3_walk_shapes():
+    """The depthwise 3x3 kernel whose threads walk down the image (weight zero point 128): widths that are not multiples
+    of the 4-column strip, one to three rows, no padding, both strides on even and odd sizes, channel counts that fill a
+    wave unevenly; with and without the accumulator dump, a ReLU clamp (one-multiply requantisation with clamps), the
+    plain [0, 255] range (saturating packs) and a scale outside the one-multiply range (64-bit form).  A weight zero
+    point other than 128 takes the older kernel and is checked beside it."""
+    rng = np.random.default_rng(77)
+    shapes = [  # N, C, H, W, pad, stride
+        (2, 32, 14, 14, 1, 1), (1, 96, 9, 9, 1, 2), (3, 8, 5, 7, 1, 1), (1, 4, 1, 1, 1, 1), (1, 12, 2, 13, 1, 1),
+        (2, 20, 3, 5, 1, 2), (1, 16, 8, 8, 1, 2), (1, 144, 6, 10, 0, 1), (1, 24, 7, 9, 0, 2), (1, 260, 4, 6, 1, 1),
+        (1, 8, 33, 4, 1, 1), (2, 8, 12, 21, 1, 2),
+    ]
+    kerns = set()
+    for i, (N, C, H, W, pad, st) in enumerate(shapes):
+        x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+        w = rng.integers(0, 256, (C, 1, 3, 3), dtype=np.uint8)
+        b = rng.integers(-3000, 3000, C).astype(np.int32)
+        izp, ozp = int(rng.integers(0, 256)), int(rng.integers(0, 200))
+        ia, wa = rand_q(rng), rand_q(rng)
+        oa = float(np.float32(ia * wa * 3000.0 / 200.0))     # sums of +-3000 land on the byte range: one-multiply form
+        for wzp in (128, 131):
+            q = (ia, izp, wa, wzp, oa, ozp)
+            kerns.add(check_conv(x, w, b, pad, st, C, q, tag="dw%d" % i))
+            want = orc.conv2d_u8(x, w, b, pad, st, C, *q)
+            plan = hipq.Conv2d(x.shape, w, b, pad, st, C, *q)
+            xd = hipq.to_device_nhwc(x)
+            assert np.array_equal(hipq.from_device_nhwc(plan(xd), C), want), (i, wzp, plan.kernel)          # no dump
+            assert np.array_equal(hipq.from_device_nhwc(plan.run_relu(xd), C), np.maximum(want, ozp)), (i, wzp, plan.kernel)
+            assert len(np.unique(want)) > 8 or want.size < 64, (i, "degenerate case")
+        q = (ia, izp, wa, 128, float(np.float32(oa * 2.0 ** 22)), ozp)   # shift beyond the one-multiply range
+        kerns.add(check_conv(x, w, b, pad, st, C, q, tag="dw%d_wide_shift" % i))
+    assert kerns == {"conv_depthwise3x3_u8_s1", "conv_depthwise3x3_u8_s2", "conv_depthwise3x3_u8_s1_wzp",
+                     "conv_depthwise3x3_u8_s2_wzp"}, kerns
+
+
 def test_ip_as_1x1():
     rng = np.random.default_rng(14)
     for M, Kd, No in ((128, 512, 256), (5, 300, 37), (1, 2048, 1000)):
