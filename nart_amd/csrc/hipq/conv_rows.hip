@@ -11,11 +11,13 @@
 //   * a work-group owns `rb` output rows of one image (the host picks rb so that the grid fills the chip in whole
 //     rounds); the rb + 2 input rows go into LDS ONCE with the load unit, 1 KB per instruction, beside a pad pixel left
 //     and right of every row and pad rows above / below the image that hold the byte izp;
-//   * the weights of all nine taps (both k-steps, both halves of the 64 output channels) are loaded into registers once
-//     and stay there;
+//   * the weights of all nine taps (both k-steps, both halves of the 64 output channels) go into LDS once per work-group
+//     with the load unit - into the space of the input rows that are not needed yet - and from there into every wave's
+//     registers, where they stay (eight waves of a CU fetching 36 KB each straight from memory kept the CU's load path
+//     busy for 2 us before the first multiply);
 //   * a wave computes 32 pixels of an output row x 64 channels at a time: per tap and k-step its pixel operand - lane
 //     (p, h): bytes [32 s + 16 h, +16) of pixel (row + dr, col + ds) - is one 128-bit LDS read, closed-form addressing,
-//     no border tests, no barrier anywhere in the loop;
+//     no border tests, no barrier anywhere in the loop; the reads run three steps ahead of the multiplies;
 //   * the 32 x 64 result bytes are transposed through a 2 KB LDS patch private to the wave (no barrier either) and leave
 //     as two 128-bit stores per lane, 2 KB contiguous in memory.
 // Requirements (checked by the host): 3x3, stride 1, pad 1, one group, input and output channel stride 64, image rows
@@ -25,17 +27,20 @@
 namespace hipq {
 
 namespace {
-constexpr int kMaxRB = 8;                   // output rows per work-group, at most
+constexpr int kMaxRB = 9;                   // output rows per work-group, at most (rows 4 .. 10 of the patch first hold the weights)
 constexpr int kRowPitch = 64 + 5 * 1024;    // bytes of an input row in LDS: the left pad pixel, then up to 5 loads of 1 KB
                                             // (64 pixels and the pad pixel to their right)
 constexpr int kPatch = 32 * 64;             // a wave's output staging: 32 pixels x 64 channels
+constexpr int kWBytes = 9 * 64 * 64;        // the weights: 9 taps x 64 channels x 64 bytes
+static_assert(4 * kRowPitch + kWBytes <= (kMaxRB + 2) * kRowPitch + 4 * kPatch,
+              "the weights pass through the space of the rows behind the first four (and of the patches, unused until then)");
 }
 
 template <bool PLAIN_SAT>
 __global__ __launch_bounds__(256, 2) void conv3x3_c64_rows_kernel(const ConvArgs a, const int nrb, const int rb)
 {
     constexpr int P_OFF = (kMaxRB + 2) * kRowPitch;
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[P_OFF + 4 * kPatch];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[P_OFF + 4 * kPatch + 256]; // rows, the waves' patches, the bias
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int half = lane >> 5, p = lane & 31, swz = (lane >> 2) & 3;
@@ -43,8 +48,39 @@ __global__ __launch_bounds__(256, 2) void conv3x3_c64_rows_kernel(const ConvArgs
     const int nrows = min(rb, a.H - r0);      // output rows of this work-group
     const int nin = nrows + 2;                // input rows r0 - 1 .. r0 + nrows
 
-    // ---- this lane's weight operands for the whole kernel: [tap][k-step][channel half]; issued before the rows, so that
-    // a wait that leaves the LAST loads outstanding (below) covers them ----
+    // ---- the first four input rows (all that the first two output rows need) and, behind them, the weights: row j of the
+    // patch = image row r0 - 1 + j; beyond the image: the byte izp.  Item i = (row j, 1 KB block) goes to wave i % 4 ----
+    const int nblk = (a.W * 64 + 64 + 1023) >> 10; // 1 KB loads per row: its pixels and the pad pixel to their right
+    auto load_rows = [&](int j0, int j1) {
+        for (int i = j0 * nblk + wave; i < j1 * nblk; i += 4) {
+            const int j = i / nblk, blk = i - j * nblk, ir = r0 - 1 + j;
+            const int off = blk * 1024 + lane * 16;
+            const bool ok = (unsigned)ir < (unsigned)a.H && off < a.W * 64;
+            // the lanes of a row's loads that lie beyond its pixels read the pad source: that is the pad pixel to the right
+            const uint8_t *src = ok ? a.x + ((size_t)(n * a.H + ir) * a.W) * 64 + off : a.padbuf;
+            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(lds + j * kRowPitch + 64 + blk * 1024), 16, 0, 0);
+        }
+    };
+    const int nfirst = min(nin, 4);
+    load_rows(0, nfirst);
+    uint8_t *wl = lds + 4 * kRowPitch; // tap t: 64 channel rows of 64 bytes, in the packed (swizzled) order
+#pragma unroll
+    for (int i = 0; i < 9; i++) {
+        const int blk = wave + 4 * i, t = blk >> 2, q = blk & 3; // 1 KB block q of tap t
+        __builtin_amdgcn_global_load_lds((gptr_t)(a.wpack + (size_t)t * a.kout_pad * 64 + q * 1024 + lane * 16),
+                                         (lptr_t)(wl + blk * 1024), 16, 0, 0);
+    }
+    int32_t *lbias = reinterpret_cast<int32_t *>(lds + P_OFF + 4 * kPatch);
+    if (tid < 64)
+        lbias[tid] = a.bias2[tid];
+    if (tid < nin * 4) { // the pad pixel left of every row
+        const uint32_t pw = a.padword;
+        *reinterpret_cast<u32x4 *>(lds + (tid >> 2) * kRowPitch + (tid & 3) * 16) = u32x4{pw, pw, pw, pw};
+    }
+    wait_vmcnt<0>();
+    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    // ---- this lane's weight operands for the whole kernel: [tap][k-step][channel half] ----
     v4i wreg[9][2][2];
 #pragma unroll
     for (int t = 0; t < 9; t++)
@@ -52,53 +88,10 @@ __global__ __launch_bounds__(256, 2) void conv3x3_c64_rows_kernel(const ConvArgs
         for (int s = 0; s < 2; s++)
 #pragma unroll
             for (int tn = 0; tn < 2; tn++)
-                wreg[t][s][tn] = ldg128(a.wpack + (size_t)t * a.kout_pad * 64 + (tn * 32 + p) * 64 + (((2 * s + half) ^ swz) << 4));
-    v16i bias[2];
-#pragma unroll
-    for (int tn = 0; tn < 2; tn++)
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-            const v4i b = *reinterpret_cast<const v4i *>(a.bias2 + tn * 32 + g * 8 + half * 4);
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-                bias[tn][g * 4 + e] = b[e];
-        }
-
-    // ---- the input rows, once: row j of the patch = image row r0 - 1 + j; beyond the image: the byte izp.  Item
-    // i = (row j, 1 KB block) goes to wave i % 4, rows ascending: of the first four rows every wave loads nblk items ----
-    const int nblk = (a.W * 64 + 64 + 1023) >> 10; // 1 KB loads per row: its pixels and the pad pixel to their right
-    const int items = nin * nblk;
-    for (int i = wave; i < items; i += 4) {
-        const int j = i / nblk, blk = i - j * nblk, ir = r0 - 1 + j;
-        const int off = blk * 1024 + lane * 16;
-        const bool ok = (unsigned)ir < (unsigned)a.H && off < a.W * 64;
-        // the lanes of a row's loads that lie beyond its pixels read the pad source: that is the pad pixel to the right
-        const uint8_t *src = ok ? a.x + ((size_t)(n * a.H + ir) * a.W) * 64 + off : a.padbuf;
-        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(lds + j * kRowPitch + 64 + blk * 1024), 16, 0, 0);
-    }
-    if (tid < nin * 4) { // the pad pixel left of every row
-        const uint32_t pw = a.padword;
-        *reinterpret_cast<u32x4 *>(lds + (tid >> 2) * kRowPitch + (tid & 3) * 16) = u32x4{pw, pw, pw, pw};
-    }
-    // The first two output rows need the first four input rows only: wait for those (this wave's loads beyond them may
-    // stay in flight), compute, and take the rest of the rows when they have had that long to arrive.
-    const int mine = (items - wave + 3) >> 2, later = mine > nblk ? mine - nblk : 0;
-    switch (later) {
-    case 0: wait_vmcnt<0>(); break;
-    case 1: wait_vmcnt<1>(); break;
-    case 2: wait_vmcnt<2>(); break;
-    case 3: wait_vmcnt<3>(); break;
-    case 4: wait_vmcnt<4>(); break;
-    case 5: wait_vmcnt<5>(); break;
-    case 6: wait_vmcnt<6>(); break;
-    case 7: wait_vmcnt<7>(); break;
-    case 8: wait_vmcnt<8>(); break;
-    case 9: wait_vmcnt<9>(); break;
-    case 10: wait_vmcnt<10>(); break;
-    default: wait_vmcnt<0>(); break; // more than that cannot be outstanding with 10 rows of 5 blocks over 4 waves... be safe
-    }
-    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
+                wreg[t][s][tn] = *reinterpret_cast<const v4i *>(wl + t * 4096 + (tn * 32 + p) * 64 + (((2 * s + half) ^ swz) << 4));
+    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): every wave holds its weights, then the rows may overwrite them
     __builtin_amdgcn_s_barrier();
+    load_rows(nfirst, nin); // in flight while the first two output rows are computed
 
     const int nseg = (a.W + 31) >> 5;         // 32-pixel segments of a row
     uint8_t *patch = lds + P_OFF + wave * kPatch;
@@ -108,17 +101,32 @@ __global__ __launch_bounds__(256, 2) void conv3x3_c64_rows_kernel(const ConvArgs
         const int col = min(seg * 32 + p, a.W - 1); // lanes beyond the row compute a copy that is never stored
         // pixel (row + dr, col + ds) of the patch, ds = -1 .. 1: patch row row + dr, pixel slot col + ds + 1
         const uint8_t *base = lds + row * kRowPitch + col * 64 + half * 16;
-        v16i acc[2] = {bias[0], bias[1]};
+        v16i acc[2];
 #pragma unroll
-        for (int dr = 0; dr < 3; dr++)
+        for (int tn = 0; tn < 2; tn++)
 #pragma unroll
-            for (int ds = 0; ds < 3; ds++)
+            for (int g = 0; g < 4; g++) {
+                const v4i b = *reinterpret_cast<const v4i *>(lbias + tn * 32 + g * 8 + half * 4);
 #pragma unroll
-                for (int s = 0; s < 2; s++) {
-                    const v4i bf = *reinterpret_cast<const v4i *>(base + dr * kRowPitch + ds * 64 + s * 32) ^ (int)a.xmask;
-                    acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[dr * 3 + ds][s][0], bf, acc[0], 0, 0, 0);
-                    acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[dr * 3 + ds][s][1], bf, acc[1], 0, 0, 0);
-                }
+                for (int e = 0; e < 4; e++)
+                    acc[tn][g * 4 + e] = b[e];
+            }
+        // step k = (tap, k-step): the pixel operand is read three steps before its two multiplies
+        auto rd = [&](int k) {
+            const int t = k >> 1;
+            return *reinterpret_cast<const v4i *>(base + (t / 3) * kRowPitch + (t % 3) * 64 + (k & 1) * 32);
+        };
+        v4i bfr[4];
+        bfr[0] = rd(0), bfr[1] = rd(1), bfr[2] = rd(2);
+#pragma unroll
+        for (int k = 0; k < 18; k++) {
+            if (k + 3 < 18)
+                bfr[(k + 3) & 3] = rd(k + 3);
+            __builtin_amdgcn_sched_barrier(0); // keep the read ahead of the multiplies (the scheduler would sink it to its use)
+            const v4i bf = bfr[k & 3] ^ (int)a.xmask;
+            acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[k >> 1][k & 1][0], bf, acc[0], 0, 0, 0);
+            acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[k >> 1][k & 1][1], bf, acc[1], 0, 0, 0);
+        }
         // requantise, transpose through the wave's own patch (16-byte piece c of pixel q at piece c ^ (q & 3)), store
 #pragma unroll
         for (int tn = 0; tn < 2; tn++)
@@ -161,7 +169,7 @@ __global__ __launch_bounds__(256, 2) void conv3x3_c64_rows_kernel(const ConvArgs
     int u = wave;
     for (; u < early; u += 4)
         compute(u);
-    wait_vmcnt<0>(); // this wave's remaining loads have landed (its stores so far as well), then everybody's
+    wait_vmcnt<0>(); // this wave's loads of the remaining rows have landed (its stores so far as well), then everybody's
     __builtin_amdgcn_s_barrier();
     for (; u < units; u += 4)
         compute(u);
