@@ -20,6 +20,13 @@
 //     no border tests, no barrier anywhere in the loop; the reads run three steps ahead of the multiplies;
 //   * the 32 x 64 result bytes are transposed through a 2 KB LDS patch private to the wave (no barrier either) and leave
 //     as two 128-bit stores per lane, 2 KB contiguous in memory.
+// Where the time goes (cycle stamps in a throw-away build, 64 x 56 x 56, 7 output rows per work-group, two work-groups
+// per CU, 12 us inside the kernel): 1.9 us until the weights and the first four rows are in LDS, 1.1 us for the eight
+// waves of a CU to read their 36 KB of weights out of it (LDS bandwidth), then 1.7 - 2.1 us per unit and wave against
+// 0.5 us of multiplies: a unit's multiplies and its requantisation (a quarter-rate 32-bit multiply per output) follow
+// one another, and the two waves of a SIMD run in step.  Interleaving the previous unit's epilogue with the multiplies
+// needs a second set of accumulators, i.e. more than the 256 registers a wave has at two waves per SIMD; at one wave
+// per SIMD (512 registers) the interleaved form measured 16 us against 13.4: nothing fills a single wave's stalls.
 // Requirements (checked by the host): 3x3, stride 1, pad 1, one group, input and output channel stride 64, image rows
 // of at most 64 pixels, weight zero point 128 (or int8), one-multiply requantisation, per-tensor weight scale.
 #include "conv_rows.h"
@@ -73,10 +80,14 @@ __global__ __launch_bounds__(256, 2) void conv3x3_c64_rows_kernel(const ConvArgs
     int32_t *lbias = reinterpret_cast<int32_t *>(lds + P_OFF + 4 * kPatch);
     if (tid < 64)
         lbias[tid] = a.bias2[tid];
-    if (tid < nin * 4) { // the pad pixel left of every row
-        const uint32_t pw = a.padword;
-        *reinterpret_cast<u32x4 *>(lds + (tid >> 2) * kRowPitch + (tid & 3) * 16) = u32x4{pw, pw, pw, pw};
-    }
+    // the pad pixel left of every row (those of rows 4 and up once the weights have left that space)
+    auto left_pads = [&](int j0, int j1) {
+        if (tid < (j1 - j0) * 4) {
+            const uint32_t pw = a.padword;
+            *reinterpret_cast<u32x4 *>(lds + (j0 + (tid >> 2)) * kRowPitch + (tid & 3) * 16) = u32x4{pw, pw, pw, pw};
+        }
+    };
+    left_pads(0, nfirst);
     wait_vmcnt<0>();
     __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
@@ -92,6 +103,7 @@ __global__ __launch_bounds__(256, 2) void conv3x3_c64_rows_kernel(const ConvArgs
     __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): every wave holds its weights, then the rows may overwrite them
     __builtin_amdgcn_s_barrier();
     load_rows(nfirst, nin); // in flight while the first two output rows are computed
+    left_pads(nfirst, nin);
 
     const int nseg = (a.W + 31) >> 5;         // 32-pixel segments of a row
     uint8_t *patch = lds + P_OFF + wave * kPatch;
@@ -201,8 +213,7 @@ static int rows_per_wg(int N, int H)
 
 void launch_conv_rows(const ConvArgs &a, hipStream_t st)
 {
-    static const int rb_env = getenv("HIPQ_ROWS_RB") ? atoi(getenv("HIPQ_ROWS_RB")) : 0;
-    const int rb = rb_env ? rb_env : rows_per_wg(a.N, a.H), nrb = (a.H + rb - 1) / rb;
+    const int rb = rows_per_wg(a.N, a.H), nrb = (a.H + rb - 1) / rb;
     const dim3 grid(a.N * nrb), block(256);
     if (a.lo == 0 && a.q.hi == 255)
         hipLaunchKernelGGL(conv3x3_c64_rows_kernel<true>, grid, block, 0, st, a, nrb, rb);

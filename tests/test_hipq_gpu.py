@@ -704,7 +704,10 @@ def test_conv3x3_rows_kernel():
     images, row blocks that do not divide the height, several images, ReLU, fewer output bits, int8 tensors."""
     rng = np.random.default_rng(47)
     shapes = [(2, 56, 56, 64), (1, 9, 64, 64), (3, 17, 63, 52), (1, 1, 1, 64), (2, 5, 32, 49), (1, 30, 16, 64), (4, 3, 33, 60),
-              (1, 64, 48, 64), (64, 8, 8, 64)]
+              (1, 64, 48, 64), (64, 8, 8, 64),
+              # batches large enough for the host to give a work-group 3, 4 and 6 output rows (5, 6 and 8 input rows: the
+              # rows behind the first four arrive after the weights have passed through their space)
+              (40, 28, 20, 64), (64, 28, 8, 64), (96, 27, 12, 56)]
     for i, (N, H, W, K) in enumerate(shapes):
         print("rows case", N, H, W, K, flush=True)
         x = rng.integers(0, 256, (N, 64, H, W), dtype=np.uint8)
