@@ -130,10 +130,13 @@ int hipq_conv2d_plan_select(hipq_conv2d_plan *plan, int tile, int stages);
  * at least twice as many and 256 to 1024 output channels over at least 1024 pixels (weight zero point 128) keep a wave's
  * pixel operands in registers while a work-group walks a contiguous range of 128-pixel x 64-channel output tiles, with
  * the residual add of hipq_conv2d_run_add applied in place on a prefetched residual tile.
- * mode 1 (the default) uses them where they measured faster: the halo kernel for 64-channel inputs up to 63 pixels
- * wide, the pointwise kernel wherever it applies, the two-group kernel for layers with at most one tile per CU (256),
+ * Rows kernel (name "..._rows3x3"): 3x3 / stride 1 / pad 1 convolutions with an input and output channel stride of 64
+ * on rows of at most 64 pixels (weight zero point 128, one-multiply requantisation, no fused add) keep the input rows
+ * of a work-group in LDS and all weights in registers.
+ * mode 1 (the default) uses them where they measured faster: the rows kernel wherever it applies, the halo kernel for
+ * the other 64-channel inputs up to 63 pixels wide, the pointwise kernel wherever it applies, the two-group kernel for layers with at most one tile per CU (256),
  * the widening kernel with the add at 64 input channels and without it at 256;
- * mode 2 the halo kernel also for 128, 256 and 512 channels (128-channel tiles, images up to 31 pixels wide), the
+ * mode 2 the halo kernel instead of the rows kernel and also for 128, 256 and 512 channels (128-channel tiles, images up to 31 pixels wide), the
  * two-group kernel whatever the number of tiles and the widening kernel wherever it applies; mode 0 none of them.
  * Identical results in every mode.  Plans that do not run the MFMA kernel return an error.
  */
