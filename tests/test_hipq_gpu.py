@@ -585,6 +585,40 @@ def test_quantize_dequantize():
         assert np.array_equal(fd.cpu().numpy().view(np.uint32), orc.dequantize_u8(want, oa, oz).view(np.uint32))
 
 
+def test_quantize_division_free_form_is_exact():
+    """quantize_u8 divides by multiplying with the correctly rounded reciprocal and two FMA corrections, clamps before
+    the division and rounds without the reference's double: checked against the reference arithmetic on the values where
+    such shortcuts would show - the fp32 neighbours (five ulps either side) of every rounding boundary (k + 0.5) * alpha
+    and of both clamps, zeros, subnormals, huge values, infinities and NaN, random bit patterns - for scales that are and
+    are not powers of two, including ones whose reciprocal rounds awkwardly, and for fewer output bits."""
+    rng = np.random.default_rng(171)
+    scales = [0.0078125, 0.1, 1.0 / 3.0, 0.05, 0.007843137718737125, 1.9999998807907104, 1.0000001192092896, 3.0e-5,
+              float(np.float32(1.0) / np.float32(255.0)), 123.456] + [rand_q(rng, 1e-4, 10.0) for _ in range(6)]
+    for i, oa in enumerate(scales):
+        oa = float(np.float32(oa))
+        for oz, obits in ((0, 8), (128, 8), (255, 8), (int(rng.integers(0, 128)), 7), (3, 4)):
+            hi = (1 << obits) - 1
+            k = np.arange(-3, hi + 4, dtype=np.float64)
+            centres = np.concatenate([(k + 0.5 - oz) * oa, (k - oz) * oa]).astype(np.float32)
+            near = centres.view(np.int32)[:, None] + np.arange(-5, 6, dtype=np.int32)[None, :]
+            special = np.array([0.0, -0.0, 1e-45, -1e-45, 1e-38, -1e-38, 3e38, -3e38, np.inf, -np.inf, np.nan, 65504.0, -65504.0],
+                               np.float32)
+            rnd = rng.integers(0, 1 << 32, 200000, dtype=np.uint64).astype(np.uint32).view(np.float32)
+            norm = (rng.standard_normal(200000) * 80 * oa).astype(np.float32)
+            x = np.concatenate([near.reshape(-1).view(np.float32), special, rnd, norm]).astype(np.float32)
+            x = np.concatenate([x, np.zeros((-x.size) % 4, np.float32)]).reshape(1, 1, -1, 4)
+            with np.errstate(all="ignore"):
+                want = orc.quantize_u8(x, oa, oz, obits)
+            xd = torch.from_numpy(x).cuda()
+            yd = torch.empty((1, x.shape[2], 4, 4), dtype=torch.uint8, device="cuda")
+            hipq.quantize_u8(xd, yd, oa, oz, obits)
+            got = hipq.from_device_nhwc(yd, 1)
+            bad = np.flatnonzero(got.reshape(-1) != want.reshape(-1))
+            assert bad.size == 0, (oa, oz, obits, bad.size, x.reshape(-1)[bad[:5]], got.reshape(-1)[bad[:5]], want.reshape(-1)[bad[:5]])
+    with pytest.raises(hipq.HipqError, match="scale"):
+        hipq.quantize_u8(xd, yd, -0.5, 0)
+
+
 def test_layout_round_trip_and_errors():
     rng = np.random.default_rng(18)
     x = rng.integers(0, 256, (2, 19, 5, 7), dtype=np.uint8)
