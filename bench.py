@@ -11,6 +11,8 @@ Prints ONE JSON line:
                         their measured durations, against the chip's dense int8 MFMA peak
   kernel_families       every family's time, TOP/s and GB/s (launch-by-launch timing, see per_kernel_times)
   sustained             the same replay loop kept running for at least two seconds
+  machine_probes        what this box delivers on the library's own probes: MFMA rate on constant and random operands, the
+                        cost of a launch in a graph chain, load-unit streaming per CU, vector-memory instruction rates
   library_int8_gemm     a yardstick: the vendor library's plain int8 GEMM (int32 output) on every layer's GEMM shape, summed,
                         beside the sum of this build's convolution-family launches
   module_path           the same network as an engine file run by nart_promark on the `hip` workspace (the drop-in path),
@@ -268,6 +270,57 @@ def library_gemm(case, ex, kt):
                     "this build: its convolution-family launches, which include all of those"}
 
 
+def machine_probes():
+    """What the box delivers on the library's own probes (include/hipq.h: hipq_probe_launch): HIP events around graph
+    replays of a few launches each.  The published peaks stay the roofs; these say how far below them a perfect kernel
+    of the same shape would land on this machine."""
+    import ctypes
+    import torch
+    from nart_amd import hipq
+    lib = hipq.lib()
+    buf = torch.randint(0, 256, (64 << 20,), dtype=torch.uint8, device="cuda")
+    st = torch.cuda.Stream()
+    units = ctypes.c_double(0)
+
+    def run(which, iters, param=0, reps=3):
+        def one():
+            hipq.check(lib.hipq_probe_launch(which, buf.data_ptr(), buf.numel(), iters, param, ctypes.byref(units), st.cuda_stream))
+        with torch.cuda.stream(st):
+            one()
+            torch.cuda.synchronize()
+            g = graph_of(one, reps, st)
+            g.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record(st)
+            for _ in range(3):
+                g.replay()
+            e1.record(st)
+            torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e-3 / (3 * reps), units.value   # seconds per launch, work per launch
+
+    out = {}
+    t, u = run(0, 4000)
+    out["mfma_i8_constant_operands_TOPs"] = round(u / t / 1e12, 1)
+    t, u = run(1, 4000)
+    out["mfma_i8_random_operands_TOPs"] = round(u / t / 1e12, 1)
+    t, _ = run(2, 1, reps=200)
+    out["launch_in_graph_chain_us"] = round(t * 1e6, 2)
+    for name, region in (("l2_resident_2MB", 2 << 20), ("beyond_l2_32MB", 32 << 20)):
+        t, u = run(3, 1536, region)
+        out["lds_dma_%s_KB_per_us_per_CU" % name] = round(u / t / 1e9 / 256, 1)
+    names = ("load_32bit_contiguous", "load_32bit_eight_pieces", "load_128bit", "store_32bit_contiguous", "store_32bit_eight_pieces",
+             "store_128bit")
+    widths = (256, 256, 1024, 256, 256, 1024)
+    for i, (nm, w) in enumerate(zip(names, widths)):
+        t, u = run(4 + i, 2000)
+        ns = t * 1e9 / u
+        out["vmem_" + nm] = {"ns_per_wave_instruction_per_CU": round(ns, 2), "TBs_chip": round(w / ns * 256 / 1e3, 2)}
+    out["note"] = ("8 waves per CU; MFMA: four independent accumulators per wave; lds_dma: global_load_lds_dwordx4, three stages of 2 KB "
+                   "per wave; vmem: 4 KB per wave, resident in the CU's L1")
+    return out
+
+
 def module_path(build, batch, steps):
     """The drop-in path: the network as an engine file, run by nart_promark (the counterpart of the reference's
     tools/promark.cpp) on the `hip` workspace through hip_module_tp, every operator launched by the module's run
@@ -466,6 +519,7 @@ def main():
 
     if not args.no_extras and not args.no_graph:
         extra("library_int8_gemm", lambda: library_gemm(case, ex, kt))
+        extra("machine_probes", machine_probes)
 
     if not args.no_extras and args.workload == "resnet50":
         extra("module_path", lambda: module_path(build, args.batch, 50))

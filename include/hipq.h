@@ -273,6 +273,20 @@ int hipq_dequantize_i8(const void *x_nhwc, float *y_nchw, int N, int C, int H, i
 /* A plain device-to-device copy kernel of known size; the calibration reference for HBM counters. */
 int hipq_copy_bytes(const void *src, void *dst, size_t count, void *stream);
 
+/*
+ * Machine probes (no counterpart in the reference; bench.py reports them as `machine_probes`): one launch of a few
+ * lines of HIP around one loop, so that the rates this library's kernels are judged against are measured on the box
+ * the benchmark runs on.  `buf`: a 1 KB aligned device buffer of at least 64 MiB that the probes read and write (fill
+ * it with random bytes for probe 1); `iters`: trip count of the probe's loop; `*units` receives the work of the launch.
+ *   0  v_mfma_i32_32x32x32_i8 on constant operands, 8 waves per CU            units: integer operations
+ *   1  the same on operands taken from the buffer (the sustained rate depends on the data)
+ *   2  an empty kernel (time a chain of them for the cost of a launch)         units: 0
+ *   3  the load unit streaming the first `param` bytes (a power of two) into LDS, global_load_lds_dwordx4   units: bytes
+ *   4, 5, 6  loads in a loop: 32-bit on 256 contiguous bytes, 32-bit as eight pieces of 32 bytes, 128-bit on 1 KB
+ *   7, 8, 9  stores in a loop, the same three shapes                           units: wave instructions per CU
+ */
+int hipq_probe_launch(int which, void *buf, size_t bytes, int iters, size_t param, double *units, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -74,6 +74,7 @@ _SIGS = {
     "hipq_quantize_i8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_float, C.c_int, C.c_void_p]),
     "hipq_dequantize_i8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_float, C.c_void_p]),
     "hipq_copy_bytes": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
+    "hipq_probe_launch": (C.c_int, [C.c_int, C.c_void_p, C.c_size_t, C.c_int, C.c_size_t, C.POINTER(C.c_double), C.c_void_p]),
 }
 EXPORTS = tuple(_SIGS)
 

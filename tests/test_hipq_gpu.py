@@ -1016,3 +1016,21 @@ def test_two_group_kernel_matches_the_oracle():
     w = rng.integers(0, 256, (64, 256, 3, 3), dtype=np.uint8)
     plan = hipq.Conv2d(x.shape, w, None, 1, 1, 1, 0.02, 7, 0.005, 100, 0.05, 3)
     assert not plan.kernel.endswith("_k2"), plan.kernel
+
+
+def test_machine_probes_launch_and_refuse_bad_arguments():
+    """hipq_probe_launch (the probes bench.py reports as machine_probes): every probe launches, ends and reports its
+    work; a buffer that is too small, a probe number out of range and a streamed region that is not a power of two
+    are refused before anything is launched."""
+    import ctypes
+    lib = hipq.lib()
+    buf = torch.randint(0, 256, (64 << 20,), dtype=torch.uint8, device="cuda")
+    units = ctypes.c_double(-1)
+    st = torch.cuda.current_stream().cuda_stream
+    for which, iters, param in [(0, 50, 0), (1, 50, 0), (2, 1, 0), (3, 64, 1 << 20)] + [(w, 20, 0) for w in range(4, 10)]:
+        hipq.check(lib.hipq_probe_launch(which, buf.data_ptr(), buf.numel(), iters, param, ctypes.byref(units), st))
+        torch.cuda.synchronize()
+        assert (units.value == 0) == (which == 2), (which, units.value)
+    for bad in [(10, buf.numel(), 10, 0), (0, 1 << 20, 10, 0), (3, buf.numel(), 10, 3 << 20), (0, buf.numel(), 0, 0)]:
+        with pytest.raises(hipq.HipqError, match="hipq_probe_launch"):
+            hipq.check(lib.hipq_probe_launch(bad[0], buf.data_ptr(), bad[1], bad[2], bad[3], ctypes.byref(units), st))
