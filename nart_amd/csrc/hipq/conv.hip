@@ -1002,7 +1002,7 @@ __device__ static inline void pointwise_strips(const ConvArgs &a, const uint8_t 
                     asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(r[2]), "v"(r[3]));
                     asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
                     asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
-                    cv[g] = (b01 & 0xffffu) | (b23 << 16);
+                    cv[g] = __builtin_amdgcn_perm(b23, b01, 0x05040100u); // the low halves of both, one instruction
                 } else {
                     int32_t rq[4];
 #pragma unroll

@@ -63,7 +63,7 @@ __device__ inline void plain_to_staging(const ConvArgs &a, const v16i (&acc)[TN]
                 asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(r[2]), "v"(r[3]));
                 asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
                 asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
-                packed = (b01 & 0xffffu) | (b23 << 16);
+                packed = __builtin_amdgcn_perm(b23, b01, 0x05040100u); // the low halves of both, one instruction
             } else {
                 int32_t rq[4];
 #pragma unroll
@@ -112,7 +112,7 @@ __device__ inline void fused_in_place(const ConvArgs &a, const v16i (&acc)[2], u
                 asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(y[2]), "v"(y[3]));
                 asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
                 asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
-                packed = (b01 & 0xffffu) | (b23 << 16);
+                packed = __builtin_amdgcn_perm(b23, b01, 0x05040100u); // the low halves of both, one instruction
             } else {
                 packed = 0;
 #pragma unroll
@@ -188,10 +188,14 @@ __global__ __launch_bounds__(256) void conv_mfma_expand_kernel(const ConvArgs a,
     int mt = t0 / ntiles, nt = t0 - mt * ntiles; // the current tile; the list is walked without further divisions
     issue(mt, nt, 0);
 
-    // ---- the folded biases -> LDS; the wave's pixel operands -> registers ----
+    // ---- the folded biases -> LDS; the wave's pixel operands -> registers.  Every global load of the prologue is issued
+    // before the first result is used (bias values wait in registers, the pixel operands are re-centred after the
+    // loop's first wait): one round trip to memory instead of three in a row ----
     int32_t *lbias = reinterpret_cast<int32_t *>(lds + B_OFF);
-    for (int i = tid; i < ntiles * kBN; i += 256)
-        lbias[i] = a.bias2[i];
+    int32_t bv[kMaxTiles * kBN / 256];
+#pragma unroll
+    for (int j = 0; j < kMaxTiles * kBN / 256; j++)
+        bv[j] = tid + 256 * j < ntiles * kBN ? a.bias2[tid + 256 * j] : 0;
     const int pl = wave * 32 + p;                 // this lane's pixel within the tile's 128
     v4i bf[NSLAB][2];
     auto load_pixels = [&](int mt) {
@@ -209,9 +213,14 @@ __global__ __launch_bounds__(256) void conv_mfma_expand_kernel(const ConvArgs a,
         for (int s = 0; s < NSLAB; s++)
 #pragma unroll
             for (int k = 0; k < 2; k++)
-                bf[s][k] = ldg128(xrow + s * 64 + k * 32 + half * 16) ^ (int)a.xmask;
+                bf[s][k] = ldg128(xrow + s * 64 + k * 32 + half * 16); // raw bytes: re-centred at the top of the next tile
     };
     load_pixels(mt);
+    bool fresh = true; // bf holds raw bytes
+#pragma unroll
+    for (int j = 0; j < kMaxTiles * kBN / 256; j++)
+        if (tid + 256 * j < ntiles * kBN)
+            lbias[tid + 256 * j] = bv[j];
     v16i acc2[MID ? TN2 : 1]; // chained: 32 pixels x MID channels of the next layer, from its folded bias
     if (MID) {
 #pragma unroll
@@ -256,6 +265,14 @@ __global__ __launch_bounds__(256) void conv_mfma_expand_kernel(const ConvArgs a,
         wait_vmcnt<0>();
         __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
         __builtin_amdgcn_s_barrier();
+        if (fresh) { // the pixel operands loaded during the previous tile (or the prologue) have landed with that wait
+#pragma unroll
+            for (int s = 0; s < NSLAB; s++)
+#pragma unroll
+                for (int k = 0; k < 2; k++)
+                    bf[s][k] ^= (int)a.xmask;
+            fresh = false;
+        }
         const uint8_t *wb = lds + buf * WBYTES;
         v16i acc[2];
 #pragma unroll
@@ -276,8 +293,10 @@ __global__ __launch_bounds__(256) void conv_mfma_expand_kernel(const ConvArgs a,
                 acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af0, bf[s][k], acc[0], 0, 0, 0);
                 acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af1, bf[s][k], acc[1], 0, 0, 0);
             }
-        if (t + 1 < t1 && wrap)
+        if (t + 1 < t1 && wrap) {
             load_pixels(nmt); // the range moves on to the next 128 pixels: their operands arrive during this tile's arithmetic
+            fresh = true;
+        }
         v4i staged[2];
         if (t > t0)
             read_staged(buf ^ 1, staged);

@@ -155,7 +155,7 @@ __global__ __launch_bounds__(256, 2) void conv3x3_c64_rows_kernel(const ConvArgs
                     asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(r[2]), "v"(r[3]));
                     asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
                     asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
-                    packed = (b01 & 0xffffu) | (b23 << 16);
+                    packed = __builtin_amdgcn_perm(b23, b01, 0x05040100u); // the low halves of both, one instruction
                 } else {
                     int32_t rq[4];
 #pragma unroll

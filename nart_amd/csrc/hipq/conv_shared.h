@@ -163,7 +163,7 @@ __device__ static inline void conv_epilogue(const ConvArgs &a, v16i (&acc)[TN][T
                     asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(r[2]), "v"(r[3]));
                     asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
                     asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
-                    packed = (b01 & 0xffffu) | (b23 << 16);
+                    packed = __builtin_amdgcn_perm(b23, b01, 0x05040100u); // the low halves of both, one instruction
                 } else {
                     int32_t rq[4];
 #pragma unroll
