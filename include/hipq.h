@@ -54,6 +54,12 @@ void hipq_quant_scale(float scale, int bits, uint32_t *mult, int *shift);
 
 /* Channel stride of the device layout for a tensor with C channels. */
 int hipq_channel_stride(int C);
+/*
+ * Host helper (no counterpart in the reference): the reciprocal with which the kernels divide by a run-time constant,
+ * floor(x / d) == (uint32_t)(((uint64_t)x * *m) >> 32) >> *s for every 0 <= x < 2^31 (*m == 0: d is 1, the quotient
+ * is x).  Returns -1 for d == 0 or a null pointer.
+ */
+int hipq_div_magic(uint32_t d, uint32_t *m, int *s);
 
 /* ---- layout conversion at the host boundary (no counterpart in the reference, which is NCHW only) */
 int hipq_nchw_to_nhwc_u8(const void *src_nchw, void *dst_nhwc, int N, int C, int H, int W, int cs,

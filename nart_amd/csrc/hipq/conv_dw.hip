@@ -6,16 +6,17 @@
 // transposes them once into per-channel dwords of four consecutive pixels (8 v_perm_b32 per 4x4 block), and feeds
 // them to the partial sums of every output row that input row belongs to: three rows in flight for stride 1 (kernel
 // rows 0, 1, 2 of output rows i, i-1, i-2), two for stride 2.  An output row is requantised and stored when its last
-// kernel row is in.  Compared with computing two output rows per thread from four freshly loaded and transposed input
-// rows, loads and transposes per output row drop from 2 to (RB + 2) / RB input rows.
+// kernel row is in: every loaded and transposed input row serves all the output rows it belongs to, and none of the
+// work is for rows that the thread does not produce (RB = 2 measured fastest: see kRowsPerThread).
 //   stride 1: T0 = [x0 x1 x2 x3], T1 = [x2 x3 x4 x5] per channel; outputs 0 / 1 are v_dot4_i32_i8 of T0 with the packed
 //             weights [w0 w1 w2 0] / [0 w0 w1 w2], outputs 2 / 3 the same with T1;
 //   stride 2: T0 = [x0..x3], T1 = [x4..x7]; outputs 0 and 2 use T0 and T1, output 1 v_alignbyte(T1, T0) = [x2 x3 x4 x5],
 //             output 3 a v_perm of T1 and the ninth column = [x6 x7 x8 0]; all with [w0 w1 w2 0].
 // Bytes are re-centred (x ^ 0x80, w - 128); bias + 128 * sum(w - 128) is folded per channel by the host.  Columns and
 // rows outside the image are loaded from a clamped address and replaced by the zero-point byte (a select per dword,
-// no divergent branch).  Rows two ahead are requested before the current row is used.
+// no divergent branch).  Rows three ahead are requested before the current row is used.
 #include "conv_dw.h"
+#include "hipq.h"
 
 #include <algorithm>
 #include <cstdlib>
@@ -93,21 +94,37 @@ __device__ static inline void emit_row(const ConvArgs &a, const int32_t (&acc)[4
     }
 }
 
+// How the grid maps to work: a work-group is ONE wave and takes 64 consecutive (strip, channel quad) items of one row block
+// of one image, so image and row block are the same for all its lanes and everything derived from them - row addresses,
+// row validity, the output row's base - is scalar-unit arithmetic, off the vector ALU that bounds this kernel.  The two
+// divisions that take a block number apart, and the one that splits an item, are multiplications by reciprocals the
+// host has computed (and verified for every dividend that can occur).
+struct DwMap {
+    int nrb, chunks, per_img, items; // row blocks per image, waves per row block, their product, items per row block
+    uint32_t m_img, m_chunk, m_cq;   // floor(x / d) = (x * m) >> (32 + s)
+    int s_img, s_chunk, s_cq;
+    int cq;
+};
+
+// m == 0: the divisor is 1 (no 32-bit reciprocal multiplies to the identity)
+__device__ static inline uint32_t div_magic(uint32_t x, uint32_t m, int s) { return m ? (uint32_t)(((uint64_t)x * m) >> 32) >> s : x; }
+
 template <int STRIDE, int QMODE, bool DUMP, int RB>
-__global__ __launch_bounds__(256) void conv_depthwise3x3_slide_kernel(const ConvArgs a, const int nrb, const int total)
+__global__ __launch_bounds__(64) void conv_depthwise3x3_slide_kernel(const ConvArgs a, const DwMap mp)
 {
     constexpr int NCOL = 3 * STRIDE + 3; // input columns under a strip of 4 outputs
     // work-groups go to the 8 XCDs in turn: renumbered so that each XCD works on one contiguous eighth of the
-    // (image-major) index space (the grid is a multiple of 8)
-    const int L = (int)(blockIdx.x & 7) * (int)(gridDim.x >> 3) + (int)(blockIdx.x >> 3);
-    const int idx = L * 256 + (int)threadIdx.x;
-    if (idx >= total)
+    // (image-major) block list (the grid is a multiple of 8; blocks beyond the list end at once)
+    const uint32_t L = (blockIdx.x & 7) * (gridDim.x >> 3) + (blockIdx.x >> 3);
+    const uint32_t n = div_magic(L, mp.m_img, mp.s_img), r1 = L - n * mp.per_img;
+    const uint32_t rb = div_magic(r1, mp.m_chunk, mp.s_chunk), chunk = r1 - rb * mp.chunks;
+    if ((int)n >= a.N)
         return;
-    const int cq = a.in_cs >> 2, nstrip = (a.OW + 3) >> 2;
-    const int t0 = fast_div(idx, cq, a.inv_ow), quad = idx - t0 * cq; // inv_ow holds 1 / cq for the depthwise kernels
-    const int t1 = t0 / nstrip, strip = t0 - t1 * nstrip;
-    const int n = t1 / nrb, rb = t1 - n * nrb;
-    const int oh0 = rb * RB, ow0 = strip * 4, c0 = quad * 4;
+    const uint32_t item = chunk * 64 + threadIdx.x;
+    if ((int)item >= mp.items)
+        return;
+    const int strip = (int)div_magic(item, mp.m_cq, mp.s_cq), quad = (int)item - strip * mp.cq;
+    const int oh0 = (int)rb * RB, ow0 = strip * 4, c0 = quad * 4;
     const int ih0 = oh0 * STRIDE - a.pad_h, iw0 = ow0 * STRIDE - a.pad_w;
     const int ncols = min(4, a.OW - ow0);
 
@@ -127,11 +144,11 @@ __global__ __launch_bounds__(256) void conv_depthwise3x3_slide_kernel(const Conv
     const uint32_t padx = a.padword ^ 0x80808080u;
     uint32_t coff[NCOL];
     bool cok[NCOL];
+    const int off0 = iw0 * a.in_cs, offmax = (a.W - 1) * a.in_cs; // one multiply per thread: the clamp commutes with the scaling
 #pragma unroll
     for (int j = 0; j < NCOL; j++) {
-        const int iw = iw0 + j;
-        cok[j] = (unsigned)iw < (unsigned)a.W;
-        coff[j] = (uint32_t)(min(max(iw, 0), a.W - 1) * a.in_cs);
+        cok[j] = (unsigned)(iw0 + j) < (unsigned)a.W;
+        coff[j] = (uint32_t)min(max(off0 + j * a.in_cs, 0), offmax);
     }
     auto issue = [&](int i, uint32_t (&dst)[NCOL]) {
         const uint32_t rbase = nbase + (uint32_t)min(max(ih0 + i, 0), a.H - 1) * rowbytes;
@@ -247,18 +264,27 @@ bool conv_dw_slide_applies(const ConvArgs &a)
 template <int STRIDE, int RB>
 static void launch_rb(const ConvArgs &a, hipStream_t st)
 {
-    const int nrb = (a.OH + RB - 1) / RB;
-    const long long total = (long long)a.N * nrb * ((a.OW + 3) / 4) * (a.in_cs / 4); // the plan guarantees 31 bits for RB = 1
-    const dim3 grid((unsigned)(((total + 255) / 256 + 7) / 8 * 8)), block(256);
+    DwMap mp;
+    mp.nrb = (a.OH + RB - 1) / RB;
+    mp.cq = a.in_cs / 4;
+    mp.items = ((a.OW + 3) / 4) * mp.cq;
+    mp.chunks = (mp.items + 63) / 64;
+    mp.per_img = mp.nrb * mp.chunks;
+    const long long grid_l = ((long long)a.N * mp.per_img + 7) / 8 * 8; // the plan bounds N * OH * strips * quads by 2^31
+    // reciprocals for the three divisions (include/hipq.h: hipq_div_magic)
+    hipq_div_magic((uint32_t)mp.per_img, &mp.m_img, &mp.s_img);
+    hipq_div_magic((uint32_t)mp.chunks, &mp.m_chunk, &mp.s_chunk);
+    hipq_div_magic((uint32_t)mp.cq, &mp.m_cq, &mp.s_cq);
+    const dim3 grid((unsigned)grid_l), block(64);
     const int qmode = (a.fastq && a.qmult == nullptr) ? (a.lo == 0 && a.q.hi == 255 ? 2 : 1) : 0;
     if (a.acc_out)
-        hipLaunchKernelGGL((conv_depthwise3x3_slide_kernel<STRIDE, 0, true, RB>), grid, block, 0, st, a, nrb, (int)total);
+        hipLaunchKernelGGL((conv_depthwise3x3_slide_kernel<STRIDE, 0, true, RB>), grid, block, 0, st, a, mp);
     else if (qmode == 2)
-        hipLaunchKernelGGL((conv_depthwise3x3_slide_kernel<STRIDE, 2, false, RB>), grid, block, 0, st, a, nrb, (int)total);
+        hipLaunchKernelGGL((conv_depthwise3x3_slide_kernel<STRIDE, 2, false, RB>), grid, block, 0, st, a, mp);
     else if (qmode == 1)
-        hipLaunchKernelGGL((conv_depthwise3x3_slide_kernel<STRIDE, 1, false, RB>), grid, block, 0, st, a, nrb, (int)total);
+        hipLaunchKernelGGL((conv_depthwise3x3_slide_kernel<STRIDE, 1, false, RB>), grid, block, 0, st, a, mp);
     else
-        hipLaunchKernelGGL((conv_depthwise3x3_slide_kernel<STRIDE, 0, false, RB>), grid, block, 0, st, a, nrb, (int)total);
+        hipLaunchKernelGGL((conv_depthwise3x3_slide_kernel<STRIDE, 0, false, RB>), grid, block, 0, st, a, mp);
 }
 
 // Output rows per thread.  Longer walks share loaded and transposed rows among more output rows (4 rows: 25 % fewer

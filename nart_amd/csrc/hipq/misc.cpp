@@ -71,3 +71,25 @@ bool hipq::make_add_params(float ia0, int iz0, float ia1, int iz1, float oa, int
 }
 
 extern "C" int hipq_channel_stride(int C) { return C <= 4 ? 4 : (C + 15) / 16 * 16; }
+
+// A power of two 2^k: m = 2^(32 - k), s = 0.  Otherwise s = floor(log2 d) and m = ceil(2^(32 + s) / d): m fits 32 bits
+// because d > 2^s, and the round-up error e = m * d - 2^(32 + s) is below d < 2^(s + 1), so x * e < 2^(32 + s) for
+// x < 2^31, which is the condition for the quotient to be exact.  d == 1 has no such m: m = 0 means "x itself".
+extern "C" int hipq_div_magic(uint32_t d, uint32_t *m, int *s)
+{
+    if (d == 0 || m == nullptr || s == nullptr)
+        return -1;
+    *m = 0, *s = 0;
+    if (d == 1)
+        return 0;
+    int lg = 31;
+    while (!(d >> lg))
+        lg--;
+    if ((d & (d - 1)) == 0) {
+        *m = 1u << (32 - lg);
+        return 0;
+    }
+    *s = lg;
+    *m = (uint32_t)(((1ull << (32 + lg)) + d - 1) / d);
+    return 0;
+}

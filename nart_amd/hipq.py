@@ -36,6 +36,7 @@ _SIGS = {
     "hipq_last_error": (C.c_char_p, []),
     "hipq_quant_scale": (None, [C.c_float, C.c_int, C.POINTER(C.c_uint32), C.POINTER(C.c_int)]),
     "hipq_channel_stride": (C.c_int, [C.c_int]),
+    "hipq_div_magic": (C.c_int, [C.c_uint32, C.POINTER(C.c_uint32), C.POINTER(C.c_int)]),
     "hipq_nchw_to_nhwc_u8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_void_p]),
     "hipq_nhwc_to_nchw_u8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_void_p]),
     "hipq_conv2d_plan_create": (C.c_int, [C.POINTER(ConvDesc), C.c_void_p, C.c_void_p, C.POINTER(C.c_void_p)]),

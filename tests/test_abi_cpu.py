@@ -40,6 +40,26 @@ def test_channel_stride_rule():
     assert [hipq.channel_stride(c) for c in (1, 3, 4, 5, 16, 17, 24, 64, 1000)] == [4, 4, 4, 16, 16, 32, 32, 64, 1008]
 
 
+def test_division_reciprocals_are_exact():
+    """hipq_div_magic: the multiply-and-shift that replaces a division by a run-time constant inside the kernels equals
+    the division for every dividend below 2^31 - checked at the dividends where a rounded-up reciprocal fails first (one
+    below and exactly at multiples of the divisor), at the ends of the range and at random ones, for small divisors,
+    powers of two and their neighbours, and large ones."""
+    import ctypes
+    rng = np.random.default_rng(5)
+    ds = list(range(1, 700)) + [2 ** k + e for k in range(2, 31) for e in (-1, 0, 1)] + [int(v) for v in rng.integers(1, 2 ** 31 - 1, 300)]
+    m, s = ctypes.c_uint32(), ctypes.c_int()
+    for d in ds:
+        assert hipq.lib().hipq_div_magic(d, ctypes.byref(m), ctypes.byref(s)) == 0
+        q = np.unique(np.concatenate([np.arange(0, min(2 ** 31 // d + 1, 3000)), rng.integers(0, 2 ** 31 // d + 1, 3000)])).astype(np.uint64)
+        x = np.concatenate([q * np.uint64(d), q * np.uint64(d) + np.uint64(d - 1), rng.integers(0, 2 ** 31, 3000).astype(np.uint64),
+                            np.array([0, 1, 2 ** 31 - 1], np.uint64)])
+        x = x[x < 2 ** 31]
+        got = ((x * np.uint64(m.value)) >> np.uint64(32)) >> np.uint64(s.value) if m.value else x
+        assert np.array_equal(got, x // np.uint64(d)), (d, m.value, s.value)
+    assert hipq.lib().hipq_div_magic(0, ctypes.byref(m), ctypes.byref(s)) == -1
+
+
 def test_ip_weight_reorder_host():
     rng = np.random.default_rng(1)
     No, C, H, W, cs = 5, 6, 2, 3, 16
