@@ -131,7 +131,8 @@ int hipq_conv2d_plan_select(hipq_conv2d_plan *plan, int tile, int stages);
  * feed the MFMA from global memory wave by wave, without LDS staging or barriers (hipq_conv2d_run only: the fused add
  * of hipq_conv2d_run_add and accumulator dumps take the tile kernel).  Two-group kernel (name "..._k2"): the tile
  * kernel with 512 threads, two groups of four waves that each reduce every other 64-byte slab of k and add their partial
- * accumulators through LDS (plain convolutions with an even number of at least 8 slabs; not with an explicit stage count).
+ * accumulators through LDS (convolutions, with or without a fused residual add, with an even number of at least 8 slabs;
+ * not with an explicit stage count).
  * Widening kernel (name "..._expand"): 1x1 convolutions without padding from 64, 128 or 256 input channels (stride) to
  * at least twice as many and 256 to 1024 output channels over at least 1024 pixels (weight zero point 128) keep a wave's
  * pixel operands in registers while a work-group walks a contiguous range of 128-pixel x 64-channel output tiles, with

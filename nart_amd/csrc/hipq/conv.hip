@@ -1590,7 +1590,7 @@ static void set_mfma_name(hipq_conv2d_plan *p, bool smallc)
     else
         snprintf(nm, sizeof nm, "conv_mfma_i8_%dx%d%s%s%s%s", kTiles[p->tile].bm, kTiles[p->tile].bn, smallc ? "_c4" : "",
                  p->has_wzp ? "_wzp" : "", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "",
-                 halo_applies(p) ? "_halo" : (!smallc && k2_applies(p)) ? "_k2" : ""); // _k2: unless a residual add is fused
+                 halo_applies(p) ? "_halo" : (!smallc && k2_applies(p)) ? "_k2" : "");
     p->name = nm;
     if (p->d_q)
         p->name += "_perchannel";
@@ -1869,8 +1869,9 @@ extern "C" const char *hipq_conv2d_plan_kernel_add(const hipq_conv2d_plan *p)
     if (expand_applies(p, a))
         snprintf(buf, sizeof buf, "conv_mfma_i8_expand%s+add", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
     else
-        snprintf(buf, sizeof buf, "conv_mfma_i8_%dx%d%s%s%s+add", kTiles[p->tile].bm, kTiles[p->tile].bn,
-                 p->variant == kMfmaSmallC ? "_c4" : "", p->has_wzp ? "_wzp" : "", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
+        snprintf(buf, sizeof buf, "conv_mfma_i8_%dx%d%s%s%s%s+add", kTiles[p->tile].bm, kTiles[p->tile].bn,
+                 p->variant == kMfmaSmallC ? "_c4" : "", p->has_wzp ? "_wzp" : "", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "",
+                 p->variant == kMfma && k2_applies(p) ? "_k2" : "");
     nm = buf;
     if (p->d_q)
         nm += "_perchannel";
@@ -1993,8 +1994,8 @@ static bool launch_halo(const hipq_conv2d_plan *p, const ConvArgs &a, const dim3
     }
 }
 
-// conv_mfma_dma_k2_kernel (the reduction shared by two groups of four waves): plain convolutions (no fused residual)
-// with aligned addressing, an even number of at least 8 slabs, a tile of at most 128 + 64 or 64 + 128 rows per stage
+// conv_mfma_dma_k2_kernel (the reduction shared by two groups of four waves): convolutions - with or without a fused
+// residual add, which its epilogue applies to the staged tile like the generic kernels' - with aligned addressing, an even number of at least 8 slabs, a tile of at most 128 + 64 or 64 + 128 rows per stage
 // pair, and - by the built-in rule - no more tiles than the chip has CUs, i.e. layers that would otherwise run one wave
 // per SIMD.  Measured inside the ResNet-50 pass the 7x7 layers gain 20 %; layers with one to two tiles per CU gain
 // nothing (two four-wave work-groups already share their CUs) and 128x128 tiles lose.  An explicit stage count
@@ -2016,7 +2017,7 @@ static bool launch_k2(const hipq_conv2d_plan *p, const ConvArgs &a, const dim3 g
     if constexpr (BM + BN > 256) {
         return false;
     } else {
-        if (!k2_applies(p) || a.res != nullptr)
+        if (!k2_applies(p))
             return false;
         if (a.nbm * a.nbn <= kCUs || BM + BN > 192) {
             // one work-group per CU: LDS is no constraint, so the deepest stream the stages allow
@@ -2078,6 +2079,8 @@ static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_
             hipLaunchKernelGGL((conv_mfma_kernel<BM, BN, WM, WN, false, true>), grid, block, 0, st, a);
     } else if (p->has_wzp) { // rare (asymmetric weights): generic addressing only
         hipLaunchKernelGGL((conv_mfma_dma_kernel<BM, BN, WM, WN, kStages, true, false>), grid, block, 0, st, a);
+    } else if (aligned && a.res != nullptr && launch_k2<BM, BN, WM, WN>(p, a, grid, st)) {
+        // few tiles and a long reduction: the two-group kernel, the add applied to its staged tile
     } else if (aligned && a.res != nullptr && a.fastq && a.addq.fast && !plain_epilogue(a)) {
         // residual add in the accumulator layout, residual tile prefetched into LDS
         const int ns = p->stages ? p->stages : (a.nslab >= kDeepFrom ? 3 : kStages);

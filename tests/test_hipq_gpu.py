@@ -988,6 +988,14 @@ def test_two_group_kernel_matches_the_oracle():
         assert plan.kernel.endswith("_k2") == (eligible and not stream), (plan.kernel, nslab)  # every case has at most 256 tiles of the rule's own tile
         xd = hipq.to_device_nhwc(x)
         assert np.array_equal(hipq.from_device_nhwc(plan(xd), K), want), (x.shape, K, plan.kernel)
+        if not stream:  # the fused residual add takes the same kernel where it applies, in both operand orders
+            assert plan.kernel_add.endswith("_k2+add") == eligible, plan.kernel_add
+            res = rng.integers(0, 256, want.shape, dtype=np.uint8)
+            ra, rz, sa, sz = rand_q(rng, 1e-2, 1e-1), int(rng.integers(0, 256)), rand_q(rng, 3e-2, 3e-1), int(rng.integers(0, 256))
+            for first in (False, True):
+                yd = plan.run_add(xd, hipq.to_device_nhwc(res), first, ra, rz, sa, sz, plan.empty_output())
+                want_add = orc.add_u8(res, want, ra, rz, q[4], q[5], sa, sz) if first else orc.add_u8(want, res, q[4], q[5], ra, rz, sa, sz)
+                assert np.array_equal(hipq.from_device_nhwc(yd, K), want_add), (x.shape, K, first, plan.kernel_add)
         plan.special(2)
         for tile in (0, 2, 3, 4):
             plan.select(tile, 0)
