@@ -140,6 +140,9 @@ int hipq_conv2d_plan_select(hipq_conv2d_plan *plan, int tile, int stages);
  * Rows kernel (name "..._rows3x3"): 3x3 / stride 1 / pad 1 convolutions with an input and output channel stride of 64
  * on rows of at most 64 pixels (weight zero point 128, one-multiply requantisation, no fused add) keep the input rows
  * of a work-group in LDS and all weights in registers.
+ * 3x3 stem kernel (name "..._stem3x3"): 3x3 / stride 2 convolutions of an image with at most 4 channels (channel stride 4,
+ * rows of at most 248 pixels, a multiple of 4) to at most 32 channels (stride 32), weight zero point 128: the input rows
+ * of a work-group in LDS, two multiplies per 32 pixels, 128-bit stores straight from the accumulators; modes 1 and 2.
  * mode 1 (the default) uses them where they measured faster: the rows kernel wherever it applies, the halo kernel for
  * the other 64-channel inputs up to 63 pixels wide, the pointwise kernel wherever it applies, the two-group kernel for layers with at most one tile per CU (256),
  * the widening kernel with the add at 64 input channels and without it at 256;

@@ -1575,6 +1575,12 @@ static bool rows_applies(const hipq_conv2d_plan *p, const ConvArgs &a)
     return p->variant == kMfma && p->special == 1 && !p->tile_selected && !p->has_wzp && conv_rows_applies(a);
 }
 
+// conv_stem3x3_kernel (conv_stem.hip): 3x3 / stride 2 from an image with at most 4 channels to at most 32
+static bool stem3_applies(const hipq_conv2d_plan *p, const ConvArgs &a)
+{
+    return p->variant == kMfmaSmallC && p->special >= 1 && !p->tile_selected && !p->has_wzp && conv_stem3x3_applies(a, a.rowb);
+}
+
 static void set_mfma_name(hipq_conv2d_plan *p, bool smallc)
 {
     char nm[96];
@@ -1587,6 +1593,8 @@ static void set_mfma_name(hipq_conv2d_plan *p, bool smallc)
         snprintf(nm, sizeof nm, "conv_mfma_i8_expand%s", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
     else if (pointwise_applies(p))
         snprintf(nm, sizeof nm, "conv_mfma_i8_pointwise%s", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
+    else if (smallc && stem3_applies(p, p->args))
+        snprintf(nm, sizeof nm, "conv_mfma_i8_stem3x3");
     else
         snprintf(nm, sizeof nm, "conv_mfma_i8_%dx%d%s%s%s%s", kTiles[p->tile].bm, kTiles[p->tile].bn, smallc ? "_c4" : "",
                  p->has_wzp ? "_wzp" : "", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "",
@@ -1901,11 +1909,11 @@ extern "C" int hipq_conv2d_plan_special(hipq_conv2d_plan *p, int mode)
 {
     clear_error();
     HIPQ_REQUIRE(p, "hipq_conv2d_plan_special: null plan");
-    HIPQ_REQUIRE(p->variant == kMfma, "hipq_conv2d_plan_special: only the DMA-fed MFMA kernel has variants (this plan runs %s)",
-                 p->name.c_str());
+    HIPQ_REQUIRE(p->variant == kMfma || p->variant == kMfmaSmallC,
+                 "hipq_conv2d_plan_special: only the MFMA kernels have variants (this plan runs %s)", p->name.c_str());
     HIPQ_REQUIRE(mode >= 0 && mode <= 2, "hipq_conv2d_plan_special: mode must be 0 (never), 1 (built-in rule) or 2 (wherever they apply)");
     p->special = mode;
-    set_mfma_name(p, false);
+    set_mfma_name(p, p->variant == kMfmaSmallC);
     return 0;
 }
 
@@ -2253,6 +2261,10 @@ static int run_conv(const hipq_conv2d_plan *p, ConvArgs &a, hipStream_t st)
         }
         if (expand_applies(p, a)) {
             launch_conv_expand(a, st); // a channel-widening 1x1 layer: pixel operands in registers, channel tiles in a loop
+            break;
+        }
+        if (stem3_applies(p, a)) {
+            launch_conv_stem3x3(a, st); // 3x3 / stride 2 on an RGB image: the input rows stay in LDS
             break;
         }
         switch (p->tile) {

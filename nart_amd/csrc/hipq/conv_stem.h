@@ -1,4 +1,4 @@
-// The stem convolution fused with its 3x3 / stride 2 / pad 1 max pooling (conv_stem.hip).
+// The stem convolutions (conv_stem.hip): 5 to 8 taps fused with the 3x3 / stride 2 / pad 1 max pooling behind them; 3x3 / stride 2.
 #pragma once
 
 #include "conv_shared.h"
@@ -9,5 +9,9 @@ namespace hipq {
 bool conv_stem_maxpool_applies(const ConvArgs &a, int smallc_rowb);
 // yp: pooled output, NHWC with channel stride 64, POH x POW pixels per image
 void launch_conv_stem_maxpool(const ConvArgs &a, uint8_t *yp, int POH, int POW, hipStream_t st);
+
+// true when conv_stem3x3_kernel serves this convolution: 3x3 / stride 2 from at most 4 to at most 32 channels, no pooling
+bool conv_stem3x3_applies(const ConvArgs &a, int smallc_rowb);
+void launch_conv_stem3x3(const ConvArgs &a, hipStream_t st);
 
 } // namespace hipq

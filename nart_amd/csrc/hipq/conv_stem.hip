@@ -211,4 +211,134 @@ void launch_conv_stem_maxpool(const ConvArgs &a, uint8_t *yp, int POH, int POW, 
     }
 }
 
+
+// ---------------------------------------------------------------------------------------------------------------------
+// A 3x3 / stride 2 stem with no pooling behind it (MobileNet-style: RGB to 32 channels): the same idea, smaller.  Such a
+// layer is all memory traffic (27 multiplies per output byte) and the register-staged tile kernel spends its time
+// gathering taps with per-dword border tests.  Here a work-group owns `rb` output rows of one image; the 2 rb + 1 input
+// rows go into LDS once (one row per load-unit instruction, pad columns and rows outside the image holding the byte
+// izp); k = (kernel row, 4 taps, 4 channels) as the plan packs it for 3-tap rows, so a k-step of 32 bytes is TWO kernel
+// rows - lane (p, h) reads 16 consecutive bytes of input row 2 oh - pad + 2 step + h - and the whole reduction is two
+// multiplies (the fourth kernel row and every fourth tap carry weight zero: whatever bytes stand there count for
+// nothing).  MFMA row i computes channel 16 ((i >> 2) & 1) + 4 (i >> 3) + (i & 3), so the 16 accumulators of a lane are
+// 16 consecutive channels of its pixel and leave as one 128-bit store, a wave writing 1 KB of consecutive bytes.
+// Requirements (checked by the host): uint8 tensors, input channel stride 4, output channel stride 32, 3 x 3, stride 2,
+// horizontal pad at most 4, output rows of at most 128 pixels, image rows of at most 248 pixels (a multiple of 4),
+// weight zero point 128, one scale for all channels.
+constexpr int kStem3MaxRB = 8;                    // output rows per work-group, at most
+constexpr int kStem3PatchRows = 2 * kStem3MaxRB + 2; // + 1 row of the last window, + 1 that only zero weights ever meet
+
+template <bool FAST, bool SAT>
+__global__ __launch_bounds__(256) void conv_stem3x3_kernel(const ConvArgs a, const int nrb, const int rb)
+{
+    constexpr int PITCH = kStemPitch;
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[kStem3PatchRows * PITCH];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int n = (int)blockIdx.x / nrb, oh0 = ((int)blockIdx.x % nrb) * rb;
+    const int nrows = min(rb, a.OH - oh0);
+    const int ir0 = oh0 * 2 - a.pad_h;
+    const int prows = 2 * nrows + 1;
+
+    const int wq = a.W >> 2;
+    for (int j = wave; j < prows; j += 4) {
+        const int ir = ir0 + j;
+        const bool ok = (unsigned)ir < (unsigned)a.H && lane < wq;
+        const uint8_t *src = ok ? a.x + ((size_t)(n * a.H + ir) * a.W) * 4 + lane * 16 : a.padbuf;
+        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(lds + j * PITCH + 16), 16, 0, 0);
+    }
+    if (tid < prows) {
+        const uint32_t pw = a.padword;
+        *reinterpret_cast<u32x4 *>(lds + tid * PITCH) = u32x4{pw, pw, pw, pw};
+    }
+
+    const int half = lane >> 5, p = lane & 31;
+    const int ch = 16 * ((p >> 2) & 1) + 4 * (p >> 3) + (p & 3); // the channel MFMA row p computes
+    v4i wreg[2];
+#pragma unroll
+    for (int ks = 0; ks < 2; ks++)
+        wreg[ks] = ldg128(a.wpack + ch * 64 + (((2 * ks + half) ^ ((ch >> 2) & 3)) << 4));
+    v16i bias;
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        const v4i b = *reinterpret_cast<const v4i *>(a.bias2 + 16 * half + 4 * g);
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+            bias[g * 4 + e] = b[e];
+    }
+    __builtin_amdgcn_s_waitcnt(0); // vmcnt(0), lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+
+    const int px = wave * 32 + p;
+    const int owc = min(px, a.OW - 1); // lanes beyond the row compute a copy that is never stored
+    const uint8_t *bbase = lds + 16 + (owc * 2 - a.pad_w) * 4 + half * PITCH;
+    uint8_t *yrow = a.y + ((size_t)(n * a.OH + oh0) * a.OW + px) * 32 + 16 * half;
+    for (int i = 0; i < nrows; i++) {
+        const uint32_t *b0 = reinterpret_cast<const uint32_t *>(bbase + (2 * i) * PITCH);
+        const uint32_t *b1 = reinterpret_cast<const uint32_t *>(bbase + (2 * i + 2) * PITCH);
+        const v4i bf0 = v4i{(int)b0[0], (int)b0[1], (int)b0[2], (int)b0[3]} ^ (int)a.xmask;
+        const v4i bf1 = v4i{(int)b1[0], (int)b1[1], (int)b1[2], (int)b1[3]} ^ (int)a.xmask;
+        v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[0], bf0, bias, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[1], bf1, acc, 0, 0, 0);
+        u32x4 out;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            if (SAT) { // clamp range exactly [0, 255]: saturating packs instead of clamps
+                int32_t r[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    r[e] = (__mulhi(acc[g * 4 + e], (int)a.q.mult) + a.qadd) >> a.qt;
+                uint32_t p01, p23, b01, b23;
+                asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p01) : "v"(r[0]), "v"(r[1]));
+                asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(r[2]), "v"(r[3]));
+                asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
+                asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
+                out[g] = __builtin_amdgcn_perm(b23, b01, 0x05040100u);
+            } else {
+                out[g] = pack_low_bytes(conv_requant<FAST>(a, acc[g * 4]), conv_requant<FAST>(a, acc[g * 4 + 1]),
+                                        conv_requant<FAST>(a, acc[g * 4 + 2]), conv_requant<FAST>(a, acc[g * 4 + 3]));
+            }
+        }
+        if (px < a.OW)
+            *reinterpret_cast<u32x4 *>(yrow + (size_t)i * a.OW * 32) = out;
+    }
+}
+
+bool conv_stem3x3_applies(const ConvArgs &a, int smallc_rowb)
+{
+    return a.in_cs == 4 && a.out_cs == 32 && a.K <= 32 && a.R == 3 && a.S == 3 && smallc_rowb == 16 && a.stride_h == 2
+        && a.stride_w == 2 && a.pad_w <= 4 && a.OW <= 128 && a.OW >= 1 && a.W % 4 == 0 && a.W <= 248 && a.nslab == 1
+        && a.qmult == nullptr && a.group == 1 && (a.OW - 1) * 2 - a.pad_w + 3 < 256 && a.xmask != 0 && a.bwz == 0
+        && a.res == nullptr && !plain_epilogue(a);
+}
+
+// Output rows per work-group: four work-groups fit a CU, so the grid runs in rounds of 1024; the cost of a choice is its
+// number of rounds times the rows a work-group loads and computes.
+static int stem3_rows_per_wg(int N, int OH)
+{
+    int best = 1;
+    long best_cost = 0;
+    for (int rb = 1; rb <= kStem3MaxRB; rb++) {
+        const long wgs = (long)N * ((OH + rb - 1) / rb);
+        const long cost = ((wgs + 1023) / 1024) * (rb + 2); // + 2: the fixed part of a work-group (loads, weights)
+        if (rb == 1 || cost < best_cost) {
+            best = rb;
+            best_cost = cost;
+        }
+    }
+    return best;
+}
+
+void launch_conv_stem3x3(const ConvArgs &a, hipStream_t st)
+{
+    const int rb = stem3_rows_per_wg(a.N, a.OH), nrb = (a.OH + rb - 1) / rb;
+    const dim3 grid(a.N * nrb), block(256);
+    if (a.fastq && a.lo == 0 && a.q.hi == 255)
+        hipLaunchKernelGGL((conv_stem3x3_kernel<true, true>), grid, block, 0, st, a, nrb, rb);
+    else if (a.fastq)
+        hipLaunchKernelGGL((conv_stem3x3_kernel<true, false>), grid, block, 0, st, a, nrb, rb);
+    else
+        hipLaunchKernelGGL((conv_stem3x3_kernel<false, false>), grid, block, 0, st, a, nrb, rb);
+}
+
 } // namespace hipq

@@ -709,6 +709,7 @@ def test_relu_decided_at_run_time():
     kerns = set()
     #         N, C,  H,  W,  K,  R, pad, stride, group
     shapes = [(2, 64, 12, 12, 64, 3, 1, 1, 1), (1, 64, 9, 9, 48, 3, 1, 1, 1), (1, 32, 9, 9, 96, 1, 0, 1, 1), (2, 256, 7, 7, 128, 1, 0, 1, 1), (1, 3, 20, 20, 32, 3, 1, 2, 1),
+              (1, 3, 20, 20, 32, 3, 1, 1, 1),
               (2, 48, 10, 10, 48, 3, 1, 1, 48), (1, 32, 9, 9, 32, 3, 1, 2, 32), (1, 24, 7, 7, 24, 5, 2, 1, 24), (1, 16, 8, 8, 32, 3, 1, 1, 4)]
     for N, C, H, W, K, R, pad, st, g in shapes:
         x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
@@ -724,6 +725,7 @@ def test_relu_decided_at_run_time():
             assert np.array_equal(hipq.from_device_nhwc(plain.run_relu(xd), K), want), (plain.kernel, obits, ozp)
             assert np.array_equal(hipq.from_device_nhwc(fused(xd), K), want), (fused.kernel, obits, ozp)
     assert any("halo" in k for k in kerns) and any("pointwise" in k for k in kerns) and any("_c4" in k for k in kerns)
+    assert any("stem3x3" in k for k in kerns)
     assert any("depthwise3x3" in k for k in kerns) and "conv_depthwise_u8" in kerns and "conv_direct_u8" in kerns
     p8 = hipq.Conv2d((1, 16, 4, 4), rng.integers(-128, 128, (16, 16, 1, 1), dtype=np.int8), None, 0, 1, 1, 0.1, 0, 0.1, 0, 0.1, 0,
                      dtype=hipq.DTYPE_I8)
@@ -769,6 +771,46 @@ def test_conv3x3_rows_kernel():
         assert plan.kernel == "conv_mfma_i8_rows3x3_signed", plan.kernel
         got = hipq.from_device_nhwc(plan(hipq.to_device_nhwc(x)), 64).view(np.int8)
         assert np.array_equal(got, orc.conv2d_i8(x, w, b, 1, 1, 1, 0.02, 0.004, 2.0, obits=obits)), obits
+
+
+def test_stem3x3_stride2_kernel():
+    """conv_stem3x3_kernel (3x3 / stride 2 from an image with at most 4 channels to at most 32; input rows resident in
+    LDS, two multiplies per 32 pixels x 32 channels) against the oracle and against the tile kernel: with and without
+    padding, odd and even heights, rows shorter than / equal to / a ragged multiple of a wave's 32 pixels, 1 to 3 input
+    channels, 17 to 32 output channels, row blocks that do not divide the height, ReLU, fewer output bits, a
+    scale that takes the 64-bit requantisation; the accumulator dump falls back to the tile kernel."""
+    rng = np.random.default_rng(53)
+    shapes = [(2, 3, 224, 224, 32, 1), (1, 3, 32, 32, 32, 1), (3, 3, 31, 44, 24, 1), (1, 1, 9, 12, 32, 0), (2, 2, 65, 248, 17, 1),
+              (1, 3, 3, 4, 32, 1), (5, 3, 30, 132, 32, 0), (64, 3, 48, 40, 32, 1), (1, 4, 20, 200, 20, 1)]
+    for i, (N, C, H, W, K, pad) in enumerate(shapes):
+        print("stem3x3 case", N, C, H, W, K, pad, flush=True)
+        x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+        w = rng.integers(0, 256, (K, C, 3, 3), dtype=np.uint8)
+        b = rng.integers(-3000, 3000, K).astype(np.int32)
+        ia, wa = rand_q(rng), rand_q(rng)
+        relu, obits = bool(i & 1), (8, 8, 7)[i % 3]
+        # requantisation shifts below 33 (the 64-bit form), in the one-multiply range, and far up in it
+        oa = float(np.float32(ia * wa * (200.0, 2000.0, 3e6)[i % 3]))
+        q = (ia, int(rng.integers(0, 256)), wa, 128, oa, int(rng.integers(0, 1 << obits)))
+        want = orc.conv2d_u8(x, w, b, pad, 2, 1, *q, obits=obits)
+        if relu:
+            want = orc.relu_u8(want, q[4], q[5], q[4], q[5], obits)
+        plan = hipq.Conv2d(x.shape, w, b, pad, 2, 1, *q, relu=relu, obits=obits)
+        assert plan.kernel == "conv_mfma_i8_stem3x3", plan.kernel
+        xd = hipq.to_device_nhwc(x)
+        got = hipq.from_device_nhwc(plan(xd), K)
+        assert np.array_equal(got, want), (N, C, H, W, K, pad, relu, obits, int((got != want).sum()))
+        plan.special(0)
+        assert "stem3x3" not in plan.kernel
+        assert np.array_equal(hipq.from_device_nhwc(plan(xd), K), want)
+    # the accumulators come from the tile kernel (this kernel never writes them); bytes and sums both match
+    x = rng.integers(0, 256, (2, 3, 40, 40), dtype=np.uint8)
+    w = rng.integers(0, 256, (32, 3, 3, 3), dtype=np.uint8)
+    b = rng.integers(-3000, 3000, 32).astype(np.int32)
+    check_conv(x, w, b, 1, 2, 1, (0.02, 7, 0.004, 128, 0.5, 3), "stem3x3 shape with accumulators")
+    # a weight zero point other than 128 stays with the tile kernel
+    plan = hipq.Conv2d(x.shape, w, b, 1, 2, 1, 0.02, 7, 0.004, 120, 0.5, 3)
+    assert "stem3x3" not in plan.kernel
 
 
 def test_conv3x3_halo_kernel_matches_the_streaming_kernel_and_the_oracle():
