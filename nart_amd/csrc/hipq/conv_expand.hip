@@ -360,10 +360,13 @@ bool conv_expand_applies(const ConvArgs &a, bool wherever)
     return a.R == 1 && a.S == 1 && a.pad_h == 0 && a.pad_w == 0 && a.group == 1 && a.bwz == 0
         && (a.in_cs == 64 || a.in_cs == 128 || a.in_cs == 256) && a.nslab == a.in_cs / 64 && a.fastq && !plain_epilogue(a)
         && ntiles >= 4 && ntiles <= kMaxTiles && a.out_cs >= 2 * a.in_cs && a.P >= 1024 && (a.res == nullptr || a.addq.fast)
-        // where it beats the kernels it replaces (batch 64): with the add at 64 input channels (31.7 against 35.7 us at
-        // 64 -> 256 on 200 704 pixels; level at 128 -> 512, behind at 256 -> 1024), without at 256 (16.7 against 19.7 us
-        // at 256 -> 512 on 50 176 pixels; level with the pointwise kernel at 64 -> 256)
-        && (wherever || (a.res != nullptr ? a.in_cs == 64 : a.in_cs == 256));
+        // where it beats the kernels it replaces: with the add at 64 input channels (31.7 against 35.7 us at 64 -> 256
+        // on 200 704 pixels; level at 128 -> 512, behind at 256 -> 1024), without at 256 (16.7 against 19.7 us at
+        // 256 -> 512 on 50 176 pixels; level with the pointwise kernel at 64 -> 256) - and only on many pixels: its grid is
+        // three work-groups per CU whatever the size, a launch of it takes 6.6 us or more, and the tile kernels need
+        // 4 to 7 us up to some 12 000 pixels (256 -> 512: level at 25 000; 64 -> 256 with the add: 19.6 against 18.7 us
+        // at 100 352)
+        && (wherever || (a.res != nullptr ? a.in_cs == 64 && a.P >= 150000 : a.in_cs == 256 && a.P >= 20000));
 }
 
 template <int NSLAB, int MID>
