@@ -138,8 +138,8 @@ int hipq_conv2d_plan_select(hipq_conv2d_plan *plan, int tile, int stages);
  * pixel operands in registers while a work-group walks a contiguous range of 128-pixel x 64-channel output tiles, with
  * the residual add of hipq_conv2d_run_add applied in place on a prefetched residual tile.
  * Rows kernel (name "..._rows3x3"): 3x3 / stride 1 / pad 1 convolutions with an input and output channel stride of 64
- * on rows of at most 64 pixels (weight zero point 128, one-multiply requantisation, no fused add) keep the input rows
- * of a work-group in LDS and all weights in registers.
+ * on rows of at most 64 pixels (weight zero point 128, one-multiply requantisation) keep the input rows of a work-group
+ * in LDS and all weights in registers; the residual add of hipq_conv2d_run_add is applied to the bytes on their way out.
  * 3x3 stem kernel (name "..._stem3x3"): 3x3 / stride 2 convolutions of an image with at most 4 channels (channel stride 4,
  * rows of at most 248 pixels, a multiple of 4) to at most 32 channels (stride 32), weight zero point 128: the input rows
  * of a work-group in LDS, two multiplies per 32 pixels, 128-bit stores straight from the accumulators; modes 1 and 2.

@@ -1874,7 +1874,9 @@ extern "C" const char *hipq_conv2d_plan_kernel_add(const hipq_conv2d_plan *p)
     a.res = a.padbuf; // any non-null pointer: the question is which kernel a launch with a residual goes to
     a.addq.fast = 1;  // the 32-bit form of the add, which ordinary scale ratios allow
     char buf[96];
-    if (expand_applies(p, a))
+    if (rows_applies(p, a))
+        snprintf(buf, sizeof buf, "conv_mfma_i8_rows3x3+add");
+    else if (expand_applies(p, a))
         snprintf(buf, sizeof buf, "conv_mfma_i8_expand%s+add", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
     else
         snprintf(buf, sizeof buf, "conv_mfma_i8_%dx%d%s%s%s%s+add", kTiles[p->tile].bm, kTiles[p->tile].bn,

@@ -19,7 +19,9 @@
 //     (p, h): bytes [32 s + 16 h, +16) of pixel (row + dr, col + ds) - is one 128-bit LDS read, closed-form addressing,
 //     no border tests, no barrier anywhere in the loop; the reads run three steps ahead of the multiplies;
 //   * the 32 x 64 result bytes are transposed through a 2 KB LDS patch private to the wave (no barrier either) and leave
-//     as two 128-bit stores per lane, 2 KB contiguous in memory.
+//     as two 128-bit stores per lane, 2 KB contiguous in memory - after the residual add of hipq_conv2d_run_add
+//     (op_quant_add_run, art/modules/quant/src/op/add.c:116-152) where one is fused: the other operand's bytes are
+//     requested before the requantisation and added to the transposed bytes.
 // Where the time goes (cycle stamps in a throw-away build, 64 x 56 x 56, 7 output rows per work-group, two work-groups
 // per CU, 12 us inside the kernel): 1.9 us until the weights and the first four rows are in LDS, 1.1 us for the eight
 // waves of a CU to read their 36 KB of weights out of it (LDS bandwidth), then 1.7 - 2.1 us per unit and wave against
@@ -43,7 +45,7 @@ static_assert(4 * kRowPitch + kWBytes <= (kMaxRB + 2) * kRowPitch + 4 * kPatch,
               "the weights pass through the space of the rows behind the first four (and of the patches, unused until then)");
 }
 
-template <bool PLAIN_SAT>
+template <bool PLAIN_SAT, bool ADD>
 __global__ __launch_bounds__(256, 2) void conv3x3_c64_rows_kernel(const ConvArgs a, const int nrb, const int rb)
 {
     constexpr int P_OFF = (kMaxRB + 2) * kRowPitch;
@@ -139,6 +141,19 @@ __global__ __launch_bounds__(256, 2) void conv3x3_c64_rows_kernel(const ConvArgs
             acc[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[k >> 1][k & 1][0], bf, acc[0], 0, 0, 0);
             acc[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wreg[k >> 1][k & 1][1], bf, acc[1], 0, 0, 0);
         }
+        uint8_t *yrow = a.y + ((size_t)(n * a.H + r0 + row) * a.W + seg * 32) * 64;
+        // fused residual add: the other operand's bytes for the two 16-byte pieces this lane will store, requested now
+        // and used after the requantisation
+        u32x4 rv[2] = {};
+        if (ADD) {
+            const uint8_t *rrow = a.res + (yrow - a.y);
+#pragma unroll
+            for (int k = 0; k < 2; k++) {
+                const int q = (lane >> 2) + 16 * k, c = lane & 3;
+                if (seg * 32 + q < a.W)
+                    rv[k] = *reinterpret_cast<const u32x4 *>(rrow + q * 64 + c * 16);
+            }
+        }
         // requantise, transpose through the wave's own patch (16-byte piece c of pixel q at piece c ^ (q & 3)), store
 #pragma unroll
         for (int tn = 0; tn < 2; tn++)
@@ -167,13 +182,18 @@ __global__ __launch_bounds__(256, 2) void conv3x3_c64_rows_kernel(const ConvArgs
                 *reinterpret_cast<uint32_t *>(patch + p * 64 + (((ch >> 4) ^ (p & 3)) << 4) + (ch & 15)) = packed;
             }
         __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): the wave's own writes
-        uint8_t *yrow = a.y + ((size_t)(n * a.H + r0 + row) * a.W + seg * 32) * 64;
 #pragma unroll
         for (int k = 0; k < 2; k++) {
             const int q = (lane >> 2) + 16 * k, c = lane & 3; // pixel of the segment, 16-byte piece
-            const v4i v = *reinterpret_cast<const v4i *>(patch + q * 64 + ((c ^ (q & 3)) << 4));
+            u32x4 v = *reinterpret_cast<const u32x4 *>(patch + q * 64 + ((c ^ (q & 3)) << 4));
+            if (ADD) { // exactly what the add operator computes from the convolution's stored bytes
+                if (a.addq.fast)
+                    v = a.res_first ? add_16<true>(rv[k], v, a.addq) : add_16<true>(v, rv[k], a.addq);
+                else
+                    v = a.res_first ? add_16<false>(rv[k], v, a.addq) : add_16<false>(v, rv[k], a.addq);
+            }
             if (seg * 32 + q < a.W)
-                *reinterpret_cast<v4i *>(yrow + q * 64 + c * 16) = v;
+                *reinterpret_cast<u32x4 *>(yrow + q * 64 + c * 16) = v;
         }
         __builtin_amdgcn_s_waitcnt(0xC07F); // the patch is read before the next unit overwrites it
     };
@@ -191,7 +211,7 @@ bool conv_rows_applies(const ConvArgs &a)
 {
     return a.R == 3 && a.S == 3 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 1 && a.pad_w == 1 && a.group == 1
         && a.in_cs == 64 && a.out_cs == 64 && a.K <= 64 && a.nslab == 9 && a.W <= 64 && a.W >= 1 && a.OH == a.H && a.OW == a.W
-        && a.bwz == 0 && a.fastq && !plain_epilogue(a) && a.res == nullptr;
+        && a.bwz == 0 && a.fastq && !plain_epilogue(a);
 }
 
 // Output rows per work-group: two work-groups fit a CU (their registers), so the grid runs in rounds of 512; the cost of
@@ -215,10 +235,17 @@ void launch_conv_rows(const ConvArgs &a, hipStream_t st)
 {
     const int rb = rows_per_wg(a.N, a.H), nrb = (a.H + rb - 1) / rb;
     const dim3 grid(a.N * nrb), block(256);
-    if (a.lo == 0 && a.q.hi == 255)
-        hipLaunchKernelGGL(conv3x3_c64_rows_kernel<true>, grid, block, 0, st, a, nrb, rb);
-    else
-        hipLaunchKernelGGL(conv3x3_c64_rows_kernel<false>, grid, block, 0, st, a, nrb, rb);
+    const bool sat = a.lo == 0 && a.q.hi == 255;
+    if (a.res != nullptr) { // the residual add of hipq_conv2d_run_add applied to the bytes on their way out
+        if (sat)
+            hipLaunchKernelGGL((conv3x3_c64_rows_kernel<true, true>), grid, block, 0, st, a, nrb, rb);
+        else
+            hipLaunchKernelGGL((conv3x3_c64_rows_kernel<false, true>), grid, block, 0, st, a, nrb, rb);
+    } else if (sat) {
+        hipLaunchKernelGGL((conv3x3_c64_rows_kernel<true, false>), grid, block, 0, st, a, nrb, rb);
+    } else {
+        hipLaunchKernelGGL((conv3x3_c64_rows_kernel<false, false>), grid, block, 0, st, a, nrb, rb);
+    }
 }
 
 } // namespace hipq

@@ -768,9 +768,26 @@ def test_conv3x3_rows_kernel():
         xd = hipq.to_device_nhwc(x)
         got = hipq.from_device_nhwc(plan(xd), K)
         assert np.array_equal(got, want), (N, H, W, K, relu, obits, int((got != want).sum()))
+        # the residual add fused into the same kernel, both operand orders, scale ratios that do and do not fit the
+        # add's 32-bit form
+        res = rng.integers(0, 1 << obits, want.shape, dtype=np.uint8)
+        rd = hipq.to_device_nhwc(res)
+        ra, rz = float(np.float32(q[4] * (1.0, 1.7, 300.0)[i % 3])), int(rng.integers(0, 256))
+        sa, sz = float(np.float32(max(q[4], ra) * 1.3)), int(rng.integers(0, 1 << obits))
+        assert plan.kernel_add == "conv_mfma_i8_rows3x3+add", plan.kernel_add
+        for res_first in (False, True):
+            want_sum = (orc.add_u8(res, want, ra, rz, q[4], q[5], sa, sz, obits) if res_first
+                        else orc.add_u8(want, res, q[4], q[5], ra, rz, sa, sz, obits))
+            y = plan.empty_output()
+            plan.run_add(xd, rd, res_first, ra, rz, sa, sz, y, obits=obits)
+            got = hipq.from_device_nhwc(y, K)
+            assert np.array_equal(got, want_sum), (N, H, W, K, relu, obits, res_first, int((got != want_sum).sum()))
         plan.special(0)
-        assert "rows3x3" not in plan.kernel
+        assert "rows3x3" not in plan.kernel and "rows3x3" not in plan.kernel_add
         assert np.array_equal(hipq.from_device_nhwc(plan(xd), K), want)
+        y = plan.empty_output()
+        plan.run_add(xd, rd, True, ra, rz, sa, sz, y, obits=obits)
+        assert np.array_equal(hipq.from_device_nhwc(y, K), want_sum), (N, H, W, K, "tile kernel with the add")
     x = rng.integers(-128, 128, (2, 64, 20, 24), dtype=np.int8)
     w = rng.integers(-127, 128, (64, 64, 3, 3), dtype=np.int8)
     b = rng.integers(-30000, 30000, 64).astype(np.int32)
