@@ -152,9 +152,11 @@ int hipq_conv2d_plan_select(hipq_conv2d_plan *plan, int tile, int stages);
  */
 int hipq_conv2d_plan_special(hipq_conv2d_plan *plan, int mode);
 /*
- * Tuning hook (no counterpart in the reference) for the streaming kernel (name "..._stream_<rows>x<cols>"): 1x1 / stride 1
- * layers over at most 256 pixels whose input rows are multiples of 128 bytes (weight zero point 128, or int8) - in
- * practice the fully-connected layers, op_quant_ip_u8xu8_run (src/op/ip.cpp:133-209), whose pixels are the batch.  They
+ * Tuning hook (no counterpart in the reference) for the streaming kernel (name "..._stream_<rows>x<cols>"): layers over
+ * at most 256 output pixels (1024 where a pixel's reduction is at least 512 bytes long) whose input pixels are multiples
+ * of 128 bytes (weight zero point 128, or int8) - the fully-connected layers, op_quant_ip_u8xu8_run
+ * (src/op/ip.cpp:133-209), whose pixels are the batch, and convolutions of any kernel size, stride and padding over small
+ * images (the late stages of a network at batch 1); hipq_conv2d_run_add fuses the residual add into it.  They
  * are bound by the weight stream, so the output is cut into strips of 16 or 32 channels, one work-group each, whose waves
  * split the reduction and stream their shares through LDS stages of their own into the 16x16x64 MFMA.  rows: pixel rows
  * per work-group (16, 32, 64 or 128), cols: 16 or 32 (128 x 32 does not exist), waves: 4; 0, 0, 0 returns to the built-in rule (one strip

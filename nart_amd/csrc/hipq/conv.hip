@@ -1066,7 +1066,10 @@ struct StreamCfg {
     static_assert(R >= 2 && (R - 1) * PER <= 63, "stage count / vmcnt range");
 };
 
-template <int MB, int NB>
+// CONVX: any kernel size, stride and padding (a convolution over few pixels - the last stages of a network at batch 1 -
+// is the same weight stream): chunk c of a pixel's reduction is 128 bytes of the channels of ONE tap, read from the
+// neighbouring pixel that tap points at, or from the pad source where it points outside the image.
+template <int MB, int NB, bool CONVX>
 __global__ __launch_bounds__(256) void conv_mfma_stream_kernel(const ConvArgs a, const int mtiles)
 {
     using Cfg = StreamCfg<MB, NB>;
@@ -1099,14 +1102,39 @@ __global__ __launch_bounds__(256) void conv_mfma_stream_kernel(const ConvArgs a,
     const int xrow = lane >> 3, xoff = ((lane & 7) ^ xrow) << 4;
     const uint8_t *wsrc = a.wpack + (size_t)n0 * 64 + lane * 16;
     const size_t wslab = (size_t)a.kout_pad * 64;
+    // CONVX: this lane's pixel of load j - first input row and column of its window, pixel index of its image's origin
+    int wih[CONVX ? XI : 1], wiw[CONVX ? XI : 1], wpix[CONVX ? XI : 1];
+    if (CONVX) {
+        const int ohw = a.OH * a.OW;
+#pragma unroll
+        for (int j = 0; j < XI; j++) {
+            const int m = min(m0 + 8 * j + xrow, a.P - 1);
+            const int n = fast_div(m, ohw, a.inv_ohw), rem = m - n * ohw;
+            const int oh = fast_div(rem, a.OW, a.inv_ow), ow = rem - oh * a.OW;
+            wih[j] = oh * a.stride_h - a.pad_h, wiw[j] = ow * a.stride_w - a.pad_w, wpix[j] = n * a.H * a.W;
+        }
+    }
+    const int cpt = a.in_cs >> 7; // chunks per tap
     auto issue = [&](int t) {
         const int chunk = chunk_of(t);
         uint8_t *st = wl + (t % R) * STAGE;
+        if (CONVX) {
+            const int tap = chunk / cpt, coff = (chunk - tap * cpt) * 128 + xoff;
+            const int kr = tap / a.S, ks = tap - kr * a.S;
 #pragma unroll
-        for (int j = 0; j < XI; j++) {
-            const int m = min(m0 + 8 * j + xrow, a.P - 1); // rows beyond the last pixel repeat it; their results are dropped
-            const uint8_t *src = a.x + (uint32_t)(m * a.in_cs + chunk * 128 + xoff);
-            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(st + j * 1024 + ((j + 1) >> 1) * 128), 16, 0, 0);
+            for (int j = 0; j < XI; j++) {
+                const int ih = wih[j] + kr, iw = wiw[j] + ks;
+                const bool ok = (unsigned)ih < (unsigned)a.H && (unsigned)iw < (unsigned)a.W;
+                const uint8_t *src = ok ? a.x + (uint32_t)((wpix[j] + ih * a.W + iw) * a.in_cs + coff) : a.padbuf + (xoff & 48);
+                __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(st + j * 1024 + ((j + 1) >> 1) * 128), 16, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < XI; j++) {
+                const int m = min(m0 + 8 * j + xrow, a.P - 1); // rows beyond the last pixel repeat it; their results are dropped
+                const uint8_t *src = a.x + (uint32_t)(m * a.in_cs + chunk * 128 + xoff);
+                __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(st + j * 1024 + ((j + 1) >> 1) * 128), 16, 0, 0);
+            }
         }
 #pragma unroll
         for (int h = 0; h < 2; h++)
@@ -1197,7 +1225,12 @@ __global__ __launch_bounds__(256) void conv_mfma_stream_kernel(const ConvArgs a,
 #pragma unroll
         for (int e = 0; e < 4; e++)
             rq[e] = a.qmult ? conv_requant_ch(a, v[e], ko + e) : a.fastq ? conv_requant<true>(a, v[e]) : conv_requant<false>(a, v[e]);
-        *reinterpret_cast<uint32_t *>(a.y + (size_t)m * a.out_cs + ko) = pack_low_bytes(rq[0], rq[1], rq[2], rq[3]);
+        uint32_t packed = pack_low_bytes(rq[0], rq[1], rq[2], rq[3]);
+        if (a.res) { // fused residual add: exactly what the add operator computes from the convolution's stored bytes
+            const uint32_t rv = *reinterpret_cast<const uint32_t *>(a.res + (size_t)m * a.out_cs + ko);
+            packed = a.res_first ? add_dword<false>(rv, packed, a.addq) : add_dword<false>(packed, rv, a.addq);
+        }
+        *reinterpret_cast<uint32_t *>(a.y + (size_t)m * a.out_cs + ko) = packed;
     }
 }
 
@@ -1526,8 +1559,8 @@ static bool pointwise_applies(const hipq_conv2d_plan *p)
 constexpr int kCUs = 256;
 static bool k2_applies(const hipq_conv2d_plan *p);
 
-// conv_mfma_stream_kernel: 1x1 / stride 1 layers over at most 256 pixels (fully-connected layers: the pixels are the
-// batch) whose rows are whole 128-byte lines, weight zero point 128 (or int8).  Shape of a work-group's share: 16 * mb
+// conv_mfma_stream_kernel: layers over at most 256 pixels (fully-connected layers: the pixels are the batch; the last
+// stages of a network at batch 1) whose pixels are whole 128-byte lines, weight zero point 128 (or int8).  Shape of a work-group's share: 16 * mb
 // pixel rows by 16 * nb output channels.  A strip that holds every pixel row reads each weight byte once; two m-tiles
 // per strip halve the pixel bytes a CU pulls through its L1 (what bounds the kernel once the weights stream at full
 // rate) and read the weights twice, the second time from L2.
@@ -1535,8 +1568,11 @@ static bool stream_applies(const hipq_conv2d_plan *p, StreamShape *shape = nullp
 {
     const hipq_conv2d_desc &d = p->d;
     const ConvArgs &a = p->args;
-    if (!(p->special && !p->tile_selected && p->variant == kMfma && !p->has_wzp && d.R == 1 && d.S == 1 && d.stride_h == 1
-          && d.stride_w == 1 && d.pad_h == 0 && d.pad_w == 0 && d.in_cs % 128 == 0 && a.P <= 256))
+    // up to 256 pixels whatever the layer; up to 1024 where the reduction is at least 512 bytes long (measured against the
+    // tile kernels: 3x3 on 784 pixels 4.8 against 7.0 us at 128 channels, 6.2 against 10.7 at 256, 12.3 against 18.4 at
+    // 512; 1x1 1024 -> 256 on 784 pixels 3.9 against 6.3; behind from 1568 pixels on, and at 256 -> 1024 from 392)
+    if (!(p->special && !p->tile_selected && p->variant == kMfma && !p->has_wzp && d.in_cs % 128 == 0
+          && (a.P <= 256 || (a.P <= 1024 && d.R * d.S * d.in_cs >= 512)) && (long long)d.N * d.H * d.W * d.in_cs < (1ll << 31)))
         return false;
     if (shape) {
         if (p->stream.mb) {
@@ -1875,7 +1911,10 @@ extern "C" const char *hipq_conv2d_plan_kernel_add(const hipq_conv2d_plan *p)
     a.res = a.padbuf; // any non-null pointer: the question is which kernel a launch with a residual goes to
     a.addq.fast = 1;  // the 32-bit form of the add, which ordinary scale ratios allow
     char buf[96];
-    if (rows_applies(p, a))
+    StreamShape ss;
+    if (stream_applies(p, &ss))
+        snprintf(buf, sizeof buf, "conv_mfma_i8_stream_%dx%d%s+add", 16 * ss.mb, 16 * ss.nb, p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
+    else if (rows_applies(p, a))
         snprintf(buf, sizeof buf, "conv_mfma_i8_rows3x3+add");
     else if (expand_applies(p, a))
         snprintf(buf, sizeof buf, "conv_mfma_i8_expand%s+add", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
@@ -2049,14 +2088,18 @@ static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_
     if (p->variant == kMfma && launch_halo<BM, BN, WM, WN>(p, a, grid, st))
         return;
     StreamShape ss;
-    if (a.res == nullptr && stream_applies(p, &ss)) {
+    if (stream_applies(p, &ss)) {
+        const bool fc = a.R == 1 && a.S == 1 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 0 && a.pad_w == 0;
         const int mtiles = (a.P + 16 * ss.mb - 1) / (16 * ss.mb), ntiles = (a.out_cs + 16 * ss.nb - 1) / (16 * ss.nb);
         const dim3 sgrid((ntiles + 7) / 8 * 8 * mtiles);
         const int key = ss.mb * 100 + ss.nb * 10 + ss.nw;
         switch (key) {
 #define HIPQ_STREAM_CASE(MB_, NB_)                                                                                       \
     case MB_ * 100 + NB_ * 10 + 4:                                                                                      \
-        hipLaunchKernelGGL((conv_mfma_stream_kernel<MB_, NB_>), sgrid, dim3(256), 0, st, a, mtiles);                    \
+        if (fc)                                                                                                         \
+            hipLaunchKernelGGL((conv_mfma_stream_kernel<MB_, NB_, false>), sgrid, dim3(256), 0, st, a, mtiles);         \
+        else                                                                                                            \
+            hipLaunchKernelGGL((conv_mfma_stream_kernel<MB_, NB_, true>), sgrid, dim3(256), 0, st, a, mtiles);          \
         return;
             HIPQ_STREAM_CASE(8, 1)
             HIPQ_STREAM_CASE(4, 2)

@@ -394,6 +394,42 @@ def test_fc_streaming_kernel():
         hipq.Conv2d((4, 128, 1, 1), np.zeros((16, 128, 1, 1), np.uint8), None, 0, 1, 1, 0.1, 0, 0.1, 128, 0.1, 0).stream(128, 32, 4)
 
 
+def test_streaming_kernel_on_convolutions_over_few_pixels():
+    """conv_mfma_stream_kernel with the general pixel gather: any kernel size, stride and padding over at most 256 output
+    pixels (1024 for long reductions) whose channels are whole 128-byte lines (the late stages of a network at batch 1), accumulators and
+    bytes against the oracle; with the residual add fused, both operand orders; special(0) gives the same bytes."""
+    rng = np.random.default_rng(91)
+    cases = [  # N, C, H, W, K, R, pad, stride
+        (1, 512, 7, 7, 512, 3, 1, 1), (1, 256, 14, 14, 512, 3, 1, 2), (1, 256, 14, 14, 256, 3, 1, 1), (2, 128, 9, 9, 64, 3, 1, 1),
+        (1, 128, 5, 7, 40, 5, 2, 1), (1, 256, 14, 14, 512, 1, 0, 2), (3, 128, 6, 5, 136, 3, 0, 1), (1, 384, 16, 16, 96, 3, 1, 1),
+        (1, 128, 28, 28, 128, 3, 1, 1), (3, 512, 17, 19, 72, 1, 0, 1),  # 257 to 1024 pixels: reductions of 512 bytes or more
+    ]
+    for i, (N, C, H, W, K, R, pad, st) in enumerate(cases):
+        x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+        w = rng.integers(0, 256, (K, C, R, R), dtype=np.uint8)
+        b = rng.integers(-30000, 30000, K).astype(np.int32)
+        ia, wa = rand_q(rng), rand_q(rng)
+        q = (ia, int(rng.integers(0, 256)), wa, 128, float(np.float32(ia * wa * np.sqrt(C * R * R) * 40.0)), int(rng.integers(0, 256)))
+        kern = check_conv(x, w, b, pad, st, 1, q, tag="stream conv %d" % i)
+        assert "_stream_" in kern, kern
+        plan = hipq.Conv2d(x.shape, w, b, pad, st, 1, *q)
+        conv = orc.conv2d_u8(x, w, b, pad, st, 1, *q)
+        xd = hipq.to_device_nhwc(x)
+        res = rng.integers(0, 256, conv.shape, dtype=np.uint8)
+        rd = hipq.to_device_nhwc(res)
+        ra, rz = float(np.float32(q[4] * (1.0, 1.7, 300.0)[i % 3])), int(rng.integers(0, 256))
+        sa, sz = float(np.float32(max(q[4], ra) * 1.3)), int(rng.integers(0, 256))
+        assert "_stream_" in plan.kernel_add and plan.kernel_add.endswith("+add"), plan.kernel_add
+        for res_first in (False, True):
+            want = orc.add_u8(res, conv, ra, rz, q[4], q[5], sa, sz) if res_first else orc.add_u8(conv, res, q[4], q[5], ra, rz, sa, sz)
+            y = plan.empty_output()
+            plan.run_add(xd, rd, res_first, ra, rz, sa, sz, y)
+            assert np.array_equal(hipq.from_device_nhwc(y, K), want), (i, res_first, plan.kernel_add)
+        plan.special(0)
+        assert "_stream_" not in plan.kernel
+        assert np.array_equal(hipq.from_device_nhwc(plan(xd), K), conv), (i, plan.kernel)
+
+
 def test_output_stride_wider_than_the_channels():
     """A caller may write a convolution's output into a buffer with a wider channel stride than the layout rule gives
     (hipq_conv2d_desc.out_cs): the packed weights and folded constants cover every output-channel tile of that stride."""
@@ -1050,7 +1086,9 @@ def test_two_group_kernel_matches_the_oracle():
         plan = hipq.Conv2d(x.shape, w, b, pad, stride, 1, *q)
         nslab = (R * R * plan.desc.in_cs + 63) // 64
         eligible = nslab % 2 == 0 and nslab >= 8
-        stream = H * W == 1  # the fully-connected shape goes to the streaming kernel unless a tile is named
+        # few pixels of whole 128-byte lines go to the streaming kernel unless a tile is named
+        npix = N * plan.OH * plan.OW
+        stream = plan.desc.in_cs % 128 == 0 and (npix <= 256 or (npix <= 1024 and R * R * plan.desc.in_cs >= 512))
         assert ("_stream_" in plan.kernel) == stream
         assert plan.kernel.endswith("_k2") == (eligible and not stream), (plan.kernel, nslab)  # every case has at most 256 tiles of the rule's own tile
         xd = hipq.to_device_nhwc(x)
