@@ -185,6 +185,15 @@ int hipq_conv2d_run(const hipq_conv2d_plan *plan, const void *x, void *y, int32_
 int hipq_conv2d_run_relu(const hipq_conv2d_plan *plan, const void *x, void *y, void *stream);
 
 /*
+ * A fully-connected layer followed by the dequantize that reads it, in one launch: op_quant_ip_u8xu8_run
+ * (art/modules/quant/src/op/ip.cpp:133-209), then op_dequantize_run (src/op/dequantize.c:110-136) on its bytes -
+ * y[n][k] = (byte - ozp) * oalpha as float32, N x K dense; the uint8 output itself is not written.  Serves uint8 plans
+ * whose output is one pixel per image and that run the streaming kernel; hipq_conv2d_dequant_fusable returns 1 for
+ * those, given the dequantize's own scale and zero point (they must equal the plan's output parameters).
+ */
+int hipq_conv2d_dequant_fusable(const hipq_conv2d_plan *plan, float alpha, int zp);
+int hipq_conv2d_run_dequant(const hipq_conv2d_plan *plan, const void *x, float *y, void *stream);
+/*
  * Convolution with the residual add fused into its epilogue: y = add(conv(x), residual), bit-identical to
  * hipq_conv2d_run followed by hipq_add_u8 on the stored bytes (op_conv_2d_u8xu8_run, then op_quant_add_run —
  * src/op/add.c:83-148), but the convolution's own uint8 result never travels to memory.  `residual` has the

@@ -1225,6 +1225,13 @@ __global__ __launch_bounds__(256) void conv_mfma_stream_kernel(const ConvArgs a,
 #pragma unroll
         for (int e = 0; e < 4; e++)
             rq[e] = a.qmult ? conv_requant_ch(a, v[e], ko + e) : a.fastq ? conv_requant<true>(a, v[e]) : conv_requant<false>(a, v[e]);
+        if (a.deq_out != nullptr) { // fused dequantize (op_dequantize_run, art/modules/quant/src/op/dequantize.c:110-136)
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                if (ko + e < a.K)
+                    a.deq_out[(size_t)m * a.K + ko + e] = __fmul_rn((float)(rq[e] - a.q.zp), a.deq_alpha);
+            continue;
+        }
         uint32_t packed = pack_low_bytes(rq[0], rq[1], rq[2], rq[3]);
         if (a.res) { // fused residual add: exactly what the add operator computes from the convolution's stored bytes
             const uint32_t rv = *reinterpret_cast<const uint32_t *>(a.res + (size_t)m * a.out_cs + ko);
@@ -2187,6 +2194,29 @@ extern "C" int hipq_conv2d_run_relu(const hipq_conv2d_plan *p, const void *x, vo
     a.y = static_cast<uint8_t *>(y);
     a.acc_out = nullptr;
     a.lo = std::min(p->d.ozp, a.q.hi); // what plan creation sets for relu = 1
+    return run_conv(p, a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int hipq_conv2d_dequant_fusable(const hipq_conv2d_plan *p, float alpha, int zp)
+{
+    if (!p || p->variant != kMfma || p->d.dtype != HIPQ_DTYPE_U8 || p->args.OH * p->args.OW != 1 || p->args.qmult != nullptr)
+        return 0;
+    // the dequantize must read the bytes with the scale and zero point they are written with
+    return stream_applies(p) && alpha == p->d.oalpha && zp == p->d.ozp ? 1 : 0;
+}
+
+extern "C" int hipq_conv2d_run_dequant(const hipq_conv2d_plan *p, const void *x, float *y, void *stream)
+{
+    clear_error();
+    HIPQ_REQUIRE(p && x && y, "hipq_conv2d_run_dequant: null argument");
+    HIPQ_REQUIRE(hipq_conv2d_dequant_fusable(p, p->d.oalpha, p->d.ozp),
+                 "hipq_conv2d_run_dequant: only fully-connected uint8 plans on the streaming kernel (this plan runs %s)", p->name.c_str());
+    ConvArgs a = p->args;
+    a.x = static_cast<const uint8_t *>(x);
+    a.y = nullptr; // never written
+    a.acc_out = nullptr;
+    a.deq_out = y;
+    a.deq_alpha = p->d.oalpha;
     return run_conv(p, a, static_cast<hipStream_t>(stream));
 }
 

@@ -47,6 +47,10 @@ struct ConvArgs {
     const uint8_t *res; // fused residual add: the other operand (same layout as y), or nullptr
     int res_first;      // 1: the residual is input 0 of the add, the convolution's output input 1
     AddParams addq;
+    // fused dequantize (streaming kernel only): the float value of every output byte, (byte - zero point) * deq_alpha, goes
+    // to deq_out[pixel][K] and the bytes themselves are not written; nullptr = off
+    float *deq_out;
+    float deq_alpha;
 };
 
 // x / d for 0 <= x < 2^31, d >= 1, inv = 1.0 / d: the double product is within one of the quotient, one

@@ -93,7 +93,7 @@ typedef std::map<const mem_t *, std::set<const op_t *>> reader_map;
 
 // keyed by workspace (the runtime is single-threaded, art/include/art/workspace.h has no locking either)
 std::map<const workspace_t *, reader_map> g_readers;
-long g_fused_adds = 0, g_fused_relus = 0, g_fused_pools = 0, g_chained_convs = 0; // fused launches so far (hip_module_fused_*)
+long g_fused_adds = 0, g_fused_relus = 0, g_fused_pools = 0, g_chained_convs = 0, g_fused_dequants = 0; // fused launches so far (hip_module_fused_*)
 
 reader_map &readers_of(op_t *op) { return g_readers[op->workspace]; }
 
@@ -187,6 +187,8 @@ void conv_launch_plain(void *ctx)
 }
 
 bool eltwise_is_plain_sum(const op_t *op); // two inputs, SUM, unit coefficients: computes what add computes
+// a dequantize that the fully-connected layer's kernel can compute in its epilogue (hipq_conv2d_dequant_fusable)
+bool dequantize_fuses_with(const op_t *deq_op, const hipq_conv2d_plan *plan);
 // a max pooling that the stem convolution's kernel can compute as well (hipq_conv2d_maxpool_fusable)
 bool pool_fuses_with(const op_t *pool_op, const hipq_conv2d_plan *plan);
 // the convolution `op` as the tail of the kernel that computes the add it reads (hipq_conv2d_run_add_conv); y: where its
@@ -211,6 +213,8 @@ bool sole_reader_fuses(op_t *op)
         return true; // any plan runs with the ReLU clamp (hipq_conv2d_run_relu)
     if (r->entry->tp == &op_pool_tp)
         return pool_fuses_with(r, c->plan);
+    if (r->entry->tp == &op_hip_dequantize_tp)
+        return dequantize_fuses_with(r, c->plan);
     // hipq_conv2d_run_add exists for the MFMA plans
     return (r->entry->tp == &op_add_tp || eltwise_is_plain_sum(r)) && r->input_size == 2
         && r->input_tensors[0]->mem != r->input_tensors[1]->mem && strncmp(hipq_conv2d_plan_kernel(c->plan), "conv_mfma", 9) == 0;
@@ -930,10 +934,28 @@ void dequantize_config(op_t *op)
     HIPM_CHECK(op_setting_single_get(op, SETTING_QUANT_QTYPE, dtINT32, &q->qtype));
 }
 
+bool dequantize_fuses_with(const op_t *deq_op, const hipq_conv2d_plan *plan)
+{
+    const qdq_op_t *q = reinterpret_cast<const qdq_op_t *>(deq_op);
+    return qdq_row(q->qtype << 8 | q->q.bits[0]) == 1 && hipq_conv2d_dequant_fusable(plan, q->q.alpha[0], q->q.zp[0]) != 0;
+}
+
 void dequantize_run(op_t *op)
 {
     qdq_op_t *q = reinterpret_cast<qdq_op_t *>(op);
-    const hip_mem_t *x = as_hip(op->input_tensors[0]->mem);
+    hip_mem_t *xm = as_hip(op->input_tensors[0]->mem);
+    if (xm->pending == conv_launch_plain) {
+        // a fully-connected layer left its launch to this operator (conv_run): one kernel computes the layer and writes
+        // the float values; the layer's own bytes stay unwritten, its hook stays for whoever asks for them
+        op_t *cop = static_cast<op_t *>(xm->pending_ctx);
+        conv_op_t *c = reinterpret_cast<conv_op_t *>(cop);
+        if (dequantize_fuses_with(op, c->plan)
+            && hipq_conv2d_run_dequant(c->plan, in_ptr(cop, 0), static_cast<float *>(out_ptr(op)), op_stream(op)) == 0) {
+            ++g_fused_dequants;
+            return;
+        }
+    }
+    const hip_mem_t *x = xm;
     if (qdq_row(q->qtype << 8 | q->q.bits[0]) == 2) // chosen from the settings, not from the tensor's dtype (dequantize.c:141-163)
         HIPM_HIPQ(hipq_dequantize_i8(in_ptr(op, 0), static_cast<float *>(out_ptr(op)), x->N, x->C, x->H, x->W, x->cs,
                                      q->q.alpha[0], op_stream(op)));
@@ -1007,6 +1029,7 @@ ART_PUBLIC long hip_module_fused_adds(void) { return g_fused_adds; }
 ART_PUBLIC long hip_module_fused_relus(void) { return g_fused_relus; }
 ART_PUBLIC long hip_module_fused_pools(void) { return g_fused_pools; }
 ART_PUBLIC long hip_module_chained_convs(void) { return g_chained_convs; }
+ART_PUBLIC long hip_module_fused_dequants(void) { return g_fused_dequants; }
 
 ART_PUBLIC void *hip_workspace_stream(workspace_t *w) { return reinterpret_cast<hip_workspace_t *>(w)->stream; }
 

@@ -45,6 +45,8 @@ _SIGS = {
     "hipq_conv2d_plan_destroy": (None, [C.c_void_p]),
     "hipq_conv2d_plan_kernel": (C.c_char_p, [C.c_void_p]),
     "hipq_conv2d_plan_kernel_add": (C.c_char_p, [C.c_void_p]),
+    "hipq_conv2d_dequant_fusable": (C.c_int, [C.c_void_p, C.c_float, C.c_int]),
+    "hipq_conv2d_run_dequant": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]),
     "hipq_conv2d_plan_select": (C.c_int, [C.c_void_p, C.c_int, C.c_int]),
     "hipq_conv2d_plan_special": (C.c_int, [C.c_void_p, C.c_int]),
     "hipq_conv2d_plan_stream": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_int]),
@@ -191,6 +193,17 @@ class Conv2d:
         check(lib().hipq_conv2d_plan_select(self.handle, tile, stages))
         self.kernel = lib().hipq_conv2d_plan_kernel(self.handle).decode()
         return self
+
+    def dequant_fusable(self, alpha, zp):
+        """True if run_dequant serves this plan and a dequantize with these settings (include/hipq.h)."""
+        return bool(lib().hipq_conv2d_dequant_fusable(self.handle, float(alpha), int(zp)))
+
+    def run_dequant(self, x, y):
+        """The layer and the dequantize of its output in one launch: y (float32, N x K) receives the values."""
+        import torch
+        assert y.dtype == torch.float32 and y.is_contiguous() and y.numel() == self.desc.N * self.desc.K
+        check(lib().hipq_conv2d_run_dequant(self.handle, _ptr(x), _ptr(y), _stream()))
+        return y
 
     def special(self, mode=1):
         """Tuning hook: the halo-tile (3x3 stride 1), pointwise (small 1x1) and two-group (few tiles, long reduction)

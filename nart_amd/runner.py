@@ -36,6 +36,7 @@ class HipqExecutor:
                         and not any(a is u[0] for a in self.fused.values())):  # one convolution per add
                     self.fused[node.output] = u[0]  # launched at the add's position: both operands exist by then
         self.pooled = {}     # conv output name -> the max-pooling node computed inside the convolution's kernel
+        self.dequantized = {}  # fully-connected output name -> the dequantize node computed in the layer's epilogue
         self.chained = {}    # add output name -> the 1x1 convolution node computed inside the fused add's kernel
         self._early = {}     # id(conv node) -> its plan, created ahead of its turn (when an add looked at it)
         self._pending = {}   # id(add node) -> the deferred convolution
@@ -69,6 +70,11 @@ class HipqExecutor:
             if node.kind == "quantize":
                 fn = (lambda i=ins[0], o=out, y=y: hipq.quantize_u8(i, o, y.alpha, y.zp))
                 self._add(node, "quantize_u8_kernel", fn, 0, 5 * int(np.prod(y.shape)))
+            elif node.kind == "dequantize" and id(node) in self._pending:
+                plan, xin, ops, nbytes, xname = self._pending.pop(id(node))
+                fn = (lambda p=plan, i=xin, o=out: p.run_dequant(i, o))
+                self.steps.append({"label": node.output, "kind": "ip+dequantize", "kernel": plan.kernel + "+dequantize", "fn": fn,
+                                   "ops": ops, "bytes": nbytes, "plan": plan})
             elif node.kind == "dequantize":
                 x = xs[0]
                 fn = (lambda i=ins[0], o=out, x=x: hipq.dequantize_u8(i, o, x.alpha, x.zp))
@@ -117,9 +123,18 @@ class HipqExecutor:
                 plan = hipq.Conv2d((Nn, kd, 1, 1), w.reshape(a["K"], kd, 1, 1), case.weights[a["b"]], 0, 1, 1, x.alpha,
                                    x.zp, a["walpha"], a["wzp"], y.alpha, y.zp, in_cs=kd)
                 self.plans.append(plan)
+                ip_ops = 2 * Nn * a["K"] * Cc * Hh * Ww
+                ip_bytes = Nn * Cc * Hh * Ww + Nn * a["K"] + a["K"] * Cc * Hh * Ww + 4 * a["K"]
+                u = [nd for nd in case.nodes if node.output in nd.inputs]
+                if (fuse_add and len(u) == 1 and u[0].kind == "dequantize" and node.output != case.output.name
+                        and plan.dequant_fusable(y.alpha, y.zp)):
+                    # the dequantize that reads the layer runs in its epilogue (hipq_conv2d_run_dequant); the bytes are never written
+                    self.dequantized[node.output] = u[0]
+                    self._pending[id(u[0])] = (plan, ins[0], ip_ops, ip_bytes + 3 * Nn * a["K"], node.inputs[0])
+                    self.buf.pop(y.name, None)
+                    continue
                 fn = (lambda p=plan, i=ins[0], o=out: p(i, o))
-                self._add(node, plan.kernel, fn, 2 * Nn * a["K"] * Cc * Hh * Ww,
-                          Nn * Cc * Hh * Ww + Nn * a["K"] + a["K"] * Cc * Hh * Ww + 4 * a["K"])
+                self._add(node, plan.kernel, fn, ip_ops, ip_bytes)
             elif node.kind == "pool" and id(node) in self._pending:
                 plan, xin, nbytes = self._pending.pop(id(node))
                 fn = (lambda p=plan, i=xin, o=out: p.run_maxpool(i, o))
@@ -187,7 +202,7 @@ class HipqExecutor:
     @property
     def elided(self):
         """Names of the tensors that are never materialised (absorbed into a fused kernel)."""
-        return set(self.fused) | set(self.pooled)
+        return set(self.fused) | set(self.pooled) | set(self.dequantized)
 
     def set_input(self, x):
         inp = self.case.input

@@ -382,9 +382,17 @@ def test_fc_streaming_kernel():
             y2 = plan(xd).cpu().numpy().reshape(M, -1)
             assert np.array_equal(y2[:, :No], want_y), (M, Kd, No, rows, cols, waves)
         plan.stream()
+        # the dequantize that reads the layer, in the layer's epilogue (hipq_conv2d_run_dequant): the float bit patterns of
+        # op_dequantize_run on the layer's bytes; refused for another scale or zero point than the bytes are written with
+        assert plan.dequant_fusable(q[4], q[5]) and not plan.dequant_fusable(float(np.float32(q[4] * 1.5)), q[5])
+        assert not plan.dequant_fusable(q[4], (q[5] + 1) % 256)
+        yf = torch.full((M, No), 7.0, dtype=torch.float32, device="cuda")
+        plan.run_dequant(xd, yf)
+        want_f = orc.dequantize_u8(want_y, q[4], q[5])
+        assert np.array_equal(yf.cpu().numpy().view(np.uint32), np.ascontiguousarray(want_f).reshape(M, No).view(np.uint32)), (M, Kd, No)
         # the tile kernels serve the same plan when the streaming kernel is switched off, with the same bytes
         plan.special(0)
-        assert "_stream_" not in plan.kernel
+        assert "_stream_" not in plan.kernel and not plan.dequant_fusable(q[4], q[5])
         y3 = plan(xd).cpu().numpy().reshape(M, -1)
         assert np.array_equal(y3[:, :No], want_y), (M, Kd, No, plan.kernel)
         plan.close()

@@ -313,6 +313,39 @@ def test_convolution_and_relu_run_as_one_kernel(own_rt):
     ws.delete()
 
 
+def test_fully_connected_layer_and_dequantize_run_as_one_kernel(own_rt):
+    """A fully-connected layer whose output only a dequantize reads leaves its launch to that operator: one kernel computes
+    the layer and writes the float values (op_dequantize_run on the layer's bytes, bit for bit); the layer's own bytes are
+    computed when somebody asks for them.  A dequantize with another scale runs as an operator of its own."""
+    import ctypes as C
+    from oracle import orc
+    fused = own_rt.libs[1].hip_module_fused_dequants
+    fused.restype = C.c_long
+    ws = own_rt.workspace("hip")
+    rng = np.random.default_rng(29)
+    x = rng.integers(0, 256, (6, 256), dtype=np.uint8)
+    w = rng.integers(0, 256, (37, 256), dtype=np.uint8)
+    b = rng.integers(-5000, 5000, 37).astype(np.int32)
+    q = dict(ialpha=0.02, izp=121, walpha=0.004, wzp=128, oalpha=0.35, ozp=100)
+    want_ip = orc.ip_u8(x, w, b, 0.02, 121, 0.004, 128, 0.35, 100)
+    assert len(np.unique(want_ip)) > 8
+    for alpha, expect in ((0.35, 1), (0.36, 0)):
+        tx = ws.tensor(x)
+        ip = ws.ip(tx, ws.tensor(w), ws.tensor(b), q).prepare()
+        dq = ws.dequantize(ip.output(0), alpha, 100).prepare()
+        want = orc.dequantize_u8(want_ip, alpha, 100)
+        n0 = fused()
+        for _ in range(2):
+            ip.run()
+            dq.run()
+            assert same_bits(dq.output(0).numpy().reshape(6, 37), np.ascontiguousarray(want).reshape(6, 37)), alpha
+        assert fused() == n0 + 2 * expect
+        assert same_bits(ip.output(0).numpy().reshape(6, 37), want_ip)  # elided when fused: computed now
+        for o in (dq, ip):
+            o.delete()
+    ws.delete()
+
+
 def test_stem_convolution_relu_and_max_pooling_run_as_one_kernel(own_rt):
     """conv_2d (3 channels, 7x7, stride 2) -> relu -> max pooling 3x3 / 2 / 1 with equal scales: the relu passes the
     convolution's launch on to the pooling, which runs all three in the convolution's kernel (no relu in between: the
