@@ -186,7 +186,7 @@ int hipq_conv2d_run_relu(const hipq_conv2d_plan *plan, const void *x, void *y, v
 
 /*
  * A fully-connected layer followed by the dequantize that reads it, in one launch: op_quant_ip_u8xu8_run
- * (art/modules/quant/src/op/ip.cpp:133-209), then op_dequantize_run (src/op/dequantize.c:110-136) on its bytes -
+ * (art/modules/quant/src/op/ip.cpp:133-209), then op_dequantize_run_u8 (src/op/dequantize.c:111-123) on its bytes -
  * y[n][k] = (byte - ozp) * oalpha as float32, N x K dense; the uint8 output itself is not written.  Serves uint8 plans
  * whose output is one pixel per image and that run the streaming kernel; hipq_conv2d_dequant_fusable returns 1 for
  * those, given the dequantize's own scale and zero point (they must equal the plan's output parameters).

@@ -1225,7 +1225,7 @@ __global__ __launch_bounds__(256) void conv_mfma_stream_kernel(const ConvArgs a,
 #pragma unroll
         for (int e = 0; e < 4; e++)
             rq[e] = a.qmult ? conv_requant_ch(a, v[e], ko + e) : a.fastq ? conv_requant<true>(a, v[e]) : conv_requant<false>(a, v[e]);
-        if (a.deq_out != nullptr) { // fused dequantize (op_dequantize_run, art/modules/quant/src/op/dequantize.c:110-136)
+        if (a.deq_out != nullptr) { // fused dequantize (op_dequantize_run_u8, art/modules/quant/src/op/dequantize.c:111-123)
 #pragma unroll
             for (int e = 0; e < 4; e++)
                 if (ko + e < a.K)

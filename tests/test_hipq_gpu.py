@@ -383,7 +383,7 @@ def test_fc_streaming_kernel():
             assert np.array_equal(y2[:, :No], want_y), (M, Kd, No, rows, cols, waves)
         plan.stream()
         # the dequantize that reads the layer, in the layer's epilogue (hipq_conv2d_run_dequant): the float bit patterns of
-        # op_dequantize_run on the layer's bytes; refused for another scale or zero point than the bytes are written with
+        # op_dequantize_run_u8 on the layer's bytes; refused for another scale or zero point than the bytes are written with
         assert plan.dequant_fusable(q[4], q[5]) and not plan.dequant_fusable(float(np.float32(q[4] * 1.5)), q[5])
         assert not plan.dequant_fusable(q[4], (q[5] + 1) % 256)
         yf = torch.full((M, No), 7.0, dtype=torch.float32, device="cuda")

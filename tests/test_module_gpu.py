@@ -315,7 +315,7 @@ def test_convolution_and_relu_run_as_one_kernel(own_rt):
 
 def test_fully_connected_layer_and_dequantize_run_as_one_kernel(own_rt):
     """A fully-connected layer whose output only a dequantize reads leaves its launch to that operator: one kernel computes
-    the layer and writes the float values (op_dequantize_run on the layer's bytes, bit for bit); the layer's own bytes are
+    the layer and writes the float values (op_dequantize_run_u8 on the layer's bytes, bit for bit); the layer's own bytes are
     computed when somebody asks for them.  A dequantize with another scale runs as an operator of its own."""
     import ctypes as C
     from oracle import orc
