@@ -1667,6 +1667,9 @@ static int choose_tile(long long P, int out_cs, bool expand, int in_cs)
         return count(2) >= 1024 ? 2 : 4; // 128x64, or 64x64 for small images
     if (expand && P >= 8000) // short reduction, wide output: store-bound, many small work-groups overlap best; from 512
         return in_cs >= 512 ? 3 : 4; // input channels on the reduction is long enough for the wider tile (17.4 -> 14.9 us)
+    if (expand && count(0) >= 200 && count(0) < kCUs)
+        return 4; // a widening layer whose 128x128 tiles would leave CUs idle: small tiles (MobileNetV2's 160 -> 960 and
+                  // 320 -> 1280 at 7x7, batch 64: the pass 0.470 -> 0.463 ms; 64x128 tiles 0.465)
     if (count(3) <= 128)
         return 4; // tiles for at most half the CUs (fully-connected layers, 7x7 layers at batch 32): the smallest tile, to
                   // put more CUs on the weight stream (512 -> 512 3x3 on 1568 pixels: 16.1 -> 14.3 us)
