@@ -183,10 +183,11 @@ def measure_workload(build, batch, inner, kernel_reps, check_rows):
     st = torch.cuda.Stream()
     with torch.cuda.stream(st):
         g = graph_of(ex.run, inner, st)
-        g.replay()
+        for _ in range(10):  # clocks and caches as in a loop that keeps running
+            g.replay()
         torch.cuda.synchronize()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        reps = 5
+        reps = 50
         e0.record(st)
         for _ in range(reps):
             g.replay()
