@@ -145,7 +145,8 @@ int hipq_conv2d_plan_select(hipq_conv2d_plan *plan, int tile, int stages);
  * of a work-group in LDS, two multiplies per 32 pixels, 128-bit stores straight from the accumulators; modes 1 and 2.
  * mode 1 (the default) uses them where they measured faster: the rows kernel wherever it applies, the halo kernel for
  * the other 64-channel inputs up to 63 pixels wide, the pointwise kernel wherever it applies, the two-group kernel for layers with at most one tile per CU (256),
- * the widening kernel at 64 input channels with or without the add (from 150 000 pixels) and without it at 256 (from 20 000);
+ * the widening kernel at 64 input channels with or without the add (from 150 000 pixels), with it at 128 (from 50 000)
+ * and without it at 256 (from 20 000);
  * mode 2 the halo kernel instead of the rows kernel and also for 128, 256 and 512 channels (128-channel tiles, images up to 31 pixels wide), the
  * two-group kernel whatever the number of tiles and the widening kernel wherever it applies; mode 0 none of them.
  * Identical results in every mode.  Plans that do not run the MFMA kernel return an error.

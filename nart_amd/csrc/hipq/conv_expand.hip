@@ -363,11 +363,12 @@ bool conv_expand_applies(const ConvArgs &a, bool wherever)
         // where it beats the kernels it replaces: with the add at 64 input channels (31.7 against 35.7 us at 64 -> 256
         // on 200 704 pixels; level at 128 -> 512, behind at 256 -> 1024), without at 256 (16.7 against 19.7 us at
         // 256 -> 512 on 50 176 pixels) and at 64 on very many pixels (64 -> 256 on 200 704: 16.3 against the pointwise
-        // kernel's 17.8 us alone, and the ResNet-50 pass it sits in 0.880 -> 0.869 ms) - and only on many pixels: its grid is
+        // kernel's 17.8 us alone, and the ResNet-50 pass it sits in 0.880 -> 0.869 ms); inside that pass the add at 128 input
+        // channels on 50 176 pixels gains 0.25 %, the one at 256 on 12 544 loses 0.5 % - and only on many pixels: its grid is
         // three work-groups per CU whatever the size, a launch of it takes 6.6 us or more, and the tile kernels need
         // 4 to 7 us up to some 12 000 pixels (256 -> 512: level at 25 000; 64 -> 256 with the add: 19.6 against 18.7 us
         // at 100 352)
-        && (wherever || (a.res != nullptr ? a.in_cs == 64 && a.P >= 150000 : (a.in_cs == 256 && a.P >= 20000) || (a.in_cs == 64 && a.P >= 150000)));
+        && (wherever || (a.res != nullptr ? (a.in_cs == 64 && a.P >= 150000) || (a.in_cs == 128 && a.P >= 50000) : (a.in_cs == 256 && a.P >= 20000) || (a.in_cs == 64 && a.P >= 150000)));
 }
 
 template <int NSLAB, int MID>

@@ -198,10 +198,11 @@ def test_channel_widening_1x1_layers():
                 got = hipq.from_device_nhwc(y, K)
                 assert np.array_equal(got, want), (i, res_first, ratio, obits, mode, int((got != want).sum()))
     # the built-in rule: a launch of this kernel has a floor of 6.6 us, so it is chosen on many pixels only - without the
-    # add at 256 input channels from 20 000 pixels, at 64 input channels (with or without the add) from 150 000
+    # add at 256 input channels from 20 000 pixels, at 64 input channels (with or without the add) from 150 000, with the
+    # add at 128 input channels from 50 000
     for (N, C, H, K, st), plain, added in (((64, 256, 56, 512, 2), True, False), ((16, 256, 56, 512, 2), False, False),
                                            ((64, 64, 56, 256, 1), True, True), ((32, 64, 56, 256, 1), False, False),
-                                           ((64, 128, 28, 512, 1), False, False)):
+                                           ((64, 128, 28, 512, 1), False, True), ((32, 128, 28, 512, 1), False, False)):
         plan = hipq.Conv2d((N, C, H, H), rng.integers(0, 256, (K, C, 1, 1), dtype=np.uint8), None, 0, st, 1, 0.02, 3, 0.004, 128, 0.3, 5)
         assert (plan.kernel == "conv_mfma_i8_expand") == plain, (N, C, H, K, st, plan.kernel)
         assert (plan.kernel_add == "conv_mfma_i8_expand+add") == added, (N, C, H, K, st, plan.kernel_add)
