@@ -38,7 +38,7 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s (published)
 # HBM bytes per launch of the dominant kernel family, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this very
 # command.  A counter run cannot be made from inside the benchmark, so the figure is carried here together with the
 # file that holds the counter readings; it only applies to the default workload with default flags.
-TRAFFIC_FROM_PROFILE = {"workload": "resnet50", "batch": 64, "bytes_per_launch": 34.52e6,
+TRAFFIC_FROM_PROFILE = {"workload": "resnet50", "batch": 64, "bytes_per_launch": 34.85e6,
                         "source": "profiles/conv_mfma_i8_resnet50_n64.md"}
 
 
