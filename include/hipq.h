@@ -225,6 +225,24 @@ int hipq_conv2d_run_add_conv(const hipq_conv2d_plan *plan, const void *x, const 
                              const hipq_conv2d_plan *next, int next_relu, void *y_next, void *stream);
 
 /*
+ * An identity bottleneck block of a residual network in one launch: y = add(widen(mid(reduce(x))), x), bit-identical to
+ * hipq_conv2d_run(reduce, x, t1), hipq_conv2d_run(mid, t1, t2) and hipq_conv2d_run_add(widen, t2, residual = x, ...) -
+ * op_conv_2d_u8xu8_run (src/op/conv_2d_uint8_impl.c:39-165) three times, then op_quant_add_run (src/op/add.c:83-148) -
+ * but t1, t2 and the widening layer's own output never travel to memory.  `reduce`: a 1x1 / stride 1 convolution from
+ * CW = 256, 512 or 1024 channels to CM = CW / 4; `mid`: 3x3 / stride 1 / pad 1, CM -> CM; `widen`: 1x1, CM -> CW; all on
+ * images whose height and width are multiples of 7, uint8 tensors with dense channel strides, weight zero points 128,
+ * per-tensor weight scales, each layer reading its input with the scale and zero point the previous one writes.  The
+ * residual is x itself, read with `reduce`'s input scale and zero point; the add's inputs are (widen(...), x), or
+ * (x, widen(...)) when residual_is_input0 != 0; oalpha / ozp / obits (8) describe the sum.  y must not be x.
+ * hipq_bottleneck_fusable answers (1 / 0) whether three plans and an add can run this way; hipq_bottleneck_run fails
+ * with an error otherwise (run the operators separately).
+ */
+int hipq_bottleneck_fusable(const hipq_conv2d_plan *reduce, const hipq_conv2d_plan *mid, const hipq_conv2d_plan *widen,
+                            int residual_is_input0, float oalpha, int ozp, int obits);
+int hipq_bottleneck_run(const hipq_conv2d_plan *reduce, const hipq_conv2d_plan *mid, const hipq_conv2d_plan *widen,
+                        const void *x, int residual_is_input0, float oalpha, int ozp, int obits, void *y, void *stream);
+
+/*
  * Convolution with the max pooling that follows it in one kernel: y = maxpool3x3/2/1(conv(x)), bit-identical to
  * hipq_conv2d_run followed by hipq_pool_u8(HIPQ_POOL_MAX, kernel 3, stride 2, pad 1) whose input and output scale and
  * zero point both equal the convolution's output parameters (op_conv_2d_u8xu8_run, then op_quant_pool_max_run -

@@ -53,6 +53,7 @@
 #include "common.h"
 #include "conv_shared.h"
 #include "conv_stem.h"
+#include "conv_block.h"
 #include "conv_expand.h"
 #include "conv_dw.h"
 #include "conv_rows.h"
@@ -1763,7 +1764,7 @@ static int plan_create(const hipq_conv2d_desc *dp, const uint8_t *w, const int32
     const int cg = d.C / d.group;
     std::vector<uint8_t> wbuf;
     std::vector<int32_t> bbuf;
-    size_t pad_off = 0;
+    size_t pad_off = 0, frag_off = 0;
     if (d.group == 1 && (d.in_cs % 16 == 0 || d.in_cs == 4)) {
         const bool smallc = d.in_cs == 4;
         p->variant = smallc ? kMfmaSmallC : kMfma;
@@ -1808,6 +1809,22 @@ static int plan_create(const hipq_conv2d_desc *dp, const uint8_t *w, const int32
         }
         pad_off = wbuf.size();
         wbuf.resize(pad_off + 64, (uint8_t)pad_byte); // source of out-of-image taps
+        // the same weights in fragment order (ConvArgs::wfrag) for the kernels whose waves load their MFMA weight
+        // operands straight from memory: layers of a bottleneck block
+        if (!smallc && boff == 0 && d.in_cs % 64 == 0 && d.in_cs <= 1024 && d.out_cs <= 1024 && d.C == d.in_cs
+            && ((d.R == 1 && d.S == 1) || (d.R == 3 && d.S == 3))) {
+            frag_off = (wbuf.size() + 255) / 256 * 256;
+            wbuf.resize(frag_off + pad_off, 0);
+            for (int sl = 0; sl < a.nslab; sl++)
+                for (int T = 0; T < a.kout_pad / 32; T++)
+                    for (int kk = 0; kk < 2; kk++)
+                        for (int l = 0; l < 64; l++) {
+                            const int pp = l & 31, hh = l >> 5;
+                            const int ko = 32 * T + 16 * ((pp >> 2) & 1) + 4 * (pp >> 3) + (pp & 3);
+                            const uint8_t *src = &wbuf[((size_t)sl * a.kout_pad + ko) * 64 + (((2 * kk + hh) ^ ((ko >> 2) & 3)) << 4)];
+                            memcpy(&wbuf[frag_off + ((((size_t)sl * (a.kout_pad / 32) + T) * 2 + kk) * 64 + l) * 16], src, 16);
+                        }
+        }
         static const bool no_halo = getenv("HIPQ_NO_SPECIAL_KERNELS") != nullptr; // A/B measurements: tile kernels only
         p->special = no_halo ? 0 : 1;
         set_mfma_name(p, smallc);
@@ -1874,6 +1891,7 @@ static int plan_create(const hipq_conv2d_desc *dp, const uint8_t *w, const int32
     a.wpack = static_cast<const uint8_t *>(p->d_w);
     a.bias2 = static_cast<const int32_t *>(p->d_bias);
     a.padbuf = a.wpack + pad_off;
+    a.wfrag = frag_off ? a.wpack + frag_off : nullptr;
     if (p->d_q) {
         a.qmult = static_cast<const uint32_t *>(p->d_q);
         a.qshift = reinterpret_cast<const int32_t *>(a.qmult + qbuf.size() / 2);
@@ -2302,6 +2320,57 @@ extern "C" int hipq_conv2d_run_add_conv(const hipq_conv2d_plan *p, const void *x
         a2.lo = std::min(next->d.ozp, a2.q.hi); // the ReLU clamp, as in hipq_conv2d_run_relu
     launch_conv_expand_chain(a, a2, static_cast<hipStream_t>(stream));
     return launch_status("conv_mfma_expand_kernel (chained)");
+}
+
+// the launch arguments of the three layers of an identity bottleneck block (hipq_bottleneck_run); false if the add's
+// scales are outside the fixed-point range
+static bool block_args(const hipq_conv2d_plan *p1, const hipq_conv2d_plan *p2, const hipq_conv2d_plan *p3, int residual_is_input0,
+                       float oalpha, int ozp, int obits, ConvArgs *a1, ConvArgs *a2, ConvArgs *a3)
+{
+    *a1 = p1->args, *a2 = p2->args;
+    // the residual is the block's input: the tensor the first layer reads, with that layer's input scale and zero point
+    return add_args(p3, residual_is_input0, p1->d.ialpha, p1->d.izp, oalpha, ozp, obits, a3);
+}
+
+extern "C" int hipq_bottleneck_fusable(const hipq_conv2d_plan *p1, const hipq_conv2d_plan *p2, const hipq_conv2d_plan *p3,
+                                       int residual_is_input0, float oalpha, int ozp, int obits)
+{
+    for (const hipq_conv2d_plan *p : {p1, p2, p3})
+        if (!p || p->variant != kMfma || !p->special || p->tile_selected || p->has_wzp || p->d.dtype != HIPQ_DTYPE_U8 || p->d.obits != 8)
+            return 0;
+    if (obits != 8 || ozp < 0 || ozp > 255)
+        return 0;
+    // each layer must read its input with the zero point the previous one writes it with
+    if (p2->d.izp != p1->d.ozp || p3->d.izp != p2->d.ozp || p2->d.ialpha != p1->d.oalpha || p3->d.ialpha != p2->d.oalpha)
+        return 0;
+    ConvArgs a1, a2, a3;
+    if (!block_args(p1, p2, p3, residual_is_input0, oalpha, ozp, obits, &a1, &a2, &a3))
+        return 0;
+    if (!conv_block_applies(a1, a2, a3))
+        return 0;
+    // built-in rule: where it measured faster than the three launches it replaces - blocks of 256 middle channels (14x14
+    // images at batch 64: 31 against 41 us and two launch gaps); hipq_conv2d_plan_special(reduce, 2): wherever it applies
+    return p1->special == 2 || a1.out_cs == 256 ? 1 : 0;
+}
+
+extern "C" int hipq_bottleneck_run(const hipq_conv2d_plan *p1, const hipq_conv2d_plan *p2, const hipq_conv2d_plan *p3, const void *x,
+                                   int residual_is_input0, float oalpha, int ozp, int obits, void *y, void *stream)
+{
+    clear_error();
+    HIPQ_REQUIRE(p1 && p2 && p3 && x && y, "hipq_bottleneck_run: null argument");
+    HIPQ_REQUIRE(x != y, "hipq_bottleneck_run: the sum cannot overwrite the block's input (neighbouring patches read it)");
+    HIPQ_REQUIRE(hipq_bottleneck_fusable(p1, p2, p3, residual_is_input0, oalpha, ozp, obits),
+                 "hipq_bottleneck_run: these three plans (%s, %s, %s) and this add do not run as one kernel: run hipq_conv2d_run "
+                 "twice and hipq_conv2d_run_add", p1->name.c_str(), p2->name.c_str(), p3->name.c_str());
+    ConvArgs a1, a2, a3;
+    block_args(p1, p2, p3, residual_is_input0, oalpha, ozp, obits, &a1, &a2, &a3);
+    a1.x = static_cast<const uint8_t *>(x);
+    a1.y = a2.y = nullptr;
+    a1.acc_out = a2.acc_out = a3.acc_out = nullptr;
+    a3.res = a1.x;
+    a3.y = static_cast<uint8_t *>(y);
+    launch_conv_block(a1, a2, a3, static_cast<hipStream_t>(stream));
+    return launch_status("conv_bottleneck_kernel");
 }
 
 extern "C" int hipq_conv2d_maxpool_fusable(const hipq_conv2d_plan *p, int OH, int OW, int kernel, int stride, int pad,

@@ -1,0 +1,14 @@
+// A whole identity bottleneck block - 1x1 reduction, 3x3, 1x1 widening, residual add - in one kernel (conv_block.hip).
+#pragma once
+
+#include "conv_shared.h"
+
+namespace hipq {
+
+// a1: the 1x1 convolution that reads the block's input x (a1.x), a2: the 3x3 / stride 1 / pad 1 convolution, a3: the
+// widening 1x1 convolution with the add's parameters in a3.addq / a3.res_first; the residual is x itself and the sum goes
+// to a3.y.  true when conv_bottleneck_kernel computes this chain.
+bool conv_block_applies(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3);
+void launch_conv_block(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3, hipStream_t st);
+
+} // namespace hipq

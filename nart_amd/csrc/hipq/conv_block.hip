@@ -1,0 +1,505 @@
+// An identity bottleneck block of a residual network in ONE kernel: the 1x1 convolution that reduces the channels, the
+// 3x3 convolution, the 1x1 convolution that widens them again and the residual add with the block's input.  gfx950 only.
+//
+// Reproduces, bit for bit, op_conv_2d_u8xu8_run (art/modules/quant/src/op/conv_2d_uint8_impl.c:39-165) three times and
+// op_quant_add_run (art/modules/quant/src/op/add.c:83-148) on their bytes: every intermediate value is requantised,
+// clamped and re-read exactly as if it had travelled through memory.
+//
+// Why: at 14x14 (and 28x28, 56x56) pixels per image and batch 64 the three layers are three launches that each find a
+// few microseconds of matrix work per CU behind a launch, a cold start and a drain, and that hand 3 to 13 MB to one
+// another through memory.  Here a work-group owns a 7x7 patch of ONE image through the whole block:
+//   * x: the patch with a one-pixel border (at most 9x9 pixels, clipped to the image), all CW channels, is fetched once
+//     into LDS by the load unit; it is the pixel operand of the first layer and, later, the residual;
+//   * layer 1 (CW -> CM, CM = CW / 4) is computed for every pixel of that region - the border pixels are computed again by
+//     the neighbouring patches' work-groups, which is the price of never synchronising work-groups - and its bytes go to
+//     a 9x9 grid of pixel rows in LDS whose out-of-image positions hold the 3x3 layer's pad byte;
+//   * layer 2 (3x3) reads its nine taps as nine shifted windows of that grid: output index m = 9 * row + column over
+//     7 rows of 9 (two columns of each row are computed and dropped), so tap (dr, ds) of output m is grid row
+//     m + 9 (dr + 1) + (ds + 1) - closed-form addressing, consecutive lanes on consecutive LDS rows; its bytes go to LDS;
+//   * layer 3 (CM -> CW) reads them as its pixel operand, requantises, adds the residual from the x tile in LDS with
+//     the reference's arithmetic and stores the sum.
+// Weights never pass through LDS: the waves of a work-group split the OUTPUT CHANNELS, so no two waves want the same
+// weight bytes, and a wave loads its MFMA weight operands straight from global memory (L2) into registers, a ring of
+// slabs ahead of its multiplies; LDS bandwidth is left to the pixel operands.  The work-group has 2 waves per 64
+// middle channels: the pair shares a 64-channel x all-pixel tile of layers 1 and 2 and splits the REDUCTION (every other
+// 64-byte slab of k), so that two waves per SIMD overlap each other's loads, LDS reads and multiplies without reading
+// any pixel operand twice; the partial sums meet once per layer in LDS, each wave keeping 32 of the 64 channels.  In
+// layer 3 every wave owns 128 output channels, keeps its pixel operands for the whole reduction in registers and works
+// through 4 chunks of 32 channels: multiplies of one wave run under the other's vector arithmetic of the add.
+// MFMA rows are permuted (row i computes channel 16 ((i >> 2) & 1) + 4 (i >> 3) + (i & 3) of its 32) so that a lane's 16
+// accumulators are 16 consecutive channels of one pixel: one 128-bit LDS or global store, no transpose.
+// Requirements (checked by the host): uint8 tensors, weight zero points 128, per-tensor scales, one-multiply
+// requantisation in all three layers, 32-bit form of the add to 8 bits, CM of 64, 128 or 256, image height and width
+// multiples of 7.
+#include "conv_block.h"
+
+#include <algorithm>
+#include <cstdlib>
+
+namespace hipq {
+
+namespace {
+
+constexpr int kPatch = 7;          // a work-group's output pixels: kPatch x kPatch of one image
+constexpr int kGridW = kPatch + 2; // the patch with its border: kGridW x kGridW pixel rows in LDS
+constexpr int kGridRows = 96;      // rows held for that grid (81 positions; the row-padded output index reaches row 83)
+
+struct BlockGeom {
+    int H, W, PY, PX, npatch;
+#ifdef HIPQ_BLOCK_STAMPS
+    unsigned long long *stamps;
+#endif
+};
+#ifdef HIPQ_BLOCK_STAMPS
+#define STAMP(k)                                                                                   \
+    do {                                                                                           \
+        if (geo.stamps && lane == 0)                                                               \
+            geo.stamps[((size_t)gid * 8 + wave) * 16 + (k)] = __builtin_readcyclecounter();         \
+    } while (0)
+#else
+#define STAMP(k)
+#endif
+
+// chunk (16 bytes) c of pixel row `row` is kept at chunk c ^ swz(row) of its LDS row, so that 16 lanes that read the same
+// chunk of 16 consecutive rows fall on 16 different bank groups whatever the row length
+template <int ROWBYTES>
+__device__ inline int swz(int row)
+{
+    return ROWBYTES >= 256 ? (row & 15) : ROWBYTES == 128 ? ((row >> 1) & 7) : ((row >> 2) & 3);
+}
+
+// 16 accumulators (16 consecutive channels of one pixel) -> 16 requantised bytes, each XORed with the low byte of flip
+__device__ inline v4i requant16(const ConvArgs &a, const v16i &acc, uint32_t flip)
+{
+    v4i o;
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        int32_t r[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+            r[e] = conv_requant<true>(a, acc[g * 4 + e]);
+        o[g] = (int)(pack_low_bytes(r[0], r[1], r[2], r[3]) ^ flip);
+    }
+    return o;
+}
+
+// The same followed by the residual add (op_quant_add_run on the requantised bytes and the residual's 16 bytes `res`),
+// in the 32-bit form: per element the convolution's clamped result minus its zero point is clamp(q, lo - zp, hi - zp)
+// with q = (mulhi(acc, mult) + 2^(t-1)) >> t; the add's terms are (d * m + c) >> s; the sum saturates to [0, 255].
+__device__ inline v4i requant_add16(const ConvArgs &a, const v16i &acc, const v4i res)
+{
+    const AddParams &q = a.addq;
+    const int mc = (int)(a.res_first ? q.m1 : q.m0), sc = a.res_first ? q.s1 : q.s0;
+    const int mr = (int)(a.res_first ? q.m0 : q.m1), sr = a.res_first ? q.s0 : q.s1, cr = a.res_first ? q.c0 : q.c1;
+    const int rc = 1 << (sc - 1); // rounding of the convolution's term (its zero point cancels)
+    const int qround = 1 << (a.qt - 1);
+    const int dlo = a.lo - a.q.zp, dhi = a.q.hi - a.q.zp;
+    v4i o;
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        const uint32_t rv = (uint32_t)res[g];
+        int32_t y[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            int32_t d = (__mulhi(acc[g * 4 + e], (int)a.q.mult) + qround) >> a.qt;
+            asm("v_med3_i32 %0, %1, %2, %3" : "=v"(d) : "v"(d), "s"(dlo), "v"(dhi));
+            const int32_t t0 = (__mul24(d, mc) + rc) >> sc;
+            const int32_t t1 = (__mul24((int)((rv >> (8 * e)) & 255), mr) + cr) >> sr;
+            y[e] = (t0 + t1 + q.cadd) >> q.sh;
+        }
+        uint32_t p01, p23, b01, b23;
+        asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p01) : "v"(y[0]), "v"(y[1]));
+        asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(y[2]), "v"(y[3]));
+        asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
+        asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
+        o[g] = (int)__builtin_amdgcn_perm(b23, b01, 0x05040100u);
+    }
+    return o;
+}
+
+// accumulators of a lane <- the folded bias of its 16 consecutive channels (or zero for the wave that does not carry it)
+__device__ inline void init_acc(v16i &acc, const int32_t *bias16, bool zero)
+{
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        const v4i bv = *reinterpret_cast<const v4i *>(bias16 + g * 4);
+#pragma unroll
+        for (int e = 0; e < 4; e++)
+            acc[g * 4 + e] = zero ? 0 : bv[e];
+    }
+}
+
+// The weight operands a wave holds ahead of its multiplies: D slabs of four (channel tile nt, k-step kk at [2 nt + kk]),
+// and the two of an odd slab count's last half slab.
+template <int D>
+struct WeightRing {
+    v4i w[D][4], wt[2];
+};
+
+// One wave's half of a layer's reduction, accumulated into acc[pixel tile][channel tile] (MT pixel tiles of 32, 2
+// channel tiles of 32): the slabs kh, kh + 2, ... of the first STOT - (STOT & 1), and, when STOT is odd, k-step kh of
+// the last slab - both waves of a pair do the same amount of work and the code has no branch, so the compiler's wait
+// counts stay exact.  ldw(s, kk, nt): the weight operand of slab s, k-step kk, channel tile nt, from global memory, D
+// slabs ahead of its multiplies (ring_fill issues the first D, as early as the caller likes); ldb(s, kk, t): the pixel
+// operand of pixel tile t from LDS, one slab ahead; flip is XORed onto the pixel operands (0x80808080 re-centres raw
+// uint8 bytes, 0 leaves re-centred ones alone).
+template <int STOT, int D, class FW>
+__device__ inline void ring_fill(WeightRing<D> &r, const int kh, FW ldw)
+{
+    constexpr int NS = STOT / 2;
+#pragma unroll
+    for (int i = 0; i < D && i < NS; i++)
+#pragma unroll
+        for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++)
+                r.w[i][2 * nt + kk] = ldw(2 * i + kh, kk, nt);
+    if ((STOT & 1) && NS <= D)
+        r.wt[0] = ldw(STOT - 1, kh, 0), r.wt[1] = ldw(STOT - 1, kh, 1);
+}
+
+template <int STOT, int MT, int D, class FW, class FB>
+__device__ inline void reduce_half(v16i (&acc)[MT][2], WeightRing<D> &r, const int kh, const int flip, FW ldw, FB ldb)
+{
+    constexpr int NS = STOT / 2;
+    constexpr bool TAIL = (STOT & 1) != 0;
+    v4i br[2][MT][2], bt[MT];
+    auto loadb = [&](int i, v4i(&b)[MT][2]) {
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++)
+                b[t][kk] = ldb(2 * i + kh, kk, t);
+    };
+    loadb(0, br[0]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < NS; i++) {
+        if (i + 1 < NS) {
+            loadb(i + 1, br[(i + 1) & 1]);
+        } else if (TAIL) {
+#pragma unroll
+            for (int t = 0; t < MT; t++)
+                bt[t] = ldb(STOT - 1, kh, t);
+        }
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+            for (int t = 0; t < MT; t++)
+#pragma unroll
+                for (int nt = 0; nt < 2; nt++)
+                    acc[t][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(r.w[i % D][2 * nt + kk], br[i & 1][t][kk] ^ flip, acc[t][nt], 0, 0, 0);
+        if (i + D < NS) {
+#pragma unroll
+            for (int nt = 0; nt < 2; nt++)
+#pragma unroll
+                for (int kk = 0; kk < 2; kk++)
+                    r.w[i % D][2 * nt + kk] = ldw(2 * (i + D) + kh, kk, nt);
+        } else if (TAIL && i + D == NS) {
+            r.wt[0] = ldw(STOT - 1, kh, 0), r.wt[1] = ldw(STOT - 1, kh, 1);
+        }
+        __builtin_amdgcn_sched_barrier(0); // keep every slab's loads, reads and multiplies where they are written
+    }
+    if (TAIL) {
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+#pragma unroll
+            for (int nt = 0; nt < 2; nt++)
+                acc[t][nt] = __builtin_amdgcn_mfma_i32_32x32x32_i8(r.wt[nt], bt[t] ^ flip, acc[t][nt], 0, 0, 0);
+    }
+}
+
+// The two waves of a pair add their partial sums: each sends its channel tile 1 and keeps tile 0 (the pair's waves order
+// their channel tiles oppositely, so one wave's tile 1 is the other's tile 0) through 4 KB slots in LDS - all pixel
+// tiles at once where the slots hold them (ONE_ROUND: MT slots per wave), else one pixel tile per round with a barrier
+// before a slot is written again.  No barrier at the end: the caller has one before it reuses the slots.
+template <int MT, bool ONE_ROUND>
+__device__ inline void pair_reduce(v16i (&acc)[MT][2], uint8_t *scr, const int wave, const int partner, const int lane)
+{
+    constexpr int SLOT = ONE_ROUND ? MT * 4096 : 4096;
+    auto send = [&](int t) {
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            v4i v;
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                v[e] = acc[t][1][g * 4 + e];
+            *reinterpret_cast<v4i *>(scr + wave * SLOT + (ONE_ROUND ? t * 4096 : 0) + g * 1024 + lane * 16) = v;
+        }
+    };
+    auto receive = [&](int t) {
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const v4i v = *reinterpret_cast<const v4i *>(scr + partner * SLOT + (ONE_ROUND ? t * 4096 : 0) + g * 1024 + lane * 16);
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                acc[t][0][g * 4 + e] += v[e];
+        }
+    };
+    if (ONE_ROUND) {
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+            send(t);
+        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
+        __builtin_amdgcn_s_barrier();
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+            receive(t);
+        return;
+    }
+#pragma unroll
+    for (int t = 0; t < MT; t++) {
+        if (t > 0) { // every wave has read the previous round's slots
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_s_barrier();
+        }
+        send(t);
+        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
+        __builtin_amdgcn_s_barrier();
+        receive(t);
+    }
+}
+
+} // namespace
+
+// G = CM / 64 (1, 2, 4): 2 G waves.  MT1: pixel tiles of layer 1 (2: regions of at most 64 pixels, i.e. images of at
+// most 2 x 2 patches; 3: up to 9 x 9 = 81).
+template <int G, int MT1>
+__global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvArgs a1, const ConvArgs a2, const ConvArgs a3,
+                                                                    const BlockGeom geo)
+{
+    constexpr int NW = 2 * G, NT = 128 * G, CM = 64 * G, CW = 256 * G;
+    constexpr bool ONE_ROUND = G == 4 && MT1 == 2;          // LDS holds every exchange slot at once
+    constexpr int X_BYTES = 32 * MT1 * CW;                  // the region's pixel rows, CW bytes each
+    constexpr int G_OFF = X_BYTES, G_BYTES = kGridRows * CM; // layer 1's bytes on the 9 x 9 grid, CM bytes a row; later layer 2's
+    constexpr int S_OFF = G_OFF + G_BYTES, S_BYTES = NW * 4096 * (ONE_ROUND ? MT1 : 1); // the pairs' exchange slots
+    constexpr int D1 = MT1 == 2 ? 6 : 4, D2 = 6;            // slabs of weights a wave holds ahead, layers 1 and 2
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[S_OFF + S_BYTES];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int p = lane & 31, h = lane >> 5;
+    const int ng = wave % G, kh = wave / G, partner = (wave + G) % NW;
+
+    // work-groups go to the 8 XCDs in turn: XCD x takes the x-th contiguous eighth of the patches, so the patches of an
+    // image - which share border pixels - and all weights are read through one L2
+    const int gid = (int)(blockIdx.x % 8) * (int)(gridDim.x / 8) + (int)(blockIdx.x / 8);
+    if (gid >= geo.npatch)
+        return;
+    STAMP(0);
+    const int ppi = geo.PY * geo.PX;
+    const int n = gid / ppi, pr = gid - n * ppi, pi = pr / geo.PX, pj = pr - pi * geo.PX;
+    const int y0 = pi * kPatch, x0 = pj * kPatch;
+    const int ry0 = max(y0 - 1, 0), rx0 = max(x0 - 1, 0);
+    const int RW = min(x0 + kPatch, geo.W - 1) - rx0 + 1, RH = min(y0 + kPatch, geo.H - 1) - ry0 + 1;
+    const int M1 = RW * RH;          // pixels of the region: at most 81 (64 when MT1 == 2: the host checks)
+    const int rwinv = 65536 / RW + 1; // j / RW == (j * rwinv) >> 16 for 0 <= j < 128, 7 <= RW <= 9
+
+    // ---- x region -> LDS: region pixel j at row j, its 16-byte piece c at piece c ^ (j & 15) of every 256 bytes ----
+    {
+        constexpr int LPR = CW / 16 >= 64 ? 64 : CW / 16, RPI = 64 / LPR; // lanes per pixel row, rows per wave instruction
+        constexpr int NINST = X_BYTES / 1024;
+        static_assert(CW <= 1024 && NINST % NW == 0, "a pixel row is at most one wave instruction");
+        const int pos = lane % LPR;
+#pragma unroll
+        for (int q = 0; q < NINST / NW; q++) {
+            const int i = wave + NW * q;
+            const int j = i * RPI + lane / LPR;
+            const int jj = min(j, M1 - 1); // rows beyond the region repeat its last pixel: computed, never used
+            const int jy = (jj * rwinv) >> 16, jx = jj - jy * RW;
+            const uint8_t *src = a1.x + (size_t)((n * geo.H + ry0 + jy) * geo.W + rx0 + jx) * CW + ((pos ^ (j & 15)) << 4);
+            __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(lds + i * 1024), 16, 0, 0);
+        }
+    }
+    // ---- the grid starts as the 3x3 layer's pad byte everywhere (re-centred like every byte kept there) ----
+    {
+        const int padw = (int)(a2.padword ^ a2.xmask);
+        const v4i pv = {padw, padw, padw, padw};
+#pragma unroll
+        for (int o = tid * 16; o < G_BYTES; o += NT * 16)
+            *reinterpret_cast<v4i *>(lds + G_OFF + o) = pv;
+    }
+
+    // Weight operands come in fragment order (ConvArgs::wfrag): the 1 KB a wave's load instruction fetches for slab s,
+    // 32-channel tile T, k-step kk is contiguous at ((s * tiles + T) * 2 + kk) * 1024, lane l's 16 bytes at 16 l.
+    // the wave's two channel tiles of layers 1 and 2: tile 0 (kept after the pair's exchange) and tile 1 (sent)
+    const int ct0 = 64 * ng + 32 * kh, ct1 = 64 * ng + 32 * (1 - kh);
+    const size_t wslab1 = (size_t)a1.kout_pad * 64, wslab2 = (size_t)a2.kout_pad * 64, wslab3 = (size_t)a3.kout_pad * 64;
+    const uint8_t *w10 = a1.wfrag + (size_t)ct0 * 64 + lane * 16, *w11 = a1.wfrag + (size_t)ct1 * 64 + lane * 16;
+    const uint8_t *w20 = a2.wfrag + (size_t)ct0 * 64 + lane * 16, *w21 = a2.wfrag + (size_t)ct1 * 64 + lane * 16;
+    auto ldw1 = [&](int s, int kk, int nt) { return ldg128((nt ? w11 : w10) + (size_t)s * wslab1 + kk * 1024); };
+    auto ldw2 = [&](int s, int kk, int nt) { return ldg128((nt ? w21 : w20) + (size_t)s * wslab2 + kk * 1024); };
+    // layer 1, slab s: pieces 4 s .. 4 s + 3 of every pixel row of the x tile
+    auto ldb1 = [&](int s, int kk, int t) {
+        const int j = 32 * t + p, hs = h ^ (j & 15);
+        return *reinterpret_cast<const v4i *>(lds + j * CW + (s >> 2) * 256 + (((4 * (s & 3) + 2 * kk) ^ hs) << 4));
+    };
+    // layer 2, slab s: channels 64 cb .. + 63 of tap (tap / 3, tap % 3), read at the tap's shift on the grid
+    auto ldb2 = [&](int s, int kk, int t) {
+        const int tap = s / G, cb = s % G, tr = (tap * 11) >> 5, off = tr * kGridW + (tap - 3 * tr);
+        const int gr = 32 * t + p + off, hs = h ^ swz<CM>(gr);
+        return *reinterpret_cast<const v4i *>(lds + G_OFF + gr * CM + (((4 * cb + 2 * kk) ^ hs) << 4));
+    };
+
+    // ================= layer 1: CW -> CM on the region's pixels =================
+    v16i acc1[MT1][2];
+#pragma unroll
+    for (int t = 0; t < MT1; t++) {
+        init_acc(acc1[t][0], a1.bias2 + ct0 + 16 * h, kh != 0);
+        init_acc(acc1[t][1], a1.bias2 + ct1 + 16 * h, kh != 0);
+    }
+    WeightRing<D1> r1;
+    ring_fill<4 * G, D1>(r1, kh, ldw1);
+    // the region's bytes have landed (and this wave's pad bytes are written) before anyone reads LDS
+    wait_vmcnt<0>();
+    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    STAMP(1);
+    reduce_half<4 * G, MT1, D1>(acc1, r1, kh, (int)a1.xmask, ldw1, ldb1);
+    STAMP(2);
+    // layer 2's first weights and folded biases travel while layer 1 is finished
+    WeightRing<D2> r2;
+    ring_fill<9 * G, D2>(r2, kh, ldw2);
+    v16i acc2[2][2];
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        init_acc(acc2[t][0], a2.bias2 + ct0 + 16 * h, kh != 0);
+        init_acc(acc2[t][1], a2.bias2 + ct1 + 16 * h, kh != 0);
+    }
+    pair_reduce<MT1, ONE_ROUND>(acc1, lds + S_OFF, wave, partner, lane);
+    STAMP(3);
+    // channels ct0 + 16 h .. + 15 of region pixel j -> the grid position of that pixel
+#pragma unroll
+    for (int t = 0; t < MT1; t++) {
+        const int j = 32 * t + p;
+        if (j < M1) {
+            const int jy = (j * rwinv) >> 16, jx = j - jy * RW;
+            const int g = (ry0 + jy - y0 + 1) * kGridW + (rx0 + jx - x0 + 1);
+            const v4i o = requant16(a1, acc1[t][0], a2.xmask);
+            *reinterpret_cast<v4i *>(lds + G_OFF + g * CM + ((((ct0 >> 4) + h) ^ swz<CM>(g)) << 4)) = o;
+        }
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    STAMP(4);
+
+    // ================= layer 2: 3x3, CM -> CM, output index m = 9 * row + column =================
+    reduce_half<9 * G, 2, D2>(acc2, r2, kh, 0, ldw2, ldb2);
+    STAMP(5);
+    // layer 3: this wave's 128 output channels in 4 chunks of 32; the first chunk's weights and biases travel now
+    const uint8_t *w3 = a3.wfrag + (size_t)(128 * wave) * 64 + lane * 16;
+    v4i wf[2 * G], b3[4];
+    auto load_chunk = [&](int cc) {
+#pragma unroll
+        for (int ks = 0; ks < 2 * G; ks++)
+            wf[ks] = ldg128(w3 + (size_t)(ks >> 1) * wslab3 + (size_t)cc * 2048 + (ks & 1) * 1024);
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+            b3[g] = *reinterpret_cast<const v4i *>(a3.bias2 + 128 * wave + 32 * cc + 16 * h + 4 * g);
+    };
+    load_chunk(0);
+    pair_reduce<2, ONE_ROUND>(acc2, lds + S_OFF, wave, partner, lane);
+    STAMP(6);
+    // every wave has passed the exchange's barrier, i.e. is done reading the grid: layer 2's bytes go there, row m
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const int m = 32 * t + p;
+        const v4i o = requant16(a2, acc2[t][0], a3.xmask);
+        *reinterpret_cast<v4i *>(lds + G_OFF + m * CM + ((((ct0 >> 4) + h) ^ swz<CM>(m)) << 4)) = o;
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+    STAMP(7);
+
+    // ================= layer 3: CM -> CW and the residual add =================
+    {
+        v4i bf[2][2 * G]; // pixel operands of the whole reduction
+        int jres[2];      // the output pixel's row in the x tile
+        size_t yoff[2];
+        bool valid[2];
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            const int m = 32 * t + p;
+#pragma unroll
+            for (int ks = 0; ks < 2 * G; ks++)
+                bf[t][ks] = *reinterpret_cast<const v4i *>(lds + G_OFF + m * CM + (((2 * ks + h) ^ swz<CM>(m)) << 4));
+            const int py = (m * 57) >> 9, px = m - py * kGridW; // m / 9 for m < 64
+            valid[t] = py < kPatch && px < kPatch;
+            jres[t] = valid[t] ? (y0 + py - ry0) * RW + (x0 + px - rx0) : 0;
+            yoff[t] = (size_t)((n * geo.H + y0 + py) * geo.W + x0 + px) * CW;
+        }
+        STAMP(8);
+        for (int cc = 0; cc < 4; cc++) {
+            const int ch = 128 * wave + 32 * cc; // first of the chunk's 32 channels
+            v16i acc[2];
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    acc[0][4 * g + e] = b3[g][e];
+            acc[1] = acc[0];
+#pragma unroll
+            for (int ks = 0; ks < 2 * G; ks++)
+#pragma unroll
+                for (int t = 0; t < 2; t++)
+                    acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[ks], bf[t][ks], acc[t], 0, 0, 0);
+            if (cc + 1 < 4)
+                load_chunk(cc + 1); // into the registers the multiplies above have read: they arrive during the arithmetic below
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                const int c16 = (ch >> 4) + h; // the 16-byte piece of the pixel's CW bytes
+                const v4i res = *reinterpret_cast<const v4i *>(lds + jres[t] * CW + (c16 & ~15) * 16 + (((c16 & 15) ^ (jres[t] & 15)) << 4));
+                const v4i o = requant_add16(a3, acc[t], res);
+                if (valid[t])
+                    *reinterpret_cast<v4i *>(a3.y + yoff[t] + ch + 16 * h) = o;
+            }
+            STAMP(9 + cc);
+        }
+    }
+}
+
+bool conv_block_applies(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3)
+{
+    const int cm = a1.out_cs, cw = a1.in_cs;
+    auto plain = [](const ConvArgs &a) {
+        return a.group == 1 && a.bwz == 0 && a.xmask != 0 && a.fastq && a.qmult == nullptr && a.acc_out == nullptr && a.deq_out == nullptr && a.wfrag != nullptr;
+    };
+    auto one = [](const ConvArgs &a) {
+        return a.R == 1 && a.S == 1 && a.pad_h == 0 && a.pad_w == 0 && a.stride_h == 1 && a.stride_w == 1;
+    };
+    auto same_image = [&](const ConvArgs &a) { return a.N == a1.N && a.H == a1.H && a.W == a1.W && a.OH == a1.H && a.OW == a1.W; };
+    return plain(a1) && plain(a2) && plain(a3) && (cm == 64 || cm == 128 || cm == 256) && cw == 4 * cm
+        && one(a1) && a1.C == cw && a1.K == cm && a1.nslab == cw / 64 && a1.kout_pad >= cm && a1.res == nullptr && same_image(a1)
+        && a2.R == 3 && a2.S == 3 && a2.pad_h == 1 && a2.pad_w == 1 && a2.stride_h == 1 && a2.stride_w == 1 && a2.C == cm
+        && a2.in_cs == cm && a2.K == cm && a2.out_cs == cm && a2.nslab == 9 * cm / 64 && a2.kout_pad >= cm && a2.res == nullptr
+        && same_image(a2)
+        && one(a3) && a3.C == cm && a3.in_cs == cm && a3.K == cw && a3.out_cs == cw && a3.nslab == cm / 64 && a3.kout_pad >= cw
+        && same_image(a3) && a3.res != nullptr && a3.addq.fast && a3.addq.hi == 255
+        && a1.H % kPatch == 0 && a1.W % kPatch == 0 && (long long)a1.N * a1.H * a1.W * cw < (1ll << 31);
+}
+
+template <int G>
+static void launch_block_g(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3, hipStream_t st)
+{
+    BlockGeom geo;
+    geo.H = a1.H, geo.W = a1.W, geo.PY = a1.H / kPatch, geo.PX = a1.W / kPatch;
+    geo.npatch = a1.N * geo.PY * geo.PX;
+#ifdef HIPQ_BLOCK_STAMPS
+    geo.stamps = getenv("HIPQ_BLOCK_STAMPS") ? (unsigned long long *)strtoull(getenv("HIPQ_BLOCK_STAMPS"), nullptr, 0) : nullptr;
+#endif
+    const dim3 grid((unsigned)((geo.npatch + 7) / 8 * 8)), block(128 * G);
+    if (geo.PY <= 2 && geo.PX <= 2) // every region is at most 8 x 8 pixels
+        hipLaunchKernelGGL((conv_bottleneck_kernel<G, 2>), grid, block, 0, st, a1, a2, a3, geo);
+    else
+        hipLaunchKernelGGL((conv_bottleneck_kernel<G, 3>), grid, block, 0, st, a1, a2, a3, geo);
+}
+
+void launch_conv_block(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3, hipStream_t st)
+{
+    switch (a1.out_cs) {
+    case 64: launch_block_g<1>(a1, a2, a3, st); break;
+    case 128: launch_block_g<2>(a1, a2, a3, st); break;
+    default: launch_block_g<4>(a1, a2, a3, st); break; // conv_block_applies: 64, 128 or 256 middle channels
+    }
+}
+
+} // namespace hipq

@@ -17,6 +17,11 @@ struct ConvArgs {
     uint8_t *y;
     int32_t *acc_out;
     const uint8_t *wpack; // MFMA: [slab][kout_pad][64] swizzled int8; depthwise: [tap][cs] int16
+    // MFMA plans over whole 64-byte channel slabs with at most 1024 input and output channels: the same weights in
+    // fragment order - the 1 KB that a wave loads as one MFMA operand (32-channel tile T, k-step kk of slab s: lane
+    // 32 h + p holds bytes [32 kk + 16 h, + 16) of channel 32 T + 16 ((p >> 2) & 1) + 4 (p >> 3) + (p & 3), so that a lane's 16
+    // accumulators are 16 consecutive channels) contiguous at ((s * kout_pad / 32 + T) * 2 + kk) * 1024; else nullptr
+    const uint8_t *wfrag;
     const int32_t *bias2; // per output channel, padded to kout_pad
     const uint8_t *padbuf; // 64 bytes of the byte izp (source of out-of-image taps)
     int N, C, H, W, K, OH, OW;

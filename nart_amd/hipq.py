@@ -57,6 +57,9 @@ _SIGS = {
     "hipq_conv2d_add_conv_fusable": (C.c_int, [C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_float, C.c_int, C.c_int, C.c_void_p]),
     "hipq_conv2d_run_add_conv": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_float, C.c_int,
                                            C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
+    "hipq_bottleneck_fusable": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_int]),
+    "hipq_bottleneck_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_int,
+                                      C.c_void_p, C.c_void_p]),
     "hipq_conv2d_maxpool_fusable": (C.c_int, [C.c_void_p] + [C.c_int] * 5 + [C.c_float, C.c_int, C.c_float, C.c_int, C.c_int]),
     "hipq_conv2d_run_maxpool": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
     "hipq_ip_reorder_weights": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 6),
@@ -273,6 +276,18 @@ class Conv2d:
             self.close()
         except Exception:
             pass
+
+
+def bottleneck_fusable(reduce, mid, widen, residual_first, oalpha, ozp, obits=8):
+    """Can the identity bottleneck block reduce -> mid -> widen -> add(., x) run as one kernel (include/hipq.h)?"""
+    return bool(lib().hipq_bottleneck_fusable(reduce.handle, mid.handle, widen.handle, int(bool(residual_first)), oalpha, ozp, obits))
+
+
+def bottleneck_run(reduce, mid, widen, x, residual_first, oalpha, ozp, y, obits=8):
+    """y = add(widen(mid(reduce(x))), x) in one launch (include/hipq.h: hipq_bottleneck_run)."""
+    check(lib().hipq_bottleneck_run(reduce.handle, mid.handle, widen.handle, _ptr(x), int(bool(residual_first)), oalpha, ozp,
+                                    obits, _ptr(y), _stream()))
+    return y
 
 
 def add_u8(a, b, y, ialpha0, izp0, ialpha1, izp1, oalpha, ozp, obits=8):

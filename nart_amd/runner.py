@@ -36,6 +36,8 @@ class HipqExecutor:
                         and not any(a is u[0] for a in self.fused.values())):  # one convolution per add
                     self.fused[node.output] = u[0]  # launched at the add's position: both operands exist by then
         self.pooled = {}     # conv output name -> the max-pooling node computed inside the convolution's kernel
+        self.blocks = {}     # id(add node) -> (reduce, mid, widen conv nodes) of an identity bottleneck block run as one kernel
+        self.in_block = {}   # id(conv node) -> the add node of its block
         self.dequantized = {}  # fully-connected output name -> the dequantize node computed in the layer's epilogue
         self.chained = {}    # add output name -> the 1x1 convolution node computed inside the fused add's kernel
         self._early = {}     # id(conv node) -> its plan, created ahead of its turn (when an add looked at it)
@@ -56,6 +58,8 @@ class HipqExecutor:
             nbytes = int(np.prod(x.shape)) + int(np.prod(y.shape)) + case.weights[a["w"]].size + 4 * a["K"]
             return plan, nbytes
 
+        if fuse_add:
+            self._find_blocks(conv_plan)
         done = set()  # nodes computed inside an earlier node's kernel
         for node in case.nodes:
             if id(node) in done:
@@ -79,6 +83,19 @@ class HipqExecutor:
                 x = xs[0]
                 fn = (lambda i=ins[0], o=out, x=x: hipq.dequantize_u8(i, o, x.alpha, x.zp))
                 self._add(node, "dequantize_u8_kernel", fn, 0, 5 * int(np.prod(y.shape)))
+            elif node.kind == "conv" and id(node) in self.in_block:
+                self.buf.pop(y.name, None)  # computed inside the block's kernel, never materialised
+                continue
+            elif node.kind == "add" and id(node) in self.blocks:
+                c1, c2, c3 = self.blocks[id(node)]
+                plans = [self._early.pop(id(c)) for c in (c1, c2, c3)]
+                self.plans += plans
+                xin = self.buf[c1.inputs[0]]
+                res_first = node.inputs[0] == c1.inputs[0]
+                fn = (lambda ps=plans, i=xin, rf=res_first, y=y, o=out: hipq.bottleneck_run(ps[0], ps[1], ps[2], i, rf, y.alpha, y.zp, o))
+                nb = 2 * int(np.prod(y.shape)) + sum(case.weights[c.attrs["w"]].size + 4 * c.attrs["K"] for c in (c1, c2, c3))
+                self.steps.append({"label": node.output, "kind": "block", "kernel": "conv_mfma_i8_bottleneck", "fn": fn,
+                                   "ops": sum(p.ops for p in plans), "bytes": nb, "plan": plans[0]})
             elif node.kind == "conv":
                 x = xs[0]
                 plan, nbytes = conv_plan(node)
@@ -152,7 +169,8 @@ class HipqExecutor:
                 for nd in case.nodes:
                     na = nd.attrs
                     if (nd.kind == "conv" and nd.inputs[0] == node.output and na["k"] == 1 and na["stride"] == 1
-                            and na["pad"] == 0 and na["group"] == 1 and nd.output != case.output.name):
+                            and na["pad"] == 0 and na["group"] == 1 and nd.output != case.output.name
+                            and id(nd) not in self.in_block):
                         p2, nb2 = conv_plan(nd)
                         if plan.add_conv_fusable(res_first, ot.alpha, ot.zp, st.alpha, st.zp, p2):
                             nxt = (nd, p2, nb2)
@@ -184,6 +202,46 @@ class HipqExecutor:
             else:
                 raise ValueError("unknown node kind " + node.kind)
 
+    def _find_blocks(self, conv_plan):
+        """Identity bottleneck blocks - 1x1, 3x3, 1x1 and the add of the last one's output with the first one's input,
+        every intermediate tensor read by nobody else - that hipq_bottleneck_run computes in one launch."""
+        case = self.case
+        T = case.tensors
+        prod = {n.output: n for n in case.nodes}
+        uses = {}
+        for n in case.nodes:
+            for i in n.inputs:
+                uses.setdefault(i, []).append(n)
+
+        def only_conv(name, k):
+            n = prod.get(name)
+            if (n is None or n.kind != "conv" or n.attrs["k"] != k or n.attrs["stride"] != 1 or n.attrs["group"] != 1
+                    or n.attrs["relu"] or len(uses.get(name, [])) != 1 or name == case.output.name):
+                return None
+            return n
+        for add in case.nodes:
+            if add.kind != "add" or len(add.inputs) != 2 or add.inputs[0] == add.inputs[1]:
+                continue
+            for ci in (0, 1):
+                c3 = only_conv(add.inputs[ci], 1)
+                c2 = only_conv(c3.inputs[0], 3) if c3 else None
+                c1 = only_conv(c2.inputs[0], 1) if c2 else None
+                if c1 is None or c1.inputs[0] != add.inputs[1 - ci] or any(id(c) in self.in_block for c in (c1, c2, c3)):
+                    continue
+                if T[c1.inputs[0]].dtype != "u8" or c1.attrs["pad"] != 0 or c3.attrs["pad"] != 0 or c2.attrs["pad"] != 1:
+                    continue
+                plans = [conv_plan(c)[0] for c in (c1, c2, c3)]
+                st = T[add.output]
+                if hipq.bottleneck_fusable(plans[0], plans[1], plans[2], ci == 1, st.alpha, st.zp):
+                    self.blocks[id(add)] = (c1, c2, c3)
+                    for c, p in zip((c1, c2, c3), plans):
+                        self.in_block[id(c)] = add
+                        self._early[id(c)] = p
+                        self.fused.pop(c.output, None)
+                    break
+                for c, p in zip((c1, c2, c3), plans):
+                    self._early.setdefault(id(c), p)  # keep the plans for the operators' own turns
+
     def _tensor(self, t):
         N, C, H, W = t.shape
         if self.share is not None:
@@ -202,7 +260,7 @@ class HipqExecutor:
     @property
     def elided(self):
         """Names of the tensors that are never materialised (absorbed into a fused kernel)."""
-        return set(self.fused) | set(self.pooled) | set(self.dequantized)
+        return set(self.fused) | set(self.pooled) | set(self.dequantized) | {c.output for cs in self.blocks.values() for c in cs}
 
     def set_input(self, x):
         inp = self.case.input
