@@ -243,6 +243,25 @@ int hipq_bottleneck_run(const hipq_conv2d_plan *reduce, const hipq_conv2d_plan *
                         const void *x, int residual_is_input0, float oalpha, int ozp, int obits, void *y, void *stream);
 
 /*
+ * The rest of a bottleneck block in one launch, from its 3x3 convolution on: y = add(widen(mid(x)), residual) and, when
+ * `next` is not NULL, y_next = next(y) - bit-identical to hipq_conv2d_run(mid, x, t), hipq_conv2d_run_add(widen, t,
+ * residual, ...) and hipq_conv2d_run(next, y, y_next): op_conv_2d_u8xu8_run (src/op/conv_2d_uint8_impl.c:39-165), then
+ * op_quant_add_run (src/op/add.c:83-148), then op_conv_2d_u8xu8_run again; t never travels to memory and y is written
+ * but not read back.  `mid`: 3x3 / stride 1 / pad 1, CM -> CM with CM = 64, 128 or 256; `widen`: 1x1, CM -> 4 CM;
+ * `next`: 1x1 / stride 1, 4 CM -> CM (the first layer of the next block); images of 8 x 8, 4 x 14 or 7 x 7 pixel patches
+ * (height and width multiples of 8 and 8, of 4 and 14, or of 7 and 7); uint8 tensors with dense channel strides, weight
+ * zero points 128, per-tensor weight scales, each layer reading its input with the scale and zero point it is written
+ * with.  The residual (any tensor of y's shape, e.g. a projection shortcut) and the add are described as in
+ * hipq_conv2d_run_add; next_relu as in hipq_conv2d_run_add_conv.  hipq_bottleneck_tail_fusable answers (1 / 0);
+ * hipq_bottleneck_tail_run fails with an error otherwise (run the operators separately).
+ */
+int hipq_bottleneck_tail_fusable(const hipq_conv2d_plan *mid, const hipq_conv2d_plan *widen, int residual_is_input0,
+                                 float res_alpha, int res_zp, float oalpha, int ozp, int obits, const hipq_conv2d_plan *next);
+int hipq_bottleneck_tail_run(const hipq_conv2d_plan *mid, const hipq_conv2d_plan *widen, const void *x, const void *residual,
+                             int residual_is_input0, float res_alpha, int res_zp, float oalpha, int ozp, int obits, void *y,
+                             const hipq_conv2d_plan *next, int next_relu, void *y_next, void *stream);
+
+/*
  * Convolution with the max pooling that follows it in one kernel: y = maxpool3x3/2/1(conv(x)), bit-identical to
  * hipq_conv2d_run followed by hipq_pool_u8(HIPQ_POOL_MAX, kernel 3, stride 2, pad 1) whose input and output scale and
  * zero point both equal the convolution's output parameters (op_conv_2d_u8xu8_run, then op_quant_pool_max_run -

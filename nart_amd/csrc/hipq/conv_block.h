@@ -11,4 +11,9 @@ namespace hipq {
 bool conv_block_applies(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3);
 void launch_conv_block(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3, hipStream_t st);
 
+// The chain cut one layer later: a2 (3x3 / stride 1 / pad 1, reads a2.x), a3 (the widening 1x1 with the residual a3.res and
+// the add's parameters, sum to a3.y) and - an != nullptr - the 1x1 convolution that reads the sum (output to an->y).
+bool conv_block_tail_applies(const ConvArgs &a2, const ConvArgs &a3, const ConvArgs *an);
+void launch_conv_block_tail(const ConvArgs &a2, const ConvArgs &a3, const ConvArgs *an, hipStream_t st);
+
 } // namespace hipq

@@ -457,6 +457,273 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// The same machinery cut one layer later: the 3x3 convolution of a bottleneck block, its widening 1x1 convolution with
+// the residual add, and - CHAIN - the 1x1 convolution that reads the sum (the first layer of the NEXT block), for the
+// stages with many pixels per image (56x56, 28x28).  Cutting the chain at the narrowest tensor means that a work-group
+// re-reads a border of 64 G bytes per pixel instead of recomputing a layer on it, needs no x tile in LDS (the residual
+// may be any tensor, e.g. a projection shortcut, and comes straight from memory a chunk ahead of its use), and - the
+// next layer being 1x1 - can finish that layer for exactly its own pixels.  A work-group owns a PH x PW patch of one
+// image (8x8, 4x14 or 7x7: 64, 56 or 49 of its 64 pixel slots do useful vector arithmetic):
+//   * the patch of the 3x3 layer's input with its border, (PH + 2) x (PW + 2) pixel rows of CM bytes, goes to LDS
+//     (out-of-image positions hold the pad byte);
+//   * layer 2 (3x3) as above, on the compact pixel index q = PW * row + column, its bytes to LDS;
+//   * layer 3 + add as above, the sum stored and - CHAIN - kept in LDS, 64 pixel rows of CW bytes;
+//   * CHAIN: the next layer (CW -> CM) reads that tile as its pixel operand, the pairs splitting the reduction again.
+template <int G, int PH, int PW, bool CHAIN>
+__global__ __launch_bounds__(128 * G, (G <= 2 ? 3 : 2)) void conv_bottleneck_tail_kernel(const ConvArgs a2, const ConvArgs a3, const ConvArgs an,
+                                                                         const BlockGeom geo)
+{
+    constexpr int NW = 2 * G, NT = 128 * G, CM = 64 * G, CW = 256 * G;
+    constexpr int GW = PW + 2, GH = PH + 2, NPIX = PH * PW, GROWS = (GH * GW + 7) / 8 * 8;
+    constexpr int G_OFF = 0, G_BYTES = GROWS * CM;            // layer 2's input on the bordered grid
+    constexpr int M_OFF = G_OFF + G_BYTES, M_BYTES = 64 * CM; // layer 2's bytes, row = pixel
+    constexpr int S_OFF = M_OFF + M_BYTES, S_BYTES = CHAIN ? 64 * CW : NW * 4096; // layer 2's exchange slots, then the sum tile
+    constexpr int D2 = G == 1 ? 4 : G == 2 ? 3 : 6, DN = D2; // slabs of weights a wave holds ahead (three waves per SIMD: fewer registers)
+    static_assert(NPIX <= 64 && NW * 4096 <= S_BYTES && NW * 4096 <= G_BYTES + M_BYTES, "slot reuse");
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[S_OFF + S_BYTES];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int p = lane & 31, h = lane >> 5;
+    const int ng = wave % G, kh = wave / G, partner = (wave + G) % NW;
+    const int gid = (int)(blockIdx.x % 8) * (int)(gridDim.x / 8) + (int)(blockIdx.x / 8); // XCD x: the x-th eighth of the patches
+    if (gid >= geo.npatch)
+        return;
+    const int ppi = geo.PY * geo.PX;
+    const int n = gid / ppi, pr = gid - n * ppi, pi = pr / geo.PX, pj = pr - pi * geo.PX;
+    const int y0 = pi * PH, x0 = pj * PW;
+    STAMP(0);
+
+    // ---- the 3x3 layer's input patch with its border -> LDS, re-centred; out-of-image positions read the pad source ----
+    {
+        constexpr int CPR = CM / 16, ITEMS = GROWS * CPR;
+#pragma unroll
+        for (int k = 0; k < (ITEMS + NT - 1) / NT; k++) {
+            const int it = tid + k * NT;
+            if (ITEMS % NT == 0 || it < ITEMS) {
+                const int g = it / CPR, c = it % CPR;
+                const int gy = g / GW, gx = g - gy * GW;
+                const int iy = y0 - 1 + gy, ix = x0 - 1 + gx;
+                const bool in = g < GH * GW && (unsigned)iy < (unsigned)geo.H && (unsigned)ix < (unsigned)geo.W;
+                const uint8_t *src = in ? a2.x + (size_t)((n * geo.H + iy) * geo.W + ix) * CM + c * 16 : a2.padbuf;
+                *reinterpret_cast<v4i *>(lds + G_OFF + g * CM + ((c ^ swz<CM>(g)) << 4)) = ldg128(src) ^ (int)a2.xmask;
+            }
+        }
+    }
+    const int ct0 = 64 * ng + 32 * kh, ct1 = 64 * ng + 32 * (1 - kh);
+    const size_t wslab2 = (size_t)a2.kout_pad * 64, wslab3 = (size_t)a3.kout_pad * 64, wslabn = (size_t)an.kout_pad * 64;
+    const uint8_t *w20 = a2.wfrag + (size_t)ct0 * 64 + lane * 16, *w21 = a2.wfrag + (size_t)ct1 * 64 + lane * 16;
+    auto ldw2 = [&](int s, int kk, int nt) { return ldg128((nt ? w21 : w20) + (size_t)s * wslab2 + kk * 1024); };
+    // the lane's pixels q = 32 t + p (slots beyond the patch repeat its last pixel and are never stored)
+    int grow[2];
+    size_t pix[2];
+    bool valid[2];
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const int q = 32 * t + p, qq = min(q, NPIX - 1), py = qq / PW, px = qq - py * PW;
+        valid[t] = q < NPIX;
+        grow[t] = (py + 1) * GW + px + 1; // the centre tap's grid row
+        pix[t] = (size_t)((n * geo.H + y0 + py) * geo.W + x0 + px);
+    }
+    auto ldb2 = [&](int s, int kk, int t) {
+        const int tap = s / G, cb = s % G, tr = (tap * 11) >> 5;
+        const int gr = grow[t] + (tr - 1) * GW + (tap - 3 * tr - 1), hs = h ^ swz<CM>(gr);
+        return *reinterpret_cast<const v4i *>(lds + G_OFF + gr * CM + (((4 * cb + 2 * kk) ^ hs) << 4));
+    };
+
+    // ================= layer 2: 3x3, CM -> CM =================
+    WeightRing<D2> r2;
+    ring_fill<9 * G, D2>(r2, kh, ldw2);
+    v16i acc2[2][2];
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        init_acc(acc2[t][0], a2.bias2 + ct0 + 16 * h, kh != 0);
+        init_acc(acc2[t][1], a2.bias2 + ct1 + 16 * h, kh != 0);
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): this thread's part of the grid is written
+    __builtin_amdgcn_s_barrier();
+    STAMP(1);
+    reduce_half<9 * G, 2, D2>(acc2, r2, kh, 0, ldw2, ldb2);
+    STAMP(2);
+    // layer 3: this wave's 128 output channels in 4 chunks of 32; the first chunk's weights, biases and residual travel now
+    const uint8_t *w3 = a3.wfrag + (size_t)(128 * wave) * 64 + lane * 16;
+    v4i wf[2 * G], b3[4], rn[2];
+    auto load_chunk = [&](int cc) {
+#pragma unroll
+        for (int ks = 0; ks < 2 * G; ks++)
+            wf[ks] = ldg128(w3 + (size_t)(ks >> 1) * wslab3 + (size_t)cc * 2048 + (ks & 1) * 1024);
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+            b3[g] = *reinterpret_cast<const v4i *>(a3.bias2 + 128 * wave + 32 * cc + 16 * h + 4 * g);
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+            rn[t] = ldg128(a3.res + pix[t] * CW + 128 * wave + 32 * cc + 16 * h);
+    };
+    load_chunk(0);
+    pair_reduce<2, false>(acc2, lds + S_OFF, wave, partner, lane);
+    STAMP(3);
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        const int q = 32 * t + p;
+        const v4i o = requant16(a2, acc2[t][0], a3.xmask);
+        *reinterpret_cast<v4i *>(lds + M_OFF + q * CM + ((((ct0 >> 4) + h) ^ swz<CM>(q)) << 4)) = o;
+    }
+    __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
+    __builtin_amdgcn_s_barrier();
+
+    STAMP(4);
+    // ================= layer 3: CM -> CW and the residual add =================
+    {
+        v4i bf[2][2 * G];
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            const int q = 32 * t + p;
+#pragma unroll
+            for (int ks = 0; ks < 2 * G; ks++)
+                bf[t][ks] = *reinterpret_cast<const v4i *>(lds + M_OFF + q * CM + (((2 * ks + h) ^ swz<CM>(q)) << 4));
+        }
+        for (int cc = 0; cc < 4; cc++) {
+            const int ch = 128 * wave + 32 * cc;
+            v16i acc[2];
+#pragma unroll
+            for (int g = 0; g < 4; g++)
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    acc[0][4 * g + e] = b3[g][e];
+            acc[1] = acc[0];
+#pragma unroll
+            for (int ks = 0; ks < 2 * G; ks++)
+#pragma unroll
+                for (int t = 0; t < 2; t++)
+                    acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[ks], bf[t][ks], acc[t], 0, 0, 0);
+            const v4i rc[2] = {rn[0], rn[1]};
+            if (cc + 1 < 4)
+                load_chunk(cc + 1); // the next chunk's operands arrive during the arithmetic below
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                const v4i o = requant_add16(a3, acc[t], rc[t]);
+                if (valid[t])
+                    *reinterpret_cast<v4i *>(a3.y + pix[t] * CW + ch + 16 * h) = o;
+                if (CHAIN) { // the sum tile: pixel row q, 16-byte piece c at piece c ^ (q & 15) of every 256 bytes
+                    const int q = 32 * t + p, c16 = (ch >> 4) + h;
+                    *reinterpret_cast<v4i *>(lds + S_OFF + q * CW + (c16 & ~15) * 16 + (((c16 & 15) ^ (q & 15)) << 4)) = o;
+                }
+            }
+            STAMP(5 + cc);
+        }
+    }
+    if (!CHAIN)
+        return;
+
+    // ================= the next block's first layer: CW -> CM on the sum tile =================
+    {
+        const uint8_t *wn0 = an.wfrag + (size_t)ct0 * 64 + lane * 16, *wn1 = an.wfrag + (size_t)ct1 * 64 + lane * 16;
+        auto ldwn = [&](int s, int kk, int nt) { return ldg128((nt ? wn1 : wn0) + (size_t)s * wslabn + kk * 1024); };
+        auto ldbn = [&](int s, int kk, int t) {
+            const int j = 32 * t + p, hs = h ^ (j & 15);
+            return *reinterpret_cast<const v4i *>(lds + S_OFF + j * CW + (s >> 2) * 256 + (((4 * (s & 3) + 2 * kk) ^ hs) << 4));
+        };
+        WeightRing<DN> rr;
+        ring_fill<4 * G, DN>(rr, kh, ldwn);
+        v16i accn[2][2];
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            init_acc(accn[t][0], an.bias2 + ct0 + 16 * h, kh != 0);
+            init_acc(accn[t][1], an.bias2 + ct1 + 16 * h, kh != 0);
+        }
+        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): this wave's part of the sum tile is written
+        __builtin_amdgcn_s_barrier();
+        STAMP(9);
+        reduce_half<4 * G, 2, DN>(accn, rr, kh, (int)an.xmask, ldwn, ldbn);
+        STAMP(10);
+        pair_reduce<2, false>(accn, lds + G_OFF, wave, partner, lane); // the grid and layer 2's tile are long read
+        STAMP(11);
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            const v4i o = requant16(an, accn[t][0], 0);
+            if (valid[t])
+                *reinterpret_cast<v4i *>(an.y + pix[t] * CM + ct0 + 16 * h) = o;
+        }
+        STAMP(12);
+    }
+}
+
+// the patch shape of the tail kernel for an H x W image: 8x8 fills every pixel slot, 4x14 seven in eight, 7x7 three in four
+static bool tail_patch(int H, int W, int *ph, int *pw)
+{
+    if (H % 8 == 0 && W % 8 == 0)
+        *ph = 8, *pw = 8;
+    else if (H % 4 == 0 && W % 14 == 0)
+        *ph = 4, *pw = 14;
+    else if (H % 7 == 0 && W % 7 == 0)
+        *ph = 7, *pw = 7;
+    else
+        return false;
+    return true;
+}
+
+bool conv_block_tail_applies(const ConvArgs &a2, const ConvArgs &a3, const ConvArgs *an)
+{
+    const int cm = a2.in_cs, cw = a3.out_cs;
+    auto plain = [](const ConvArgs &a) {
+        return a.group == 1 && a.bwz == 0 && a.xmask != 0 && a.fastq && a.qmult == nullptr && a.acc_out == nullptr && a.deq_out == nullptr && a.wfrag != nullptr;
+    };
+    auto one = [](const ConvArgs &a) {
+        return a.R == 1 && a.S == 1 && a.pad_h == 0 && a.pad_w == 0 && a.stride_h == 1 && a.stride_w == 1;
+    };
+    auto same_image = [&](const ConvArgs &a) { return a.N == a2.N && a.H == a2.H && a.W == a2.W && a.OH == a2.H && a.OW == a2.W; };
+    int ph, pw;
+    if (!(plain(a2) && plain(a3) && (cm == 64 || cm == 128 || cm == 256) && cw == 4 * cm
+          && a2.R == 3 && a2.S == 3 && a2.pad_h == 1 && a2.pad_w == 1 && a2.stride_h == 1 && a2.stride_w == 1 && a2.C == cm
+          && a2.K == cm && a2.out_cs == cm && a2.nslab == 9 * cm / 64 && a2.kout_pad >= cm && a2.res == nullptr && same_image(a2)
+          && one(a3) && a3.C == cm && a3.in_cs == cm && a3.K == cw && a3.nslab == cm / 64 && a3.kout_pad >= cw && same_image(a3)
+          && a3.res != nullptr && a3.addq.fast && a3.addq.hi == 255 && tail_patch(a2.H, a2.W, &ph, &pw)
+          && (long long)a2.N * a2.H * a2.W * cw < (1ll << 31)))
+        return false;
+    if (an == nullptr)
+        return true;
+    return plain(*an) && one(*an) && an->C == cw && an->in_cs == cw && an->K == cm && an->out_cs == cm && an->nslab == cw / 64
+        && an->kout_pad >= cm && an->res == nullptr && same_image(*an);
+}
+
+template <int G, int PH, int PW>
+static void launch_tail_gp(const ConvArgs &a2, const ConvArgs &a3, const ConvArgs *an, hipStream_t st)
+{
+    BlockGeom geo;
+    geo.H = a2.H, geo.W = a2.W, geo.PY = a2.H / PH, geo.PX = a2.W / PW;
+    geo.npatch = a2.N * geo.PY * geo.PX;
+#ifdef HIPQ_BLOCK_STAMPS
+    geo.stamps = getenv("HIPQ_BLOCK_STAMPS") ? (unsigned long long *)strtoull(getenv("HIPQ_BLOCK_STAMPS"), nullptr, 0) : nullptr;
+#endif
+    const dim3 grid((unsigned)((geo.npatch + 7) / 8 * 8)), block(128 * G);
+    if (an)
+        hipLaunchKernelGGL((conv_bottleneck_tail_kernel<G, PH, PW, true>), grid, block, 0, st, a2, a3, *an, geo);
+    else
+        hipLaunchKernelGGL((conv_bottleneck_tail_kernel<G, PH, PW, false>), grid, block, 0, st, a2, a3, a3, geo);
+}
+
+template <int G>
+static void launch_tail_g(const ConvArgs &a2, const ConvArgs &a3, const ConvArgs *an, hipStream_t st)
+{
+    int ph = 0, pw = 0;
+    tail_patch(a2.H, a2.W, &ph, &pw);
+    if (ph == 8)
+        launch_tail_gp<G, 8, 8>(a2, a3, an, st);
+    else if (ph == 4)
+        launch_tail_gp<G, 4, 14>(a2, a3, an, st);
+    else
+        launch_tail_gp<G, 7, 7>(a2, a3, an, st);
+}
+
+void launch_conv_block_tail(const ConvArgs &a2, const ConvArgs &a3, const ConvArgs *an, hipStream_t st)
+{
+    switch (a2.in_cs) {
+    case 64: launch_tail_g<1>(a2, a3, an, st); break;
+    case 128: launch_tail_g<2>(a2, a3, an, st); break;
+    default: launch_tail_g<4>(a2, a3, an, st); break; // conv_block_tail_applies: 64, 128 or 256 middle channels
+    }
+}
+
 bool conv_block_applies(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3)
 {
     const int cm = a1.out_cs, cw = a1.in_cs;

@@ -60,6 +60,10 @@ _SIGS = {
     "hipq_bottleneck_fusable": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_int]),
     "hipq_bottleneck_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_int,
                                       C.c_void_p, C.c_void_p]),
+    "hipq_bottleneck_tail_fusable": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_float, C.c_int, C.c_int,
+                                               C.c_void_p]),
+    "hipq_bottleneck_tail_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_float,
+                                           C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
     "hipq_conv2d_maxpool_fusable": (C.c_int, [C.c_void_p] + [C.c_int] * 5 + [C.c_float, C.c_int, C.c_float, C.c_int, C.c_int]),
     "hipq_conv2d_run_maxpool": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
     "hipq_ip_reorder_weights": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 6),
@@ -287,6 +291,21 @@ def bottleneck_run(reduce, mid, widen, x, residual_first, oalpha, ozp, y, obits=
     """y = add(widen(mid(reduce(x))), x) in one launch (include/hipq.h: hipq_bottleneck_run)."""
     check(lib().hipq_bottleneck_run(reduce.handle, mid.handle, widen.handle, _ptr(x), int(bool(residual_first)), oalpha, ozp,
                                     obits, _ptr(y), _stream()))
+    return y
+
+
+def bottleneck_tail_fusable(mid, widen, residual_first, res_alpha, res_zp, oalpha, ozp, nxt=None, obits=8):
+    """Can mid (3x3) -> widen (1x1) -> add(., residual) [-> nxt (1x1)] run as one kernel (include/hipq.h)?"""
+    return bool(lib().hipq_bottleneck_tail_fusable(mid.handle, widen.handle, int(bool(residual_first)), res_alpha, res_zp, oalpha,
+                                                   ozp, obits, nxt.handle if nxt is not None else None))
+
+
+def bottleneck_tail_run(mid, widen, x, residual, residual_first, res_alpha, res_zp, oalpha, ozp, y, nxt=None, y_next=None,
+                        next_relu=False, obits=8):
+    """y = add(widen(mid(x)), residual) and y_next = nxt(y) in one launch (include/hipq.h: hipq_bottleneck_tail_run)."""
+    check(lib().hipq_bottleneck_tail_run(mid.handle, widen.handle, _ptr(x), _ptr(residual), int(bool(residual_first)), res_alpha,
+                                         res_zp, oalpha, ozp, obits, _ptr(y), nxt.handle if nxt is not None else None,
+                                         int(bool(next_relu)), _ptr(y_next), _stream()))
     return y
 
 

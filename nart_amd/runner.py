@@ -38,6 +38,7 @@ class HipqExecutor:
         self.pooled = {}     # conv output name -> the max-pooling node computed inside the convolution's kernel
         self.blocks = {}     # id(add node) -> (reduce, mid, widen conv nodes) of an identity bottleneck block run as one kernel
         self.in_block = {}   # id(conv node) -> the add node of its block
+        self.tails = {}      # id(add node) -> (mid, widen, next or None): the block from its 3x3 layer on as one kernel
         self.dequantized = {}  # fully-connected output name -> the dequantize node computed in the layer's epilogue
         self.chained = {}    # add output name -> the 1x1 convolution node computed inside the fused add's kernel
         self._early = {}     # id(conv node) -> its plan, created ahead of its turn (when an add looked at it)
@@ -96,6 +97,29 @@ class HipqExecutor:
                 nb = 2 * int(np.prod(y.shape)) + sum(case.weights[c.attrs["w"]].size + 4 * c.attrs["K"] for c in (c1, c2, c3))
                 self.steps.append({"label": node.output, "kind": "block", "kernel": "conv_mfma_i8_bottleneck", "fn": fn,
                                    "ops": sum(p.ops for p in plans), "bytes": nb, "plan": plans[0]})
+            elif node.kind == "add" and id(node) in self.tails:
+                c2, c3, nxt = self.tails[id(node)]
+                convs = [c for c in (c2, c3, nxt) if c is not None]
+                plans = [self._early.pop(id(c)) for c in convs]
+                self.plans += plans
+                other = [i for i in node.inputs if i != c3.output][0]
+                res_first = node.inputs[0] == other
+                ot = T[other]
+                y2 = None
+                if nxt is not None:
+                    y2 = self._tensor(T[nxt.output])
+                    if y2 is None:
+                        raise RuntimeError("shared executor: %s is fused away in the parent but not here" % nxt.output)
+                    self.buf[nxt.output] = y2
+                    self.chained[node.output] = nxt
+                    done.add(id(nxt))
+                fn = (lambda ps=plans, i=self.buf[c2.inputs[0]], r=self.buf[other], rf=res_first, ot=ot, y=y, o=out, y2=y2:
+                      hipq.bottleneck_tail_run(ps[0], ps[1], i, r, rf, ot.alpha, ot.zp, y.alpha, y.zp, o,
+                                               ps[2] if len(ps) > 2 else None, y2))
+                nb = (int(np.prod(T[c2.inputs[0]].shape)) + 2 * int(np.prod(y.shape)) + (int(np.prod(T[nxt.output].shape)) if nxt else 0)
+                      + sum(case.weights[c.attrs["w"]].size + 4 * c.attrs["K"] for c in convs))
+                self.steps.append({"label": node.output, "kind": "block tail", "kernel": "conv_mfma_i8_bottleneck_tail" + ("+conv" if nxt else ""),
+                                   "fn": fn, "ops": sum(p.ops for p in plans), "bytes": nb, "plan": plans[0]})
             elif node.kind == "conv":
                 x = xs[0]
                 plan, nbytes = conv_plan(node)
@@ -241,6 +265,36 @@ class HipqExecutor:
                     break
                 for c, p in zip((c1, c2, c3), plans):
                     self._early.setdefault(id(c), p)  # keep the plans for the operators' own turns
+            if id(add) in self.blocks:
+                continue
+            # the block from its 3x3 layer on, with any residual, and the 1x1 layer that reads the sum
+            for ci in (0, 1):
+                c3 = only_conv(add.inputs[ci], 1)
+                c2 = only_conv(c3.inputs[0], 3) if c3 else None
+                if c2 is None or any(id(c) in self.in_block for c in (c2, c3)) or c3.attrs["pad"] != 0 or c2.attrs["pad"] != 1:
+                    continue
+                p2, p3 = conv_plan(c2)[0], conv_plan(c3)[0]
+                st, ot = T[add.output], T[add.inputs[1 - ci]]
+                nxt, pn = None, None
+                for nd in uses.get(add.output, []):
+                    na = nd.attrs
+                    if (nd.kind == "conv" and na["k"] == 1 and na["stride"] == 1 and na["pad"] == 0 and na["group"] == 1
+                            and not na["relu"] and nd.output != case.output.name and id(nd) not in self.in_block
+                            and not any(t[2] is nd for t in self.tails.values())):
+                        cand = conv_plan(nd)[0]
+                        self._early[id(nd)] = cand
+                        if hipq.bottleneck_tail_fusable(p2, p3, ci == 1, ot.alpha, ot.zp, st.alpha, st.zp, cand):
+                            nxt, pn = nd, cand
+                            break
+                if nxt is not None or hipq.bottleneck_tail_fusable(p2, p3, ci == 1, ot.alpha, ot.zp, st.alpha, st.zp):
+                    self.tails[id(add)] = (c2, c3, nxt)
+                    for c, pl in ((c2, p2), (c3, p3)):
+                        self.in_block[id(c)] = add
+                        self._early[id(c)] = pl
+                        self.fused.pop(c.output, None)
+                    break
+                self._early.setdefault(id(c2), p2)
+                self._early.setdefault(id(c3), p3)
 
     def _tensor(self, t):
         N, C, H, W = t.shape
@@ -260,7 +314,7 @@ class HipqExecutor:
     @property
     def elided(self):
         """Names of the tensors that are never materialised (absorbed into a fused kernel)."""
-        return set(self.fused) | set(self.pooled) | set(self.dequantized) | {c.output for cs in self.blocks.values() for c in cs}
+        return set(self.fused) | set(self.pooled) | set(self.dequantized) | {c.output for cs in self.blocks.values() for c in cs} | {c.output for cs in self.tails.values() for c in cs[:2]}
 
     def set_input(self, x):
         inp = self.case.input

@@ -88,6 +88,146 @@ def test_bottleneck_block(case):
         assert torch.equal(y, y2)
 
 
+TAIL_CASES = [  # N, CW, H, W: patches of 8 x 8, 4 x 14 and 7 x 7 pixels; 64, 128 and 256 middle channels
+    (1, 256, 16, 24), (2, 512, 8, 28), (2, 256, 14, 21), (1, 1024, 8, 8), (1, 512, 56, 8), (3, 256, 4, 14), (1, 1024, 7, 7),
+]
+
+
+def make_tail(rng, N, CW, H, W, relu_next):
+    """The block from its 3x3 layer on: t1 [N, CM, H, W] -> 3x3 -> 1x1 to CW -> add(., residual) -> 1x1 back to CM."""
+    CM = CW // 4
+    t1 = rng.integers(0, 256, (N, CM, H, W), dtype=np.uint8)
+    res = rng.integers(0, 256, (N, CW, H, W), dtype=np.uint8)
+    ia, iz = 0.04, int(rng.integers(0, 256))
+    layers = []
+    for (K, C, k), oz in zip(((CM, CM, 3), (CW, CM, 1)), (int(rng.integers(0, 30)), None)):
+        w = rng.integers(1, 256, (K, C, k, k), dtype=np.uint8)
+        sigma = 74.0 * 74.0 * math.sqrt(C * k * k)
+        b = rng.integers(-int(sigma), int(sigma) + 1, K).astype(np.int32)
+        oa = float(np.float32(ia * rng.uniform(0.75, 1.35)))
+        wa = float(np.float32(oa * 40.0 / (ia * sigma)))
+        oz = int(rng.integers(96, 160)) if oz is None else oz
+        layers.append(dict(w=w, b=b, pad=k // 2, q=(ia, iz, wa, 128, oa, oz)))
+        ia, iz = oa, oz
+    ra, rz = float(np.float32(ia * rng.uniform(0.6, 1.6))), int(rng.integers(0, 256))
+    sa, sz = float(np.float32(math.hypot(ia, ra) * 1.1)), int(rng.integers(0, 40))
+    w = rng.integers(1, 256, (CM, CW, 1, 1), dtype=np.uint8)
+    sigma = 74.0 * 74.0 * math.sqrt(CW)
+    b = rng.integers(-int(sigma), int(sigma) + 1, CM).astype(np.int32)
+    oa = float(np.float32(sa * rng.uniform(0.75, 1.35)))
+    nxt = dict(w=w, b=b, pad=0, q=(sa, sz, float(np.float32(oa * 40.0 / (sa * sigma))), 128, oa, int(rng.integers(20, 60))), relu=relu_next)
+    return t1, res, layers, (ra, rz), (sa, sz), nxt
+
+
+@pytest.mark.parametrize("case", TAIL_CASES, ids=lambda c: "x".join(map(str, c)))
+def test_bottleneck_tail(case):
+    """hipq_bottleneck_tail_run == 3x3 convolution, widening convolution, add with any residual and - chained - the next
+    1x1 convolution run one by one by the oracle: both operand orders of the add, with and without the chained layer, a
+    ReLU on the chained layer, every patch shape and channel count."""
+    N, CW, H, W = case
+    CM = CW // 4
+    rng = np.random.default_rng(2000 + CW + H)
+    for res_first, chain, relu_next in ((False, True, False), (True, True, True), (True, False, False)):
+        t1, res, layers, rq, sq, nx = make_tail(rng, N, CW, H, W, relu_next)
+        plans = plans_of(t1, layers)
+        pn = hipq.Conv2d((N, CW, H, W), nx["w"], nx["b"], 0, 1, 1, *nx["q"])
+        print("tail case", case, res_first, chain, relu_next, [p.kernel for p in plans], flush=True)
+        assert hipq.bottleneck_tail_fusable(plans[0], plans[1], res_first, rq[0], rq[1], sq[0], sq[1], pn if chain else None)
+        t = orc.conv2d_u8(t1, layers[0]["w"], layers[0]["b"], 1, 1, 1, *layers[0]["q"])
+        c = orc.conv2d_u8(t, layers[1]["w"], layers[1]["b"], 0, 1, 1, *layers[1]["q"])
+        q3 = layers[1]["q"]
+        want = orc.add_u8(res, c, rq[0], rq[1], q3[4], q3[5], sq[0], sq[1]) if res_first else orc.add_u8(c, res, q3[4], q3[5], rq[0], rq[1], sq[0], sq[1])
+        xd, rd = hipq.to_device_nhwc(t1), hipq.to_device_nhwc(res)
+        y = torch.zeros_like(rd)
+        yn = torch.zeros_like(xd) if chain else None
+        hipq.bottleneck_tail_run(plans[0], plans[1], xd, rd, res_first, rq[0], rq[1], sq[0], sq[1], y, pn if chain else None, yn,
+                                 next_relu=relu_next)
+        torch.cuda.synchronize()
+        got = hipq.from_device_nhwc(y, CW)
+        bad = got != want
+        assert not bad.any(), (case, res_first, chain, int(bad.sum()), np.argwhere(bad)[:8].tolist())
+        if chain:
+            wantn = orc.conv2d_u8(want, nx["w"], nx["b"], 0, 1, 1, *nx["q"])
+            if relu_next:
+                wantn = np.maximum(wantn, nx["q"][5]).astype(np.uint8)
+            gotn = hipq.from_device_nhwc(yn, CM)
+            bad = gotn != wantn
+            assert not bad.any(), (case, "next layer", relu_next, int(bad.sum()), np.argwhere(bad)[:8].tolist())
+
+
+def test_bottleneck_refusals():
+    """What the one-launch forms do not serve is refused by the predicates and fails loudly in the run entry points."""
+    rng = np.random.default_rng(7)
+    x, xq, layers, sq = make_block(rng, 1, 256, 10, 14)  # a height that is no multiple of 7
+    plans = plans_of(x, layers)
+    assert not hipq.bottleneck_fusable(*plans, False, sq[0], sq[1])
+    xd = hipq.to_device_nhwc(x)
+    with pytest.raises(hipq.HipqError, match="do not run as one kernel"):
+        hipq.bottleneck_run(*plans, xd, False, sq[0], sq[1], torch.zeros_like(xd))
+    x, xq, layers, sq = make_block(rng, 1, 256, 14, 14)
+    plans = plans_of(x, layers)
+    xd = hipq.to_device_nhwc(x)
+    with pytest.raises(hipq.HipqError, match="cannot overwrite"):
+        hipq.bottleneck_run(*plans, xd, False, sq[0], sq[1], xd)
+    assert not hipq.bottleneck_fusable(*plans, False, sq[0], sq[1], obits=7)
+    # the tail form: a stride-2 3x3 layer, and a chained layer that reads the sum with another zero point
+    t1, res, tl, rq, sq2, nx = make_tail(rng, 1, 256, 16, 16, False)
+    p2s = hipq.Conv2d(t1.shape, tl[0]["w"], tl[0]["b"], 1, 2, 1, *tl[0]["q"]).special(2)
+    p3 = hipq.Conv2d((1, 64, 8, 8), tl[1]["w"], tl[1]["b"], 0, 1, 1, *tl[1]["q"])
+    assert not hipq.bottleneck_tail_fusable(p2s, p3, False, rq[0], rq[1], sq2[0], sq2[1])
+    plans = plans_of(t1, tl)
+    q = list(nx["q"])
+    q[1] = (q[1] + 1) % 256
+    pn = hipq.Conv2d((1, 256, 16, 16), nx["w"], nx["b"], 0, 1, 1, *q)
+    assert hipq.bottleneck_tail_fusable(plans[0], plans[1], False, rq[0], rq[1], sq2[0], sq2[1])
+    assert not hipq.bottleneck_tail_fusable(plans[0], plans[1], False, rq[0], rq[1], sq2[0], sq2[1], pn)
+    xd, rd = hipq.to_device_nhwc(t1), hipq.to_device_nhwc(res)
+    with pytest.raises(hipq.HipqError, match="do not run as one kernel"):
+        hipq.bottleneck_tail_run(plans[0], plans[1], xd, rd, False, rq[0], rq[1], sq2[0], sq2[1], torch.zeros_like(rd), pn, torch.zeros_like(xd))
+
+
+def time_tail(N, CW, HW, reps=50):
+    rng = np.random.default_rng(6)
+    t1, res, layers, rq, sq, nx = make_tail(rng, N, CW, HW, HW, False)
+    plans = plans_of(t1, layers)
+    pn = hipq.Conv2d((N, CW, HW, HW), nx["w"], nx["b"], 0, 1, 1, *nx["q"])
+    xd, rd = hipq.to_device_nhwc(t1), hipq.to_device_nhwc(res)
+    y, yn, t = torch.zeros_like(rd), torch.zeros_like(xd), torch.zeros_like(xd)
+    fusable = plans[1].add_conv_fusable(False, rq[0], rq[1], sq[0], sq[1], pn)
+
+    def fused():
+        hipq.bottleneck_tail_run(plans[0], plans[1], xd, rd, False, rq[0], rq[1], sq[0], sq[1], y, pn, yn)
+
+    def separate():
+        plans[0](xd, t)
+        if fusable:
+            plans[1].run_add_conv(t, rd, False, rq[0], rq[1], sq[0], sq[1], y, pn, yn)
+        else:
+            plans[1].run_add(t, rd, False, rq[0], rq[1], sq[0], sq[1], y)
+            pn(y, yn)
+
+    out = {}
+    for name, fn in (("fused", fused), ("separate", separate)):
+        fn()
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for _ in range(10):
+                fn()
+        for _ in range(3):
+            g.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(reps):
+            g.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        out[name] = e0.elapsed_time(e1) / reps / 10 * 1e3
+    print("tail N=%d CW=%d %dx%d: fused %.1f us, separate (%s, %s) %.1f us" % (
+        N, CW, HW, HW, out["fused"], plans[0].kernel, "expand+add+conv" if fusable else "add, conv", out["separate"]), flush=True)
+
+
 def time_block(N, CW, HW, reps=50):
     rng = np.random.default_rng(5)
     x, xq, layers, sq = make_block(rng, N, CW, HW, HW)
@@ -129,3 +269,5 @@ def time_block(N, CW, HW, reps=50):
 if __name__ == "__main__":
     for N, CW, HW in ((64, 1024, 14), (64, 512, 28), (64, 256, 56)):
         time_block(N, CW, HW)
+    for N, CW, HW in ((64, 1024, 14), (64, 512, 28), (64, 256, 56)):
+        time_tail(N, CW, HW)
