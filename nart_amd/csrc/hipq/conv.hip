@@ -57,6 +57,7 @@
 #include "conv_expand.h"
 #include "conv_dw.h"
 #include "conv_rows.h"
+#include "conv_wreg.h"
 
 namespace hipq {
 
@@ -1619,6 +1620,26 @@ static bool rows_applies(const hipq_conv2d_plan *p, const ConvArgs &a)
     return p->variant == kMfma && p->special == 1 && !p->tile_selected && !p->has_wzp && conv_rows_applies(a);
 }
 
+// conv_wreg_kernel (conv_wreg.hip): 1x1 / 3x3 layers whose weight operands go straight from memory to the waves' registers
+static bool wreg_applies(const hipq_conv2d_plan *p, const ConvArgs &a)
+{
+    if (!(p->variant == kMfma && p->special && !p->tile_selected && !p->has_wzp && p->d.dtype == HIPQ_DTYPE_U8 && conv_wreg_applies(a)))
+        return false;
+    if (p->special == 3)
+        return true;
+    if (p->special == 2)
+        return false; // mode 2 asks for the halo / two-group / widening kernels wherever they apply
+    // built-in rule (measured at batch 64 against the tile kernels): the 3x3 layers of the 14x14 and 7x7 stages (256 -> 256 at
+    // 14x14 16.5 -> 13.2 us, 512 -> 512 at 7x7 18.2 -> 13.7, the stride-2 layers into them 17.2 -> 15.3 and 18.1 -> 15.6) and the
+    // 1x1 layers there that reduce the channels four times (1024 -> 256: 9.0 -> 7.9 us, 2048 -> 512: 10.1 -> 8.0); level or behind
+    // on the other 1x1 layers and on larger images
+    if (a.P > 16384 || a.P <= 1024)
+        return false;
+    if (a.R == 3)
+        return true;
+    return a.res == nullptr && a.stride_h == 1 && a.in_cs >= 4 * a.out_cs;
+}
+
 // conv_stem3x3_kernel (conv_stem.hip): 3x3 / stride 2 from an image with at most 4 channels to at most 32
 static bool stem3_applies(const hipq_conv2d_plan *p, const ConvArgs &a)
 {
@@ -1629,7 +1650,9 @@ static void set_mfma_name(hipq_conv2d_plan *p, bool smallc)
 {
     char nm[96];
     StreamShape ss;
-    if (!smallc && stream_applies(p, &ss))
+    if (!smallc && wreg_applies(p, p->args))
+        snprintf(nm, sizeof nm, "conv_mfma_i8_wreg");
+    else if (!smallc && stream_applies(p, &ss))
         snprintf(nm, sizeof nm, "conv_mfma_i8_stream_%dx%d%s", 16 * ss.mb, 16 * ss.nb, p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
     else if (!smallc && rows_applies(p, p->args))
         snprintf(nm, sizeof nm, "conv_mfma_i8_rows3x3%s", p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
@@ -1811,7 +1834,7 @@ static int plan_create(const hipq_conv2d_desc *dp, const uint8_t *w, const int32
         wbuf.resize(pad_off + 64, (uint8_t)pad_byte); // source of out-of-image taps
         // the same weights in fragment order (ConvArgs::wfrag) for the kernels whose waves load their MFMA weight
         // operands straight from memory: layers of a bottleneck block
-        if (!smallc && boff == 0 && d.in_cs % 64 == 0 && d.in_cs <= 1024 && d.out_cs <= 1024 && d.C == d.in_cs
+        if (!smallc && boff == 0 && d.in_cs % 64 == 0 && d.in_cs <= 2048 && d.out_cs <= 2048 && d.C == d.in_cs
             && ((d.R == 1 && d.S == 1) || (d.R == 3 && d.S == 3))) {
             frag_off = (wbuf.size() + 255) / 256 * 256;
             wbuf.resize(frag_off + pad_off, 0);
@@ -1892,6 +1915,8 @@ static int plan_create(const hipq_conv2d_desc *dp, const uint8_t *w, const int32
     a.bias2 = static_cast<const int32_t *>(p->d_bias);
     a.padbuf = a.wpack + pad_off;
     a.wfrag = frag_off ? a.wpack + frag_off : nullptr;
+    if (frag_off)
+        set_mfma_name(p, false); // the register-fed kernel's rule looks at the fragment-order copy
     if (p->d_q) {
         a.qmult = static_cast<const uint32_t *>(p->d_q);
         a.qshift = reinterpret_cast<const int32_t *>(a.qmult + qbuf.size() / 2);
@@ -1941,9 +1966,12 @@ extern "C" const char *hipq_conv2d_plan_kernel_add(const hipq_conv2d_plan *p)
     ConvArgs a = p->args;
     a.res = a.padbuf; // any non-null pointer: the question is which kernel a launch with a residual goes to
     a.addq.fast = 1;  // the 32-bit form of the add, which ordinary scale ratios allow
+    a.addq.hi = 255;  // to 8 bits
     char buf[96];
     StreamShape ss;
-    if (stream_applies(p, &ss))
+    if (wreg_applies(p, a))
+        snprintf(buf, sizeof buf, "conv_mfma_i8_wreg+add");
+    else if (stream_applies(p, &ss))
         snprintf(buf, sizeof buf, "conv_mfma_i8_stream_%dx%d%s+add", 16 * ss.mb, 16 * ss.nb, p->d.dtype == HIPQ_DTYPE_I8 ? "_signed" : "");
     else if (rows_applies(p, a))
         snprintf(buf, sizeof buf, "conv_mfma_i8_rows3x3+add");
@@ -1984,7 +2012,7 @@ extern "C" int hipq_conv2d_plan_special(hipq_conv2d_plan *p, int mode)
     HIPQ_REQUIRE(p, "hipq_conv2d_plan_special: null plan");
     HIPQ_REQUIRE(p->variant == kMfma || p->variant == kMfmaSmallC,
                  "hipq_conv2d_plan_special: only the MFMA kernels have variants (this plan runs %s)", p->name.c_str());
-    HIPQ_REQUIRE(mode >= 0 && mode <= 2, "hipq_conv2d_plan_special: mode must be 0 (never), 1 (built-in rule) or 2 (wherever they apply)");
+    HIPQ_REQUIRE(mode >= 0 && mode <= 3, "hipq_conv2d_plan_special: mode must be 0 (never), 1 (built-in rule), 2 (wherever they apply) or 3 (the register-fed kernel wherever it applies)");
     p->special = mode;
     set_mfma_name(p, p->variant == kMfmaSmallC);
     return 0;
@@ -2470,6 +2498,10 @@ static int run_conv(const hipq_conv2d_plan *p, ConvArgs &a, hipStream_t st)
     switch (p->variant) {
     case kMfma:
     case kMfmaSmallC:
+        if (wreg_applies(p, a)) {
+            launch_conv_wreg(a, st); // few pixels: the pixel operand in LDS once, weight operands straight into registers
+            break;
+        }
         if (rows_applies(p, a)) {
             launch_conv_rows(a, st); // 3x3 with 64 channels: the input rows stay in LDS, the weights in registers
             break;

@@ -228,6 +228,94 @@ def time_tail(N, CW, HW, reps=50):
         N, CW, HW, HW, out["fused"], plans[0].kernel, "expand+add+conv" if fusable else "add, conv", out["separate"]), flush=True)
 
 
+WREG_CASES = [  # N, C, H, W, K, kernel, stride: 1x1 and 3x3 layers of the 14x14 and 7x7 stages
+    (2, 1024, 14, 14, 256, 1, 1), (1, 2048, 7, 7, 512, 1, 1), (3, 512, 7, 7, 2048, 1, 1), (2, 512, 28, 28, 1024, 1, 2),
+    (1, 256, 9, 13, 128, 1, 1), (2, 1024, 14, 14, 2048, 1, 2), (2, 512, 7, 7, 512, 3, 1), (1, 256, 28, 28, 256, 3, 2),
+    (2, 128, 14, 21, 128, 3, 1), (1, 512, 14, 14, 512, 3, 2), (1, 128, 56, 28, 128, 3, 2), (2, 256, 14, 14, 256, 3, 1),
+]
+
+
+@pytest.mark.parametrize("case", WREG_CASES, ids=lambda c: "x".join(map(str, c)))
+def test_register_fed_convolution(case):
+    """conv_wreg_kernel (special(3)) against the oracle's convolution and, for 1x1 layers, convolution + add."""
+    N, C, H, W, K, k, st = case
+    rng = np.random.default_rng(3000 + C + K + k)
+    x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+    w = rng.integers(1, 256, (K, C, k, k), dtype=np.uint8)
+    sigma = 74.0 * 74.0 * math.sqrt(C * k * k)
+    b = rng.integers(-int(sigma), int(sigma) + 1, K).astype(np.int32)
+    for relu in (False, True):
+        ia, iz = 0.03, int(rng.integers(0, 256))
+        oa = float(np.float32(ia * rng.uniform(0.75, 1.35)))
+        q = (ia, iz, float(np.float32(oa * 40.0 / (ia * sigma))), 128, oa, int(rng.integers(0, 200)))
+        plan = hipq.Conv2d(x.shape, w, b, k // 2, st, 1, *q, relu=relu).special(3)
+        print("register-fed case", case, relu, plan.kernel, flush=True)
+        assert plan.kernel == "conv_mfma_i8_wreg", plan.kernel
+        want = orc.conv2d_u8(x, w, b, k // 2, st, 1, *q)
+        if relu:
+            want = np.maximum(want, q[5]).astype(np.uint8)
+        xd = hipq.to_device_nhwc(x)
+        y = plan(xd)
+        torch.cuda.synchronize()
+        got = hipq.from_device_nhwc(y, K)
+        bad = got != want
+        assert not bad.any(), (case, relu, int(bad.sum()), np.argwhere(bad)[:8].tolist())
+        if k == 1 and not relu:
+            for res_first in (False, True):
+                res = rng.integers(0, 256, want.shape, dtype=np.uint8)
+                ra, rz = float(np.float32(oa * rng.uniform(0.6, 1.6))), int(rng.integers(0, 256))
+                sa, sz = float(np.float32(math.hypot(oa, ra) * 1.1)), int(rng.integers(0, 40))
+                assert plan.kernel_add == "conv_mfma_i8_wreg+add", plan.kernel_add
+                wanta = orc.add_u8(res, want, ra, rz, q[4], q[5], sa, sz) if res_first else orc.add_u8(want, res, q[4], q[5], ra, rz, sa, sz)
+                ya = torch.zeros_like(y)
+                plan.run_add(xd, hipq.to_device_nhwc(res), res_first, ra, rz, sa, sz, ya)
+                torch.cuda.synchronize()
+                gota = hipq.from_device_nhwc(ya, K)
+                assert np.array_equal(gota, wanta), (case, "add", res_first, int((gota != wanta).sum()))
+
+
+def time_layers():
+    """Every convolution of the 28x28-and-smaller stages of ResNet-50 at batch 64: the built-in kernel against special(3)."""
+    rng = np.random.default_rng(9)
+    layers = [  # C, H, K, k, stride, with add
+        (256, 56, 128, 1, 1, False), (128, 56, 128, 3, 2, False), (256, 56, 512, 1, 2, False), (512, 28, 128, 1, 1, False),
+        (512, 28, 256, 1, 1, False), (256, 28, 256, 3, 2, False), (512, 28, 1024, 1, 2, False), (256, 14, 1024, 1, 1, True),
+        (1024, 14, 256, 1, 1, False), (256, 14, 256, 3, 1, False), (1024, 14, 512, 1, 1, False), (512, 14, 512, 3, 2, False),
+        (1024, 14, 2048, 1, 2, False), (512, 7, 2048, 1, 1, True), (2048, 7, 512, 1, 1, False), (512, 7, 512, 3, 1, False),
+    ]
+    for C, HW, K, k, st, add in layers:
+        N = 64
+        x = torch.randint(0, 256, (N, HW, HW, C), dtype=torch.uint8, device="cuda")
+        w = rng.integers(1, 256, (K, C, k, k), dtype=np.uint8)
+        sigma = 74.0 * 74.0 * math.sqrt(C * k * k)
+        b = rng.integers(-int(sigma), int(sigma) + 1, K).astype(np.int32)
+        q = (0.03, 120, float(np.float32(40.0 / sigma)), 128, 0.03, 0 if not add else 128)
+        out = {}
+        for mode in (1, 3):
+            plan = hipq.Conv2d((N, C, HW, HW), w, b, k // 2, st, 1, *q).special(mode)
+            y = plan.empty_output()
+            res = torch.randint(0, 256, y.shape, dtype=torch.uint8, device="cuda")
+            fn = (lambda: plan.run_add(x, res, False, 0.04, 100, 0.06, 0, y)) if add else (lambda: plan(x, y))
+            fn()
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g):
+                for _ in range(10):
+                    fn()
+            for _ in range(3):
+                g.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(20):
+                g.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            out[mode] = (e0.elapsed_time(e1) / 200 * 1e3, plan.kernel_add if add else plan.kernel)
+        print("layer C=%4d %2dx%2d K=%4d k=%d s=%d add=%d: %-34s %6.1f us | %-22s %6.1f us" % (
+            C, HW, HW, K, k, st, add, out[1][1], out[1][0], out[3][1], out[3][0]), flush=True)
+
+
 def time_block(N, CW, HW, reps=50):
     rng = np.random.default_rng(5)
     x, xq, layers, sq = make_block(rng, N, CW, HW, HW)
@@ -271,3 +359,4 @@ if __name__ == "__main__":
         time_block(N, CW, HW)
     for N, CW, HW in ((64, 1024, 14), (64, 512, 28), (64, 256, 56)):
         time_tail(N, CW, HW)
+    time_layers()
