@@ -11,8 +11,6 @@ Prints ONE JSON line:
                         their measured durations, against the chip's dense int8 MFMA peak
   kernel_families       every family's time, TOP/s and GB/s (launch-by-launch timing, see per_kernel_times)
   sustained             the same replay loop kept running for at least two seconds
-  machine_probes        what this box delivers on the library's own probes: MFMA rate on constant and random operands, the
-                        cost of a launch in a graph chain, load-unit streaming per CU, vector-memory instruction rates
   library_int8_gemm     a yardstick: the vendor library's plain int8 GEMM (int32 output) on every layer's GEMM shape, summed,
                         beside the sum of this build's convolution-family launches
   module_path           the same network as an engine file run by nart_promark on the `hip` workspace (the drop-in path),
@@ -37,9 +35,25 @@ PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA, TOP/s (published)
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s (published)
 # HBM bytes per launch of the dominant kernel family, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this very
 # command.  A counter run cannot be made from inside the benchmark, so the figure is carried here together with the
-# file that holds the counter readings; it only applies to the default workload with default flags.
+# file that holds the counter readings and a digest of the kernel sources it was taken with: the line reports it only
+# for the default workload with default flags and only while the sources under nart_amd/csrc/hipq still have that digest
+# (traffic is null, with the reason, once a kernel has changed and the profile has not been taken again).
 TRAFFIC_FROM_PROFILE = {"workload": "resnet50", "batch": 64, "bytes_per_launch": 34.85e6,
-                        "source": "profiles/conv_mfma_i8_resnet50_n64.md"}
+                        "source": "profiles/conv_mfma_i8_resnet50_n64.md",
+                        "sources_sha256": "stale"}
+
+
+def kernel_sources_digest():
+    """sha256 over the kernel sources (names and contents, in name order): ties a profile to the code it measured."""
+    import hashlib
+    d = os.path.join(ROOT, "nart_amd", "csrc", "hipq")
+    h = hashlib.sha256()
+    for f in sorted(os.listdir(d)):
+        if f.endswith((".hip", ".h", ".cpp")):
+            h.update(f.encode())
+            with open(os.path.join(d, f), "rb") as fh:
+                h.update(fh.read())
+    return h.hexdigest()[:16]
 
 
 def time_steps(fn, steps, warmup):
@@ -81,15 +95,22 @@ def per_kernel_times(ex, reps):
         torch.cuda.synchronize()
         with torch.cuda.stream(st):
             g = graph_of(s["fn"], reps, st)
-            g.replay()
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(st)
-            for _ in range(3):
-                g.replay()
-            e1.record(st)
-            torch.cuda.synchronize()
-        out.append(e0.elapsed_time(e1) / (3 * reps))
+
+            def timed(warm, n):
+                for _ in range(warm):
+                    g.replay()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(st)
+                for _ in range(n):
+                    g.replay()
+                e1.record(st)
+                torch.cuda.synchronize()
+                return e0.elapsed_time(e1) / (n * reps)
+            t = timed(3, 5)
+            if t < 0.010:  # a kernel under 10 us: clocks and caches settle over more replays, and more are averaged
+                t = timed(10, 20)
+        out.append(t)
         del g
     return out
 
@@ -123,7 +144,20 @@ def roofline_of(fam, kt):
     roof["avg_launch_us"] = round(d["ms"] / d["launches"] * 1e3, 2)
     roof["sum_kernel_ms"] = round(sum(kt), 4)
     roof["timing"] = "HIP events on the launch stream around graph replays of back-to-back launches of each operator, inputs warm"
+    roof["family_ms"] = round(d["ms"], 4)
+    roof["other_kernels_ms"] = round(sum(kt) - d["ms"], 4)
     return roof
+
+
+def add_in_pass(roof, ms_per_step):
+    """The same fraction with the family's launches timed INSIDE the replayed step: the step minus the other kernels'
+    durations, i.e. with every launch gap and every cold input of the pass charged to the family."""
+    in_pass = ms_per_step - roof["other_kernels_ms"]
+    if roof["bound"] == "mfma" and roof["algorithmic_ops_per_launch"] and in_pass > 0:
+        ach = roof["algorithmic_ops_per_launch"] * roof["launches_per_step"] / (in_pass * 1e-3) / 1e12
+        roof["achieved_in_pass"] = round(ach, 2)
+        roof["frac_in_pass"] = round(ach / roof["peak"], 4)
+        roof["avg_launch_us_in_pass"] = round(in_pass / roof["launches_per_step"] * 1e3, 2)
 
 
 def cpu_baseline(case_builder, gpu_first_image, budget_s=30.0):
@@ -271,57 +305,6 @@ def library_gemm(case, ex, kt):
                     "this build: its convolution-family launches, which include all of those"}
 
 
-def machine_probes():
-    """What the box delivers on the library's own probes (include/hipq.h: hipq_probe_launch): HIP events around graph
-    replays of a few launches each.  The published peaks stay the roofs; these say how far below them a perfect kernel
-    of the same shape would land on this machine."""
-    import ctypes
-    import torch
-    from nart_amd import hipq
-    lib = hipq.lib()
-    buf = torch.randint(0, 256, (64 << 20,), dtype=torch.uint8, device="cuda")
-    st = torch.cuda.Stream()
-    units = ctypes.c_double(0)
-
-    def run(which, iters, param=0, reps=3):
-        def one():
-            hipq.check(lib.hipq_probe_launch(which, buf.data_ptr(), buf.numel(), iters, param, ctypes.byref(units), st.cuda_stream))
-        with torch.cuda.stream(st):
-            one()
-            torch.cuda.synchronize()
-            g = graph_of(one, reps, st)
-            g.replay()
-            torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            e0.record(st)
-            for _ in range(3):
-                g.replay()
-            e1.record(st)
-            torch.cuda.synchronize()
-        return e0.elapsed_time(e1) * 1e-3 / (3 * reps), units.value   # seconds per launch, work per launch
-
-    out = {}
-    t, u = run(0, 4000)
-    out["mfma_i8_constant_operands_TOPs"] = round(u / t / 1e12, 1)
-    t, u = run(1, 4000)
-    out["mfma_i8_random_operands_TOPs"] = round(u / t / 1e12, 1)
-    t, _ = run(2, 1, reps=200)
-    out["launch_in_graph_chain_us"] = round(t * 1e6, 2)
-    for name, region in (("l2_resident_2MB", 2 << 20), ("beyond_l2_32MB", 32 << 20)):
-        t, u = run(3, 1536, region)
-        out["lds_dma_%s_KB_per_us_per_CU" % name] = round(u / t / 1e9 / 256, 1)
-    names = ("load_32bit_contiguous", "load_32bit_eight_pieces", "load_128bit", "store_32bit_contiguous", "store_32bit_eight_pieces",
-             "store_128bit")
-    widths = (256, 256, 1024, 256, 256, 1024)
-    for i, (nm, w) in enumerate(zip(names, widths)):
-        t, u = run(4 + i, 2000)
-        ns = t * 1e9 / u
-        out["vmem_" + nm] = {"ns_per_wave_instruction_per_CU": round(ns, 2), "TBs_chip": round(w / ns * 256 / 1e3, 2)}
-    out["note"] = ("8 waves per CU; MFMA: four independent accumulators per wave; lds_dma: global_load_lds_dwordx4, three stages of 2 KB "
-                   "per wave; vmem: 4 KB per wave, resident in the CU's L1")
-    return out
-
-
 def module_path(build, batch, steps):
     """The drop-in path: the network as an engine file, run by nart_promark (the counterpart of the reference's
     tools/promark.cpp) on the `hip` workspace through hip_module_tp, every operator launched by the module's run
@@ -422,11 +405,18 @@ def main():
     fam = families_of(ex, kt)
     roof = roofline_of(fam, kt)
     default_flags = not (args.tune or args.no_graph or args.no_fuse)
+    add_in_pass(roof, ms)
     if (default_flags and args.workload == TRAFFIC_FROM_PROFILE["workload"] and args.batch == TRAFFIC_FROM_PROFILE["batch"]
             and roof["kernel"] == "conv_mfma_i8"):
-        roof["traffic"] = TRAFFIC_FROM_PROFILE["bytes_per_launch"]
-        roof["traffic_source"] = (TRAFFIC_FROM_PROFILE["source"]
-                                  + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, copy-kernel calibrated)")
+        digest = kernel_sources_digest()
+        roof["kernel_sources_sha256"] = digest
+        if digest == TRAFFIC_FROM_PROFILE["sources_sha256"]:
+            roof["traffic"] = TRAFFIC_FROM_PROFILE["bytes_per_launch"]
+            roof["traffic_source"] = (TRAFFIC_FROM_PROFILE["source"]
+                                      + " (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, copy-kernel calibrated)")
+        else:
+            roof["traffic_source"] = ("null: the kernel sources changed since %s was taken (digest %s there)"
+                                      % (TRAFFIC_FROM_PROFILE["source"], TRAFFIC_FROM_PROFILE["sources_sha256"]))
     families = {k: {"ms": round(v["ms"], 4), "launches": v["launches"],
                     "TOPs": round(v["ops"] / (v["ms"] * 1e-3) / 1e12, 2) if v["ops"] else None,
                     "GBs": round(v["bytes"] / (v["ms"] * 1e-3) / 1e9, 1)} for k, v in fam.items()}
@@ -520,7 +510,6 @@ def main():
 
     if not args.no_extras and not args.no_graph:
         extra("library_int8_gemm", lambda: library_gemm(case, ex, kt))
-        extra("machine_probes", machine_probes)
 
     if not args.no_extras and args.workload == "resnet50":
         extra("module_path", lambda: module_path(build, args.batch, 50))

@@ -1678,14 +1678,9 @@ static int conv_out_dim(int in, int pad, int k, int stride)
 }
 
 // Largest tile that still gives every CU a few work-groups to overlap (two waves per SIMD hide the
-// global-load latency of one another); HIPQ_CONV_TILE=<index into kTiles> overrides for tuning runs.
+// global-load latency of one another).
 static int choose_tile(long long P, int out_cs, bool expand, int in_cs)
 {
-    if (const char *e = getenv("HIPQ_CONV_TILE")) {
-        const int t = atoi(e);
-        if (t >= 0 && t < kNumTiles)
-            return t;
-    }
     auto count = [&](int t) { return ((P + kTiles[t].bm - 1) / kTiles[t].bm) * ((out_cs + kTiles[t].bn - 1) / kTiles[t].bn); };
     // one tile of channels, or a width that would leave 15 % or more of the 128-channel tiles' columns empty (96, 160,
     // 320 channels): 64x64 tiles (MobileNetV2 at batch 64, inside the network: 0.463 -> 0.459 ms for the first, -> 0.460
@@ -1770,9 +1765,10 @@ static int plan_create(const hipq_conv2d_desc *dp, const uint8_t *w, const int32
     if (!valid_shift(a.q.shift)) {
         delete p;
         return fail("conv: requantisation shift %d outside 1..62 (scale %g)", a.q.shift,
-                    (double)(d.ialpha * d.walpha / d.oalpha));
+                    (double)(d.ialpha * (walpha_pc ? walpha_pc[0] : d.walpha) / d.oalpha));
     }
-    a.fastq = a.q.shift >= 33 && a.q.shift <= 52;
+    // the one-multiply form needs one shift for the whole tensor: never for per-channel scales, whatever channel 0's is
+    a.fastq = walpha_pc == nullptr && a.q.shift >= 33 && a.q.shift <= 52;
     a.qt = a.fastq ? a.q.shift - 32 : 1;
     a.qadd = a.fastq ? (1 << (a.qt - 1)) + (a.q.zp << a.qt) : 0;
     a.inv_ohw = 1.0 / ((double)a.OH * a.OW);
@@ -1848,8 +1844,7 @@ static int plan_create(const hipq_conv2d_desc *dp, const uint8_t *w, const int32
                             memcpy(&wbuf[frag_off + ((((size_t)sl * (a.kout_pad / 32) + T) * 2 + kk) * 64 + l) * 16], src, 16);
                         }
         }
-        static const bool no_halo = getenv("HIPQ_NO_SPECIAL_KERNELS") != nullptr; // A/B measurements: tile kernels only
-        p->special = no_halo ? 0 : 1;
+        p->special = 1;
         set_mfma_name(p, smallc);
     } else if (!sgn && d.group == d.C && d.K == d.C && d.in_cs == d.out_cs && d.R == 3 && d.S == 3 && d.stride_h == d.stride_w
                && (d.stride_h == 1 || d.stride_h == 2)
@@ -2148,10 +2143,11 @@ static void launch_mfma(const hipq_conv2d_plan *p, const ConvArgs &a, hipStream_
 {
     const int nblk = a.nbm * a.nbn;
     const dim3 grid((nblk + 7) / 8 * 8), block(256);
-    if (p->variant == kMfma && launch_halo<BM, BN, WM, WN>(p, a, grid, st))
-        return;
     StreamShape ss;
-    if (stream_applies(p, &ss)) {
+    const bool streams = stream_applies(p, &ss); // the kernel the plan is named after wins over the halo kernel
+    if (p->variant == kMfma && !streams && launch_halo<BM, BN, WM, WN>(p, a, grid, st))
+        return;
+    if (streams) {
         const bool fc = a.R == 1 && a.S == 1 && a.stride_h == 1 && a.stride_w == 1 && a.pad_h == 0 && a.pad_w == 0;
         const int mtiles = (a.P + 16 * ss.mb - 1) / (16 * ss.mb), ntiles = (a.out_cs + 16 * ss.nb - 1) / (16 * ss.nb);
         const dim3 sgrid((ntiles + 7) / 8 * 8 * mtiles);

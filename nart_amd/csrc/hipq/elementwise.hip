@@ -545,6 +545,25 @@ __global__ __launch_bounds__(256) void dequantize_u8_kernel(const DequantArgs p)
     }
 }
 
+// int32 accumulators (NHWC, as hipq_conv2d_run's acc_out writes them) -> fp32 dense NCHW: (float)acc * alpha
+struct DequantI32Args {
+    const int32_t *x;
+    float *y;
+    int N, C, H, W, cs;
+    float alpha;
+};
+
+__global__ __launch_bounds__(256) void dequantize_i32_kernel(const DequantI32Args p)
+{
+    const size_t hw = (size_t)p.H * p.W, total = (size_t)p.N * p.C * hw;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+         idx += (size_t)gridDim.x * blockDim.x) {
+        const size_t pix = idx % hw, rest = idx / hw;
+        const int c = (int)(rest % p.C), n = (int)(rest / p.C);
+        p.y[idx] = __fmul_rn(__int2float_rn(p.x[((size_t)n * hw + pix) * p.cs + c]), p.alpha);
+    }
+}
+
 // ---- layout conversion ---------------------------------------------------------------------------
 struct LayoutArgs {
     const uint8_t *src;
@@ -855,6 +874,17 @@ extern "C" int hipq_dequantize_u8(const void *x, float *y, int N, int C, int H, 
 extern "C" int hipq_dequantize_i8(const void *x, float *y, int N, int C, int H, int W, int cs, float ia, void *stream)
 {
     return launch_dequantize("hipq_dequantize_i8", 1, x, y, N, C, H, W, cs, ia, 0, stream);
+}
+
+extern "C" int hipq_dequantize_i32(const int32_t *x, float *y, int N, int C, int H, int W, int cs, float alpha, void *stream)
+{
+    clear_error();
+    HIPQ_REQUIRE(x && y && N > 0 && C > 0 && H > 0 && W > 0 && cs >= C, "hipq_dequantize_i32: bad argument");
+    DequantI32Args p;
+    p.x = x, p.y = y, p.N = N, p.C = C, p.H = H, p.W = W, p.cs = cs, p.alpha = alpha;
+    hipLaunchKernelGGL(dequantize_i32_kernel, dim3(grid_for((size_t)N * C * H * W)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), p);
+    return launch_status("dequantize_i32_kernel");
 }
 
 static int layout_args(LayoutArgs &p, const void *src, void *dst, int N, int C, int H, int W, int cs)

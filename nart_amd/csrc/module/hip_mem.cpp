@@ -1,8 +1,46 @@
 // hip_mem_tp: the memory type of the `hip` workspace — a device buffer plus a pinned host mirror, kept
 // coherent on demand.  Implements the mem_tp vtable of art/include/art/mem.h:48-64.
+#include <algorithm>
 #include <cstring>
+#include <vector>
 
 #include "hip_module.h"
+
+// The streams of the live `hip` workspaces.  A memory remembers the stream that last wrote its device side and the one
+// that last read its host mirror, and may outlive the workspace that owned it: a stream that has been retired was
+// synchronised when its workspace went away, so there is nothing left to wait for (and nothing valid to wait on).
+static std::vector<hipStream_t> &live_streams()
+{
+    static std::vector<hipStream_t> v;
+    return v;
+}
+
+void hip_stream_register(hipStream_t st) { live_streams().push_back(st); }
+
+void hip_stream_retire(hipStream_t st)
+{
+    HIPM_HIP(hipStreamSynchronize(st));
+    auto &v = live_streams();
+    v.erase(std::remove(v.begin(), v.end(), st), v.end());
+}
+
+void hip_stream_forget(hipStream_t st)
+{
+    auto &v = live_streams();
+    v.erase(std::remove(v.begin(), v.end(), st), v.end());
+}
+
+// wait for the work queued on st - and only on st: another workspace's kernels keep running.  A stream this module no
+// longer knows (its workspace is gone, or it was a caller's stream that has been replaced) cannot be named any more:
+// then the whole device is waited for, as the runtime's other GPU modules always do.
+static void wait_stream(hipStream_t st)
+{
+    auto &v = live_streams();
+    if (st == nullptr || std::find(v.begin(), v.end(), st) != v.end())
+        HIPM_HIP(hipStreamSynchronize(st));
+    else
+        HIPM_HIP(hipDeviceSynchronize());
+}
 
 static void grow_dev(void **p, size_t *cap, size_t need)
 {
@@ -67,7 +105,7 @@ static void ensure_host(hip_mem_t *m)
     memset(p, 0, m->size);
     if (m->host) {
         if (m->up_pending) { // an upload may still read the old mirror
-            HIPM_HIP(hipStreamSynchronize(m->up_stream));
+            wait_stream(m->up_stream);
             m->up_pending = false;
         }
         memcpy(p, m->host, m->host_cap);
@@ -104,13 +142,14 @@ static void upload(hip_mem_t *m, hipStream_t st)
     m->dev_valid = true;
     m->up_pending = true; // the copy still reads the mirror
     m->up_stream = st;
+    m->prod_stream = st;
 }
 
 // the mirror is about to be handed out for writing: an upload that still reads it must finish first
 static void finish_upload(hip_mem_t *m)
 {
     if (m->up_pending) {
-        HIPM_HIP(hipStreamSynchronize(m->up_stream));
+        wait_stream(m->up_stream);
         m->up_pending = false;
     }
 }
@@ -122,7 +161,7 @@ static void *hm_cpu_data(const mem_t *mm)
     hip_mem_t *m = as_hip(const_cast<mem_t *>(mm));
     hip_mem_settle(m);
     if (m->dev_valid && !m->host_valid) {
-        HIPM_HIP(hipDeviceSynchronize()); // the producing kernels run on a workspace stream
+        wait_stream(m->prod_stream); // the producing kernels run on that workspace's stream; other workspaces are not waited for
         download(m);
     }
     ensure_host(m);
@@ -137,7 +176,7 @@ const void *hip_mem_host_in(mem_t *mm)
     hip_mem_t *m = as_hip(mm);
     hip_mem_settle(m);
     if (m->dev_valid && !m->host_valid) {
-        HIPM_HIP(hipDeviceSynchronize());
+        wait_stream(m->prod_stream);
         download(m);
     }
     ensure_host(m);
@@ -157,10 +196,11 @@ const void *hip_mem_dev_in(mem_t *mm, hipStream_t st)
     return m->dev;
 }
 
-void *hip_mem_dev_out(mem_t *mm, hipStream_t)
+void *hip_mem_dev_out(mem_t *mm, hipStream_t st)
 {
     hip_mem_t *m = as_hip(mm);
     m->pending = nullptr; // about to be overwritten: a deferred producer's result is dead
+    m->prod_stream = st;  // whoever reads the contents from outside that stream waits for it first
     grow_dev(&m->dev, &m->dev_cap, dev_bytes(m));
     m->dev_valid = true;
     m->host_valid = false;
@@ -221,7 +261,7 @@ void hip_mem_tag(tensor_t *t)
             m->dev_valid = false;
         }
         if (m->dev_valid && !m->host_valid && m->dev) {
-            HIPM_HIP(hipDeviceSynchronize()); // the producing kernels run on a workspace stream
+            wait_stream(m->prod_stream); // the producing kernels run on that workspace's stream
             download(m);
         }
         m->dev_valid = false;

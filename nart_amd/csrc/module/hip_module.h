@@ -87,6 +87,9 @@ struct hip_mem_t {
     // once that copy has finished.
     bool up_pending;
     hipStream_t up_stream;
+    // The stream whose work last wrote `dev` (a workspace's, or the null stream for an upload on behalf of foreign code):
+    // a reader outside that stream waits for it, and for nothing else.
+    hipStream_t prod_stream;
     // Deferred producer.  A convolution whose only reader is an add does not launch at its own run(): it leaves this
     // hook, and the add runs both as one fused kernel (hip_ops.cpp).  Whoever else asks for the contents first - the
     // host, another workspace, a re-run - makes the hook launch the plain convolution into `dev` (hip_mem_settle).
@@ -110,6 +113,11 @@ extern const mem_tp hip_mem_tp_st;
 // An existing tag with the same element count is kept: a reshape()d view shares its producer's geometry.
 void hip_mem_tag(tensor_t *t);
 // Device pointer for reading (uploads / converts the host mirror if that is the newer side).
+// the streams hip_mem_tp may wait on by name: a workspace registers the stream it launches on, retires the one it owns
+// (synchronise, then forget) before destroying it and forgets a caller's stream when it stops using it
+void hip_stream_register(hipStream_t st);
+void hip_stream_retire(hipStream_t st);
+void hip_stream_forget(hipStream_t st);
 const void *hip_mem_dev_in(mem_t *m, hipStream_t st);
 // Device pointer for writing: the device side becomes the valid one.
 void *hip_mem_dev_out(mem_t *m, hipStream_t st);

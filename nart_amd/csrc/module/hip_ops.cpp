@@ -239,10 +239,17 @@ void conv_run(op_t *op)
 
 // A walpha array with one entry per output channel (and more than one channel) selects per-channel requantisation, the
 // convention of the reference's CUDA sibling (cuda_quant/src/op/conv_2d_quant.cu:751-764); a single entry is the
-// per-tensor scale the reference CPU module reads (conv_2d_uint8_impl.c:57-66).
+// per-tensor scale the reference CPU module reads (conv_2d_uint8_impl.c:57-66).  The reference's converter writes one
+// entry per CONSTANT input (python/nart/modules/quant.py:178-208: the weights' scale, then the bias's), of which the CPU
+// module reads the first (conv_2d_uint8_impl.c:61, ip.cpp:148): an array of that length is that convention and stays
+// per tensor even when it happens to equal the channel count (a two-channel layer with a bias).
 const float *per_channel_walpha(const conv_op_t *c)
 {
-    return c->num_output > 1 && c->qw.n_alpha == c->num_output ? c->qw.alpha : nullptr;
+    const op_t *op = reinterpret_cast<const op_t *>(c);
+    const uint32_t n_const = op->input_size > 0 ? (uint32_t)op->input_size - 1 : 0;
+    if (c->num_output <= 1 || (uint32_t)c->qw.n_alpha != (uint32_t)c->num_output || (uint32_t)c->qw.n_alpha == n_const)
+        return nullptr;
+    return c->qw.alpha;
 }
 
 void build_plan(op_t *op, const hipq_conv2d_desc &d, const uint8_t *w, const void *w_id)
@@ -986,8 +993,12 @@ const mem_tp *ws_memtype(const workspace_t *) { return &hip_mem_tp_st; }
 void ws_delete(workspace_t *w)
 {
     hip_workspace_t *ws = reinterpret_cast<hip_workspace_t *>(w);
-    if (ws->own_stream && ws->stream)
+    if (ws->own_stream && ws->stream) {
+        hip_stream_retire(ws->stream); // memories that outlive the workspace remember this stream
         (void)hipStreamDestroy(ws->stream);
+    } else if (ws->stream) {
+        hip_stream_forget(ws->stream);
+    }
     g_readers.erase(w);
     free(ws);
 }
@@ -1020,6 +1031,7 @@ static workspace_t *ws_new(const setting_entry_t *settings)
     HIPM_HIP(hipSetDevice(ws->dev_id));
     HIPM_HIP(hipStreamCreateWithFlags(&ws->stream, hipStreamNonBlocking)); // default priority
     ws->own_stream = true;
+    hip_stream_register(ws->stream);
     return &ws->ws;
 }
 
@@ -1036,10 +1048,16 @@ ART_PUBLIC void *hip_workspace_stream(workspace_t *w) { return reinterpret_cast<
 ART_PUBLIC void hip_workspace_set_stream(workspace_t *w, void *stream)
 {
     hip_workspace_t *ws = reinterpret_cast<hip_workspace_t *>(w);
-    if (ws->own_stream && ws->stream)
+    if (ws->own_stream && ws->stream) {
+        hip_stream_retire(ws->stream);
         (void)hipStreamDestroy(ws->stream);
+    } else if (ws->stream) {
+        hip_stream_forget(ws->stream);
+    }
     ws->stream = static_cast<hipStream_t>(stream);
     ws->own_stream = false;
+    if (ws->stream)
+        hip_stream_register(ws->stream);
 }
 
 // Blocks until everything the workspace has launched is done; runners that time a run call it (operators return

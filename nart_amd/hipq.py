@@ -83,8 +83,8 @@ _SIGS = {
     "hipq_dequantize_u8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_float, C.c_int, C.c_void_p]),
     "hipq_quantize_i8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_float, C.c_int, C.c_void_p]),
     "hipq_dequantize_i8": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_float, C.c_void_p]),
+    "hipq_dequantize_i32": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 5 + [C.c_float, C.c_void_p]),
     "hipq_copy_bytes": (C.c_int, [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]),
-    "hipq_probe_launch": (C.c_int, [C.c_int, C.c_void_p, C.c_size_t, C.c_int, C.c_size_t, C.POINTER(C.c_double), C.c_void_p]),
 }
 EXPORTS = tuple(_SIGS)
 
@@ -376,6 +376,13 @@ def quantize_i8(x_nchw, y, oalpha, obits=8):
 def dequantize_i8(x, y_nchw, ialpha):
     N, Cc, H, W = y_nchw.shape
     check(lib().hipq_dequantize_i8(_ptr(x), _ptr(y_nchw), N, Cc, H, W, x.shape[-1], ialpha, _stream()))
+    return y_nchw
+
+
+def dequantize_i32(acc, y_nchw, alpha):
+    """int32 accumulators NHWC -> fp32 NCHW: (float)acc * alpha (include/hipq.h: hipq_dequantize_i32)."""
+    N, Cc, H, W = y_nchw.shape
+    check(lib().hipq_dequantize_i32(_ptr(acc), _ptr(y_nchw), N, Cc, H, W, acc.shape[-1], float(np.float32(alpha)), _stream()))
     return y_nchw
 
 

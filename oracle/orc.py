@@ -174,6 +174,14 @@ def dequantize_u8(x, ialpha, izp):
     return y
 
 
+def dequantize_i32(acc, alpha):
+    """int32 accumulators -> fp32: (float)acc * alpha.  No counterpart in the reference (closed form only)."""
+    acc = np.ascontiguousarray(acc, np.int32)
+    y = np.empty(acc.shape, np.float32)
+    lib().orc_dequantize_i32(_p(acc), _p(y), C.c_size_t(acc.size), _f(alpha))
+    return y
+
+
 def concat_u8(ins, ialpha, izp, oalpha, ozp, obits=8):
     """Concatenation along dimension 1 with per-input rescaling (the reference ignores `axis`, concat.c:99-121)."""
     ins = [np.ascontiguousarray(a, np.uint8) for a in ins]

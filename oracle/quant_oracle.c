@@ -390,6 +390,18 @@ void orc_dequantize_u8(const uint8_t *x, float *y, size_t count, float ialpha, i
         y[i] = (float)((int)x[i] - izp) * ialpha; /* dequantize.c:121 */
 }
 
+/* Dequantize of int32 accumulators.  NO counterpart in the reference: op_dequantize_run_u8 / _i8 (dequantize.c:111-136)
+ * read bytes only.  An accumulator of a convolution or inner product counts units of ialpha * walpha (the scale its
+ * int32 bias is quantised with, python/docs/tutorial/switch/cuda_quant.rst:60), so its real value is the closed form
+ * y = (float)acc * alpha with alpha = ialpha * walpha formed in fp32 by the caller: one int32 -> fp32 conversion (round to
+ * nearest even beyond 2^24) and one fp32 multiply, like dequantize.c:121.  Pinned by that closed form only (numpy's
+ * astype(float32) * float32 in tests/test_oracle.py): parity unpinned against any reference output. */
+void orc_dequantize_i32(const int32_t *x, float *y, size_t count, float alpha)
+{
+    for (size_t i = 0; i < count; i++)
+        y[i] = (float)x[i] * alpha;
+}
+
 /* op_quant_concat_run — concat.c:82-124: whatever `axis` says, the loop copies image by image and input by input,
  * i.e. it concatenates along dimension 1; every input is rescaled: (mult, shift) = gqs(ialpha_j / oalpha, 16),
  * y = sat(rrn(mult * (x - izp_j), shift) + ozp).  mult is a uint16_t, the product an int. */

@@ -93,6 +93,7 @@ void orc_quantize_u8(const float *x, uint8_t *y, size_t count, float oalpha, int
 
 /* op_dequantize_run_u8 — dequantize.c:111-123. */
 void orc_dequantize_u8(const uint8_t *x, float *y, size_t count, float ialpha, int izp);
+void orc_dequantize_i32(const int32_t *x, float *y, size_t count, float alpha);
 
 /* op_quant_concat_run — concat.c:82-124.  per_image[j] = elements of input j per image (C_j*H*W). */
 void orc_concat_u8(const uint8_t *const *in, int n_in, const size_t *per_image, const float *ialpha,

@@ -638,6 +638,30 @@ def test_quantize_dequantize():
         assert np.array_equal(fd.cpu().numpy().view(np.uint32), orc.dequantize_u8(want, oa, oz).view(np.uint32))
 
 
+def test_dequantize_of_int32_accumulators():
+    """hipq_dequantize_i32 (no counterpart in the reference, which dequantizes bytes only): a convolution's accumulator
+    dump times ialpha * walpha, against the oracle's closed form, plus values where int32 -> fp32 rounds."""
+    rng = np.random.default_rng(18)
+    x = rng.integers(0, 256, (2, 48, 9, 7), dtype=np.uint8)
+    w = rng.integers(0, 256, (40, 48, 3, 3), dtype=np.uint8)
+    b = rng.integers(-30000, 30000, 40).astype(np.int32)
+    q = (0.02, 128, 0.005, 128, 0.05, 0)
+    plan = hipq.Conv2d(x.shape, w, b, 1, 1, 1, *q)
+    acc = torch.zeros((2, 9, 7, plan.desc.out_cs), dtype=torch.int32, device="cuda")
+    plan(hipq.to_device_nhwc(x), acc=acc)
+    _, want_acc = orc.conv2d_u8(x, w, b, 1, 1, 1, *q, return_acc=True)
+    alpha = float(np.float32(q[0]) * np.float32(q[2]))
+    fd = torch.empty((2, 40, 9, 7), dtype=torch.float32, device="cuda")
+    hipq.dequantize_i32(acc, fd, alpha)
+    assert np.array_equal(fd.cpu().numpy().view(np.uint32), orc.dequantize_i32(want_acc, alpha).view(np.uint32))
+    big = np.concatenate([rng.integers(-2**31, 2**31, 4086), [2**24 + 1, 2**24 + 3, -(2**24) - 1, 2**31 - 1, -2**31, 0, 1, -1, 2**25 + 2,
+                                                                2**25 + 6]]).astype(np.int32).reshape(1, 4096, 1, 1)
+    bd = torch.from_numpy(big.reshape(1, 1, 1, 4096)).cuda()
+    fd = torch.empty((1, 4096, 1, 1), dtype=torch.float32, device="cuda")
+    hipq.dequantize_i32(bd, fd, 3.1e-5)
+    assert np.array_equal(fd.cpu().numpy().view(np.uint32), orc.dequantize_i32(big, 3.1e-5).view(np.uint32))
+
+
 def test_quantize_division_free_form_is_exact():
     """quantize_u8 divides by multiplying with the correctly rounded reciprocal and two FMA corrections, clamps before
     the division and rounds without the reference's double: checked against the reference arithmetic on the values where
@@ -1138,21 +1162,3 @@ def test_two_group_kernel_matches_the_oracle():
     w = rng.integers(0, 256, (64, 256, 3, 3), dtype=np.uint8)
     plan = hipq.Conv2d(x.shape, w, None, 1, 1, 1, 0.02, 7, 0.005, 100, 0.05, 3)
     assert not plan.kernel.endswith("_k2"), plan.kernel
-
-
-def test_machine_probes_launch_and_refuse_bad_arguments():
-    """hipq_probe_launch (the probes bench.py reports as machine_probes): every probe launches, ends and reports its
-    work; a buffer that is too small, a probe number out of range and a streamed region that is not a power of two
-    are refused before anything is launched."""
-    import ctypes
-    lib = hipq.lib()
-    buf = torch.randint(0, 256, (64 << 20,), dtype=torch.uint8, device="cuda")
-    units = ctypes.c_double(-1)
-    st = torch.cuda.current_stream().cuda_stream
-    for which, iters, param in [(0, 50, 0), (1, 50, 0), (2, 1, 0), (3, 64, 1 << 20)] + [(w, 20, 0) for w in range(4, 10)]:
-        hipq.check(lib.hipq_probe_launch(which, buf.data_ptr(), buf.numel(), iters, param, ctypes.byref(units), st))
-        torch.cuda.synchronize()
-        assert (units.value == 0) == (which == 2), (which, units.value)
-    for bad in [(10, buf.numel(), 10, 0), (0, 1 << 20, 10, 0), (3, buf.numel(), 10, 3 << 20), (0, buf.numel(), 0, 0)]:
-        with pytest.raises(hipq.HipqError, match="hipq_probe_launch"):
-            hipq.check(lib.hipq_probe_launch(bad[0], buf.data_ptr(), bad[1], bad[2], bad[3], ctypes.byref(units), st))

@@ -150,6 +150,30 @@ def test_per_channel_weight_scales_through_the_op_api(own_rt):
     assert same_bits(ip.output(0).numpy().reshape(6, 37), want_ip) and len(np.unique(want_ip)) > 8
     for o in (ip, conv):
         o.delete()
+    # The reference's converter writes one walpha entry per constant input - the weights' scale, then the bias's
+    # (python/nart/modules/quant.py:178-208) - and the CPU module reads the first (conv_2d_uint8_impl.c:61, ip.cpp:148): a
+    # two-channel layer with a bias carries two entries and is still per tensor.
+    x2 = rng.integers(0, 256, (1, 16, 6, 6), dtype=np.uint8)
+    w2 = rng.integers(0, 256, (2, 16, 3, 3), dtype=np.uint8)
+    b2 = rng.integers(-3000, 3000, 2).astype(np.int32)
+    wa2 = np.array([0.004, 0.004 * 0.031], np.float32)
+    conv2 = ws.conv2d(ws.tensor(x2), ws.tensor(w2), ws.tensor(b2), 1, 1, 1,
+                      dict(ialpha=0.031, izp=77, walpha=wa2, wzp=128, oalpha=0.4, ozp=13)).prepare().run()
+    want2 = orc.conv2d_u8(x2, w2, b2, 1, 1, 1, 0.031, 77, float(wa2[0]), 128, 0.4, 13)
+    assert same_bits(conv2.output(0).numpy(), want2) and len(np.unique(want2)) > 8
+    xf2 = rng.integers(0, 256, (5, 64), dtype=np.uint8)
+    wf2 = rng.integers(0, 256, (2, 64), dtype=np.uint8)
+    ip2 = ws.ip(ws.tensor(xf2), ws.tensor(wf2), ws.tensor(b2),
+                dict(ialpha=0.02, izp=128, walpha=wa2, wzp=128, oalpha=0.7, ozp=100)).prepare().run()
+    want_ip2 = orc.ip_u8(xf2, wf2, b2, 0.02, 128, float(wa2[0]), 128, 0.7, 100)
+    assert same_bits(ip2.output(0).numpy().reshape(5, 2), want_ip2.reshape(5, 2))
+    # without a bias two entries for two channels ARE one per channel
+    conv3 = ws.conv2d(ws.tensor(x2), ws.tensor(w2), None, 1, 1, 1,
+                      dict(ialpha=0.031, izp=77, walpha=wa2 * np.float32([1, 40]), wzp=128, oalpha=0.4, ozp=13)).prepare().run()
+    want3 = orc.conv2d_u8_per_channel(x2, w2, None, 1, 1, 1, 0.031, 77, wa2 * np.float32([1, 40]), 128, 0.4, 13)
+    assert same_bits(conv3.output(0).numpy(), want3)
+    for o in (conv2, ip2, conv3):
+        o.delete()
     ws.delete()
 
 

@@ -506,3 +506,19 @@ def test_per_channel_requantisation_is_pinned():
     y8 = orc.requant_per_channel_i8(acc8, ia, wa, oa, 7)
     for k in range(K):
         assert np.array_equal(y8[:, k], orc.conv2d_i8(xs, ws, b, 1, 1, 1, ia, float(wa[k]), oa, 7)[:, k]), k
+
+
+def test_dequantize_of_int32_accumulators_is_its_closed_form():
+    """orc.dequantize_i32 has no reference counterpart (op_dequantize_run_u8 / _i8 read bytes only): it is pinned by
+    what the arithmetic fixes - one int32 -> fp32 conversion, round to nearest even, and one fp32 multiply - computed
+    independently by numpy, on values on both sides of 2^24 (where the conversion starts to round), the int32 extremes
+    and ties."""
+    rng = np.random.default_rng(5)
+    acc = np.concatenate([rng.integers(-2**31, 2**31, 4000), rng.integers(-2**24 - 64, 2**24 + 64, 4000),
+                          np.array([0, 1, -1, 2**24 + 1, 2**24 + 3, -(2**24) - 1, 2**25 + 2, 2**25 + 6, 2**31 - 1, -2**31])]).astype(np.int32)
+    for alpha in (np.float32(0.02) * np.float32(0.005), np.float32(1.0), np.float32(3.1e-5)):
+        want = acc.astype(np.float32) * np.float32(alpha)
+        got = orc.dequantize_i32(acc, float(alpha))
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # the conversion is to NEAREST EVEN: 2^24 + 1 -> 2^24, 2^24 + 3 -> 2^24 + 4
+    assert orc.dequantize_i32(np.array([2**24 + 1, 2**24 + 3], np.int32), 1.0).tolist() == [2.0**24, 2.0**24 + 4]
