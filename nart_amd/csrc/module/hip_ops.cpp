@@ -94,6 +94,7 @@ typedef std::map<const mem_t *, std::set<const op_t *>> reader_map;
 // keyed by workspace (the runtime is single-threaded, art/include/art/workspace.h has no locking either)
 std::map<const workspace_t *, reader_map> g_readers;
 long g_fused_adds = 0, g_fused_relus = 0, g_fused_pools = 0, g_chained_convs = 0, g_fused_dequants = 0; // fused launches so far (hip_module_fused_*)
+long g_fused_blocks = 0, g_fused_tails = 0; // whole bottleneck blocks / blocks from their 3x3 layer on, as one launch
 
 reader_map &readers_of(op_t *op) { return g_readers[op->workspace]; }
 
@@ -132,6 +133,9 @@ struct conv_op_t {
     const void *w_seen;    // identity of the weights the plan was packed from
     uint64_t pc_seen;      // checksum of the per-channel weight scales the plan was built with (0: per tensor)
     int defer;             // 0 undecided, 1 leave the launch to the add / relu that reads the output, -1 launch at run()
+    // A convolution that heads a bottleneck block (1x1, then 3x3, then 1x1 and the add with the block's input) which
+    // hipq_bottleneck_run computes in one launch: the block's 3x3 convolution and its add (else null).
+    const op_t *blk_next, *blk_add;
 };
 
 void conv_config(op_t *op)
@@ -187,6 +191,11 @@ void conv_launch_plain(void *ctx)
 }
 
 bool eltwise_is_plain_sum(const op_t *op); // two inputs, SUM, unit coefficients: computes what add computes
+struct QSet;
+const QSet &add_inputs(const op_t *add_op);  // the input / output quantisation settings of an add or eltwise operator
+const QSet &add_output(const op_t *add_op);
+bool conv_heads_block(op_t *op, const op_t *r);
+bool conv_continues_block(op_t *op, const op_t *r);
 // a dequantize that the fully-connected layer's kernel can compute in its epilogue (hipq_conv2d_dequant_fusable)
 bool dequantize_fuses_with(const op_t *deq_op, const hipq_conv2d_plan *plan);
 // a max pooling that the stem convolution's kernel can compute as well (hipq_conv2d_maxpool_fusable)
@@ -194,6 +203,79 @@ bool pool_fuses_with(const op_t *pool_op, const hipq_conv2d_plan *plan);
 // the convolution `op` as the tail of the kernel that computes the add it reads (hipq_conv2d_run_add_conv); y: where its
 // output goes, relu: with the ReLU clamp.  false: not possible, run it plainly
 bool conv_run_chained(op_t *op, void *y, int relu);
+
+// ---- whole bottleneck blocks ---------------------------------------------------------------------------------------
+// 1x1 -> 3x3 -> 1x1 -> add(., block input), every intermediate tensor read by its successor only: the 1x1 head and the
+// 3x3 leave hooks like the widening convolution does, and the add's run() launches hipq_bottleneck_run (all three
+// convolutions and the add) or, where only that form applies, hipq_bottleneck_tail_run (from the 3x3 on, with any
+// residual; the 1x1 convolution that reads the sum may ride along, conv_run_chained).  Hooks settle in a chain: asking
+// for the 3x3's output runs the head first.
+const op_t *only_reader(const op_t *op)
+{
+    const auto wit = g_readers.find(op->workspace);
+    if (wit == g_readers.end())
+        return nullptr;
+    const auto it = wit->second.find(op->output_tensors[0].mem);
+    if (it == wit->second.end() || it->second.size() != 1 || (*it->second.begin())->workspace != op->workspace)
+        return nullptr;
+    return *it->second.begin();
+}
+
+// the add (or plain two-input SUM) that is the only reader of convolution r's output and reads it with the scale it is
+// written with; *idx: which of its inputs that is
+const op_t *add_reading(const op_t *r, int *idx)
+{
+    const op_t *a = only_reader(r);
+    if (a == nullptr || !(a->entry->tp == &op_add_tp || eltwise_is_plain_sum(a)) || a->input_size != 2
+        || a->input_tensors[0]->mem == a->input_tensors[1]->mem)
+        return nullptr;
+    const int i = a->input_tensors[0]->mem == r->output_tensors[0].mem ? 0 : 1;
+    const conv_op_t *c = reinterpret_cast<const conv_op_t *>(r);
+    const QSet &qi = add_inputs(a);
+    if (qi.alpha[i] != c->desc.oalpha || qi.zp[i] != c->desc.ozp)
+        return nullptr;
+    *idx = i;
+    return a;
+}
+
+// op: a 1x1 convolution, r (its only reader): a 3x3 convolution, then a 1x1 convolution, then the add with op's input
+bool conv_heads_block(op_t *op, const op_t *r)
+{
+    conv_op_t *c1 = reinterpret_cast<conv_op_t *>(op);
+    c1->blk_next = c1->blk_add = nullptr;
+    const op_t *r2 = only_reader(r);
+    if (r2 == nullptr || r2->entry->tp != &op_conv_2d_tp)
+        return false;
+    int i = 0;
+    const op_t *a = add_reading(r2, &i);
+    if (a == nullptr || a->input_tensors[1 - i]->mem != op->input_tensors[0]->mem)
+        return false;
+    const conv_op_t *c2 = reinterpret_cast<const conv_op_t *>(r), *c3 = reinterpret_cast<const conv_op_t *>(r2);
+    const QSet &qi = add_inputs(a), &qo = add_output(a);
+    if (!c1->plan || !c2->plan || !c3->plan || qi.alpha[1 - i] != c1->desc.ialpha || qi.zp[1 - i] != c1->desc.izp
+        || !hipq_bottleneck_fusable(c1->plan, c2->plan, c3->plan, i == 1, qo.alpha[0], qo.zp[0], qo.bits[0]))
+        return false;
+    c1->blk_next = r;
+    c1->blk_add = a;
+    return true;
+}
+
+// op: a 3x3 convolution whose only reader r is a 1x1 convolution read by an add only - the middle of a block whose head
+// has just left its launch to this chain, or of one that hipq_bottleneck_tail_run computes from here on
+bool conv_continues_block(op_t *op, const op_t *r)
+{
+    const conv_op_t *c2 = reinterpret_cast<const conv_op_t *>(op), *c3 = reinterpret_cast<const conv_op_t *>(r);
+    int i = 0;
+    const op_t *a = add_reading(r, &i);
+    if (a == nullptr || !c2->plan || !c3->plan)
+        return false;
+    const hip_mem_t *in = as_hip(op->input_tensors[0]->mem);
+    if (in->pending == conv_launch_plain && reinterpret_cast<const conv_op_t *>(static_cast<op_t *>(in->pending_ctx))->blk_next == op)
+        return true;
+    const QSet &qi = add_inputs(a), &qo = add_output(a);
+    return hipq_bottleneck_tail_fusable(c2->plan, c3->plan, i == 1, qi.alpha[1 - i], qi.zp[1 - i], qo.alpha[0], qo.zp[0], qo.bits[0],
+                                        nullptr) != 0;
+}
 
 // 1: the only reader of the convolution's output is an add or a relu of this workspace that can take over the launch
 bool sole_reader_fuses(op_t *op)
@@ -211,6 +293,8 @@ bool sole_reader_fuses(op_t *op)
         return false;
     if (r->entry->tp == &op_relu_tp)
         return true; // any plan runs with the ReLU clamp (hipq_conv2d_run_relu)
+    if (r->entry->tp == &op_conv_2d_tp)
+        return conv_heads_block(op, r) || conv_continues_block(op, r);
     if (r->entry->tp == &op_pool_tp)
         return pool_fuses_with(r, c->plan);
     if (r->entry->tp == &op_hip_dequantize_tp)
@@ -366,6 +450,9 @@ struct ew_op_t {
                   // convolution), -1 launch at run()
 };
 
+const QSet &add_inputs(const op_t *add_op) { return reinterpret_cast<const ew_op_t *>(add_op)->qi; }
+const QSet &add_output(const op_t *add_op) { return reinterpret_cast<const ew_op_t *>(add_op)->qo; }
+
 size_t device_bytes_of(const tensor_t *t)
 {
     const hip_mem_t *m = as_hip(t->mem);
@@ -417,6 +504,62 @@ int deferred_conv_input(op_t *op)
     return -1;
 }
 
+// the 3x3 convolution that left its launch to the widening convolution cop (which left its own to an add); null: none
+op_t *deferred_mid_of(op_t *cop)
+{
+    hip_mem_t *m2 = as_hip(cop->input_tensors[0]->mem);
+    if (m2->pending != conv_launch_plain)
+        return nullptr;
+    op_t *cop2 = static_cast<op_t *>(m2->pending_ctx);
+    return cop2->entry->tp == &op_conv_2d_tp && only_reader(cop2) == cop ? cop2 : nullptr;
+}
+
+// The add `op`, whose input i is the widening convolution cop that left it its launch, as one launch with the block's
+// earlier convolutions where those left theirs as well: the whole block (hipq_bottleneck_run) or the block from its 3x3
+// layer on (hipq_bottleneck_tail_run), the sum into y; nxt: the 1x1 convolution that reads the sum and rides along
+// (output into y_next, relu: with the ReLU clamp), or null.  false: nothing launched.
+bool block_launch(op_t *op, op_t *cop, int i, void *y, op_t *nxt, int relu, void *y_next)
+{
+    ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    op_t *cop2 = deferred_mid_of(cop);
+    if (cop2 == nullptr)
+        return false;
+    conv_op_t *c3 = reinterpret_cast<conv_op_t *>(cop), *c2 = reinterpret_cast<conv_op_t *>(cop2);
+    const int o = 1 - i;
+    hip_mem_t *m1 = as_hip(cop2->input_tensors[0]->mem);
+    if (nxt == nullptr && m1->pending == conv_launch_plain) {
+        op_t *cop1 = static_cast<op_t *>(m1->pending_ctx);
+        conv_op_t *c1 = reinterpret_cast<conv_op_t *>(cop1);
+        if (cop1->entry->tp == &op_conv_2d_tp && c1->blk_next == cop2 && c1->blk_add == op
+            && op->input_tensors[o]->mem == cop1->input_tensors[0]->mem && e->qi.alpha[o] == c1->desc.ialpha && e->qi.zp[o] == c1->desc.izp
+            && hipq_bottleneck_fusable(c1->plan, c2->plan, c3->plan, o == 0, e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0])) {
+            const void *x = in_ptr(cop1, 0);
+            if (x != y && hipq_bottleneck_run(c1->plan, c2->plan, c3->plan, x, o == 0, e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0], y,
+                                              op_stream(op)) == 0) {
+                ++g_fused_adds;
+                ++g_fused_blocks;
+                return true; // the three convolutions' outputs stay unwritten; their hooks stay for whoever asks
+            }
+        }
+    }
+    const conv_op_t *cn = reinterpret_cast<const conv_op_t *>(nxt);
+    if (!hipq_bottleneck_tail_fusable(c2->plan, c3->plan, o == 0, e->qi.alpha[o], e->qi.zp[o], e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0],
+                                      nxt ? cn->plan : nullptr))
+        return false;
+    const void *res = in_ptr(op, o);  // settles the other input if it is deferred
+    const void *x = in_ptr(cop2, 0);  // and the block's head, whose output this form reads
+    if (deferred_mid_of(cop) != cop2)
+        return false; // settling reached the 3x3 convolution itself: it has run, the caller's path reads its output
+    if (hipq_bottleneck_tail_run(c2->plan, c3->plan, x, res, o == 0, e->qi.alpha[o], e->qi.zp[o], e->qo.alpha[0], e->qo.zp[0],
+                                 e->qo.bits[0], y, nxt ? cn->plan : nullptr, relu, y_next, op_stream(op)) != 0)
+        return false;
+    ++g_fused_adds;
+    ++g_fused_tails;
+    if (nxt)
+        ++g_chained_convs;
+    return true;
+}
+
 // the add `op` as the epilogue of the convolution that left it its launch, into y; false: run it plainly
 bool run_fused_into_convolution(op_t *op, void *y)
 {
@@ -426,6 +569,8 @@ bool run_fused_into_convolution(op_t *op, void *y)
         return false;
     op_t *cop = static_cast<op_t *>(as_hip(op->input_tensors[i]->mem)->pending_ctx);
     conv_op_t *c = reinterpret_cast<conv_op_t *>(cop);
+    if (block_launch(op, cop, i, y, nullptr, 0, nullptr))
+        return true;
     const int o = 1 - i;
     const void *res = in_ptr(op, o); // settles the other input if it is deferred as well
     const void *x = in_ptr(cop, 0);
@@ -482,9 +627,13 @@ bool add_defers(op_t *op)
                 if (r->workspace != op->workspace || r->entry->tp != &op_conv_2d_tp)
                     continue;
                 const conv_op_t *rc = reinterpret_cast<const conv_op_t *>(r);
+                op_t *mid = deferred_mid_of(static_cast<op_t *>(as_hip(op->input_tensors[i]->mem)->pending_ctx));
                 if (rc->plan != nullptr && r->input_tensors[0]->mem == op->output_tensors[0].mem
-                    && hipq_conv2d_add_conv_fusable(c->plan, o == 0, e->qi.alpha[o], e->qi.zp[o], e->qo.alpha[0], e->qo.zp[0],
-                                                    e->qo.bits[0], rc->plan)) {
+                    && (hipq_conv2d_add_conv_fusable(c->plan, o == 0, e->qi.alpha[o], e->qi.zp[o], e->qo.alpha[0], e->qo.zp[0],
+                                                     e->qo.bits[0], rc->plan)
+                        || (mid != nullptr
+                            && hipq_bottleneck_tail_fusable(reinterpret_cast<conv_op_t *>(mid)->plan, c->plan, o == 0, e->qi.alpha[o],
+                                                            e->qi.zp[o], e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0], rc->plan)))) {
                     e->defer = 1;
                     break;
                 }
@@ -518,6 +667,14 @@ bool conv_run_chained(op_t *op, void *y, int relu)
     op_t *cop = static_cast<op_t *>(as_hip(aop->input_tensors[i]->mem)->pending_ctx);
     conv_op_t *c = reinterpret_cast<conv_op_t *>(cop), *c2 = reinterpret_cast<conv_op_t *>(op);
     const int o = 1 - i;
+    if (deferred_mid_of(cop) != nullptr) {
+        // the block from its 3x3 layer on, the add and this convolution as one launch
+        sm->pending = nullptr; // the sum is written by that launch
+        if (block_launch(aop, cop, i, sm->dev, op, relu, y))
+            return true;
+        sm->pending = add_launch_deferred;
+        sm->pending_ctx = aop;
+    }
     if (!hipq_conv2d_add_conv_fusable(c->plan, o == 0, e->qi.alpha[o], e->qi.zp[o], e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0],
                                       c2->plan))
         return false;
@@ -1042,6 +1199,8 @@ ART_PUBLIC long hip_module_fused_relus(void) { return g_fused_relus; }
 ART_PUBLIC long hip_module_fused_pools(void) { return g_fused_pools; }
 ART_PUBLIC long hip_module_chained_convs(void) { return g_chained_convs; }
 ART_PUBLIC long hip_module_fused_dequants(void) { return g_fused_dequants; }
+ART_PUBLIC long hip_module_fused_blocks(void) { return g_fused_blocks; }
+ART_PUBLIC long hip_module_fused_tails(void) { return g_fused_tails; }
 
 ART_PUBLIC void *hip_workspace_stream(workspace_t *w) { return reinterpret_cast<hip_workspace_t *>(w)->stream; }
 

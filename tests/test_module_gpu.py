@@ -307,6 +307,106 @@ def test_add_and_the_next_1x1_convolution_run_as_one_kernel(own_rt):
     ws.delete()
 
 
+def test_whole_bottleneck_block_runs_as_one_kernel(own_rt):
+    """conv_2d (1024 -> 256, 1x1) -> conv_2d (3x3) -> conv_2d (256 -> 1024, 1x1) -> add with the block's input: the three
+    convolutions leave their launches to the add, whose run() launches hipq_bottleneck_run.  A host that reads an
+    intermediate tensor in between gets the operators one by one (the hooks settle in a chain); every tensor of the
+    block can still be read afterwards.  Same bytes as the oracle's four operators, pass after pass."""
+    import ctypes as C
+    from oracle import orc
+    blocks = own_rt.libs[1].hip_module_fused_blocks
+    blocks.restype = C.c_long
+    ws = own_rt.workspace("hip")
+    rng = np.random.default_rng(31)
+    x = rng.integers(0, 256, (2, 1024, 14, 14), dtype=np.uint8)
+    shapes = ((256, 1024, 1), (256, 256, 3), (1024, 256, 1))
+    ws_w = [rng.integers(1, 256, (K, Cc, k, k), dtype=np.uint8) for K, Cc, k in shapes]
+    bs = [rng.integers(-20000, 20000, K).astype(np.int32) for K, _, _ in shapes]
+    qs = [dict(ialpha=0.05, izp=9, walpha=0.0011, wzp=128, oalpha=0.06, ozp=0),
+          dict(ialpha=0.06, izp=0, walpha=0.0016, wzp=128, oalpha=0.055, ozp=0),
+          dict(ialpha=0.055, izp=0, walpha=0.0035, wzp=128, oalpha=0.07, ozp=121)]
+    t = x
+    wants = []
+    for w, b, q, (K, Cc, k) in zip(ws_w, bs, qs, shapes):
+        t = orc.conv2d_u8(t, w, b, k // 2, 1, 1, q["ialpha"], q["izp"], q["walpha"], 128, q["oalpha"], q["ozp"])
+        wants.append(t)
+    for res_first in (False, True):
+        want = orc.add_u8(x, t, 0.05, 9, 0.07, 121, 0.09, 0) if res_first else orc.add_u8(t, x, 0.07, 121, 0.05, 9, 0.09, 0)
+        assert len(np.unique(want)) > 32
+        for peek, expect in ((None, 1), (0, 0), (1, 0)):
+            tx = ws.tensor(x)
+            convs, cur = [], tx
+            for w, b, q, (K, Cc, k) in zip(ws_w, bs, qs, shapes):
+                convs.append(ws.conv2d(cur, ws.tensor(w), ws.tensor(b), k // 2, 1, 1, q).prepare())
+                cur = convs[-1].output(0)
+            ins = [tx, cur] if res_first else [cur, tx]
+            qa = dict(ialpha=[0.05, 0.07] if res_first else [0.07, 0.05], izp=[9, 121] if res_first else [121, 9], oalpha=0.09, ozp=0)
+            add = ws.add(ins[0], ins[1], qa).prepare()
+            for rep in range(2):
+                n0 = blocks()
+                for j, c in enumerate(convs):
+                    c.run()
+                    if peek == j:
+                        assert same_bits(c.output(0).numpy(), wants[j]), (res_first, peek, rep)
+                add.run()
+                assert same_bits(add.output(0).numpy(), want), (res_first, peek, rep)
+                assert blocks() == n0 + expect, (res_first, peek, rep)
+            for j, c in enumerate(convs):  # never written by the fused launch: computed on demand
+                assert same_bits(c.output(0).numpy(), wants[j]), (res_first, peek, j)
+            for o in [add] + convs[::-1]:
+                o.delete()
+    ws.delete()
+
+
+def test_block_tail_and_next_convolution_run_as_one_kernel(own_rt):
+    """conv_2d (3x3, 128 -> 128) -> conv_2d (128 -> 512, 1x1) -> add with any residual -> conv_2d (512 -> 128, 1x1): the 3x3
+    and the widening convolution leave their launches to the add, the add leaves its own to the convolution that reads
+    the sum, and that convolution's run() launches hipq_bottleneck_tail_run for all four.  Without a chained reader the
+    add launches the first three.  A host that peeks gets the operators one by one."""
+    import ctypes as C
+    from oracle import orc
+    tails = own_rt.libs[1].hip_module_fused_tails
+    tails.restype = C.c_long
+    chained = own_rt.libs[1].hip_module_chained_convs
+    chained.restype = C.c_long
+    ws = own_rt.workspace("hip")
+    rng = np.random.default_rng(32)
+    t1 = rng.integers(0, 256, (2, 128, 28, 28), dtype=np.uint8)
+    r = rng.integers(0, 256, (2, 512, 28, 28), dtype=np.uint8)
+    w2, b2 = rng.integers(1, 256, (128, 128, 3, 3), dtype=np.uint8), rng.integers(-20000, 20000, 128).astype(np.int32)
+    w3, b3 = rng.integers(1, 256, (512, 128, 1, 1), dtype=np.uint8), rng.integers(-9000, 9000, 512).astype(np.int32)
+    wn, bn = rng.integers(1, 256, (128, 512, 1, 1), dtype=np.uint8), rng.integers(-9000, 9000, 128).astype(np.int32)
+    q2 = dict(ialpha=0.05, izp=0, walpha=0.0022, wzp=128, oalpha=0.055, ozp=0)
+    q3 = dict(ialpha=0.055, izp=0, walpha=0.005, wzp=128, oalpha=0.07, ozp=121)
+    qn = dict(ialpha=0.09, izp=0, walpha=0.0024, wzp=128, oalpha=0.06, ozp=0)
+    want2 = orc.conv2d_u8(t1, w2, b2, 1, 1, 1, 0.05, 0, 0.0022, 128, 0.055, 0)
+    want3 = orc.conv2d_u8(want2, w3, b3, 0, 1, 1, 0.055, 0, 0.005, 128, 0.07, 121)
+    want_a = orc.add_u8(want3, r, 0.07, 121, 0.04, 77, 0.09, 0)
+    want_n = orc.conv2d_u8(want_a, wn, bn, 0, 1, 1, 0.09, 0, 0.0024, 128, 0.06, 0)
+    assert len(np.unique(want_n)) > 32
+    for with_next, peek, exp_tail, exp_chain in ((True, False, 1, 1), (False, False, 1, 0), (True, True, 0, 0)):
+        c2 = ws.conv2d(ws.tensor(t1), ws.tensor(w2), ws.tensor(b2), 1, 1, 1, q2).prepare()
+        c3 = ws.conv2d(c2.output(0), ws.tensor(w3), ws.tensor(b3), 0, 1, 1, q3).prepare()
+        add = ws.add(c3.output(0), ws.tensor(r), dict(ialpha=[0.07, 0.04], izp=[121, 77], oalpha=0.09, ozp=0)).prepare()
+        cn = ws.conv2d(add.output(0), ws.tensor(wn), ws.tensor(bn), 0, 1, 1, qn).prepare() if with_next else None
+        for rep in range(2):
+            t0, k0 = tails(), chained()
+            c2.run()
+            if peek:
+                assert same_bits(c2.output(0).numpy(), want2)
+            c3.run()
+            add.run()
+            if cn:
+                cn.run()
+                assert same_bits(cn.output(0).numpy(), want_n), (with_next, peek, rep)
+            assert same_bits(add.output(0).numpy(), want_a), (with_next, peek, rep)
+            assert tails() == t0 + exp_tail and chained() - k0 in (exp_chain, 1 if (peek and with_next) else exp_chain), (with_next, peek, rep)
+        assert same_bits(c3.output(0).numpy(), want3) and same_bits(c2.output(0).numpy(), want2)
+        for o in ([cn] if cn else []) + [add, c3, c2]:
+            o.delete()
+    ws.delete()
+
+
 def test_convolution_and_relu_run_as_one_kernel(own_rt):
     """A convolution whose output only a relu with the same scale and zero point on both sides reads leaves its launch
     to that relu (the clamp moves into the convolution's epilogue); other relus run as operators of their own."""
