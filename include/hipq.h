@@ -228,6 +228,22 @@ int hipq_conv2d_run_add_conv(const hipq_conv2d_plan *plan, const void *x, const 
                              const hipq_conv2d_plan *next, int next_relu, void *y_next, void *stream);
 
 /*
+ * The last layer of a bottleneck block with a projection shortcut, in one launch: y = add(plan(x), shortcut(x_shortcut)),
+ * bit-identical to hipq_conv2d_run(shortcut, x_shortcut, r) followed by hipq_conv2d_run_add(plan, x, residual = r, ...) -
+ * op_conv_2d_u8xu8_run (src/op/conv_2d_uint8_impl.c:39-165) twice, then op_quant_add_run (src/op/add.c:83-148) - but the
+ * shortcut's bytes never travel to memory.  `plan`: a 1x1 / stride 1 convolution from 256 or 512 channels; `shortcut`: a
+ * 1x1 convolution, stride 1 or 2, from twice as many channels to the same output pixels and channels (a multiple of 128);
+ * uint8 tensors with dense channel strides, weight zero points 128, per-tensor weight scales, no ReLU on the shortcut.
+ * The add's inputs are (plan(x), shortcut(...)), or the other way round when shortcut_is_input0 != 0; oalpha / ozp /
+ * obits (8) describe the sum.  hipq_conv2d_add2_fusable answers (1 / 0); hipq_conv2d_run_add2 fails with an error
+ * otherwise (run the operators separately).
+ */
+int hipq_conv2d_add2_fusable(const hipq_conv2d_plan *plan, const hipq_conv2d_plan *shortcut, int shortcut_is_input0, float oalpha,
+                             int ozp, int obits);
+int hipq_conv2d_run_add2(const hipq_conv2d_plan *plan, const void *x, const hipq_conv2d_plan *shortcut, const void *x_shortcut,
+                         int shortcut_is_input0, float oalpha, int ozp, int obits, void *y, void *stream);
+
+/*
  * An identity bottleneck block of a residual network in one launch: y = add(widen(mid(reduce(x))), x), bit-identical to
  * hipq_conv2d_run(reduce, x, t1), hipq_conv2d_run(mid, t1, t2) and hipq_conv2d_run_add(widen, t2, residual = x, ...) -
  * op_conv_2d_u8xu8_run (src/op/conv_2d_uint8_impl.c:39-165) three times, then op_quant_add_run (src/op/add.c:83-148) -

@@ -2397,6 +2397,43 @@ extern "C" int hipq_bottleneck_run(const hipq_conv2d_plan *p1, const hipq_conv2d
     return launch_status("conv_bottleneck_kernel");
 }
 
+extern "C" int hipq_conv2d_add2_fusable(const hipq_conv2d_plan *p, const hipq_conv2d_plan *sc, int shortcut_is_input0, float oalpha,
+                                        int ozp, int obits)
+{
+    for (const hipq_conv2d_plan *q : {p, sc})
+        if (!q || q->variant != kMfma || !q->special || q->tile_selected || q->has_wzp || q->d.dtype != HIPQ_DTYPE_U8 || q->d.obits != 8)
+            return 0;
+    if (obits != 8 || ozp < 0 || ozp > 255)
+        return 0;
+    ConvArgs a;
+    if (!add_args(p, shortcut_is_input0, sc->d.oalpha, sc->d.ozp, oalpha, ozp, obits, &a) || !conv_wreg_dual_applies(a, sc->args))
+        return 0;
+    // built-in rule: where it measured faster than the two launches - 256 -> 1024 with a 512-channel shortcut on 14x14
+    // images at batch 64 (28.1 us against 15.8 + 14.1 and a launch gap; 512 -> 2048 on 7x7 images loses, 28.9 against
+    // 12.6 + 10.7: its pixel operands leave LDS room for one work-group of four waves per CU);
+    // hipq_conv2d_plan_special(plan, 2): wherever it applies
+    return p->special == 2 || (a.P <= 16384 && a.in_cs == 256) ? 1 : 0;
+}
+
+extern "C" int hipq_conv2d_run_add2(const hipq_conv2d_plan *p, const void *x, const hipq_conv2d_plan *sc, const void *x_shortcut,
+                                    int shortcut_is_input0, float oalpha, int ozp, int obits, void *y, void *stream)
+{
+    clear_error();
+    HIPQ_REQUIRE(p && sc && x && x_shortcut && y, "hipq_conv2d_run_add2: null argument");
+    HIPQ_REQUIRE(hipq_conv2d_add2_fusable(p, sc, shortcut_is_input0, oalpha, ozp, obits),
+                 "hipq_conv2d_run_add2: these two plans (%s, %s) and this add do not run as one kernel: run hipq_conv2d_run and "
+                 "hipq_conv2d_run_add", p->name.c_str(), sc->name.c_str());
+    ConvArgs a, b = sc->args;
+    add_args(p, shortcut_is_input0, sc->d.oalpha, sc->d.ozp, oalpha, ozp, obits, &a);
+    a.x = static_cast<const uint8_t *>(x);
+    a.y = static_cast<uint8_t *>(y);
+    a.acc_out = b.acc_out = nullptr;
+    b.x = static_cast<const uint8_t *>(x_shortcut);
+    b.y = nullptr;
+    launch_conv_wreg_dual(a, b, static_cast<hipStream_t>(stream));
+    return launch_status("conv_wreg_dual_kernel");
+}
+
 // hipq_bottleneck_tail_*: the launch arguments of the three layers; false if the chain does not run as one kernel
 static bool tail_args(const hipq_conv2d_plan *p2, const hipq_conv2d_plan *p3, int residual_is_input0, float res_alpha, int res_zp,
                       float oalpha, int ozp, int obits, const hipq_conv2d_plan *next, ConvArgs *a2, ConvArgs *a3, ConvArgs *an)

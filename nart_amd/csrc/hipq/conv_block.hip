@@ -72,16 +72,13 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
                                                                     const BlockGeom geo)
 {
     constexpr int NW = 2 * G, NT = 128 * G, CM = 64 * G, CW = 256 * G;
-    constexpr bool ONE_ROUND = G == 4 && MT1 == 2;          // LDS holds every exchange slot at once
     constexpr int X_BYTES = 32 * MT1 * CW;                  // the region's pixel rows, CW bytes each
     constexpr int G_OFF = X_BYTES, G_BYTES = kGridRows * CM; // layer 1's bytes on the 9 x 9 grid, CM bytes a row; later layer 2's
-    constexpr int S_OFF = G_OFF + G_BYTES, S_BYTES = NW * 4096 * (ONE_ROUND ? MT1 : 1); // the pairs' exchange slots
-    constexpr int D1 = MT1 == 2 ? 6 : 4, D2 = 6;            // slabs of weights a wave holds ahead, layers 1 and 2
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[S_OFF + S_BYTES];
+    constexpr int D1 = MT1 == 2 ? 10 : 8, D2 = 10;          // slabs of weights a wave holds ahead, layers 1 and 2
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[G_OFF + G_BYTES];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int p = lane & 31, h = lane >> 5;
-    const int ng = wave % G, kh = wave / G, partner = (wave + G) % NW;
 
     // work-groups go to the 8 XCDs in turn: XCD x takes the x-th contiguous eighth of the patches, so the patches of an
     // image - which share border pixels - and all weights are read through one L2
@@ -124,13 +121,13 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
 
     // Weight operands come in fragment order (ConvArgs::wfrag): the 1 KB a wave's load instruction fetches for slab s,
     // 32-channel tile T, k-step kk is contiguous at ((s * tiles + T) * 2 + kk) * 1024, lane l's 16 bytes at 16 l.
-    // the wave's two channel tiles of layers 1 and 2: tile 0 (kept after the pair's exchange) and tile 1 (sent)
-    const int ct0 = 64 * ng + 32 * kh, ct1 = 64 * ng + 32 * (1 - kh);
+    // layers 1 and 2: a wave owns 32 of the CM channels and the whole reduction, so the waves exchange nothing
+    const int ct0 = 32 * wave;
     const size_t wslab1 = (size_t)a1.kout_pad * 64, wslab2 = (size_t)a2.kout_pad * 64, wslab3 = (size_t)a3.kout_pad * 64;
-    const uint8_t *w10 = a1.wfrag + (size_t)ct0 * 64 + lane * 16, *w11 = a1.wfrag + (size_t)ct1 * 64 + lane * 16;
-    const uint8_t *w20 = a2.wfrag + (size_t)ct0 * 64 + lane * 16, *w21 = a2.wfrag + (size_t)ct1 * 64 + lane * 16;
-    auto ldw1 = [&](int s, int kk, int nt) { return ldg128((nt ? w11 : w10) + (size_t)s * wslab1 + kk * 1024); };
-    auto ldw2 = [&](int s, int kk, int nt) { return ldg128((nt ? w21 : w20) + (size_t)s * wslab2 + kk * 1024); };
+    const uint8_t *w10 = a1.wfrag + (size_t)ct0 * 64 + lane * 16;
+    const uint8_t *w20 = a2.wfrag + (size_t)ct0 * 64 + lane * 16;
+    auto ldw1 = [&](int s, int kk) { return ldg128(w10 + (size_t)s * wslab1 + kk * 1024); };
+    auto ldw2 = [&](int s, int kk) { return ldg128(w20 + (size_t)s * wslab2 + kk * 1024); };
     // layer 1, slab s: pieces 4 s .. 4 s + 3 of every pixel row of the x tile
     auto ldb1 = [&](int s, int kk, int t) {
         const int j = 32 * t + p, hs = h ^ (j & 15);
@@ -144,31 +141,26 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
     };
 
     // ================= layer 1: CW -> CM on the region's pixels =================
-    v16i acc1[MT1][2];
+    v16i acc1[MT1];
 #pragma unroll
-    for (int t = 0; t < MT1; t++) {
-        init_acc(acc1[t][0], a1.bias2 + ct0 + 16 * h, kh != 0);
-        init_acc(acc1[t][1], a1.bias2 + ct1 + 16 * h, kh != 0);
-    }
-    WeightRing<D1> r1;
-    ring_fill<4 * G, D1>(r1, kh, ldw1);
+    for (int t = 0; t < MT1; t++)
+        init_acc(acc1[t], a1.bias2 + ct0 + 16 * h, false);
+    WeightRing1<D1> r1;
+    ring_fill1<4 * G, D1>(r1, ldw1);
     // the region's bytes have landed (and this wave's pad bytes are written) before anyone reads LDS
     wait_vmcnt<0>();
     __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
     STAMP(1);
-    reduce_half<4 * G, MT1, D1>(acc1, r1, kh, (int)a1.xmask, ldw1, ldb1);
+    reduce_all<4 * G, MT1, D1>(acc1, r1, (int)a1.xmask, ldw1, ldb1);
     STAMP(2);
     // layer 2's first weights and folded biases travel while layer 1 is finished
-    WeightRing<D2> r2;
-    ring_fill<9 * G, D2>(r2, kh, ldw2);
-    v16i acc2[2][2];
+    WeightRing1<D2> r2;
+    ring_fill1<9 * G, D2>(r2, ldw2);
+    v16i acc2[2];
 #pragma unroll
-    for (int t = 0; t < 2; t++) {
-        init_acc(acc2[t][0], a2.bias2 + ct0 + 16 * h, kh != 0);
-        init_acc(acc2[t][1], a2.bias2 + ct1 + 16 * h, kh != 0);
-    }
-    pair_reduce<MT1, ONE_ROUND>(acc1, lds + S_OFF, wave, partner, lane);
+    for (int t = 0; t < 2; t++)
+        init_acc(acc2[t], a2.bias2 + ct0 + 16 * h, false);
     STAMP(3);
     // channels ct0 + 16 h .. + 15 of region pixel j -> the grid position of that pixel
 #pragma unroll
@@ -177,7 +169,7 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
         if (j < M1) {
             const int jy = (j * rwinv) >> 16, jx = j - jy * RW;
             const int g = (ry0 + jy - y0 + 1) * kGridW + (rx0 + jx - x0 + 1);
-            const v4i o = requant16(a1, acc1[t][0], a2.xmask);
+            const v4i o = requant16(a1, acc1[t], a2.xmask);
             *reinterpret_cast<v4i *>(lds + G_OFF + g * CM + ((((ct0 >> 4) + h) ^ swz<CM>(g)) << 4)) = o;
         }
     }
@@ -186,7 +178,7 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
     STAMP(4);
 
     // ================= layer 2: 3x3, CM -> CM, output index m = 9 * row + column =================
-    reduce_half<9 * G, 2, D2>(acc2, r2, kh, 0, ldw2, ldb2);
+    reduce_all<9 * G, 2, D2>(acc2, r2, 0, ldw2, ldb2);
     STAMP(5);
     // layer 3: this wave's 128 output channels in 4 chunks of 32; the first chunk's weights and biases travel now
     const uint8_t *w3 = a3.wfrag + (size_t)(128 * wave) * 64 + lane * 16;
@@ -200,13 +192,16 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
             b3[g] = *reinterpret_cast<const v4i *>(a3.bias2 + 128 * wave + 32 * cc + 16 * h + 4 * g);
     };
     load_chunk(0);
-    pair_reduce<2, ONE_ROUND>(acc2, lds + S_OFF, wave, partner, lane);
+    v4i o2[2];
+#pragma unroll
+    for (int t = 0; t < 2; t++)
+        o2[t] = requant16(a2, acc2[t], a3.xmask);
+    __builtin_amdgcn_s_barrier(); // every wave is done reading the grid: layer 2's bytes go there, row m
     STAMP(6);
-    // every wave has passed the exchange's barrier, i.e. is done reading the grid: layer 2's bytes go there, row m
 #pragma unroll
     for (int t = 0; t < 2; t++) {
         const int m = 32 * t + p;
-        const v4i o = requant16(a2, acc2[t][0], a3.xmask);
+        const v4i o = o2[t];
         *reinterpret_cast<v4i *>(lds + G_OFF + m * CM + ((((ct0 >> 4) + h) ^ swz<CM>(m)) << 4)) = o;
     }
     __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
@@ -281,14 +276,13 @@ __global__ __launch_bounds__(128 * G, (G <= 2 ? 3 : 2)) void conv_bottleneck_tai
     constexpr int GW = PW + 2, GH = PH + 2, NPIX = PH * PW, GROWS = (GH * GW + 7) / 8 * 8;
     constexpr int G_OFF = 0, G_BYTES = GROWS * CM;            // layer 2's input on the bordered grid
     constexpr int M_OFF = G_OFF + G_BYTES, M_BYTES = 64 * CM; // layer 2's bytes, row = pixel
-    constexpr int S_OFF = M_OFF + M_BYTES, S_BYTES = CHAIN ? 64 * CW : NW * 4096; // layer 2's exchange slots, then the sum tile
-    constexpr int D2 = G == 1 ? 4 : G == 2 ? 3 : 6, DN = D2; // slabs of weights a wave holds ahead (three waves per SIMD: fewer registers)
-    static_assert(NPIX <= 64 && NW * 4096 <= S_BYTES && NW * 4096 <= G_BYTES + M_BYTES, "slot reuse");
+    constexpr int S_OFF = M_OFF + M_BYTES, S_BYTES = CHAIN ? 64 * CW : 0; // the sum tile
+    constexpr int D2 = G <= 2 ? 6 : 10, DN = D2; // slabs of weights a wave holds ahead (three waves per SIMD: fewer registers)
+    static_assert(NPIX <= 64, "pixel slots");
     __shared__ __attribute__((aligned(1024))) uint8_t lds[S_OFF + S_BYTES];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int p = lane & 31, h = lane >> 5;
-    const int ng = wave % G, kh = wave / G, partner = (wave + G) % NW;
     const int gid = (int)(blockIdx.x % 8) * (int)(gridDim.x / 8) + (int)(blockIdx.x / 8); // XCD x: the x-th eighth of the patches
     if (gid >= geo.npatch)
         return;
@@ -313,10 +307,10 @@ __global__ __launch_bounds__(128 * G, (G <= 2 ? 3 : 2)) void conv_bottleneck_tai
             }
         }
     }
-    const int ct0 = 64 * ng + 32 * kh, ct1 = 64 * ng + 32 * (1 - kh);
+    const int ct0 = 32 * wave; // layers 2 and next: a wave owns 32 of the CM channels and the whole reduction
     const size_t wslab2 = (size_t)a2.kout_pad * 64, wslab3 = (size_t)a3.kout_pad * 64, wslabn = (size_t)an.kout_pad * 64;
-    const uint8_t *w20 = a2.wfrag + (size_t)ct0 * 64 + lane * 16, *w21 = a2.wfrag + (size_t)ct1 * 64 + lane * 16;
-    auto ldw2 = [&](int s, int kk, int nt) { return ldg128((nt ? w21 : w20) + (size_t)s * wslab2 + kk * 1024); };
+    const uint8_t *w20 = a2.wfrag + (size_t)ct0 * 64 + lane * 16;
+    auto ldw2 = [&](int s, int kk) { return ldg128(w20 + (size_t)s * wslab2 + kk * 1024); };
     // the lane's pixels q = 32 t + p (slots beyond the patch repeat its last pixel and are never stored)
     int grow[2];
     size_t pix[2];
@@ -335,18 +329,16 @@ __global__ __launch_bounds__(128 * G, (G <= 2 ? 3 : 2)) void conv_bottleneck_tai
     };
 
     // ================= layer 2: 3x3, CM -> CM =================
-    WeightRing<D2> r2;
-    ring_fill<9 * G, D2>(r2, kh, ldw2);
-    v16i acc2[2][2];
+    WeightRing1<D2> r2;
+    ring_fill1<9 * G, D2>(r2, ldw2);
+    v16i acc2[2];
 #pragma unroll
-    for (int t = 0; t < 2; t++) {
-        init_acc(acc2[t][0], a2.bias2 + ct0 + 16 * h, kh != 0);
-        init_acc(acc2[t][1], a2.bias2 + ct1 + 16 * h, kh != 0);
-    }
+    for (int t = 0; t < 2; t++)
+        init_acc(acc2[t], a2.bias2 + ct0 + 16 * h, false);
     __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): this thread's part of the grid is written
     __builtin_amdgcn_s_barrier();
     STAMP(1);
-    reduce_half<9 * G, 2, D2>(acc2, r2, kh, 0, ldw2, ldb2);
+    reduce_all<9 * G, 2, D2>(acc2, r2, 0, ldw2, ldb2);
     STAMP(2);
     // layer 3: this wave's 128 output channels in 4 chunks of 32; the first chunk's weights, biases and residual travel now
     const uint8_t *w3 = a3.wfrag + (size_t)(128 * wave) * 64 + lane * 16;
@@ -363,12 +355,11 @@ __global__ __launch_bounds__(128 * G, (G <= 2 ? 3 : 2)) void conv_bottleneck_tai
             rn[t] = ldg128(a3.res + pix[t] * CW + 128 * wave + 32 * cc + 16 * h);
     };
     load_chunk(0);
-    pair_reduce<2, false>(acc2, lds + S_OFF, wave, partner, lane);
     STAMP(3);
 #pragma unroll
     for (int t = 0; t < 2; t++) {
         const int q = 32 * t + p;
-        const v4i o = requant16(a2, acc2[t][0], a3.xmask);
+        const v4i o = requant16(a2, acc2[t], a3.xmask);
         *reinterpret_cast<v4i *>(lds + M_OFF + q * CM + ((((ct0 >> 4) + h) ^ swz<CM>(q)) << 4)) = o;
     }
     __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
@@ -420,30 +411,26 @@ __global__ __launch_bounds__(128 * G, (G <= 2 ? 3 : 2)) void conv_bottleneck_tai
 
     // ================= the next block's first layer: CW -> CM on the sum tile =================
     {
-        const uint8_t *wn0 = an.wfrag + (size_t)ct0 * 64 + lane * 16, *wn1 = an.wfrag + (size_t)ct1 * 64 + lane * 16;
-        auto ldwn = [&](int s, int kk, int nt) { return ldg128((nt ? wn1 : wn0) + (size_t)s * wslabn + kk * 1024); };
+        const uint8_t *wn0 = an.wfrag + (size_t)ct0 * 64 + lane * 16;
+        auto ldwn = [&](int s, int kk) { return ldg128(wn0 + (size_t)s * wslabn + kk * 1024); };
         auto ldbn = [&](int s, int kk, int t) {
             const int j = 32 * t + p, hs = h ^ (j & 15);
             return *reinterpret_cast<const v4i *>(lds + S_OFF + j * CW + (s >> 2) * 256 + (((4 * (s & 3) + 2 * kk) ^ hs) << 4));
         };
-        WeightRing<DN> rr;
-        ring_fill<4 * G, DN>(rr, kh, ldwn);
-        v16i accn[2][2];
+        WeightRing1<DN> rr;
+        ring_fill1<4 * G, DN>(rr, ldwn);
+        v16i accn[2];
 #pragma unroll
-        for (int t = 0; t < 2; t++) {
-            init_acc(accn[t][0], an.bias2 + ct0 + 16 * h, kh != 0);
-            init_acc(accn[t][1], an.bias2 + ct1 + 16 * h, kh != 0);
-        }
+        for (int t = 0; t < 2; t++)
+            init_acc(accn[t], an.bias2 + ct0 + 16 * h, false);
         __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): this wave's part of the sum tile is written
         __builtin_amdgcn_s_barrier();
         STAMP(9);
-        reduce_half<4 * G, 2, DN>(accn, rr, kh, (int)an.xmask, ldwn, ldbn);
+        reduce_all<4 * G, 2, DN>(accn, rr, (int)an.xmask, ldwn, ldbn);
         STAMP(10);
-        pair_reduce<2, false>(accn, lds + G_OFF, wave, partner, lane); // the grid and layer 2's tile are long read
-        STAMP(11);
 #pragma unroll
         for (int t = 0; t < 2; t++) {
-            const v4i o = requant16(an, accn[t][0], 0);
+            const v4i o = requant16(an, accn[t], 0);
             if (valid[t])
                 *reinterpret_cast<v4i *>(an.y + pix[t] * CM + ct0 + 16 * h) = o;
         }

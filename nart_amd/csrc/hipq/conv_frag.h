@@ -158,6 +158,55 @@ __device__ static inline void reduce_half(v16i (&acc)[MT][2], WeightRing<D> &r, 
     }
 }
 
+// The same without sharing the reduction: a wave owns ONE 32-channel tile and all STOT slabs, so nothing is exchanged.
+// Every wave then reads every pixel operand (twice the LDS traffic of the split), which the kernels that are bound by
+// the weight stream or by vector arithmetic can afford.  ldw(s, kk): the weight operand of slab s, k-step kk; ldb as above.
+template <int D>
+struct WeightRing1 {
+    v4i w[D][2];
+};
+
+template <int STOT, int D, class FW>
+__device__ static inline void ring_fill1(WeightRing1<D> &r, FW ldw)
+{
+#pragma unroll
+    for (int i = 0; i < D && i < STOT; i++)
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++)
+            r.w[i][kk] = ldw(i, kk);
+}
+
+template <int STOT, int MT, int D, class FW, class FB>
+__device__ static inline void reduce_all(v16i (&acc)[MT], WeightRing1<D> &r, const int flip, FW ldw, FB ldb)
+{
+    v4i br[2][MT][2];
+    auto loadb = [&](int i, v4i(&b)[MT][2]) {
+#pragma unroll
+        for (int t = 0; t < MT; t++)
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++)
+                b[t][kk] = ldb(i, kk, t);
+    };
+    loadb(0, br[0]);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int i = 0; i < STOT; i++) {
+        if (i + 1 < STOT)
+            loadb(i + 1, br[(i + 1) & 1]);
+#pragma unroll
+        for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+            for (int t = 0; t < MT; t++)
+                acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(r.w[i % D][kk], br[i & 1][t][kk] ^ flip, acc[t], 0, 0, 0);
+        if (i + D < STOT) {
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++)
+                r.w[i % D][kk] = ldw(i + D, kk);
+        }
+        __builtin_amdgcn_sched_barrier(0); // keep every slab's loads, reads and multiplies where they are written
+    }
+}
+
 // The two waves of a pair add their partial sums: each sends its channel tile 1 and keeps tile 0 (the pair's waves order
 // their channel tiles oppositely, so one wave's tile 1 is the other's tile 0) through 4 KB slots in LDS - all pixel
 // tiles at once where the slots hold them (ONE_ROUND: MT slots per wave), else one pixel tile per round with a barrier

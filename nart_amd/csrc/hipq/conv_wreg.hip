@@ -35,8 +35,9 @@ namespace {
 constexpr int kWregPatch = 7; // 3x3 layers: a work-group's output pixels are a 7 x 7 patch of one image
 
 struct WregGeom {
-    int npg, nnb; // pixel groups, blocks of 128 output channels
+    int npg, nnb; // pixel groups, channel groups (a work-group's share: nbpw blocks of 128 output channels)
     int PY, PX;   // 3x3: patches per image
+    int nbpw;     // blocks of 128 output channels a work-group walks with one load of its pixel operands (1: conv_wreg_kernel)
 };
 
 } // namespace
@@ -153,6 +154,160 @@ __global__ __launch_bounds__(256, 2) void conv_wreg_kernel(const ConvArgs a, con
     }
 }
 
+// The last layer of a bottleneck block with a projection shortcut: y = add(a(x), b(xb)) with both convolutions in the
+// same kernel - a: 1x1 / stride 1 from 64 CPT channels (its add parameters in a.addq / a.res_first, the sum to a.y), b:
+// 1x1 / stride S2 from 64 CPT2 channels to the same output channels, whose requantised bytes are the add's other operand
+// and never travel to memory (a launch, and a write and a read of the widest tensor of the block, disappear).  Both pixel
+// operands go to LDS at the start; b is reduced first and its 16 bytes per lane and pixel tile wait in registers while a is
+// reduced into the same accumulators.
+template <int CPT, int CPT2, int S2>
+__global__ __launch_bounds__(256, (4096 * (CPT + CPT2) + 16384 <= 81920 ? 2 : 1)) void conv_wreg_dual_kernel(const ConvArgs a, const ConvArgs b, const WregGeom geo)
+{
+    constexpr int RB = 64 * CPT, RB2 = 64 * CPT2, X_BYTES = 64 * RB, X2_BYTES = 64 * RB2;
+    constexpr int S_OFF = X_BYTES + X2_BYTES, D = 6;
+    static_assert(CPT >= 4 && CPT2 >= 4, "pixel rows of at least 256 bytes");
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[S_OFF + 4 * 4096];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int p = lane & 31, h = lane >> 5;
+    const int ng = wave & 1, kh = wave >> 1, partner = wave ^ 2;
+    const int gid = (int)(blockIdx.x % 8) * (int)(gridDim.x / 8) + (int)(blockIdx.x / 8); // XCD x: the x-th eighth of the list
+    if (gid >= geo.npg * geo.nnb)
+        return;
+    const int pg = gid / geo.nnb, nb = gid - pg * geo.nnb;
+
+    // ---- both pixel operands -> LDS: 16-byte piece c of row r at piece c ^ (r & 15) of every 256 bytes ----
+#pragma unroll
+    for (int k = 0; k < (X_BYTES + X2_BYTES) / 4096; k++) {
+        const bool second = k >= X_BYTES / 4096;
+        const int id = ((second ? k - X_BYTES / 4096 : k) * 4 + wave) * 64 + lane;
+        const int cpr = second ? RB2 / 16 : RB / 16, row = id / cpr, c = (id % cpr) ^ (row & 15);
+        const int m = min(pg * 64 + row, a.P - 1); // rows beyond the tensor repeat its last pixel: never stored
+        const uint8_t *src;
+        if (!second) {
+            src = a.x + (size_t)m * RB + c * 16;
+        } else if (S2 == 1) {
+            src = b.x + (size_t)m * RB2 + c * 16;
+        } else {
+            const int ohw = a.OH * a.OW, ni = fast_div(m, ohw, a.inv_ohw), rem = m - ni * ohw;
+            const int oy = fast_div(rem, a.OW, a.inv_ow), ox = rem - oy * a.OW;
+            src = b.x + (size_t)((ni * b.H + oy * S2) * b.W + ox * S2) * RB2 + c * 16;
+        }
+        __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(lds + (k * 4 + wave) * 1024), 16, 0, 0);
+    }
+
+    // The work-group walks geo.nbpw blocks of 128 output channels with the pixel operands it has loaded once.  Per block
+    // the wave's two channel tiles: tile 0 (kept after the pair's exchange) and tile 1 (sent).
+    const size_t wslab = (size_t)a.kout_pad * 64, wslab2 = (size_t)b.kout_pad * 64;
+    int ct0 = 128 * nb * geo.nbpw + 64 * ng + 32 * kh, ct1 = 128 * nb * geo.nbpw + 64 * ng + 32 * (1 - kh);
+    const uint8_t *w0, *w1, *v0, *v1;
+    auto ldw = [&](int s, int kk, int nt) { return ldg128((nt ? w1 : w0) + (size_t)s * wslab + kk * 1024); };
+    auto ldw2 = [&](int s, int kk, int nt) { return ldg128((nt ? v1 : v0) + (size_t)s * wslab2 + kk * 1024); };
+    auto ldb = [&](int s, int kk, int t) {
+        const int j = 32 * t + p, hs = h ^ (j & 15);
+        return *reinterpret_cast<const v4i *>(lds + j * RB + (s >> 2) * 256 + (((4 * (s & 3) + 2 * kk) ^ hs) << 4));
+    };
+    auto ldb2 = [&](int s, int kk, int t) {
+        const int j = 32 * t + p, hs = h ^ (j & 15);
+        return *reinterpret_cast<const v4i *>(lds + X_BYTES + j * RB2 + (s >> 2) * 256 + (((4 * (s & 3) + 2 * kk) ^ hs) << 4));
+    };
+    size_t pix[2];
+    bool valid[2];
+#pragma unroll
+    for (int t = 0; t < 2; t++) {
+        valid[t] = pg * 64 + 32 * t + p < a.P;
+        pix[t] = (size_t)min(pg * 64 + 32 * t + p, a.P - 1);
+    }
+    WeightRing<D> ring, ringa;
+    v0 = b.wfrag + (size_t)ct0 * 64 + lane * 16, v1 = b.wfrag + (size_t)ct1 * 64 + lane * 16;
+    ring_fill<CPT2, D>(ring, kh, ldw2);
+    wait_vmcnt<0>(); // every wave's share of both pixel operands has landed before anyone reads them
+    __builtin_amdgcn_s_barrier();
+    for (int bi = 0; bi < geo.nbpw; bi++) {
+        // ---- the shortcut b: its bytes for this wave's 32 channels of the 64 pixels stay in registers ----
+        v16i acc[2][2];
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            init_acc(acc[t][0], b.bias2 + ct0 + 16 * h, kh != 0);
+            init_acc(acc[t][1], b.bias2 + ct1 + 16 * h, kh != 0);
+        }
+        reduce_half<CPT2, 2, D>(acc, ring, kh, (int)b.xmask, ldw2, ldb2);
+        w0 = a.wfrag + (size_t)ct0 * 64 + lane * 16, w1 = a.wfrag + (size_t)ct1 * 64 + lane * 16;
+        ring_fill<CPT, D>(ringa, kh, ldw); // a's first weights travel while b's halves meet
+        if (bi > 0) {
+            __builtin_amdgcn_s_waitcnt(0xC07F);
+            __builtin_amdgcn_s_barrier(); // every wave has read the exchange slots of the previous block
+        }
+        pair_reduce<2, false>(acc, lds + S_OFF, wave, partner, lane);
+        v4i res[2];
+#pragma unroll
+        for (int t = 0; t < 2; t++)
+            res[t] = requant16(b, acc[t][0], 0);
+        // ---- a, then the add ----
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            init_acc(acc[t][0], a.bias2 + ct0 + 16 * h, kh != 0);
+            init_acc(acc[t][1], a.bias2 + ct1 + 16 * h, kh != 0);
+        }
+        reduce_half<CPT, 2, D>(acc, ringa, kh, (int)a.xmask, ldw, ldb);
+        const int st0 = ct0; // this block's channels; the next block's shortcut weights travel during the exchange and the add
+        ct0 += 128, ct1 += 128;
+        if (bi + 1 < geo.nbpw) {
+            v0 = b.wfrag + (size_t)ct0 * 64 + lane * 16, v1 = b.wfrag + (size_t)ct1 * 64 + lane * 16;
+            ring_fill<CPT2, D>(ring, kh, ldw2);
+        }
+        __builtin_amdgcn_s_waitcnt(0xC07F);
+        __builtin_amdgcn_s_barrier(); // every wave has read the exchange slots of b
+        pair_reduce<2, false>(acc, lds + S_OFF, wave, partner, lane);
+#pragma unroll
+        for (int t = 0; t < 2; t++) {
+            const v4i o = requant_add16(a, acc[t][0], res[t]);
+            if (valid[t])
+                *reinterpret_cast<v4i *>(a.y + pix[t] * a.out_cs + st0 + 16 * h) = o;
+        }
+    }
+}
+
+// a: the widening 1x1 convolution (stride 1, add parameters set, a.res any non-null pointer), b: the shortcut
+bool conv_wreg_dual_applies(const ConvArgs &a, const ConvArgs &b)
+{
+    auto plain1x1 = [](const ConvArgs &c) {
+        return c.group == 1 && c.bwz == 0 && c.xmask != 0 && c.fastq && c.qmult == nullptr && c.acc_out == nullptr && c.deq_out == nullptr
+            && c.wfrag != nullptr && c.C == c.in_cs && c.in_cs % 64 == 0 && c.K == c.out_cs && c.out_cs % 128 == 0 && c.R == 1 && c.S == 1
+            && c.pad_h == 0 && c.pad_w == 0 && c.stride_h == c.stride_w && c.nslab == c.in_cs / 64;
+    };
+    if (!(plain1x1(a) && plain1x1(b) && a.stride_h == 1 && (b.stride_h == 1 || b.stride_h == 2) && a.res != nullptr && a.addq.fast
+          && a.addq.hi == 255 && b.res == nullptr && b.q.hi == 255 && a.out_cs == b.out_cs && a.N == b.N && a.OH == b.OH
+          && a.OW == b.OW && a.P == b.P && (long long)b.N * b.H * b.W * b.in_cs < (1ll << 31)))
+        return false;
+    const int c1 = a.in_cs / 64, c2 = b.in_cs / 64;
+    return (c1 == 4 || c1 == 8) && c2 == 2 * c1;
+}
+
+void launch_conv_wreg_dual(const ConvArgs &a, const ConvArgs &b, hipStream_t st)
+{
+    WregGeom geo;
+    geo.PY = geo.PX = 0, geo.npg = (a.P + 63) / 64;
+    // channel blocks per work-group: as many as still leave about two work-groups per CU (each reuses its pixel operands
+    // in LDS and pays the start of the kernel once), in whole divisors of the block count
+    const int nblk = a.out_cs / 128;
+    geo.nbpw = 1;
+    for (int k = 2; k <= 8; k++)
+        if (nblk % k == 0 && (long long)geo.npg * (nblk / k) >= 384)
+            geo.nbpw = k;
+    geo.nnb = nblk / geo.nbpw;
+    const dim3 grid((unsigned)((geo.npg * geo.nnb + 7) / 8 * 8)), block(256);
+    const int c1 = a.in_cs / 64;
+    if (c1 == 4 && b.stride_h == 1)
+        hipLaunchKernelGGL((conv_wreg_dual_kernel<4, 8, 1>), grid, block, 0, st, a, b, geo);
+    else if (c1 == 4)
+        hipLaunchKernelGGL((conv_wreg_dual_kernel<4, 8, 2>), grid, block, 0, st, a, b, geo);
+    else if (b.stride_h == 1)
+        hipLaunchKernelGGL((conv_wreg_dual_kernel<8, 16, 1>), grid, block, 0, st, a, b, geo);
+    else
+        hipLaunchKernelGGL((conv_wreg_dual_kernel<8, 16, 2>), grid, block, 0, st, a, b, geo);
+}
+
 bool conv_wreg_applies(const ConvArgs &a)
 {
     if (!(a.group == 1 && a.bwz == 0 && a.xmask != 0 && a.fastq && a.qmult == nullptr && a.acc_out == nullptr && a.deq_out == nullptr
@@ -171,7 +326,7 @@ template <int CPT, int TAPS, int S>
 static void launch_wreg(const ConvArgs &a, hipStream_t st)
 {
     WregGeom geo;
-    geo.nnb = a.out_cs / 128;
+    geo.nnb = a.out_cs / 128, geo.nbpw = 1;
     geo.PY = a.OH / kWregPatch, geo.PX = a.OW / kWregPatch;
     geo.npg = TAPS == 9 ? a.N * geo.PY * geo.PX : (a.P + 63) / 64;
     const dim3 grid((unsigned)((geo.npg * geo.nnb + 7) / 8 * 8)), block(256);

@@ -57,6 +57,9 @@ _SIGS = {
     "hipq_conv2d_add_conv_fusable": (C.c_int, [C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_float, C.c_int, C.c_int, C.c_void_p]),
     "hipq_conv2d_run_add_conv": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_float, C.c_int,
                                            C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
+    "hipq_conv2d_add2_fusable": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_int]),
+    "hipq_conv2d_run_add2": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_int,
+                                       C.c_void_p, C.c_void_p]),
     "hipq_bottleneck_fusable": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_int]),
     "hipq_bottleneck_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_int,
                                       C.c_void_p, C.c_void_p]),
@@ -280,6 +283,18 @@ class Conv2d:
             self.close()
         except Exception:
             pass
+
+
+def add2_fusable(plan, shortcut, shortcut_first, oalpha, ozp, obits=8):
+    """Can add(plan(x), shortcut(x_shortcut)) run as one kernel (include/hipq.h: hipq_conv2d_add2_fusable)?"""
+    return bool(lib().hipq_conv2d_add2_fusable(plan.handle, shortcut.handle, int(bool(shortcut_first)), oalpha, ozp, obits))
+
+
+def run_add2(plan, x, shortcut, x_shortcut, shortcut_first, oalpha, ozp, y, obits=8):
+    """y = add(plan(x), shortcut(x_shortcut)) in one launch (include/hipq.h: hipq_conv2d_run_add2)."""
+    check(lib().hipq_conv2d_run_add2(plan.handle, _ptr(x), shortcut.handle, _ptr(x_shortcut), int(bool(shortcut_first)), oalpha, ozp,
+                                     obits, _ptr(y), _stream()))
+    return y
 
 
 def bottleneck_fusable(reduce, mid, widen, residual_first, oalpha, ozp, obits=8):

@@ -39,6 +39,7 @@ class HipqExecutor:
         self.blocks = {}     # id(add node) -> (reduce, mid, widen conv nodes) of an identity bottleneck block run as one kernel
         self.in_block = {}   # id(conv node) -> the add node of its block
         self.tails = {}      # id(add node) -> (mid, widen, next or None): the block from its 3x3 layer on as one kernel
+        self.duals = {}      # id(add node) -> (widen, shortcut): both 1x1 convolutions and the add as one kernel
         self.dequantized = {}  # fully-connected output name -> the dequantize node computed in the layer's epilogue
         self.chained = {}    # add output name -> the 1x1 convolution node computed inside the fused add's kernel
         self._early = {}     # id(conv node) -> its plan, created ahead of its turn (when an add looked at it)
@@ -97,6 +98,17 @@ class HipqExecutor:
                 nb = 2 * int(np.prod(y.shape)) + sum(case.weights[c.attrs["w"]].size + 4 * c.attrs["K"] for c in (c1, c2, c3))
                 self.steps.append({"label": node.output, "kind": "block", "kernel": "conv_mfma_i8_bottleneck", "fn": fn,
                                    "ops": sum(p.ops for p in plans), "bytes": nb, "plan": plans[0]})
+            elif node.kind == "add" and id(node) in self.duals:
+                cm, cs = self.duals[id(node)]
+                pm, ps = self._early.pop(id(cm)), self._early.pop(id(cs))
+                self.plans += [pm, ps]
+                sc_first = node.inputs[0] == cs.output
+                fn = (lambda pm=pm, ps=ps, i=self.buf[cm.inputs[0]], j=self.buf[cs.inputs[0]], sf=sc_first, y=y, o=out:
+                      hipq.run_add2(pm, i, ps, j, sf, y.alpha, y.zp, o))
+                nb = (int(np.prod(T[cm.inputs[0]].shape)) + int(np.prod(T[cs.inputs[0]].shape)) + int(np.prod(y.shape))
+                      + sum(case.weights[c.attrs["w"]].size + 4 * c.attrs["K"] for c in (cm, cs)))
+                self.steps.append({"label": node.output, "kind": "conv+conv+add", "kernel": "conv_mfma_i8_wreg_dual+add", "fn": fn,
+                                   "ops": pm.ops + ps.ops, "bytes": nb, "plan": pm})
             elif node.kind == "add" and id(node) in self.tails:
                 c2, c3, nxt = self.tails[id(node)]
                 convs = [c for c in (c2, c3, nxt) if c is not None]
@@ -267,6 +279,24 @@ class HipqExecutor:
                     self._early.setdefault(id(c), p)  # keep the plans for the operators' own turns
             if id(add) in self.blocks:
                 continue
+            # a block with a projection shortcut: both inputs of the add are 1x1 convolutions read by nobody else
+            pair = [prod.get(i) for i in add.inputs]
+            if all(n is not None and n.kind == "conv" and n.attrs["k"] == 1 and n.attrs["group"] == 1 and not n.attrs["relu"]
+                   and n.attrs["pad"] == 0 and len(uses.get(n.output, [])) == 1 and n.output != case.output.name
+                   and id(n) not in self.in_block for n in pair):
+                plans = [conv_plan(n)[0] for n in pair]
+                st = T[add.output]
+                for mi in (0, 1):
+                    if hipq.add2_fusable(plans[mi], plans[1 - mi], mi == 1, st.alpha, st.zp):
+                        self.duals[id(add)] = (pair[mi], pair[1 - mi])
+                        break
+                for n, pl in zip(pair, plans):
+                    self._early[id(n)] = pl
+                    if id(add) in self.duals:
+                        self.in_block[id(n)] = add
+                        self.fused.pop(n.output, None)
+                if id(add) in self.duals:
+                    continue
             # the block from its 3x3 layer on, with any residual, and the 1x1 layer that reads the sum
             for ci in (0, 1):
                 c3 = only_conv(add.inputs[ci], 1)
@@ -314,7 +344,7 @@ class HipqExecutor:
     @property
     def elided(self):
         """Names of the tensors that are never materialised (absorbed into a fused kernel)."""
-        return set(self.fused) | set(self.pooled) | set(self.dequantized) | {c.output for cs in self.blocks.values() for c in cs} | {c.output for cs in self.tails.values() for c in cs[:2]}
+        return set(self.fused) | set(self.pooled) | set(self.dequantized) | {c.output for cs in self.blocks.values() for c in cs} | {c.output for cs in self.tails.values() for c in cs[:2]} | {c.output for cs in self.duals.values() for c in cs}
 
     def set_input(self, x):
         inp = self.case.input

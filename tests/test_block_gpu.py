@@ -274,6 +274,54 @@ def test_register_fed_convolution(case):
                 assert np.array_equal(gota, wanta), (case, "add", res_first, int((gota != wanta).sum()))
 
 
+ADD2_CASES = [  # N, C (widening layer's input channels), output H, W, K, the shortcut's stride
+    (2, 256, 14, 14, 1024, 2), (3, 512, 7, 7, 2048, 2), (1, 256, 9, 13, 384, 1), (2, 512, 14, 7, 1024, 1),
+]
+
+
+@pytest.mark.parametrize("case", ADD2_CASES, ids=lambda c: "x".join(map(str, c)))
+def test_widening_convolution_shortcut_and_add(case):
+    """hipq_conv2d_run_add2: the widening 1x1 convolution of a block, its projection shortcut (1x1, stride 1 or 2, from the
+    block's input) and the add, against the oracle's three operators; both operand orders."""
+    N, C, H, W, K, st = case
+    rng = np.random.default_rng(4000 + C + K + st)
+    x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+    xs = rng.integers(0, 256, (N, 2 * C, H * st - (st - 1), W * st - (st - 1)), dtype=np.uint8)
+
+    def layer(Cin):
+        w = rng.integers(1, 256, (K, Cin, 1, 1), dtype=np.uint8)
+        sigma = 74.0 * 74.0 * math.sqrt(Cin)
+        b = rng.integers(-int(sigma), int(sigma) + 1, K).astype(np.int32)
+        ia, iz = float(np.float32(rng.uniform(0.02, 0.06))), int(rng.integers(0, 256))
+        oa = float(np.float32(ia * rng.uniform(0.75, 1.35)))
+        return w, b, (ia, iz, float(np.float32(oa * 40.0 / (ia * sigma))), 128, oa, int(rng.integers(96, 160)))
+    w, b, q = layer(C)
+    ws_, bs, qs = layer(2 * C)
+    pm = hipq.Conv2d(x.shape, w, b, 0, 1, 1, *q).special(2)
+    ps = hipq.Conv2d(xs.shape, ws_, bs, 0, st, 1, *qs)
+    want_m = orc.conv2d_u8(x, w, b, 0, 1, 1, *q)
+    want_s = orc.conv2d_u8(xs, ws_, bs, 0, st, 1, *qs)
+    assert want_m.shape == want_s.shape
+    xd, xsd = hipq.to_device_nhwc(x), hipq.to_device_nhwc(xs)
+    for sc_first in (False, True):
+        sa, sz = float(np.float32(math.hypot(q[4], qs[4]) * 1.1)), int(rng.integers(0, 40))
+        print("add2 case", case, sc_first, pm.kernel, ps.kernel, flush=True)
+        assert hipq.add2_fusable(pm, ps, sc_first, sa, sz)
+        want = orc.add_u8(want_s, want_m, qs[4], qs[5], q[4], q[5], sa, sz) if sc_first else orc.add_u8(want_m, want_s, q[4], q[5], qs[4], qs[5], sa, sz)
+        y = pm.empty_output()
+        hipq.run_add2(pm, xd, ps, xsd, sc_first, sa, sz, y)
+        torch.cuda.synchronize()
+        got = hipq.from_device_nhwc(y, K)
+        bad = got != want
+        assert not bad.any(), (case, sc_first, int(bad.sum()), np.argwhere(bad)[:8].tolist())
+    # a shortcut with other output channels is refused
+    w3 = rng.integers(1, 256, (K + 128, 2 * C, 1, 1), dtype=np.uint8)
+    p3 = hipq.Conv2d(xs.shape, w3, None, 0, st, 1, *qs)
+    assert not hipq.add2_fusable(pm, p3, False, 0.1, 0)
+    with pytest.raises(hipq.HipqError, match="do not run as one kernel"):
+        hipq.run_add2(pm, xd, p3, xsd, False, 0.1, 0, pm.empty_output())
+
+
 def time_layers():
     """Every convolution of the 28x28-and-smaller stages of ResNet-50 at batch 64: the built-in kernel against special(3)."""
     rng = np.random.default_rng(9)
