@@ -2374,7 +2374,7 @@ extern "C" int hipq_bottleneck_fusable(const hipq_conv2d_plan *p1, const hipq_co
         return 0;
     // built-in rule: where it measured faster than the three launches it replaces - blocks of 256 middle channels (14x14
     // images at batch 64: 31 against 41 us and two launch gaps); hipq_conv2d_plan_special(reduce, 2): wherever it applies
-    return p1->special == 2 || a1.out_cs == 256 ? 1 : 0;
+    return p1->special == 2 || conv_block_preferred(a1) ? 1 : 0;
 }
 
 extern "C" int hipq_bottleneck_run(const hipq_conv2d_plan *p1, const hipq_conv2d_plan *p2, const hipq_conv2d_plan *p3, const void *x,
@@ -2461,10 +2461,8 @@ extern "C" int hipq_bottleneck_tail_fusable(const hipq_conv2d_plan *p2, const hi
     ConvArgs a2, a3, an;
     if (!tail_args(p2, p3, residual_is_input0, res_alpha, res_zp, oalpha, ozp, obits, next, &a2, &a3, &an))
         return 0;
-    // built-in rule: where it measured faster than the launches it replaces - blocks of 128 middle channels (28x28 images at
-    // batch 64: 38.6 us against 14.0 + 28.6 and a launch gap; level at 64 channels on 56x56: 53.1 against 13.8 + 39.1; 256
-    // channels belong to hipq_bottleneck_run); hipq_conv2d_plan_special(mid, 2): wherever it applies
-    return p2->special == 2 || a2.in_cs == 128 ? 1 : 0;
+    // hipq_conv2d_plan_special(mid, 2): wherever it applies; else the built-in rule
+    return p2->special == 2 || conv_block_tail_preferred(a2, next != nullptr) ? 1 : 0;
 }
 
 extern "C" int hipq_bottleneck_tail_run(const hipq_conv2d_plan *p2, const hipq_conv2d_plan *p3, const void *x, const void *residual,

@@ -10,10 +10,13 @@ namespace hipq {
 // to a3.y.  true when conv_bottleneck_kernel computes this chain.
 bool conv_block_applies(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3);
 void launch_conv_block(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3, hipStream_t st);
+// true where the one kernel measured faster than the launches it replaces
+bool conv_block_preferred(const ConvArgs &a1);
 
 // The chain cut one layer later: a2 (3x3 / stride 1 / pad 1, reads a2.x), a3 (the widening 1x1 with the residual a3.res and
 // the add's parameters, sum to a3.y) and - an != nullptr - the 1x1 convolution that reads the sum (output to an->y).
 bool conv_block_tail_applies(const ConvArgs &a2, const ConvArgs &a3, const ConvArgs *an);
 void launch_conv_block_tail(const ConvArgs &a2, const ConvArgs &a3, const ConvArgs *an, hipStream_t st);
+bool conv_block_tail_preferred(const ConvArgs &a2, bool chained);
 
 } // namespace hipq

@@ -269,17 +269,18 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
 //   * layer 3 + add as above, the sum stored and - CHAIN - kept in LDS, 64 pixel rows of CW bytes;
 //   * CHAIN: the next layer (CW -> CM) reads that tile as its pixel operand, the pairs splitting the reduction again.
 template <int G, int PH, int PW, bool CHAIN>
-__global__ __launch_bounds__(128 * G, (G <= 2 ? 3 : 2)) void conv_bottleneck_tail_kernel(const ConvArgs a2, const ConvArgs a3, const ConvArgs an,
+__global__ __launch_bounds__(128 * G, (G == 1 ? 4 : G == 2 ? 3 : 2)) void conv_bottleneck_tail_kernel(const ConvArgs a2, const ConvArgs a3, const ConvArgs an,
                                                                          const BlockGeom geo)
 {
     constexpr int NW = 2 * G, NT = 128 * G, CM = 64 * G, CW = 256 * G;
     constexpr int GW = PW + 2, GH = PH + 2, NPIX = PH * PW, GROWS = (GH * GW + 7) / 8 * 8;
     constexpr int G_OFF = 0, G_BYTES = GROWS * CM;            // layer 2's input on the bordered grid
     constexpr int M_OFF = G_OFF + G_BYTES, M_BYTES = 64 * CM; // layer 2's bytes, row = pixel
-    constexpr int S_OFF = M_OFF + M_BYTES, S_BYTES = CHAIN ? 64 * CW : 0; // the sum tile
-    constexpr int D2 = G <= 2 ? 6 : 10, DN = D2; // slabs of weights a wave holds ahead (three waves per SIMD: fewer registers)
+    // the sum tile takes the place of the grid and of layer 2's bytes once every wave holds its operands of layer 3
+    constexpr int S_OFF = 0, S_BYTES = CHAIN ? 64 * CW : 0;
+    constexpr int D2 = G == 1 ? 4 : G == 2 ? 6 : 10, DN = D2; // slabs of weights a wave holds ahead (four or three waves per SIMD: fewer registers)
     static_assert(NPIX <= 64, "pixel slots");
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[S_OFF + S_BYTES];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[M_OFF + M_BYTES > S_BYTES ? M_OFF + M_BYTES : S_BYTES];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int p = lane & 31, h = lane >> 5;
@@ -375,6 +376,10 @@ __global__ __launch_bounds__(128 * G, (G <= 2 ? 3 : 2)) void conv_bottleneck_tai
 #pragma unroll
             for (int ks = 0; ks < 2 * G; ks++)
                 bf[t][ks] = *reinterpret_cast<const v4i *>(lds + M_OFF + q * CM + (((2 * ks + h) ^ swz<CM>(q)) << 4));
+        }
+        if (CHAIN) { // the sum tile lies over what the waves have just read
+            __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
+            __builtin_amdgcn_s_barrier();
         }
         for (int cc = 0; cc < 4; cc++) {
             const int ch = 128 * wave + 32 * cc;
@@ -513,6 +518,15 @@ void launch_conv_block_tail(const ConvArgs &a2, const ConvArgs &a3, const ConvAr
     default: launch_tail_g<4>(a2, a3, an, st); break; // conv_block_tail_applies: 64, 128 or 256 middle channels
     }
 }
+
+// Measured at batch 64: blocks of 256 middle channels (14x14 images) 25.6 us against 8.0 + 13.2 + 14.5 and two launch
+// gaps; 128 channels (28x28) 40.6 against 49.0, where the tail form below does better still; 64 channels lose.
+bool conv_block_preferred(const ConvArgs &a1) { return a1.out_cs == 256; }
+
+// Measured at batch 64: 128 middle channels (28x28 images) 32 us with the next layer, 27 without, against 14.0 + 28.6
+// and a launch gap; 64 channels (56x56) 43 to 48 with the next layer against 13.8 + 37.3 and the gap, but 58 without
+// (the sum's pixel tile is what that form saves); 256 channels belong to the whole-block kernel.
+bool conv_block_tail_preferred(const ConvArgs &a2, bool chained) { return a2.in_cs == 128 || (a2.in_cs == 64 && chained); }
 
 bool conv_block_applies(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3)
 {
