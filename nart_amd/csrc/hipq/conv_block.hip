@@ -267,12 +267,13 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
 //     (out-of-image positions hold the pad byte);
 //   * layer 2 (3x3) as above, on the compact pixel index q = PW * row + column, its bytes to LDS;
 //   * layer 3 + add as above, the sum stored and - CHAIN - kept in LDS, 64 pixel rows of CW bytes;
-//   * CHAIN: the next layer (CW -> CM) reads that tile as its pixel operand, the pairs splitting the reduction again.
-template <int G, int PH, int PW, bool CHAIN>
+//   * CHAIN: the next layer (CW -> CM, or CW -> 2 CM where the next stage begins) reads that tile as its pixel operand.
+template <int G, int PH, int PW, int NX>
 __global__ __launch_bounds__(128 * G, (G == 1 ? 4 : G == 2 ? 3 : 2)) void conv_bottleneck_tail_kernel(const ConvArgs a2, const ConvArgs a3, const ConvArgs an,
                                                                          const BlockGeom geo)
 {
     constexpr int NW = 2 * G, NT = 128 * G, CM = 64 * G, CW = 256 * G;
+    constexpr bool CHAIN = NX != 0; // the next layer has NX * CM output channels
     constexpr int GW = PW + 2, GH = PH + 2, NPIX = PH * PW, GROWS = (GH * GW + 7) / 8 * 8;
     constexpr int G_OFF = 0, G_BYTES = GROWS * CM;            // layer 2's input on the bordered grid
     constexpr int M_OFF = G_OFF + G_BYTES, M_BYTES = 64 * CM; // layer 2's bytes, row = pixel
@@ -414,9 +415,12 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? 4 : G == 2 ? 3 : 2)) void conv_b
     if (!CHAIN)
         return;
 
-    // ================= the next block's first layer: CW -> CM on the sum tile =================
-    {
-        const uint8_t *wn0 = an.wfrag + (size_t)ct0 * 64 + lane * 16;
+    // ================= the next block's first layer: CW -> NX * CM on the sum tile =================
+    // a wave owns the 32-channel tiles wave, wave + NW, ... one after the other (the sum tile is read once per tile)
+#pragma unroll
+    for (int jx = 0; jx < (NX ? NX : 1); jx++) {
+        const int cn = 32 * (wave + NW * jx);
+        const uint8_t *wn0 = an.wfrag + (size_t)cn * 64 + lane * 16;
         auto ldwn = [&](int s, int kk) { return ldg128(wn0 + (size_t)s * wslabn + kk * 1024); };
         auto ldbn = [&](int s, int kk, int t) {
             const int j = 32 * t + p, hs = h ^ (j & 15);
@@ -427,9 +431,11 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? 4 : G == 2 ? 3 : 2)) void conv_b
         v16i accn[2];
 #pragma unroll
         for (int t = 0; t < 2; t++)
-            init_acc(accn[t], an.bias2 + ct0 + 16 * h, false);
-        __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): this wave's part of the sum tile is written
-        __builtin_amdgcn_s_barrier();
+            init_acc(accn[t], an.bias2 + cn + 16 * h, false);
+        if (jx == 0) {
+            __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): this wave's part of the sum tile is written
+            __builtin_amdgcn_s_barrier();
+        }
         STAMP(9);
         reduce_all<4 * G, 2, DN>(accn, rr, (int)an.xmask, ldwn, ldbn);
         STAMP(10);
@@ -437,7 +443,7 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? 4 : G == 2 ? 3 : 2)) void conv_b
         for (int t = 0; t < 2; t++) {
             const v4i o = requant16(an, accn[t], 0);
             if (valid[t])
-                *reinterpret_cast<v4i *>(an.y + pix[t] * CM + ct0 + 16 * h) = o;
+                *reinterpret_cast<v4i *>(an.y + pix[t] * (NX * CM) + cn + 16 * h) = o;
         }
         STAMP(12);
     }
@@ -477,8 +483,8 @@ bool conv_block_tail_applies(const ConvArgs &a2, const ConvArgs &a3, const ConvA
         return false;
     if (an == nullptr)
         return true;
-    return plain(*an) && one(*an) && an->C == cw && an->in_cs == cw && an->K == cm && an->out_cs == cm && an->nslab == cw / 64
-        && an->kout_pad >= cm && an->res == nullptr && same_image(*an);
+    return plain(*an) && one(*an) && an->C == cw && an->in_cs == cw && (an->K == cm || an->K == 2 * cm) && an->out_cs == an->K
+        && an->nslab == cw / 64 && an->kout_pad >= an->K && an->res == nullptr && same_image(*an);
 }
 
 template <int G, int PH, int PW>
@@ -491,10 +497,12 @@ static void launch_tail_gp(const ConvArgs &a2, const ConvArgs &a3, const ConvArg
     geo.stamps = getenv("HIPQ_BLOCK_STAMPS") ? (unsigned long long *)strtoull(getenv("HIPQ_BLOCK_STAMPS"), nullptr, 0) : nullptr;
 #endif
     const dim3 grid((unsigned)((geo.npatch + 7) / 8 * 8)), block(128 * G);
-    if (an)
-        hipLaunchKernelGGL((conv_bottleneck_tail_kernel<G, PH, PW, true>), grid, block, 0, st, a2, a3, *an, geo);
+    if (an && an->K == 2 * a2.in_cs)
+        hipLaunchKernelGGL((conv_bottleneck_tail_kernel<G, PH, PW, 2>), grid, block, 0, st, a2, a3, *an, geo);
+    else if (an)
+        hipLaunchKernelGGL((conv_bottleneck_tail_kernel<G, PH, PW, 1>), grid, block, 0, st, a2, a3, *an, geo);
     else
-        hipLaunchKernelGGL((conv_bottleneck_tail_kernel<G, PH, PW, false>), grid, block, 0, st, a2, a3, a3, geo);
+        hipLaunchKernelGGL((conv_bottleneck_tail_kernel<G, PH, PW, 0>), grid, block, 0, st, a2, a3, a3, geo);
 }
 
 template <int G>

@@ -93,9 +93,11 @@ TAIL_CASES = [  # N, CW, H, W: patches of 8 x 8, 4 x 14 and 7 x 7 pixels; 64, 12
 ]
 
 
-def make_tail(rng, N, CW, H, W, relu_next):
-    """The block from its 3x3 layer on: t1 [N, CM, H, W] -> 3x3 -> 1x1 to CW -> add(., residual) -> 1x1 back to CM."""
+def make_tail(rng, N, CW, H, W, relu_next, wide_next=False):
+    """The block from its 3x3 layer on: t1 [N, CM, H, W] -> 3x3 -> 1x1 to CW -> add(., residual) -> 1x1 back to CM (to
+    2 CM with wide_next: the first layer of the next stage)."""
     CM = CW // 4
+    CN = 2 * CM if wide_next else CM
     t1 = rng.integers(0, 256, (N, CM, H, W), dtype=np.uint8)
     res = rng.integers(0, 256, (N, CW, H, W), dtype=np.uint8)
     ia, iz = 0.04, int(rng.integers(0, 256))
@@ -111,9 +113,9 @@ def make_tail(rng, N, CW, H, W, relu_next):
         ia, iz = oa, oz
     ra, rz = float(np.float32(ia * rng.uniform(0.6, 1.6))), int(rng.integers(0, 256))
     sa, sz = float(np.float32(math.hypot(ia, ra) * 1.1)), int(rng.integers(0, 40))
-    w = rng.integers(1, 256, (CM, CW, 1, 1), dtype=np.uint8)
+    w = rng.integers(1, 256, (CN, CW, 1, 1), dtype=np.uint8)
     sigma = 74.0 * 74.0 * math.sqrt(CW)
-    b = rng.integers(-int(sigma), int(sigma) + 1, CM).astype(np.int32)
+    b = rng.integers(-int(sigma), int(sigma) + 1, CN).astype(np.int32)
     oa = float(np.float32(sa * rng.uniform(0.75, 1.35)))
     nxt = dict(w=w, b=b, pad=0, q=(sa, sz, float(np.float32(oa * 40.0 / (sa * sigma))), 128, oa, int(rng.integers(20, 60))), relu=relu_next)
     return t1, res, layers, (ra, rz), (sa, sz), nxt
@@ -123,12 +125,13 @@ def make_tail(rng, N, CW, H, W, relu_next):
 def test_bottleneck_tail(case):
     """hipq_bottleneck_tail_run == 3x3 convolution, widening convolution, add with any residual and - chained - the next
     1x1 convolution run one by one by the oracle: both operand orders of the add, with and without the chained layer, a
-    ReLU on the chained layer, every patch shape and channel count."""
+    ReLU on the chained layer, a chained layer of twice the channels, every patch shape and channel count."""
     N, CW, H, W = case
     CM = CW // 4
     rng = np.random.default_rng(2000 + CW + H)
-    for res_first, chain, relu_next in ((False, True, False), (True, True, True), (True, False, False)):
-        t1, res, layers, rq, sq, nx = make_tail(rng, N, CW, H, W, relu_next)
+    for res_first, chain, relu_next, wide in ((False, True, False, False), (True, True, True, False), (True, False, False, False),
+                                              (False, True, True, True)):
+        t1, res, layers, rq, sq, nx = make_tail(rng, N, CW, H, W, relu_next, wide)
         plans = plans_of(t1, layers)
         pn = hipq.Conv2d((N, CW, H, W), nx["w"], nx["b"], 0, 1, 1, *nx["q"])
         print("tail case", case, res_first, chain, relu_next, [p.kernel for p in plans], flush=True)
@@ -139,7 +142,7 @@ def test_bottleneck_tail(case):
         want = orc.add_u8(res, c, rq[0], rq[1], q3[4], q3[5], sq[0], sq[1]) if res_first else orc.add_u8(c, res, q3[4], q3[5], rq[0], rq[1], sq[0], sq[1])
         xd, rd = hipq.to_device_nhwc(t1), hipq.to_device_nhwc(res)
         y = torch.zeros_like(rd)
-        yn = torch.zeros_like(xd) if chain else None
+        yn = torch.zeros((N, H, W, nx["w"].shape[0]), dtype=torch.uint8, device="cuda") if chain else None
         hipq.bottleneck_tail_run(plans[0], plans[1], xd, rd, res_first, rq[0], rq[1], sq[0], sq[1], y, pn if chain else None, yn,
                                  next_relu=relu_next)
         torch.cuda.synchronize()
@@ -150,7 +153,7 @@ def test_bottleneck_tail(case):
             wantn = orc.conv2d_u8(want, nx["w"], nx["b"], 0, 1, 1, *nx["q"])
             if relu_next:
                 wantn = np.maximum(wantn, nx["q"][5]).astype(np.uint8)
-            gotn = hipq.from_device_nhwc(yn, CM)
+            gotn = hipq.from_device_nhwc(yn, nx["w"].shape[0])
             bad = gotn != wantn
             assert not bad.any(), (case, "next layer", relu_next, int(bad.sum()), np.argwhere(bad)[:8].tolist())
 
