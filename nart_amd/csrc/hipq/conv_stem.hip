@@ -20,10 +20,15 @@
 //     the int32 accumulators in registers (the same lane owns the same pixel column in every row, and a maximum
 //     commutes with the monotonic requantisation): only one row in 2.25 is requantised.  Its bytes go to a row buffer
 //     in LDS, from which the 256 threads take the horizontal 3-maxima and write one pooled row with 128-bit stores.
+//   * NEXT: a 1x1 convolution from the 64 pooled channels to 64 channels (the first layer of the first bottleneck
+//     block) is computed on every pooled row while it is still in LDS - two pixel tiles x two channel tiles, one per
+//     wave, two multiplies each, weights in fragment order (ConvArgs::wfrag) kept in registers - and written beside
+//     the pooled row, which its other readers (the projection shortcut) still need.
 // Requirements (checked by the host): uint8 tensors, input channel stride 4, at most 64 output channels with stride 64,
 // kernel rows of 5 to 8 taps, 5 to 8 kernel rows, stride 2, horizontal pad at most 4, convolution rows of at most 128
 // pixels, image rows of at most 248 pixels (a multiple of 4), weight zero point 128.
 #include "conv_stem.h"
+#include "conv_frag.h"
 
 namespace hipq {
 
@@ -31,14 +36,16 @@ constexpr int kStemMaxPH = 7;                     // pooled rows per work-group,
 constexpr int kStemPitch = 16 + 1024;             // bytes of a patch row: 4 pad pixels, then one 1 KB load
 constexpr int kStemMaxPatchRows = 4 * kStemMaxPH + 8; // stride 2: 2 (2 ph) + R rows, R <= 8
 constexpr int kStemRowBuf = 128 * 64;             // one requantised row: 128 pixels x 64 channels
+constexpr int kStemPoolBuf = 64 * 64;             // NEXT: one pooled row, 64 pixel slots x 64 channels
 
-template <int R, bool FAST>
+template <int R, bool FAST, bool NEXT>
 __global__ __launch_bounds__(256, 2) void conv_stem_maxpool_kernel(const ConvArgs a, uint8_t *yp, const int POH, const int POW,
-                                                                const int nrb, const int ph_per_wg)
+                                                                const int nrb, const int ph_per_wg, const ConvArgs an)
 {
     constexpr int PITCH = kStemPitch;
     constexpr int R_OFF = kStemMaxPatchRows * PITCH;
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[R_OFF + 2 * kStemRowBuf];
+    constexpr int P_OFF = R_OFF + 2 * kStemRowBuf;
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[P_OFF + (NEXT ? kStemPoolBuf : 0)];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = (int)blockIdx.x / nrb, rb = (int)blockIdx.x % nrb;
@@ -81,6 +88,17 @@ __global__ __launch_bounds__(256, 2) void conv_stem_maxpool_kernel(const ConvArg
             for (int e = 0; e < 4; e++)
                 bias[tn][g * 4 + e] = b[e];
         }
+    // NEXT: wave w computes pixel tile w & 1, channel tile w >> 1 of every pooled row; its two weight operands and its
+    // lane's 16 folded biases stay in registers
+    v4i wn[2] = {};
+    v16i bn = {};
+    if (NEXT) {
+        const uint8_t *wp = an.wfrag + (size_t)(wave >> 1) * 2048 + lane * 16;
+        wn[0] = ldg128(wp), wn[1] = ldg128(wp + 1024);
+        frag::init_acc(bn, an.bias2 + 32 * (wave >> 1) + 16 * half, false);
+        if (tid < kStemPoolBuf / 16) // pixel slots beyond the row are multiplied too: give them defined bytes
+            *reinterpret_cast<u32x4 *>(lds + P_OFF + tid * 16) = u32x4{0, 0, 0, 0};
+    }
     __builtin_amdgcn_s_waitcnt(0); // vmcnt(0), lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
 
@@ -162,6 +180,22 @@ __global__ __launch_bounds__(256, 2) void conv_stem_maxpool_kernel(const ConvArg
                     mx[d] = max_u8x4(mx[d], v[d]);
             }
             *reinterpret_cast<u32x4 *>(yp + ((size_t)(n * POH + ph0 + j) * POW + pwi) * 64 + c16 * 16) = mx;
+            if (NEXT) // 16-byte piece c of pooled pixel q at piece c ^ (q & 3)
+                *reinterpret_cast<u32x4 *>(lds + P_OFF + pwi * 64 + ((c16 ^ (pwi & 3)) << 4)) = mx;
+        }
+        if (NEXT) {
+            // every thread passes the next row's barrier only after its reads below: one buffer is enough
+            __syncthreads();
+            const int q = 32 * (wave & 1) + p;
+            v16i accn = bn;
+#pragma unroll
+            for (int kk = 0; kk < 2; kk++) {
+                const v4i b = *reinterpret_cast<const v4i *>(lds + P_OFF + q * 64 + (((2 * kk + half) ^ (q & 3)) << 4)) ^ (int)an.xmask;
+                accn = __builtin_amdgcn_mfma_i32_32x32x32_i8(wn[kk], b, accn, 0, 0, 0);
+            }
+            const v4i o = frag::requant16(an, accn, 0);
+            if (q < POW)
+                *reinterpret_cast<v4i *>(an.y + ((size_t)(n * POH + ph0 + j) * POW + q) * 64 + 32 * (wave >> 1) + 16 * half) = o;
         }
     }
 }
@@ -191,23 +225,34 @@ static int stem_rows_per_wg(int N, int POH)
 }
 
 template <int R>
-static void launch_stem_r(const ConvArgs &a, uint8_t *yp, int POH, int POW, hipStream_t st)
+static void launch_stem_r(const ConvArgs &a, uint8_t *yp, int POH, int POW, const ConvArgs *an, hipStream_t st)
 {
     const int ph = stem_rows_per_wg(a.N, POH), nrb = (POH + ph - 1) / ph;
     const dim3 grid(a.N * nrb), block(256);
-    if (a.fastq)
-        hipLaunchKernelGGL((conv_stem_maxpool_kernel<R, true>), grid, block, 0, st, a, yp, POH, POW, nrb, ph);
+    if (an && a.fastq)
+        hipLaunchKernelGGL((conv_stem_maxpool_kernel<R, true, true>), grid, block, 0, st, a, yp, POH, POW, nrb, ph, *an);
+    else if (a.fastq)
+        hipLaunchKernelGGL((conv_stem_maxpool_kernel<R, true, false>), grid, block, 0, st, a, yp, POH, POW, nrb, ph, a);
     else
-        hipLaunchKernelGGL((conv_stem_maxpool_kernel<R, false>), grid, block, 0, st, a, yp, POH, POW, nrb, ph);
+        hipLaunchKernelGGL((conv_stem_maxpool_kernel<R, false, false>), grid, block, 0, st, a, yp, POH, POW, nrb, ph, a);
 }
 
-void launch_conv_stem_maxpool(const ConvArgs &a, uint8_t *yp, int POH, int POW, hipStream_t st)
+// the 1x1 convolution that the stem's kernel computes on its pooled rows: 64 -> 64 channels, stride 1, on POH x POW pixels
+bool conv_stem_next_applies(const ConvArgs &a, int POH, int POW, const ConvArgs &an)
+{
+    return a.fastq && POW <= 64 && an.R == 1 && an.S == 1 && an.pad_h == 0 && an.pad_w == 0 && an.stride_h == 1 && an.stride_w == 1
+        && an.group == 1 && an.C == 64 && an.in_cs == 64 && an.K == 64 && an.out_cs == 64 && an.nslab == 1 && an.kout_pad >= 64
+        && an.N == a.N && an.H == POH && an.W == POW && an.OH == POH && an.OW == POW && an.bwz == 0 && an.xmask != 0 && an.fastq
+        && an.qmult == nullptr && an.acc_out == nullptr && an.deq_out == nullptr && an.res == nullptr && an.wfrag != nullptr;
+}
+
+void launch_conv_stem_maxpool(const ConvArgs &a, uint8_t *yp, int POH, int POW, const ConvArgs *an, hipStream_t st)
 {
     switch (a.R) {
-    case 5: launch_stem_r<5>(a, yp, POH, POW, st); break;
-    case 6: launch_stem_r<6>(a, yp, POH, POW, st); break;
-    case 7: launch_stem_r<7>(a, yp, POH, POW, st); break;
-    default: launch_stem_r<8>(a, yp, POH, POW, st); break; // conv_stem_maxpool_applies: 5 <= R <= 8
+    case 5: launch_stem_r<5>(a, yp, POH, POW, an, st); break;
+    case 6: launch_stem_r<6>(a, yp, POH, POW, an, st); break;
+    case 7: launch_stem_r<7>(a, yp, POH, POW, an, st); break;
+    default: launch_stem_r<8>(a, yp, POH, POW, an, st); break; // conv_stem_maxpool_applies: 5 <= R <= 8
     }
 }
 

@@ -69,6 +69,9 @@ _SIGS = {
                                            C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
     "hipq_conv2d_maxpool_fusable": (C.c_int, [C.c_void_p] + [C.c_int] * 5 + [C.c_float, C.c_int, C.c_float, C.c_int, C.c_int]),
     "hipq_conv2d_run_maxpool": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
+    "hipq_conv2d_maxpool_conv_fusable": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
+    "hipq_conv2d_run_maxpool_conv": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int,
+                                               C.c_void_p, C.c_void_p]),
     "hipq_ip_reorder_weights": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 6),
     "hipq_add_u8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_float, C.c_int, C.c_float,
                               C.c_int, C.c_float, C.c_int, C.c_int, C.c_void_p]),
@@ -272,6 +275,16 @@ class Conv2d:
         (include/hipq.h: hipq_conv2d_run_maxpool)."""
         check(lib().hipq_conv2d_run_maxpool(self.handle, _ptr(x), _ptr(y), y.shape[1], y.shape[2], int(bool(relu)), _stream()))
         return y
+
+    def maxpool_conv_fusable(self, OH, OW, nxt):
+        """Can that pooling AND the 1x1 convolution `nxt` that reads the pooled tensor run inside this convolution's kernel?"""
+        return bool(lib().hipq_conv2d_maxpool_conv_fusable(self.handle, OH, OW, nxt.handle))
+
+    def run_maxpool_conv(self, x, y, nxt, y_next, relu=False, next_relu=False):
+        """y = maxpool3x3/2/1(conv(x)) and y_next = nxt(y) in one launch (include/hipq.h: hipq_conv2d_run_maxpool_conv)."""
+        check(lib().hipq_conv2d_run_maxpool_conv(self.handle, _ptr(x), _ptr(y), y.shape[1], y.shape[2], int(bool(relu)),
+                                                 nxt.handle, int(bool(next_relu)), _ptr(y_next), _stream()))
+        return y, y_next
 
     def close(self):
         if self.handle:

@@ -568,6 +568,57 @@ def test_stem_convolution_with_fused_max_pooling():
     assert not s1.maxpool_fusable(8, 8, 3, 2, 1, 0.1, 0, 0.1, 0)
 
 
+def test_stem_with_pooling_and_the_next_convolution():
+    """hipq_conv2d_run_maxpool_conv: stem convolution, max pooling and the 1x1 convolution (64 -> 64) that reads the pooled
+    tensor in one kernel, against the oracle's three operators: pooled rows of 56, 16 and 9 pixels (two, one and a
+    ragged pixel tile), a ragged last row block, with and without ReLU on either convolution; the pooled tensor is
+    written as well; plans that do not chain refuse."""
+    rng = np.random.default_rng(152)
+    #        N  C   H    W   R pad relu relu_next
+    cases = [(2, 3, 224, 224, 7, 3, True, True), (3, 3, 64, 64, 7, 3, False, False), (1, 4, 50, 36, 5, 2, True, False),
+             (2, 3, 130, 100, 7, 3, False, True)]
+    for N, C, H, W, R, pad, relu, relu_next in cases:
+        print("stem chain case", N, C, H, W, R, pad, relu, relu_next, flush=True)
+        x = rng.integers(0, 256, (N, C, H, W), dtype=np.uint8)
+        w = rng.integers(0, 256, (64, C, R, R), dtype=np.uint8)
+        b = rng.integers(-20000, 20000, 64).astype(np.int32)
+        ia, izp, wa = rand_q(rng), int(rng.integers(0, 256)), rand_q(rng)
+        ozp = 0 if relu else int(rng.integers(0, 256))
+        oa = float(np.float32(ia * wa * np.sqrt(C * R * R) * 60.0))
+        q = (ia, izp, wa, 128, oa, ozp)
+        conv = orc.conv2d_u8(x, w, b, pad, 2, 1, *q)
+        if relu:
+            conv = np.maximum(conv, ozp).astype(np.uint8)
+        pooled = orc.pool_u8(conv, 3, 1, 2, 0, False, oa, ozp, oa, ozp)
+        w2 = rng.integers(0, 256, (64, 64, 1, 1), dtype=np.uint8)
+        b2 = rng.integers(-20000, 20000, 64).astype(np.int32)
+        wa2, oz2 = rand_q(rng), (0 if relu_next else int(rng.integers(0, 256)))
+        oa2 = float(np.float32(oa * wa2 * 8.0 * 60.0))
+        q2 = (oa, ozp, wa2, 128, oa2, oz2)
+        want2 = orc.conv2d_u8(pooled, w2, b2, 0, 1, 1, *q2)
+        if relu_next:
+            want2 = np.maximum(want2, oz2).astype(np.uint8)
+        assert len(np.unique(want2)) > 8
+        plan = hipq.Conv2d(x.shape, w, b, pad, 2, 1, *q, relu=relu)
+        nxt = hipq.Conv2d(pooled.shape, w2, b2, 0, 1, 1, *q2, relu=relu_next)
+        POH, POW = pooled.shape[2], pooled.shape[3]
+        assert plan.maxpool_conv_fusable(POH, POW, nxt), (plan.kernel, nxt.kernel)
+        yd = torch.full((N, POH, POW, 64), 7, dtype=torch.uint8, device="cuda")
+        y2 = torch.full((N, POH, POW, 64), 9, dtype=torch.uint8, device="cuda")
+        plan.run_maxpool_conv(hipq.to_device_nhwc(x), yd, nxt, y2)
+        torch.cuda.synchronize()
+        assert np.array_equal(yd.cpu().numpy().transpose(0, 3, 1, 2), pooled), (N, C, H, W, "pooled tensor")
+        got2 = y2.cpu().numpy().transpose(0, 3, 1, 2)
+        assert np.array_equal(got2, want2), (N, C, H, W, R, int((got2 != want2).sum()), np.argwhere(got2 != want2)[:6].tolist())
+        # a next layer that reads another scale, or is no 64 -> 64 1x1 layer, does not chain
+        other = hipq.Conv2d(pooled.shape, w2, b2, 0, 1, 1, float(np.float32(oa * 1.25)), ozp, wa2, 128, oa2, oz2)
+        assert not plan.maxpool_conv_fusable(POH, POW, other)
+        with pytest.raises(hipq.HipqError, match="do not run as one kernel"):
+            plan.run_maxpool_conv(hipq.to_device_nhwc(x), yd, other, y2)
+        wide = hipq.Conv2d(pooled.shape, rng.integers(0, 256, (128, 64, 1, 1), dtype=np.uint8), None, 0, 1, 1, *q2)
+        assert not plan.maxpool_conv_fusable(POH, POW, wide)
+
+
 def test_elementwise():
     rng = np.random.default_rng(15)
     for n in (1, 15, 16, 4099, 64 * 56 * 56 * 16 + 3):
