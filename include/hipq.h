@@ -261,6 +261,17 @@ int hipq_bottleneck_fusable(const hipq_conv2d_plan *reduce, const hipq_conv2d_pl
 int hipq_bottleneck_run(const hipq_conv2d_plan *reduce, const hipq_conv2d_plan *mid, const hipq_conv2d_plan *widen,
                         const void *x, int residual_is_input0, float oalpha, int ozp, int obits, void *y, void *stream);
 
+/* The same with the 1x1 / stride 1 convolution that reads the sum computed in the kernel as well: y_next = next(y), with
+ * `next` from CW to 2 CM channels (the first layer of the next stage; execute.c:43-90 runs it as one more operator),
+ * reading the sum with the scale and zero point given for it; next_relu as in hipq_conv2d_run_relu.  The sum is written
+ * too - the next stage's shortcut reads it.  x, y and y_next are three different tensors.
+ * hipq_bottleneck_conv_fusable answers (1 / 0); hipq_bottleneck_run_conv fails with an error where it answers 0. */
+int hipq_bottleneck_conv_fusable(const hipq_conv2d_plan *reduce, const hipq_conv2d_plan *mid, const hipq_conv2d_plan *widen,
+                                 int residual_is_input0, float oalpha, int ozp, int obits, const hipq_conv2d_plan *next);
+int hipq_bottleneck_run_conv(const hipq_conv2d_plan *reduce, const hipq_conv2d_plan *mid, const hipq_conv2d_plan *widen,
+                             const void *x, int residual_is_input0, float oalpha, int ozp, int obits, void *y,
+                             const hipq_conv2d_plan *next, int next_relu, void *y_next, void *stream);
+
 /*
  * The rest of a bottleneck block in one launch, from its 3x3 convolution on: y = add(widen(mid(x)), residual) and, when
  * `next` is not NULL, y_next = next(y) - bit-identical to hipq_conv2d_run(mid, x, t), hipq_conv2d_run_add(widen, t,

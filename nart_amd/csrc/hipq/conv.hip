@@ -2370,7 +2370,7 @@ extern "C" int hipq_bottleneck_fusable(const hipq_conv2d_plan *p1, const hipq_co
     ConvArgs a1, a2, a3;
     if (!block_args(p1, p2, p3, residual_is_input0, oalpha, ozp, obits, &a1, &a2, &a3))
         return 0;
-    if (!conv_block_applies(a1, a2, a3))
+    if (!conv_block_applies(a1, a2, a3, nullptr))
         return 0;
     // built-in rule: where it measured faster than the three launches it replaces - blocks of 256 middle channels (14x14
     // images at batch 64: 31 against 41 us and two launch gaps); hipq_conv2d_plan_special(reduce, 2): wherever it applies
@@ -2393,7 +2393,46 @@ extern "C" int hipq_bottleneck_run(const hipq_conv2d_plan *p1, const hipq_conv2d
     a1.acc_out = a2.acc_out = a3.acc_out = nullptr;
     a3.res = a1.x;
     a3.y = static_cast<uint8_t *>(y);
-    launch_conv_block(a1, a2, a3, static_cast<hipStream_t>(stream));
+    launch_conv_block(a1, a2, a3, nullptr, static_cast<hipStream_t>(stream));
+    return launch_status("conv_bottleneck_kernel");
+}
+
+extern "C" int hipq_bottleneck_conv_fusable(const hipq_conv2d_plan *p1, const hipq_conv2d_plan *p2, const hipq_conv2d_plan *p3,
+                                            int residual_is_input0, float oalpha, int ozp, int obits, const hipq_conv2d_plan *next)
+{
+    if (!next || !hipq_bottleneck_fusable(p1, p2, p3, residual_is_input0, oalpha, ozp, obits))
+        return 0;
+    if (next->variant != kMfma || !next->special || next->tile_selected || next->has_wzp || next->d.dtype != HIPQ_DTYPE_U8
+        || next->d.obits != 8 || next->d.izp != ozp || next->d.ialpha != oalpha)
+        return 0;
+    ConvArgs a1, a2, a3;
+    block_args(p1, p2, p3, residual_is_input0, oalpha, ozp, obits, &a1, &a2, &a3);
+    return conv_block_applies(a1, a2, a3, &next->args) ? 1 : 0;
+}
+
+extern "C" int hipq_bottleneck_run_conv(const hipq_conv2d_plan *p1, const hipq_conv2d_plan *p2, const hipq_conv2d_plan *p3, const void *x,
+                                        int residual_is_input0, float oalpha, int ozp, int obits, void *y,
+                                        const hipq_conv2d_plan *next, int next_relu, void *y_next, void *stream)
+{
+    clear_error();
+    HIPQ_REQUIRE(p1 && p2 && p3 && x && y && next && y_next, "hipq_bottleneck_run_conv: null argument");
+    HIPQ_REQUIRE(x != y && x != y_next && y != y_next,
+                 "hipq_bottleneck_run_conv: the sum and the next layer's output cannot overwrite the block's input or each other");
+    HIPQ_REQUIRE(hipq_bottleneck_conv_fusable(p1, p2, p3, residual_is_input0, oalpha, ozp, obits, next),
+                 "hipq_bottleneck_run_conv: these plans (%s, %s, %s, next layer %s) and this add do not run as one kernel: run "
+                 "hipq_bottleneck_run and hipq_conv2d_run", p1->name.c_str(), p2->name.c_str(), p3->name.c_str(), next->name.c_str());
+    ConvArgs a1, a2, a3, an = next->args;
+    block_args(p1, p2, p3, residual_is_input0, oalpha, ozp, obits, &a1, &a2, &a3);
+    a1.x = static_cast<const uint8_t *>(x);
+    a1.y = a2.y = nullptr;
+    a1.acc_out = a2.acc_out = a3.acc_out = an.acc_out = nullptr;
+    a3.res = a1.x;
+    a3.y = static_cast<uint8_t *>(y);
+    an.x = nullptr;
+    an.y = static_cast<uint8_t *>(y_next);
+    if (next_relu)
+        an.lo = std::min(next->d.ozp, an.q.hi); // the ReLU clamp, as in hipq_conv2d_run_relu
+    launch_conv_block(a1, a2, a3, &an, static_cast<hipStream_t>(stream));
     return launch_status("conv_bottleneck_kernel");
 }
 

@@ -8,8 +8,10 @@ namespace hipq {
 // a1: the 1x1 convolution that reads the block's input x (a1.x), a2: the 3x3 / stride 1 / pad 1 convolution, a3: the
 // widening 1x1 convolution with the add's parameters in a3.addq / a3.res_first; the residual is x itself and the sum goes
 // to a3.y.  true when conv_bottleneck_kernel computes this chain.
-bool conv_block_applies(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3);
-void launch_conv_block(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3, hipStream_t st);
+// an != nullptr: the 1x1 convolution that reads the sum, to twice the middle channels (the first layer of the next stage), is
+// computed in the kernel as well (output to an->y).
+bool conv_block_applies(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3, const ConvArgs *an);
+void launch_conv_block(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3, const ConvArgs *an, hipStream_t st);
 // true where the one kernel measured faster than the launches it replaces
 bool conv_block_preferred(const ConvArgs &a1);
 

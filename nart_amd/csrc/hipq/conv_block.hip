@@ -67,9 +67,11 @@ struct BlockGeom {
 
 // G = CM / 64 (1, 2, 4): 2 G waves.  MT1: pixel tiles of layer 1 (2: regions of at most 64 pixels, i.e. images of at
 // most 2 x 2 patches; 3: up to 9 x 9 = 81).
-template <int G, int MT1>
+// NX: 0, or 2 - the 1x1 convolution that reads the sum (CW -> 2 CM channels, the first layer of the next stage) is computed
+// as well: the sum tile takes the x tile's place in LDS, row = output index m, and is that layer's pixel operand.
+template <int G, int MT1, int NX>
 __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvArgs a1, const ConvArgs a2, const ConvArgs a3,
-                                                                    const BlockGeom geo)
+                                                                    const ConvArgs an, const BlockGeom geo)
 {
     constexpr int NW = 2 * G, NT = 128 * G, CM = 64 * G, CW = 256 * G;
     constexpr int X_BYTES = 32 * MT1 * CW;                  // the region's pixel rows, CW bytes each
@@ -214,6 +216,7 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
         int jres[2];      // the output pixel's row in the x tile
         size_t yoff[2];
         bool valid[2];
+        int pixo[2];
 #pragma unroll
         for (int t = 0; t < 2; t++) {
             const int m = 32 * t + p;
@@ -223,7 +226,8 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
             const int py = (m * 57) >> 9, px = m - py * kGridW; // m / 9 for m < 64
             valid[t] = py < kPatch && px < kPatch;
             jres[t] = valid[t] ? (y0 + py - ry0) * RW + (x0 + px - rx0) : 0;
-            yoff[t] = (size_t)((n * geo.H + y0 + py) * geo.W + x0 + px) * CW;
+            pixo[t] = (n * geo.H + y0 + py) * geo.W + x0 + px;
+            yoff[t] = (size_t)pixo[t] * CW;
         }
         STAMP(8);
         for (int cc = 0; cc < 4; cc++) {
@@ -242,15 +246,52 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
                     acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[ks], bf[t][ks], acc[t], 0, 0, 0);
             if (cc + 1 < 4)
                 load_chunk(cc + 1); // into the registers the multiplies above have read: they arrive during the arithmetic below
+            const int c16 = (ch >> 4) + h; // the 16-byte piece of the pixel's CW bytes
+            v4i res[2];
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+                res[t] = *reinterpret_cast<const v4i *>(lds + jres[t] * CW + (c16 & ~15) * 16 + (((c16 & 15) ^ (jres[t] & 15)) << 4));
 #pragma unroll
             for (int t = 0; t < 2; t++) {
-                const int c16 = (ch >> 4) + h; // the 16-byte piece of the pixel's CW bytes
-                const v4i res = *reinterpret_cast<const v4i *>(lds + jres[t] * CW + (c16 & ~15) * 16 + (((c16 & 15) ^ (jres[t] & 15)) << 4));
-                const v4i o = requant_add16(a3, acc[t], res);
+                const v4i o = requant_add16(a3, acc[t], res[t]);
                 if (valid[t])
                     *reinterpret_cast<v4i *>(a3.y + yoff[t] + ch + 16 * h) = o;
+                if (NX) {
+                    // the sum tile over the x tile: only this wave ever touches these 16-byte pieces (its own channels), and
+                    // every lane has read its residuals of this chunk above
+                    const int m = 32 * t + p;
+                    *reinterpret_cast<v4i *>(lds + m * CW + (c16 & ~15) * 16 + (((c16 & 15) ^ (m & 15)) << 4)) = o;
+                }
             }
             STAMP(9 + cc);
+        }
+        if (!NX)
+            return;
+        // ================= the next stage's first layer: CW -> NX * CM on the sum tile =================
+        // a wave owns the 32-channel tiles wave, wave + NW, ... one after the other
+        const size_t wslabn = (size_t)an.kout_pad * 64;
+#pragma unroll
+        for (int jx = 0; jx < (NX ? NX : 1); jx++) {
+            const int cn = 32 * (wave + NW * jx);
+            const uint8_t *wn0 = an.wfrag + (size_t)cn * 64 + lane * 16;
+            auto ldwn = [&](int s, int kk) { return ldg128(wn0 + (size_t)s * wslabn + kk * 1024); };
+            WeightRing1<D1> rr;
+            ring_fill1<4 * G, D1>(rr, ldwn);
+            v16i accn[2];
+#pragma unroll
+            for (int t = 0; t < 2; t++)
+                init_acc(accn[t], an.bias2 + cn + 16 * h, false);
+            if (jx == 0) {
+                __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): this wave's part of the sum tile is written
+                __builtin_amdgcn_s_barrier();
+            }
+            reduce_all<4 * G, 2, D1>(accn, rr, (int)an.xmask, ldwn, ldb1);
+#pragma unroll
+            for (int t = 0; t < 2; t++) {
+                const v4i o = requant16(an, accn[t], 0);
+                if (valid[t])
+                    *reinterpret_cast<v4i *>(an.y + (size_t)pixo[t] * (NX * CM) + cn + 16 * h) = o;
+            }
         }
     }
 }
@@ -536,7 +577,7 @@ bool conv_block_preferred(const ConvArgs &a1) { return a1.out_cs == 256; }
 // (the sum's pixel tile is what that form saves); 256 channels belong to the whole-block kernel.
 bool conv_block_tail_preferred(const ConvArgs &a2, bool chained) { return a2.in_cs == 128 || (a2.in_cs == 64 && chained); }
 
-bool conv_block_applies(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3)
+bool conv_block_applies(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3, const ConvArgs *an)
 {
     const int cm = a1.out_cs, cw = a1.in_cs;
     auto plain = [](const ConvArgs &a) {
@@ -546,6 +587,9 @@ bool conv_block_applies(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &
         return a.R == 1 && a.S == 1 && a.pad_h == 0 && a.pad_w == 0 && a.stride_h == 1 && a.stride_w == 1;
     };
     auto same_image = [&](const ConvArgs &a) { return a.N == a1.N && a.H == a1.H && a.W == a1.W && a.OH == a1.H && a.OW == a1.W; };
+    if (an && !(plain(*an) && one(*an) && an->C == cw && an->in_cs == cw && an->K == 2 * cm && an->out_cs == an->K
+                && an->nslab == cw / 64 && an->kout_pad >= an->K && an->res == nullptr && same_image(*an)))
+        return false;
     return plain(a1) && plain(a2) && plain(a3) && (cm == 64 || cm == 128 || cm == 256) && cw == 4 * cm
         && one(a1) && a1.C == cw && a1.K == cm && a1.nslab == cw / 64 && a1.kout_pad >= cm && a1.res == nullptr && same_image(a1)
         && a2.R == 3 && a2.S == 3 && a2.pad_h == 1 && a2.pad_w == 1 && a2.stride_h == 1 && a2.stride_w == 1 && a2.C == cm
@@ -557,7 +601,7 @@ bool conv_block_applies(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &
 }
 
 template <int G>
-static void launch_block_g(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3, hipStream_t st)
+static void launch_block_g(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3, const ConvArgs *an, hipStream_t st)
 {
     BlockGeom geo;
     geo.H = a1.H, geo.W = a1.W, geo.PY = a1.H / kPatch, geo.PX = a1.W / kPatch;
@@ -566,18 +610,23 @@ static void launch_block_g(const ConvArgs &a1, const ConvArgs &a2, const ConvArg
     geo.stamps = getenv("HIPQ_BLOCK_STAMPS") ? (unsigned long long *)strtoull(getenv("HIPQ_BLOCK_STAMPS"), nullptr, 0) : nullptr;
 #endif
     const dim3 grid((unsigned)((geo.npatch + 7) / 8 * 8)), block(128 * G);
-    if (geo.PY <= 2 && geo.PX <= 2) // every region is at most 8 x 8 pixels
-        hipLaunchKernelGGL((conv_bottleneck_kernel<G, 2>), grid, block, 0, st, a1, a2, a3, geo);
+    const bool small = geo.PY <= 2 && geo.PX <= 2; // every region is at most 8 x 8 pixels
+    if (small && an)
+        hipLaunchKernelGGL((conv_bottleneck_kernel<G, 2, 2>), grid, block, 0, st, a1, a2, a3, *an, geo);
+    else if (small)
+        hipLaunchKernelGGL((conv_bottleneck_kernel<G, 2, 0>), grid, block, 0, st, a1, a2, a3, a3, geo);
+    else if (an)
+        hipLaunchKernelGGL((conv_bottleneck_kernel<G, 3, 2>), grid, block, 0, st, a1, a2, a3, *an, geo);
     else
-        hipLaunchKernelGGL((conv_bottleneck_kernel<G, 3>), grid, block, 0, st, a1, a2, a3, geo);
+        hipLaunchKernelGGL((conv_bottleneck_kernel<G, 3, 0>), grid, block, 0, st, a1, a2, a3, a3, geo);
 }
 
-void launch_conv_block(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3, hipStream_t st)
+void launch_conv_block(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &a3, const ConvArgs *an, hipStream_t st)
 {
     switch (a1.out_cs) {
-    case 64: launch_block_g<1>(a1, a2, a3, st); break;
-    case 128: launch_block_g<2>(a1, a2, a3, st); break;
-    default: launch_block_g<4>(a1, a2, a3, st); break; // conv_block_applies: 64, 128 or 256 middle channels
+    case 64: launch_block_g<1>(a1, a2, a3, an, st); break;
+    case 128: launch_block_g<2>(a1, a2, a3, an, st); break;
+    default: launch_block_g<4>(a1, a2, a3, an, st); break; // conv_block_applies: 64, 128 or 256 middle channels
     }
 }
 

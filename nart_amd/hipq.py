@@ -61,6 +61,9 @@ _SIGS = {
     "hipq_conv2d_run_add2": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_int,
                                        C.c_void_p, C.c_void_p]),
     "hipq_bottleneck_fusable": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_int]),
+    "hipq_bottleneck_conv_fusable": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_int, C.c_void_p]),
+    "hipq_bottleneck_run_conv": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_int,
+                                           C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
     "hipq_bottleneck_run": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_int,
                                       C.c_void_p, C.c_void_p]),
     "hipq_bottleneck_tail_fusable": (C.c_int, [C.c_void_p, C.c_void_p, C.c_int, C.c_float, C.c_int, C.c_float, C.c_int, C.c_int,
@@ -320,6 +323,19 @@ def bottleneck_run(reduce, mid, widen, x, residual_first, oalpha, ozp, y, obits=
     check(lib().hipq_bottleneck_run(reduce.handle, mid.handle, widen.handle, _ptr(x), int(bool(residual_first)), oalpha, ozp,
                                     obits, _ptr(y), _stream()))
     return y
+
+
+def bottleneck_conv_fusable(reduce, mid, widen, residual_first, oalpha, ozp, nxt, obits=8):
+    """Can that block AND the 1x1 convolution `nxt` that reads its sum run as one kernel (include/hipq.h)?"""
+    return bool(lib().hipq_bottleneck_conv_fusable(reduce.handle, mid.handle, widen.handle, int(bool(residual_first)), oalpha, ozp,
+                                                   obits, nxt.handle))
+
+
+def bottleneck_run_conv(reduce, mid, widen, x, residual_first, oalpha, ozp, y, nxt, y_next, obits=8, next_relu=False):
+    """y = add(widen(mid(reduce(x))), x) and y_next = nxt(y) in one launch (include/hipq.h: hipq_bottleneck_run_conv)."""
+    check(lib().hipq_bottleneck_run_conv(reduce.handle, mid.handle, widen.handle, _ptr(x), int(bool(residual_first)), oalpha, ozp,
+                                         obits, _ptr(y), nxt.handle, int(bool(next_relu)), _ptr(y_next), _stream()))
+    return y, y_next
 
 
 def bottleneck_tail_fusable(mid, widen, residual_first, res_alpha, res_zp, oalpha, ozp, nxt=None, obits=8):

@@ -94,8 +94,35 @@ class HipqExecutor:
                 self.plans += plans
                 xin = self.buf[c1.inputs[0]]
                 res_first = node.inputs[0] == c1.inputs[0]
-                fn = (lambda ps=plans, i=xin, rf=res_first, y=y, o=out: hipq.bottleneck_run(ps[0], ps[1], ps[2], i, rf, y.alpha, y.zp, o))
                 nb = 2 * int(np.prod(y.shape)) + sum(case.weights[c.attrs["w"]].size + 4 * c.attrs["K"] for c in (c1, c2, c3))
+                # the 1x1 convolution that reads the sum (the first layer of the next stage) in the same kernel
+                nxt = None
+                for nd in case.nodes:
+                    na = nd.attrs
+                    if (nd.kind == "conv" and nd.inputs[0] == node.output and na["k"] == 1 and na["stride"] == 1
+                            and na["pad"] == 0 and na["group"] == 1 and nd.output != case.output.name
+                            and id(nd) not in self.in_block and nd.output not in self.fused):
+                        p2, nb2 = conv_plan(nd)
+                        if hipq.bottleneck_conv_fusable(plans[0], plans[1], plans[2], res_first, y.alpha, y.zp, p2):
+                            nxt = (nd, p2, nb2)
+                            break
+                        self._early[id(nd)] = p2
+                if nxt is not None:
+                    nd, p2, nb2 = nxt
+                    y2 = self._tensor(T[nd.output])
+                    if y2 is None:
+                        raise RuntimeError("shared executor: %s is fused away in the parent but not here" % nd.output)
+                    self.buf[nd.output] = y2
+                    self.plans.append(p2)
+                    self.chained[node.output] = nd
+                    done.add(id(nd))
+                    fn = (lambda ps=plans, i=xin, rf=res_first, y=y, o=out, p2=p2, y2=y2:
+                          hipq.bottleneck_run_conv(ps[0], ps[1], ps[2], i, rf, y.alpha, y.zp, o, p2, y2))
+                    self.steps.append({"label": node.output, "kind": "block+conv", "kernel": "conv_mfma_i8_bottleneck+conv", "fn": fn,
+                                       "ops": sum(p.ops for p in plans) + p2.ops, "bytes": nb + nb2 - int(np.prod(y.shape)),
+                                       "plan": plans[0]})
+                    continue
+                fn = (lambda ps=plans, i=xin, rf=res_first, y=y, o=out: hipq.bottleneck_run(ps[0], ps[1], ps[2], i, rf, y.alpha, y.zp, o))
                 self.steps.append({"label": node.output, "kind": "block", "kernel": "conv_mfma_i8_bottleneck", "fn": fn,
                                    "ops": sum(p.ops for p in plans), "bytes": nb, "plan": plans[0]})
             elif node.kind == "add" and id(node) in self.duals:

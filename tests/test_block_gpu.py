@@ -86,6 +86,26 @@ def test_bottleneck_block(case):
         plans[2].run_add(t2, xd, res_first, xq[0], xq[1], sq[0], sq[1], y2)
         torch.cuda.synchronize()
         assert torch.equal(y, y2)
+        # the same with the next stage's first layer (CW -> CW / 2) computed in the kernel as well
+        CN = CW // 2
+        wn = rng.integers(1, 256, (CN, CW, 1, 1), dtype=np.uint8)
+        sigma = 74.0 * 74.0 * math.sqrt(CW)
+        bn = rng.integers(-int(sigma), int(sigma) + 1, CN).astype(np.int32)
+        oan = float(np.float32(sq[0] * rng.uniform(0.75, 1.35)))
+        qn = (sq[0], sq[1], float(np.float32(oan * 40.0 / (sq[0] * sigma))), 128, oan, int(rng.integers(20, 60)))
+        pn = hipq.Conv2d((N, CW, H, W), wn, bn, 0, 1, 1, *qn, relu=res_first)
+        assert hipq.bottleneck_conv_fusable(*plans, res_first, sq[0], sq[1], pn), hipq.lib().hipq_last_error()
+        y3, yn = torch.zeros_like(xd), torch.zeros((N, H, W, CN), dtype=torch.uint8, device="cuda")
+        hipq.bottleneck_run_conv(*plans, xd, res_first, sq[0], sq[1], y3, pn, yn)
+        torch.cuda.synchronize()
+        assert torch.equal(y3, y)
+        wantn = orc.conv2d_u8(want, wn, bn, 0, 1, 1, *qn)
+        if res_first:
+            wantn = np.maximum(wantn, qn[5]).astype(np.uint8)
+        gotn = hipq.from_device_nhwc(yn, CN)
+        bad = gotn != wantn
+        assert not bad.any(), (case, "next layer", int(bad.sum()), np.argwhere(bad)[:8].tolist())
+        assert len(np.unique(wantn)) > 8
 
 
 TAIL_CASES = [  # N, CW, H, W: patches of 8 x 8, 4 x 14 and 7 x 7 pixels; 64, 128 and 256 middle channels
