@@ -49,6 +49,7 @@ constexpr int kGridRows = 96;      // rows held for that grid (81 positions; the
 
 struct BlockGeom {
     int H, W, PY, PX, npatch;
+    int IH, IW; // the tail kernel's input image where its 3x3 layer has stride 2 (H, W: the output image)
 #ifdef HIPQ_BLOCK_STAMPS
     unsigned long long *stamps;
 #endif
@@ -309,13 +310,14 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
 //   * layer 2 (3x3) as above, on the compact pixel index q = PW * row + column, its bytes to LDS;
 //   * layer 3 + add as above, the sum stored and - CHAIN - kept in LDS, 64 pixel rows of CW bytes;
 //   * CHAIN: the next layer (CW -> CM, or CW -> 2 CM where the next stage begins) reads that tile as its pixel operand.
-template <int G, int PH, int PW, int NX>
+// ST: the 3x3 layer's stride (1, or 2 - the first block of a stage: the grid then holds (2 PH + 1) x (2 PW + 1) input pixels).
+template <int G, int PH, int PW, int NX, int ST>
 __global__ __launch_bounds__(128 * G, (G == 1 ? 4 : G == 2 ? 3 : 2)) void conv_bottleneck_tail_kernel(const ConvArgs a2, const ConvArgs a3, const ConvArgs an,
                                                                          const BlockGeom geo)
 {
     constexpr int NW = 2 * G, NT = 128 * G, CM = 64 * G, CW = 256 * G;
     constexpr bool CHAIN = NX != 0; // the next layer has NX * CM output channels
-    constexpr int GW = PW + 2, GH = PH + 2, NPIX = PH * PW, GROWS = (GH * GW + 7) / 8 * 8;
+    constexpr int GW = ST * (PW - 1) + 3, GH = ST * (PH - 1) + 3, NPIX = PH * PW, GROWS = (GH * GW + 7) / 8 * 8;
     constexpr int G_OFF = 0, G_BYTES = GROWS * CM;            // layer 2's input on the bordered grid
     constexpr int M_OFF = G_OFF + G_BYTES, M_BYTES = 64 * CM; // layer 2's bytes, row = pixel
     // the sum tile takes the place of the grid and of layer 2's bytes once every wave holds its operands of layer 3
@@ -343,9 +345,10 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? 4 : G == 2 ? 3 : 2)) void conv_b
             if (ITEMS % NT == 0 || it < ITEMS) {
                 const int g = it / CPR, c = it % CPR;
                 const int gy = g / GW, gx = g - gy * GW;
-                const int iy = y0 - 1 + gy, ix = x0 - 1 + gx;
-                const bool in = g < GH * GW && (unsigned)iy < (unsigned)geo.H && (unsigned)ix < (unsigned)geo.W;
-                const uint8_t *src = in ? a2.x + (size_t)((n * geo.H + iy) * geo.W + ix) * CM + c * 16 : a2.padbuf;
+                const int iy = ST * y0 - 1 + gy, ix = ST * x0 - 1 + gx;
+                const int ih = ST == 1 ? geo.H : geo.IH, iw = ST == 1 ? geo.W : geo.IW;
+                const bool in = g < GH * GW && (unsigned)iy < (unsigned)ih && (unsigned)ix < (unsigned)iw;
+                const uint8_t *src = in ? a2.x + (size_t)((n * ih + iy) * iw + ix) * CM + c * 16 : a2.padbuf;
                 *reinterpret_cast<v4i *>(lds + G_OFF + g * CM + ((c ^ swz<CM>(g)) << 4)) = ldg128(src) ^ (int)a2.xmask;
             }
         }
@@ -362,7 +365,7 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? 4 : G == 2 ? 3 : 2)) void conv_b
     for (int t = 0; t < 2; t++) {
         const int q = 32 * t + p, qq = min(q, NPIX - 1), py = qq / PW, px = qq - py * PW;
         valid[t] = q < NPIX;
-        grow[t] = (py + 1) * GW + px + 1; // the centre tap's grid row
+        grow[t] = (ST * py + 1) * GW + ST * px + 1; // the centre tap's grid row
         pix[t] = (size_t)((n * geo.H + y0 + py) * geo.W + x0 + px);
     }
     auto ldb2 = [&](int s, int kk, int t) {
@@ -513,13 +516,16 @@ bool conv_block_tail_applies(const ConvArgs &a2, const ConvArgs &a3, const ConvA
     auto one = [](const ConvArgs &a) {
         return a.R == 1 && a.S == 1 && a.pad_h == 0 && a.pad_w == 0 && a.stride_h == 1 && a.stride_w == 1;
     };
-    auto same_image = [&](const ConvArgs &a) { return a.N == a2.N && a.H == a2.H && a.W == a2.W && a.OH == a2.H && a.OW == a2.W; };
+    // the layers after the 3x3 one work on its output image
+    auto same_image = [&](const ConvArgs &a) { return a.N == a2.N && a.H == a2.OH && a.W == a2.OW && a.OH == a2.OH && a.OW == a2.OW; };
+    const int st = a2.stride_h;
     int ph, pw;
     if (!(plain(a2) && plain(a3) && (cm == 64 || cm == 128 || cm == 256) && cw == 4 * cm
-          && a2.R == 3 && a2.S == 3 && a2.pad_h == 1 && a2.pad_w == 1 && a2.stride_h == 1 && a2.stride_w == 1 && a2.C == cm
-          && a2.K == cm && a2.out_cs == cm && a2.nslab == 9 * cm / 64 && a2.kout_pad >= cm && a2.res == nullptr && same_image(a2)
+          && a2.R == 3 && a2.S == 3 && a2.pad_h == 1 && a2.pad_w == 1 && a2.stride_w == st && (st == 1 || (st == 2 && cm == 128))
+          && a2.OH == (a2.H - 1) / st + 1 && a2.OW == (a2.W - 1) / st + 1 && a2.C == cm
+          && a2.K == cm && a2.out_cs == cm && a2.nslab == 9 * cm / 64 && a2.kout_pad >= cm && a2.res == nullptr
           && one(a3) && a3.C == cm && a3.in_cs == cm && a3.K == cw && a3.nslab == cm / 64 && a3.kout_pad >= cw && same_image(a3)
-          && a3.res != nullptr && a3.addq.fast && a3.addq.hi == 255 && tail_patch(a2.H, a2.W, &ph, &pw)
+          && a3.res != nullptr && a3.addq.fast && a3.addq.hi == 255 && tail_patch(a2.OH, a2.OW, &ph, &pw)
           && (long long)a2.N * a2.H * a2.W * cw < (1ll << 31)))
         return false;
     if (an == nullptr)
@@ -528,43 +534,46 @@ bool conv_block_tail_applies(const ConvArgs &a2, const ConvArgs &a3, const ConvA
         && an->nslab == cw / 64 && an->kout_pad >= an->K && an->res == nullptr && same_image(*an);
 }
 
-template <int G, int PH, int PW>
+template <int G, int PH, int PW, int ST>
 static void launch_tail_gp(const ConvArgs &a2, const ConvArgs &a3, const ConvArgs *an, hipStream_t st)
 {
     BlockGeom geo;
-    geo.H = a2.H, geo.W = a2.W, geo.PY = a2.H / PH, geo.PX = a2.W / PW;
+    geo.H = a2.OH, geo.W = a2.OW, geo.PY = a2.OH / PH, geo.PX = a2.OW / PW;
+    geo.IH = a2.H, geo.IW = a2.W;
     geo.npatch = a2.N * geo.PY * geo.PX;
 #ifdef HIPQ_BLOCK_STAMPS
     geo.stamps = getenv("HIPQ_BLOCK_STAMPS") ? (unsigned long long *)strtoull(getenv("HIPQ_BLOCK_STAMPS"), nullptr, 0) : nullptr;
 #endif
     const dim3 grid((unsigned)((geo.npatch + 7) / 8 * 8)), block(128 * G);
     if (an && an->K == 2 * a2.in_cs)
-        hipLaunchKernelGGL((conv_bottleneck_tail_kernel<G, PH, PW, 2>), grid, block, 0, st, a2, a3, *an, geo);
+        hipLaunchKernelGGL((conv_bottleneck_tail_kernel<G, PH, PW, 2, ST>), grid, block, 0, st, a2, a3, *an, geo);
     else if (an)
-        hipLaunchKernelGGL((conv_bottleneck_tail_kernel<G, PH, PW, 1>), grid, block, 0, st, a2, a3, *an, geo);
+        hipLaunchKernelGGL((conv_bottleneck_tail_kernel<G, PH, PW, 1, ST>), grid, block, 0, st, a2, a3, *an, geo);
     else
-        hipLaunchKernelGGL((conv_bottleneck_tail_kernel<G, PH, PW, 0>), grid, block, 0, st, a2, a3, a3, geo);
+        hipLaunchKernelGGL((conv_bottleneck_tail_kernel<G, PH, PW, 0, ST>), grid, block, 0, st, a2, a3, a3, geo);
 }
 
-template <int G>
+template <int G, int ST>
 static void launch_tail_g(const ConvArgs &a2, const ConvArgs &a3, const ConvArgs *an, hipStream_t st)
 {
     int ph = 0, pw = 0;
-    tail_patch(a2.H, a2.W, &ph, &pw);
+    tail_patch(a2.OH, a2.OW, &ph, &pw);
     if (ph == 8)
-        launch_tail_gp<G, 8, 8>(a2, a3, an, st);
+        launch_tail_gp<G, 8, 8, ST>(a2, a3, an, st);
     else if (ph == 4)
-        launch_tail_gp<G, 4, 14>(a2, a3, an, st);
+        launch_tail_gp<G, 4, 14, ST>(a2, a3, an, st);
     else
-        launch_tail_gp<G, 7, 7>(a2, a3, an, st);
+        launch_tail_gp<G, 7, 7, ST>(a2, a3, an, st);
 }
 
 void launch_conv_block_tail(const ConvArgs &a2, const ConvArgs &a3, const ConvArgs *an, hipStream_t st)
 {
+    if (a2.stride_h == 2) // conv_block_tail_applies: 128 middle channels only
+        return launch_tail_g<2, 2>(a2, a3, an, st);
     switch (a2.in_cs) {
-    case 64: launch_tail_g<1>(a2, a3, an, st); break;
-    case 128: launch_tail_g<2>(a2, a3, an, st); break;
-    default: launch_tail_g<4>(a2, a3, an, st); break; // conv_block_tail_applies: 64, 128 or 256 middle channels
+    case 64: launch_tail_g<1, 1>(a2, a3, an, st); break;
+    case 128: launch_tail_g<2, 1>(a2, a3, an, st); break;
+    default: launch_tail_g<4, 1>(a2, a3, an, st); break; // conv_block_tail_applies: 64, 128 or 256 middle channels
     }
 }
 

@@ -301,9 +301,9 @@ class HipqExecutor:
             for i in n.inputs:
                 uses.setdefault(i, []).append(n)
 
-        def only_conv(name, k):
+        def only_conv(name, k, strides=(1,)):
             n = prod.get(name)
-            if (n is None or n.kind != "conv" or n.attrs["k"] != k or n.attrs["stride"] != 1 or n.attrs["group"] != 1
+            if (n is None or n.kind != "conv" or n.attrs["k"] != k or n.attrs["stride"] not in strides or n.attrs["group"] != 1
                     or n.attrs["relu"] or len(uses.get(name, [])) != 1 or name == case.output.name):
                 return None
             return n
@@ -352,7 +352,7 @@ class HipqExecutor:
             # the block from its 3x3 layer on, with any residual, and the 1x1 layer that reads the sum
             for ci in (0, 1):
                 c3 = only_conv(add.inputs[ci], 1)
-                c2 = only_conv(c3.inputs[0], 3) if c3 else None
+                c2 = only_conv(c3.inputs[0], 3, (1, 2)) if c3 else None
                 if c2 is None or any(id(c) in self.in_block for c in (c2, c3)) or c3.attrs["pad"] != 0 or c2.attrs["pad"] != 1:
                     continue
                 p2, p3 = conv_plan(c2)[0], conv_plan(c3)[0]

@@ -45,15 +45,17 @@ def oracle_block(x, xq, layers, sq, res_first):
     return orc.add_u8(t, x, q3[4], q3[5], xq[0], xq[1], sq[0], sq[1])
 
 
-def plans_of(x, layers):
+def plans_of(x, layers, stride=1):
+    """stride: of the first layer (a 3x3 / pad 1 layer when it is 2)."""
     shape = x.shape
     plans = []
     for L in layers:
-        p = hipq.Conv2d(shape, L["w"], L["b"], L["pad"], 1, 1, *L["q"])
+        st = stride if not plans else 1
+        p = hipq.Conv2d(shape, L["w"], L["b"], L["pad"], st, 1, *L["q"])
         plans.append(p)
         if len(plans) == 1:
             p.special(2)  # the block kernel wherever it applies, not only where the built-in rule uses it
-        shape = (shape[0], L["w"].shape[0], shape[2], shape[3])
+        shape = (shape[0], L["w"].shape[0], (shape[2] - 1) // st + 1, (shape[3] - 1) // st + 1)
     return plans
 
 
@@ -113,12 +115,13 @@ TAIL_CASES = [  # N, CW, H, W: patches of 8 x 8, 4 x 14 and 7 x 7 pixels; 64, 12
 ]
 
 
-def make_tail(rng, N, CW, H, W, relu_next, wide_next=False):
+def make_tail(rng, N, CW, H, W, relu_next, wide_next=False, in_hw=None):
     """The block from its 3x3 layer on: t1 [N, CM, H, W] -> 3x3 -> 1x1 to CW -> add(., residual) -> 1x1 back to CM (to
-    2 CM with wide_next: the first layer of the next stage)."""
+    2 CM with wide_next: the first layer of the next stage).  in_hw: the size of t1 where the 3x3 layer has stride 2 and
+    H x W is its output."""
     CM = CW // 4
     CN = 2 * CM if wide_next else CM
-    t1 = rng.integers(0, 256, (N, CM, H, W), dtype=np.uint8)
+    t1 = rng.integers(0, 256, (N, CM) + tuple(in_hw or (H, W)), dtype=np.uint8)
     res = rng.integers(0, 256, (N, CW, H, W), dtype=np.uint8)
     ia, iz = 0.04, int(rng.integers(0, 256))
     layers = []
@@ -176,6 +179,44 @@ def test_bottleneck_tail(case):
             gotn = hipq.from_device_nhwc(yn, nx["w"].shape[0])
             bad = gotn != wantn
             assert not bad.any(), (case, "next layer", relu_next, int(bad.sum()), np.argwhere(bad)[:8].tolist())
+
+
+@pytest.mark.parametrize("case", [(2, 512, 28, 28, 56, 56), (1, 512, 8, 16, 15, 32), (2, 512, 7, 14, 13, 27), (1, 512, 4, 14, 8, 28)],
+                         ids=lambda c: "x".join(map(str, c)))
+def test_bottleneck_tail_with_a_strided_3x3_layer(case):
+    """The first block of a stage: the 3x3 layer has stride 2 (even and odd input sizes, every patch shape), the residual is
+    any tensor of the output's size (the projection shortcut), with and without the chained layer."""
+    N, CW, H, W, IH, IW = case
+    CM = CW // 4
+    rng = np.random.default_rng(2500 + H + IW)
+    for res_first, chain, wide in ((False, True, False), (True, False, False), (True, True, True)):
+        t1, res, layers, rq, sq, nx = make_tail(rng, N, CW, H, W, False, wide, (IH, IW))
+        plans = plans_of(t1, layers, stride=2)
+        pn = hipq.Conv2d((N, CW, H, W), nx["w"], nx["b"], 0, 1, 1, *nx["q"])
+        print("strided tail case", case, res_first, chain, wide, [p.kernel for p in plans], flush=True)
+        assert hipq.bottleneck_tail_fusable(plans[0], plans[1], res_first, rq[0], rq[1], sq[0], sq[1], pn if chain else None)
+        t = orc.conv2d_u8(t1, layers[0]["w"], layers[0]["b"], 1, 2, 1, *layers[0]["q"])
+        assert t.shape[2:] == (H, W)
+        c = orc.conv2d_u8(t, layers[1]["w"], layers[1]["b"], 0, 1, 1, *layers[1]["q"])
+        q3 = layers[1]["q"]
+        want = orc.add_u8(res, c, rq[0], rq[1], q3[4], q3[5], sq[0], sq[1]) if res_first else orc.add_u8(c, res, q3[4], q3[5], rq[0], rq[1], sq[0], sq[1])
+        xd, rd = hipq.to_device_nhwc(t1), hipq.to_device_nhwc(res)
+        y = torch.zeros_like(rd)
+        yn = torch.zeros((N, H, W, nx["w"].shape[0]), dtype=torch.uint8, device="cuda") if chain else None
+        hipq.bottleneck_tail_run(plans[0], plans[1], xd, rd, res_first, rq[0], rq[1], sq[0], sq[1], y, pn if chain else None, yn)
+        torch.cuda.synchronize()
+        got = hipq.from_device_nhwc(y, CW)
+        bad = got != want
+        assert not bad.any(), (case, res_first, chain, int(bad.sum()), np.argwhere(bad)[:8].tolist())
+        if chain:
+            wantn = orc.conv2d_u8(want, nx["w"], nx["b"], 0, 1, 1, *nx["q"])
+            gotn = hipq.from_device_nhwc(yn, nx["w"].shape[0])
+            bad = gotn != wantn
+            assert not bad.any(), (case, "next layer", int(bad.sum()), np.argwhere(bad)[:8].tolist())
+    # 64 or 256 middle channels with a strided 3x3 layer go through the separate entry points
+    t1, res, layers, rq, sq, nx = make_tail(rng, 1, 256, 8, 8, False, False, (16, 16))
+    plans = plans_of(t1, layers, stride=2)
+    assert not hipq.bottleneck_tail_fusable(plans[0], plans[1], False, rq[0], rq[1], sq[0], sq[1])
 
 
 def test_bottleneck_refusals():
