@@ -308,16 +308,19 @@ int hipq_conv2d_maxpool_fusable(const hipq_conv2d_plan *plan, int OH, int OW, in
                                 int izp, float oalpha, int ozp, int obits);
 int hipq_conv2d_run_maxpool(const hipq_conv2d_plan *plan, const void *x, void *y, int OH, int OW, int relu, void *stream);
 
-/* The same with the 1x1 convolution that reads the pooled tensor computed in the kernel as well (ResNet: the first layer
- * of the first bottleneck block, 64 -> 64 channels; execute.c:43-90 runs convolution, pooling and that convolution as
- * three operators): every pooled row is multiplied while it is still on the chip.  The pooled tensor is written too - its
- * other readers need it.  `next` reads the pooled tensor with the scale and zero point `plan` writes it with; next_relu as
- * in hipq_conv2d_run_relu; y_next: NHWC [N, OH, OW, 64], distinct from x and y.  hipq_conv2d_maxpool_conv_fusable answers
- * (1 / 0) whether the two plans and a 3x3 / stride 2 / pad 1 pooling to OH x OW run this way; the run entry point fails with
- * an error otherwise. */
-int hipq_conv2d_maxpool_conv_fusable(const hipq_conv2d_plan *plan, int OH, int OW, const hipq_conv2d_plan *next);
+/* The same with the 1x1 convolutions that read the pooled tensor computed in the kernel as well (ResNet: the first layer
+ * of the first bottleneck block, 64 -> 64 channels, and that block's projection shortcut, 64 -> 256; execute.c:43-90
+ * runs convolution, pooling and those convolutions as four operators): every pooled row is multiplied while it is still
+ * on the chip.  The pooled tensor is written too.  `next` and `next2` (may be NULL, then next2_relu and y_next2 are
+ * ignored) read the pooled tensor with the scale and zero point `plan` writes it with; each has a multiple of 64 output
+ * channels, 320 together at most; next_relu as in hipq_conv2d_run_relu; y_next: NHWC [N, OH, OW, K of next], y_next2
+ * likewise, all tensors distinct.  hipq_conv2d_maxpool_conv_fusable answers (1 / 0) whether the plans and a 3x3 / stride 2
+ * / pad 1 pooling to OH x OW run this way; the run entry point fails with an error otherwise. */
+int hipq_conv2d_maxpool_conv_fusable(const hipq_conv2d_plan *plan, int OH, int OW, const hipq_conv2d_plan *next,
+                                     const hipq_conv2d_plan *next2);
 int hipq_conv2d_run_maxpool_conv(const hipq_conv2d_plan *plan, const void *x, void *y, int OH, int OW, int relu,
-                                 const hipq_conv2d_plan *next, int next_relu, void *y_next, void *stream);
+                                 const hipq_conv2d_plan *next, int next_relu, void *y_next, const hipq_conv2d_plan *next2,
+                                 int next2_relu, void *y_next2, void *stream);
 
 /* ---- inner product: op_quant_ip_u8xu8_run — src/op/ip.cpp:133-209.
  * Expressed as a 1x1 convolution over M "pixels": desc {N=M, C=Kdim, H=W=1, K=Nout, R=S=1}.

@@ -2559,42 +2559,49 @@ extern "C" int hipq_conv2d_run_maxpool(const hipq_conv2d_plan *p, const void *x,
     a.acc_out = nullptr;
     if (relu)
         a.lo = std::min(p->d.ozp, a.q.hi); // the ReLU clamp, as in hipq_conv2d_run_relu
-    launch_conv_stem_maxpool(a, static_cast<uint8_t *>(y), OH, OW, nullptr, static_cast<hipStream_t>(stream));
+    launch_conv_stem_maxpool(a, static_cast<uint8_t *>(y), OH, OW, nullptr, nullptr, static_cast<hipStream_t>(stream));
     return launch_status("conv_stem_maxpool_kernel");
 }
 
-extern "C" int hipq_conv2d_maxpool_conv_fusable(const hipq_conv2d_plan *p, int OH, int OW, const hipq_conv2d_plan *next)
+extern "C" int hipq_conv2d_maxpool_conv_fusable(const hipq_conv2d_plan *p, int OH, int OW, const hipq_conv2d_plan *next,
+                                                const hipq_conv2d_plan *next2)
 {
     if (!p || !next || !hipq_conv2d_maxpool_fusable(p, OH, OW, 3, 2, 1, p->d.oalpha, p->d.ozp, p->d.oalpha, p->d.ozp, 8))
         return 0;
-    if (next->variant != kMfma || !next->special || next->tile_selected || next->has_wzp || next->d.dtype != HIPQ_DTYPE_U8
-        || next->d.obits != 8 || next->d.izp != p->d.ozp || next->d.ialpha != p->d.oalpha)
-        return 0;
-    return conv_stem_next_applies(p->args, OH, OW, next->args) ? 1 : 0;
+    for (const hipq_conv2d_plan *q : {next, next2})
+        if (q && (q->variant != kMfma || !q->special || q->tile_selected || q->has_wzp || q->d.dtype != HIPQ_DTYPE_U8 || q->d.obits != 8
+                  || q->d.izp != p->d.ozp || q->d.ialpha != p->d.oalpha))
+            return 0;
+    return conv_stem_next_applies(p->args, OH, OW, next->args, next2 ? &next2->args : nullptr) ? 1 : 0;
 }
 
 extern "C" int hipq_conv2d_run_maxpool_conv(const hipq_conv2d_plan *p, const void *x, void *y, int OH, int OW, int relu,
-                                            const hipq_conv2d_plan *next, int next_relu, void *y_next, void *stream)
+                                            const hipq_conv2d_plan *next, int next_relu, void *y_next,
+                                            const hipq_conv2d_plan *next2, int next2_relu, void *y_next2, void *stream)
 {
     clear_error();
-    HIPQ_REQUIRE(p && x && y && next && y_next, "hipq_conv2d_run_maxpool_conv: null argument");
-    HIPQ_REQUIRE(hipq_conv2d_maxpool_conv_fusable(p, OH, OW, next),
-                 "hipq_conv2d_run_maxpool_conv: these plans (%s, %s) do not run as one kernel with a 3x3 / stride 2 / pad 1 max "
+    HIPQ_REQUIRE(p && x && y && next && y_next && (!next2 || y_next2), "hipq_conv2d_run_maxpool_conv: null argument");
+    HIPQ_REQUIRE(hipq_conv2d_maxpool_conv_fusable(p, OH, OW, next, next2),
+                 "hipq_conv2d_run_maxpool_conv: these plans (%s, %s%s%s) do not run as one kernel with a 3x3 / stride 2 / pad 1 max "
                  "pooling to %d x %d between them: run hipq_conv2d_run_maxpool and hipq_conv2d_run", p->name.c_str(),
-                 next->name.c_str(), OH, OW);
-    HIPQ_REQUIRE(y_next != y && y_next != x, "hipq_conv2d_run_maxpool_conv: the next layer cannot overwrite a tensor the kernel reads or writes");
-    ConvArgs a = p->args, an = next->args;
+                 next->name.c_str(), next2 ? ", " : "", next2 ? next2->name.c_str() : "", OH, OW);
+    HIPQ_REQUIRE(y_next != y && y_next != x && (!next2 || (y_next2 != y && y_next2 != x && y_next2 != y_next)),
+                 "hipq_conv2d_run_maxpool_conv: a chained layer cannot overwrite a tensor the kernel reads or writes");
+    ConvArgs a = p->args, an = next->args, an2 = next2 ? next2->args : next->args;
     a.x = static_cast<const uint8_t *>(x);
     a.y = nullptr;
     a.acc_out = nullptr;
     if (relu)
         a.lo = std::min(p->d.ozp, a.q.hi); // the ReLU clamp, as in hipq_conv2d_run_relu
-    an.x = nullptr;
+    an.x = an2.x = nullptr;
     an.y = static_cast<uint8_t *>(y_next);
-    an.acc_out = nullptr;
+    an2.y = static_cast<uint8_t *>(y_next2);
+    an.acc_out = an2.acc_out = nullptr;
     if (next_relu)
         an.lo = std::min(next->d.ozp, an.q.hi);
-    launch_conv_stem_maxpool(a, static_cast<uint8_t *>(y), OH, OW, &an, static_cast<hipStream_t>(stream));
+    if (next2 && next2_relu)
+        an2.lo = std::min(next2->d.ozp, an2.q.hi);
+    launch_conv_stem_maxpool(a, static_cast<uint8_t *>(y), OH, OW, &an, next2 ? &an2 : nullptr, static_cast<hipStream_t>(stream));
     return launch_status("conv_stem_maxpool_kernel");
 }
 

@@ -20,13 +20,15 @@
 //     the int32 accumulators in registers (the same lane owns the same pixel column in every row, and a maximum
 //     commutes with the monotonic requantisation): only one row in 2.25 is requantised.  Its bytes go to a row buffer
 //     in LDS, from which the 256 threads take the horizontal 3-maxima and write one pooled row with 128-bit stores.
-//   * NEXT: a 1x1 convolution from the 64 pooled channels to 64 channels (the first layer of the first bottleneck
-//     block) is computed on every pooled row while it is still in LDS - two pixel tiles x two channel tiles, one per
-//     wave, two multiplies each, weights in fragment order (ConvArgs::wfrag) kept in registers - and written beside
-//     the pooled row, which its other readers (the projection shortcut) still need.
+//   * NEXT (1 or 2): the 1x1 convolutions that read the 64 pooled channels (the first layer of the first bottleneck
+//     block, 64 -> 64, and its projection shortcut, 64 -> 256) are computed on every pooled row while it is still in
+//     LDS: their weights (fragment order, ConvArgs::wfrag) and folded biases wait in LDS, a wave takes one of the two
+//     pixel tiles and every second 32-channel tile, two multiplies per tile.  The pooled row is written as well.
 // Requirements (checked by the host): uint8 tensors, input channel stride 4, at most 64 output channels with stride 64,
 // kernel rows of 5 to 8 taps, 5 to 8 kernel rows, stride 2, horizontal pad at most 4, convolution rows of at most 128
 // pixels, image rows of at most 248 pixels (a multiple of 4), weight zero point 128.
+#include <type_traits>
+
 #include "conv_stem.h"
 #include "conv_frag.h"
 
@@ -37,15 +39,19 @@ constexpr int kStemPitch = 16 + 1024;             // bytes of a patch row: 4 pad
 constexpr int kStemMaxPatchRows = 4 * kStemMaxPH + 8; // stride 2: 2 (2 ph) + R rows, R <= 8
 constexpr int kStemRowBuf = 128 * 64;             // one requantised row: 128 pixels x 64 channels
 constexpr int kStemPoolBuf = 64 * 64;             // NEXT: one pooled row, 64 pixel slots x 64 channels
+constexpr int kStemNextCh = 320;                  // NEXT: output channels of the chained layers together, at most
 
-template <int R, bool FAST, bool NEXT>
+template <int R, bool FAST, int NEXT>
 __global__ __launch_bounds__(256, 2) void conv_stem_maxpool_kernel(const ConvArgs a, uint8_t *yp, const int POH, const int POW,
-                                                                const int nrb, const int ph_per_wg, const ConvArgs an)
+                                                                const int nrb, const int ph_per_wg, const ConvArgs an,
+                                                                const ConvArgs an2)
 {
     constexpr int PITCH = kStemPitch;
     constexpr int R_OFF = kStemMaxPatchRows * PITCH;
     constexpr int P_OFF = R_OFF + 2 * kStemRowBuf;
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[P_OFF + (NEXT ? kStemPoolBuf : 0)];
+    constexpr int W_OFF = P_OFF + kStemPoolBuf;   // NEXT: the chained layers' weights, 64 bytes a channel, then their biases
+    constexpr int B_OFF = W_OFF + kStemNextCh * 64;
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[NEXT ? B_OFF + kStemNextCh * 4 : P_OFF];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int n = (int)blockIdx.x / nrb, rb = (int)blockIdx.x % nrb;
@@ -88,14 +94,16 @@ __global__ __launch_bounds__(256, 2) void conv_stem_maxpool_kernel(const ConvArg
             for (int e = 0; e < 4; e++)
                 bias[tn][g * 4 + e] = b[e];
         }
-    // NEXT: wave w computes pixel tile w & 1, channel tile w >> 1 of every pooled row; its two weight operands and its
-    // lane's 16 folded biases stay in registers
-    v4i wn[2] = {};
-    v16i bn = {};
+    // NEXT: the chained layers' weights (one slab: the 64 bytes of a channel's 64 inputs, tiles of 32 channels in
+    // fragment order) and folded biases -> LDS, layer after layer
     if (NEXT) {
-        const uint8_t *wp = an.wfrag + (size_t)(wave >> 1) * 2048 + lane * 16;
-        wn[0] = ldg128(wp), wn[1] = ldg128(wp + 1024);
-        frag::init_acc(bn, an.bias2 + 32 * (wave >> 1) + 16 * half, false);
+        const int k1 = an.K, k2 = NEXT == 2 ? an2.K : 0;
+        for (int i = tid; i < (k1 + k2) * 4; i += 256) { // 16-byte pieces
+            const uint8_t *src = i < k1 * 4 ? an.wfrag + (size_t)i * 16 : an2.wfrag + (size_t)(i - k1 * 4) * 16;
+            *reinterpret_cast<v4i *>(lds + W_OFF + i * 16) = ldg128(src);
+        }
+        for (int i = tid; i < k1 + k2; i += 256)
+            *reinterpret_cast<int32_t *>(lds + B_OFF + i * 4) = i < k1 ? an.bias2[i] : an2.bias2[i - k1];
         if (tid < kStemPoolBuf / 16) // pixel slots beyond the row are multiplied too: give them defined bytes
             *reinterpret_cast<u32x4 *>(lds + P_OFF + tid * 16) = u32x4{0, 0, 0, 0};
     }
@@ -186,16 +194,53 @@ __global__ __launch_bounds__(256, 2) void conv_stem_maxpool_kernel(const ConvArg
         if (NEXT) {
             // every thread passes the next row's barrier only after its reads below: one buffer is enough
             __syncthreads();
+            // wave w: pixel tile w & 1, the 32-channel tiles (w >> 1), (w >> 1) + 2, ... of each layer
             const int q = 32 * (wave & 1) + p;
-            v16i accn = bn;
+            v4i b[2];
 #pragma unroll
-            for (int kk = 0; kk < 2; kk++) {
-                const v4i b = *reinterpret_cast<const v4i *>(lds + P_OFF + q * 64 + (((2 * kk + half) ^ (q & 3)) << 4)) ^ (int)an.xmask;
-                accn = __builtin_amdgcn_mfma_i32_32x32x32_i8(wn[kk], b, accn, 0, 0, 0);
-            }
-            const v4i o = frag::requant16(an, accn, 0);
-            if (q < POW)
-                *reinterpret_cast<v4i *>(an.y + ((size_t)(n * POH + ph0 + j) * POW + q) * 64 + 32 * (wave >> 1) + 16 * half) = o;
+            for (int kk = 0; kk < 2; kk++) // both layers read the pooled bytes with the same zero point (the host checks)
+                b[kk] = *reinterpret_cast<const v4i *>(lds + P_OFF + q * 64 + (((2 * kk + half) ^ (q & 3)) << 4)) ^ (int)an.xmask;
+            const size_t pixn = (size_t)(n * POH + ph0 + j) * POW + q;
+            // ch0: the layer's first channel among all chained channels; U tiles at a time, so that one tile's LDS reads
+            // and multiplies run under another's requantisation
+            auto tiles = [&](const ConvArgs &al, const int ch0, const int nt0, auto U) {
+                v16i accn[U.value];
+#pragma unroll
+                for (int u = 0; u < U.value; u++) {
+                    const int c = ch0 + 32 * (nt0 + 2 * u);
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const v4i bv = *reinterpret_cast<const v4i *>(lds + B_OFF + (c + 16 * half + 4 * g) * 4);
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            accn[u][4 * g + e] = bv[e];
+                    }
+                }
+#pragma unroll
+                for (int kk = 0; kk < 2; kk++)
+#pragma unroll
+                    for (int u = 0; u < U.value; u++) {
+                        const uint8_t *wp = lds + W_OFF + (ch0 + 32 * (nt0 + 2 * u)) * 64 + lane * 16;
+                        accn[u] = __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const v4i *>(wp + kk * 1024), b[kk], accn[u], 0, 0, 0);
+                    }
+#pragma unroll
+                for (int u = 0; u < U.value; u++) {
+                    const v4i o = frag::requant16(al, accn[u], 0);
+                    if (q < POW)
+                        *reinterpret_cast<v4i *>(al.y + pixn * al.K + 32 * (nt0 + 2 * u) + 16 * half) = o;
+                }
+            };
+            auto layer = [&](const ConvArgs &al, const int ch0) {
+                const int ntl = al.K / 32; // a multiple of 2: the wave's tiles are (wave >> 1) + 2 i, i < ntl / 2
+                int nt = wave >> 1;
+                for (; nt + 2 < ntl; nt += 4)
+                    tiles(al, ch0, nt, std::integral_constant<int, 2>());
+                if (nt < ntl)
+                    tiles(al, ch0, nt, std::integral_constant<int, 1>());
+            };
+            layer(an, 0);
+            if (NEXT == 2)
+                layer(an2, an.K);
         }
     }
 }
@@ -225,34 +270,40 @@ static int stem_rows_per_wg(int N, int POH)
 }
 
 template <int R>
-static void launch_stem_r(const ConvArgs &a, uint8_t *yp, int POH, int POW, const ConvArgs *an, hipStream_t st)
+static void launch_stem_r(const ConvArgs &a, uint8_t *yp, int POH, int POW, const ConvArgs *an, const ConvArgs *an2, hipStream_t st)
 {
     const int ph = stem_rows_per_wg(a.N, POH), nrb = (POH + ph - 1) / ph;
     const dim3 grid(a.N * nrb), block(256);
-    if (an && a.fastq)
-        hipLaunchKernelGGL((conv_stem_maxpool_kernel<R, true, true>), grid, block, 0, st, a, yp, POH, POW, nrb, ph, *an);
+    if (an && an2) // conv_stem_next_applies: the one-multiply requantisation
+        hipLaunchKernelGGL((conv_stem_maxpool_kernel<R, true, 2>), grid, block, 0, st, a, yp, POH, POW, nrb, ph, *an, *an2);
+    else if (an)
+        hipLaunchKernelGGL((conv_stem_maxpool_kernel<R, true, 1>), grid, block, 0, st, a, yp, POH, POW, nrb, ph, *an, *an);
     else if (a.fastq)
-        hipLaunchKernelGGL((conv_stem_maxpool_kernel<R, true, false>), grid, block, 0, st, a, yp, POH, POW, nrb, ph, a);
+        hipLaunchKernelGGL((conv_stem_maxpool_kernel<R, true, 0>), grid, block, 0, st, a, yp, POH, POW, nrb, ph, a, a);
     else
-        hipLaunchKernelGGL((conv_stem_maxpool_kernel<R, false, false>), grid, block, 0, st, a, yp, POH, POW, nrb, ph, a);
+        hipLaunchKernelGGL((conv_stem_maxpool_kernel<R, false, 0>), grid, block, 0, st, a, yp, POH, POW, nrb, ph, a, a);
 }
 
-// the 1x1 convolution that the stem's kernel computes on its pooled rows: 64 -> 64 channels, stride 1, on POH x POW pixels
-bool conv_stem_next_applies(const ConvArgs &a, int POH, int POW, const ConvArgs &an)
+// the 1x1 convolutions that the stem's kernel computes on its pooled rows: from the 64 pooled channels to a multiple of 64
+// channels, stride 1, on POH x POW pixels; an2 may be null; together at most kStemNextCh channels
+bool conv_stem_next_applies(const ConvArgs &a, int POH, int POW, const ConvArgs &an, const ConvArgs *an2)
 {
-    return a.fastq && POW <= 64 && an.R == 1 && an.S == 1 && an.pad_h == 0 && an.pad_w == 0 && an.stride_h == 1 && an.stride_w == 1
-        && an.group == 1 && an.C == 64 && an.in_cs == 64 && an.K == 64 && an.out_cs == 64 && an.nslab == 1 && an.kout_pad >= 64
-        && an.N == a.N && an.H == POH && an.W == POW && an.OH == POH && an.OW == POW && an.bwz == 0 && an.xmask != 0 && an.fastq
-        && an.qmult == nullptr && an.acc_out == nullptr && an.deq_out == nullptr && an.res == nullptr && an.wfrag != nullptr;
+    auto ok = [&](const ConvArgs &l) {
+        return l.R == 1 && l.S == 1 && l.pad_h == 0 && l.pad_w == 0 && l.stride_h == 1 && l.stride_w == 1 && l.group == 1 && l.C == 64
+            && l.in_cs == 64 && l.K >= 64 && l.K % 64 == 0 && l.out_cs == l.K && l.nslab == 1 && l.kout_pad >= l.K && l.N == a.N
+            && l.H == POH && l.W == POW && l.OH == POH && l.OW == POW && l.bwz == 0 && l.xmask == an.xmask && l.xmask != 0 && l.fastq
+            && l.qmult == nullptr && l.acc_out == nullptr && l.deq_out == nullptr && l.res == nullptr && l.wfrag != nullptr;
+    };
+    return a.fastq && POW <= 64 && ok(an) && (!an2 || ok(*an2)) && an.K + (an2 ? an2->K : 0) <= kStemNextCh;
 }
 
-void launch_conv_stem_maxpool(const ConvArgs &a, uint8_t *yp, int POH, int POW, const ConvArgs *an, hipStream_t st)
+void launch_conv_stem_maxpool(const ConvArgs &a, uint8_t *yp, int POH, int POW, const ConvArgs *an, const ConvArgs *an2, hipStream_t st)
 {
     switch (a.R) {
-    case 5: launch_stem_r<5>(a, yp, POH, POW, an, st); break;
-    case 6: launch_stem_r<6>(a, yp, POH, POW, an, st); break;
-    case 7: launch_stem_r<7>(a, yp, POH, POW, an, st); break;
-    default: launch_stem_r<8>(a, yp, POH, POW, an, st); break; // conv_stem_maxpool_applies: 5 <= R <= 8
+    case 5: launch_stem_r<5>(a, yp, POH, POW, an, an2, st); break;
+    case 6: launch_stem_r<6>(a, yp, POH, POW, an, an2, st); break;
+    case 7: launch_stem_r<7>(a, yp, POH, POW, an, an2, st); break;
+    default: launch_stem_r<8>(a, yp, POH, POW, an, an2, st); break; // conv_stem_maxpool_applies: 5 <= R <= 8
     }
 }
 

@@ -72,9 +72,9 @@ _SIGS = {
                                            C.c_int, C.c_int, C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
     "hipq_conv2d_maxpool_fusable": (C.c_int, [C.c_void_p] + [C.c_int] * 5 + [C.c_float, C.c_int, C.c_float, C.c_int, C.c_int]),
     "hipq_conv2d_run_maxpool": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p]),
-    "hipq_conv2d_maxpool_conv_fusable": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p]),
+    "hipq_conv2d_maxpool_conv_fusable": (C.c_int, [C.c_void_p, C.c_int, C.c_int, C.c_void_p, C.c_void_p]),
     "hipq_conv2d_run_maxpool_conv": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_int, C.c_void_p, C.c_int,
-                                               C.c_void_p, C.c_void_p]),
+                                               C.c_void_p, C.c_void_p, C.c_int, C.c_void_p, C.c_void_p]),
     "hipq_ip_reorder_weights": (C.c_int, [C.c_void_p, C.c_void_p] + [C.c_int] * 6),
     "hipq_add_u8": (C.c_int, [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_float, C.c_int, C.c_float,
                               C.c_int, C.c_float, C.c_int, C.c_int, C.c_void_p]),
@@ -279,15 +279,18 @@ class Conv2d:
         check(lib().hipq_conv2d_run_maxpool(self.handle, _ptr(x), _ptr(y), y.shape[1], y.shape[2], int(bool(relu)), _stream()))
         return y
 
-    def maxpool_conv_fusable(self, OH, OW, nxt):
-        """Can that pooling AND the 1x1 convolution `nxt` that reads the pooled tensor run inside this convolution's kernel?"""
-        return bool(lib().hipq_conv2d_maxpool_conv_fusable(self.handle, OH, OW, nxt.handle))
+    def maxpool_conv_fusable(self, OH, OW, nxt, nxt2=None):
+        """Can that pooling AND the 1x1 convolutions `nxt` (and `nxt2`) that read the pooled tensor run inside this
+        convolution's kernel?"""
+        return bool(lib().hipq_conv2d_maxpool_conv_fusable(self.handle, OH, OW, nxt.handle, nxt2.handle if nxt2 else None))
 
-    def run_maxpool_conv(self, x, y, nxt, y_next, relu=False, next_relu=False):
-        """y = maxpool3x3/2/1(conv(x)) and y_next = nxt(y) in one launch (include/hipq.h: hipq_conv2d_run_maxpool_conv)."""
+    def run_maxpool_conv(self, x, y, nxt, y_next, relu=False, next_relu=False, nxt2=None, y_next2=None, next2_relu=False):
+        """y = maxpool3x3/2/1(conv(x)), y_next = nxt(y) and - given - y_next2 = nxt2(y) in one launch (include/hipq.h:
+        hipq_conv2d_run_maxpool_conv)."""
         check(lib().hipq_conv2d_run_maxpool_conv(self.handle, _ptr(x), _ptr(y), y.shape[1], y.shape[2], int(bool(relu)),
-                                                 nxt.handle, int(bool(next_relu)), _ptr(y_next), _stream()))
-        return y, y_next
+                                                 nxt.handle, int(bool(next_relu)), _ptr(y_next), nxt2.handle if nxt2 else None,
+                                                 int(bool(next2_relu)), _ptr(y_next2) if y_next2 is not None else None, _stream()))
+        return y, y_next, y_next2
 
     def close(self):
         if self.handle:

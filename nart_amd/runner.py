@@ -217,30 +217,44 @@ class HipqExecutor:
                 self._add(node, plan.kernel, fn, ip_ops, ip_bytes)
             elif node.kind == "pool" and id(node) in self._pending:
                 plan, xin, nbytes = self._pending.pop(id(node))
-                # the 1x1 convolution that reads the pooled tensor (the first layer of the first block) in the same kernel
-                nxt = None
+                # the 1x1 convolutions that read the pooled tensor (the first layer of the first block, its projection
+                # shortcut) in the same kernel
+                cands = []
                 for nd in case.nodes:
                     na = nd.attrs
                     if (nd.kind == "conv" and nd.inputs[0] == node.output and na["k"] == 1 and na["stride"] == 1
                             and na["pad"] == 0 and na["group"] == 1 and nd.output != case.output.name
-                            and id(nd) not in self.in_block and nd.output not in self.fused):
+                            and id(nd) not in self.in_block and nd.output not in self.fused and len(cands) < 2):
                         p2, nb2 = conv_plan(nd)
-                        if plan.maxpool_conv_fusable(y.shape[2], y.shape[3], p2):
-                            nxt = (nd, p2, nb2)
-                            break
-                        self._early[id(nd)] = p2
-                if nxt is not None:
-                    nd, p2, nb2 = nxt
-                    y2 = self._tensor(T[nd.output])
-                    if y2 is None:
-                        raise RuntimeError("shared executor: %s is fused away in the parent but not here" % nd.output)
-                    self.buf[nd.output] = y2
-                    self.plans.append(p2)
-                    self.chained[node.output] = nd
-                    done.add(id(nd))
-                    fn = (lambda p=plan, i=xin, o=out, p2=p2, y2=y2: p.run_maxpool_conv(i, o, p2, y2))
-                    self.steps.append({"label": node.output, "kind": "conv+pool+conv", "kernel": "conv_mfma_i8_stem+maxpool+conv",
-                                       "fn": fn, "ops": plan.ops + p2.ops, "bytes": nbytes + nb2 - int(np.prod(y.shape)), "plan": plan})
+                        cands.append((nd, p2, nb2))
+                OHp, OWp = y.shape[2], y.shape[3]
+                nxt = []
+                if len(cands) == 2 and plan.maxpool_conv_fusable(OHp, OWp, cands[0][1], cands[1][1]):
+                    nxt = cands
+                else:
+                    for c in cands:
+                        if not nxt and plan.maxpool_conv_fusable(OHp, OWp, c[1]):
+                            nxt = [c]
+                for c in cands:
+                    if not any(c is k for k in nxt):
+                        self._early[id(c[0])] = c[1]
+                if nxt:
+                    ys = []
+                    for nd, p2, nb2 in nxt:
+                        y2 = self._tensor(T[nd.output])
+                        if y2 is None:
+                            raise RuntimeError("shared executor: %s is fused away in the parent but not here" % nd.output)
+                        self.buf[nd.output] = y2
+                        self.plans.append(p2)
+                        done.add(id(nd))
+                        ys.append(y2)
+                    self.chained[node.output] = nxt[0][0]
+                    p2, pb = nxt[0][1], (nxt[1][1] if len(nxt) == 2 else None)
+                    yb = ys[1] if len(nxt) == 2 else None
+                    fn = (lambda p=plan, i=xin, o=out, p2=p2, y2=ys[0], pb=pb, yb=yb: p.run_maxpool_conv(i, o, p2, y2, nxt2=pb, y_next2=yb))
+                    self.steps.append({"label": node.output, "kind": "conv+pool+conv", "kernel": "conv_mfma_i8_stem+maxpool" + "+conv" * len(nxt),
+                                       "fn": fn, "ops": plan.ops + sum(c[1].ops for c in nxt),
+                                       "bytes": nbytes + sum(c[2] - int(np.prod(y.shape)) for c in nxt), "plan": plan})
                     continue
                 fn = (lambda p=plan, i=xin, o=out: p.run_maxpool(i, o))
                 self.steps.append({"label": node.output, "kind": "conv+pool", "kernel": "conv_mfma_i8_stem+maxpool", "fn": fn,

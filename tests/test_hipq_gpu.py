@@ -572,7 +572,7 @@ def test_stem_with_pooling_and_the_next_convolution():
     """hipq_conv2d_run_maxpool_conv: stem convolution, max pooling and the 1x1 convolution (64 -> 64) that reads the pooled
     tensor in one kernel, against the oracle's three operators: pooled rows of 56, 16 and 9 pixels (two, one and a
     ragged pixel tile), a ragged last row block, with and without ReLU on either convolution; the pooled tensor is
-    written as well; plans that do not chain refuse."""
+    written as well; a second chained layer (64 -> 256); plans that do not chain refuse."""
     rng = np.random.default_rng(152)
     #        N  C   H    W   R pad relu relu_next
     cases = [(2, 3, 224, 224, 7, 3, True, True), (3, 3, 64, 64, 7, 3, False, False), (1, 4, 50, 36, 5, 2, True, False),
@@ -615,8 +615,26 @@ def test_stem_with_pooling_and_the_next_convolution():
         assert not plan.maxpool_conv_fusable(POH, POW, other)
         with pytest.raises(hipq.HipqError, match="do not run as one kernel"):
             plan.run_maxpool_conv(hipq.to_device_nhwc(x), yd, other, y2)
-        wide = hipq.Conv2d(pooled.shape, rng.integers(0, 256, (128, 64, 1, 1), dtype=np.uint8), None, 0, 1, 1, *q2)
-        assert not plan.maxpool_conv_fusable(POH, POW, wide)
+        odd = hipq.Conv2d(pooled.shape, rng.integers(0, 256, (96, 64, 1, 1), dtype=np.uint8), None, 0, 1, 1, *q2)
+        assert not plan.maxpool_conv_fusable(POH, POW, odd)
+        # two chained layers: 64 -> 64 and 64 -> 256 (a block's first layer and its projection shortcut)
+        w3 = rng.integers(0, 256, (256, 64, 1, 1), dtype=np.uint8)
+        b3 = rng.integers(-20000, 20000, 256).astype(np.int32)
+        wa3, oz3 = rand_q(rng), int(rng.integers(0, 256))
+        q3 = (oa, ozp, wa3, 128, float(np.float32(oa * wa3 * 8.0 * 60.0)), oz3)
+        want3 = orc.conv2d_u8(pooled, w3, b3, 0, 1, 1, *q3)
+        sc = hipq.Conv2d(pooled.shape, w3, b3, 0, 1, 1, *q3)
+        assert plan.maxpool_conv_fusable(POH, POW, nxt, sc), (plan.kernel, nxt.kernel, sc.kernel)
+        yd.fill_(7), y2.fill_(9)
+        y3 = torch.full((N, POH, POW, 256), 11, dtype=torch.uint8, device="cuda")
+        plan.run_maxpool_conv(hipq.to_device_nhwc(x), yd, nxt, y2, nxt2=sc, y_next2=y3)
+        torch.cuda.synchronize()
+        assert np.array_equal(yd.cpu().numpy().transpose(0, 3, 1, 2), pooled), (N, C, H, W, "pooled tensor, two layers")
+        assert np.array_equal(y2.cpu().numpy().transpose(0, 3, 1, 2), want2), (N, C, H, W, "first chained layer of two")
+        got3 = y3.cpu().numpy().transpose(0, 3, 1, 2)
+        assert np.array_equal(got3, want3), (N, C, H, W, int((got3 != want3).sum()), np.argwhere(got3 != want3)[:6].tolist())
+        big = hipq.Conv2d(pooled.shape, rng.integers(0, 256, (320, 64, 1, 1), dtype=np.uint8), None, 0, 1, 1, *q3)
+        assert plan.maxpool_conv_fusable(POH, POW, big) and not plan.maxpool_conv_fusable(POH, POW, nxt, big)  # 384 channels
 
 
 def test_elementwise():
