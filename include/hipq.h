@@ -35,8 +35,10 @@ extern "C" {
 #endif
 
 /* 3: per-channel weight scales, the fused stem (convolution + max pooling), the streaming and channel-widening kernels'
- * hooks, hipq_conv2d_plan_kernel_add.  Every entry point of version 2 is unchanged. */
-#define HIPQ_ABI_VERSION 3
+ * hooks, hipq_conv2d_plan_kernel_add.
+ * 4: whole residual blocks in one launch (hipq_bottleneck_*, hipq_conv2d_run_add2, hipq_conv2d_run_maxpool_conv),
+ * hipq_dequantize_i32; the machine probes (hipq_probe_launch) are gone.  Every other entry point of version 3 is unchanged. */
+#define HIPQ_ABI_VERSION 4
 
 #define HIPQ_ELTWISE_SUM 1 /* SETTING_ELTWISE_OP_SUM */
 #define HIPQ_ELTWISE_MAX 2 /* SETTING_ELTWISE_OP_MAX */

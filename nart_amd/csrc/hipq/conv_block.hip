@@ -20,10 +20,10 @@
 //     the reference's arithmetic and stores the sum.
 // Weights never pass through LDS: the waves of a work-group split the OUTPUT CHANNELS, so no two waves want the same
 // weight bytes, and a wave loads its MFMA weight operands straight from global memory (L2) into registers, a ring of
-// slabs ahead of its multiplies; LDS bandwidth is left to the pixel operands.  The work-group has 2 waves per 64
-// middle channels: the pair shares a 64-channel x all-pixel tile of layers 1 and 2 and splits the REDUCTION (every other
-// 64-byte slab of k), so that two waves per SIMD overlap each other's loads, LDS reads and multiplies without reading
-// any pixel operand twice; the partial sums meet once per layer in LDS, each wave keeping 32 of the 64 channels.  In
+// slabs ahead of its multiplies; LDS bandwidth is left to the pixel operands.  The work-group has one wave per 32 middle
+// channels: in layers 1 and 2 a wave owns a 32-channel tile for all pixels and the whole reduction, so the waves
+// exchange nothing (splitting the reduction between two waves instead read every pixel operand once, not twice, but the
+// exchange of partial sums through LDS and its barriers cost more than the reads: 28 -> 25.6 us per block at 14x14).  In
 // layer 3 every wave owns 128 output channels, keeps its pixel operands for the whole reduction in registers and works
 // through 4 chunks of 32 channels: multiplies of one wave run under the other's vector arithmetic of the add.
 // MFMA rows are permuted (row i computes channel 16 ((i >> 2) & 1) + 4 (i >> 3) + (i & 3) of its 32) so that a lane's 16
@@ -35,7 +35,6 @@
 #include "conv_frag.h"
 
 #include <algorithm>
-#include <cstdlib>
 
 namespace hipq {
 
@@ -50,19 +49,7 @@ constexpr int kGridRows = 96;      // rows held for that grid (81 positions; the
 struct BlockGeom {
     int H, W, PY, PX, npatch;
     int IH, IW; // the tail kernel's input image where its 3x3 layer has stride 2 (H, W: the output image)
-#ifdef HIPQ_BLOCK_STAMPS
-    unsigned long long *stamps;
-#endif
 };
-#ifdef HIPQ_BLOCK_STAMPS
-#define STAMP(k)                                                                                   \
-    do {                                                                                           \
-        if (geo.stamps && lane == 0)                                                               \
-            geo.stamps[((size_t)gid * 8 + wave) * 16 + (k)] = __builtin_readcyclecounter();         \
-    } while (0)
-#else
-#define STAMP(k)
-#endif
 
 } // namespace
 
@@ -88,7 +75,6 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
     const int gid = (int)(blockIdx.x % 8) * (int)(gridDim.x / 8) + (int)(blockIdx.x / 8);
     if (gid >= geo.npatch)
         return;
-    STAMP(0);
     const int ppi = geo.PY * geo.PX;
     const int n = gid / ppi, pr = gid - n * ppi, pi = pr / geo.PX, pj = pr - pi * geo.PX;
     const int y0 = pi * kPatch, x0 = pj * kPatch;
@@ -154,9 +140,7 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
     wait_vmcnt<0>();
     __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
-    STAMP(1);
     reduce_all<4 * G, MT1, D1>(acc1, r1, (int)a1.xmask, ldw1, ldb1);
-    STAMP(2);
     // layer 2's first weights and folded biases travel while layer 1 is finished
     WeightRing1<D2> r2;
     ring_fill1<9 * G, D2>(r2, ldw2);
@@ -164,7 +148,6 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
 #pragma unroll
     for (int t = 0; t < 2; t++)
         init_acc(acc2[t], a2.bias2 + ct0 + 16 * h, false);
-    STAMP(3);
     // channels ct0 + 16 h .. + 15 of region pixel j -> the grid position of that pixel
 #pragma unroll
     for (int t = 0; t < MT1; t++) {
@@ -178,11 +161,9 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
     }
     __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
-    STAMP(4);
 
     // ================= layer 2: 3x3, CM -> CM, output index m = 9 * row + column =================
     reduce_all<9 * G, 2, D2>(acc2, r2, 0, ldw2, ldb2);
-    STAMP(5);
     // layer 3: this wave's 128 output channels in 4 chunks of 32; the first chunk's weights and biases travel now
     const uint8_t *w3 = a3.wfrag + (size_t)(128 * wave) * 64 + lane * 16;
     v4i wf[2 * G], b3[4];
@@ -200,7 +181,6 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
     for (int t = 0; t < 2; t++)
         o2[t] = requant16(a2, acc2[t], a3.xmask);
     __builtin_amdgcn_s_barrier(); // every wave is done reading the grid: layer 2's bytes go there, row m
-    STAMP(6);
 #pragma unroll
     for (int t = 0; t < 2; t++) {
         const int m = 32 * t + p;
@@ -209,7 +189,6 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
     }
     __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
-    STAMP(7);
 
     // ================= layer 3: CM -> CW and the residual add =================
     {
@@ -230,7 +209,6 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
             pixo[t] = (n * geo.H + y0 + py) * geo.W + x0 + px;
             yoff[t] = (size_t)pixo[t] * CW;
         }
-        STAMP(8);
         for (int cc = 0; cc < 4; cc++) {
             const int ch = 128 * wave + 32 * cc; // first of the chunk's 32 channels
             v16i acc[2];
@@ -264,7 +242,6 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
                     *reinterpret_cast<v4i *>(lds + m * CW + (c16 & ~15) * 16 + (((c16 & 15) ^ (m & 15)) << 4)) = o;
                 }
             }
-            STAMP(9 + cc);
         }
         if (!NX)
             return;
@@ -312,7 +289,7 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
 //   * CHAIN: the next layer (CW -> CM, or CW -> 2 CM where the next stage begins) reads that tile as its pixel operand.
 // ST: the 3x3 layer's stride (1, or 2 - the first block of a stage: the grid then holds (2 PH + 1) x (2 PW + 1) input pixels).
 template <int G, int PH, int PW, int NX, int ST>
-__global__ __launch_bounds__(128 * G, (G == 1 ? 4 : G == 2 ? 3 : 2)) void conv_bottleneck_tail_kernel(const ConvArgs a2, const ConvArgs a3, const ConvArgs an,
+__global__ __launch_bounds__(128 * G, (G == 1 ? (NX ? 4 : 3) : G == 2 ? 3 : 2)) void conv_bottleneck_tail_kernel(const ConvArgs a2, const ConvArgs a3, const ConvArgs an,
                                                                          const BlockGeom geo)
 {
     constexpr int NW = 2 * G, NT = 128 * G, CM = 64 * G, CW = 256 * G;
@@ -334,7 +311,6 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? 4 : G == 2 ? 3 : 2)) void conv_b
     const int ppi = geo.PY * geo.PX;
     const int n = gid / ppi, pr = gid - n * ppi, pi = pr / geo.PX, pj = pr - pi * geo.PX;
     const int y0 = pi * PH, x0 = pj * PW;
-    STAMP(0);
 
     // ---- the 3x3 layer's input patch with its border -> LDS, re-centred; out-of-image positions read the pad source ----
     {
@@ -383,9 +359,7 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? 4 : G == 2 ? 3 : 2)) void conv_b
         init_acc(acc2[t], a2.bias2 + ct0 + 16 * h, false);
     __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): this thread's part of the grid is written
     __builtin_amdgcn_s_barrier();
-    STAMP(1);
     reduce_all<9 * G, 2, D2>(acc2, r2, 0, ldw2, ldb2);
-    STAMP(2);
     // layer 3: this wave's 128 output channels in 4 chunks of 32; the first chunk's weights, biases and residual travel now
     const uint8_t *w3 = a3.wfrag + (size_t)(128 * wave) * 64 + lane * 16;
     v4i wf[2 * G], b3[4], rn[2];
@@ -401,7 +375,6 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? 4 : G == 2 ? 3 : 2)) void conv_b
             rn[t] = ldg128(a3.res + pix[t] * CW + 128 * wave + 32 * cc + 16 * h);
     };
     load_chunk(0);
-    STAMP(3);
 #pragma unroll
     for (int t = 0; t < 2; t++) {
         const int q = 32 * t + p;
@@ -411,7 +384,6 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? 4 : G == 2 ? 3 : 2)) void conv_b
     __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
 
-    STAMP(4);
     // ================= layer 3: CM -> CW and the residual add =================
     {
         v4i bf[2][2 * G];
@@ -453,7 +425,6 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? 4 : G == 2 ? 3 : 2)) void conv_b
                     *reinterpret_cast<v4i *>(lds + S_OFF + q * CW + (c16 & ~15) * 16 + (((c16 & 15) ^ (q & 15)) << 4)) = o;
                 }
             }
-            STAMP(5 + cc);
         }
     }
     if (!CHAIN)
@@ -480,16 +451,13 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? 4 : G == 2 ? 3 : 2)) void conv_b
             __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): this wave's part of the sum tile is written
             __builtin_amdgcn_s_barrier();
         }
-        STAMP(9);
         reduce_all<4 * G, 2, DN>(accn, rr, (int)an.xmask, ldwn, ldbn);
-        STAMP(10);
 #pragma unroll
         for (int t = 0; t < 2; t++) {
             const v4i o = requant16(an, accn[t], 0);
             if (valid[t])
                 *reinterpret_cast<v4i *>(an.y + pix[t] * (NX * CM) + cn + 16 * h) = o;
         }
-        STAMP(12);
     }
 }
 
@@ -541,9 +509,6 @@ static void launch_tail_gp(const ConvArgs &a2, const ConvArgs &a3, const ConvArg
     geo.H = a2.OH, geo.W = a2.OW, geo.PY = a2.OH / PH, geo.PX = a2.OW / PW;
     geo.IH = a2.H, geo.IW = a2.W;
     geo.npatch = a2.N * geo.PY * geo.PX;
-#ifdef HIPQ_BLOCK_STAMPS
-    geo.stamps = getenv("HIPQ_BLOCK_STAMPS") ? (unsigned long long *)strtoull(getenv("HIPQ_BLOCK_STAMPS"), nullptr, 0) : nullptr;
-#endif
     const dim3 grid((unsigned)((geo.npatch + 7) / 8 * 8)), block(128 * G);
     if (an && an->K == 2 * a2.in_cs)
         hipLaunchKernelGGL((conv_bottleneck_tail_kernel<G, PH, PW, 2, ST>), grid, block, 0, st, a2, a3, *an, geo);
@@ -615,9 +580,6 @@ static void launch_block_g(const ConvArgs &a1, const ConvArgs &a2, const ConvArg
     BlockGeom geo;
     geo.H = a1.H, geo.W = a1.W, geo.PY = a1.H / kPatch, geo.PX = a1.W / kPatch;
     geo.npatch = a1.N * geo.PY * geo.PX;
-#ifdef HIPQ_BLOCK_STAMPS
-    geo.stamps = getenv("HIPQ_BLOCK_STAMPS") ? (unsigned long long *)strtoull(getenv("HIPQ_BLOCK_STAMPS"), nullptr, 0) : nullptr;
-#endif
     const dim3 grid((unsigned)((geo.npatch + 7) / 8 * 8)), block(128 * G);
     const bool small = geo.PY <= 2 && geo.PX <= 2; // every region is at most 8 x 8 pixels
     if (small && an)

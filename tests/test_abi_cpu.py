@@ -24,7 +24,7 @@ def test_hipq_exports_every_declared_symbol():
     assert declared == set(hipq.EXPORTS), declared ^ set(hipq.EXPORTS)
     for name in declared:
         assert getattr(L, name) is not None
-    assert L.hipq_abi_version() == 3
+    assert L.hipq_abi_version() == 4
 
 
 def test_quant_scale_matches_oracle():
