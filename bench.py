@@ -38,9 +38,9 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s (published)
 # file that holds the counter readings and a digest of the kernel sources it was taken with: the line reports it only
 # for the default workload with default flags and only while the sources under nart_amd/csrc/hipq still have that digest
 # (traffic is null, with the reason, once a kernel has changed and the profile has not been taken again).
-TRAFFIC_FROM_PROFILE = {"workload": "resnet50", "batch": 64, "bytes_per_launch": 34.85e6,
+TRAFFIC_FROM_PROFILE = {"workload": "resnet50", "batch": 64, "bytes_per_launch": 56.91e6,
                         "source": "profiles/conv_mfma_i8_resnet50_n64.md",
-                        "sources_sha256": "stale"}
+                        "sources_sha256": "b06ad3f0772c8196"}
 
 
 def kernel_sources_digest():
@@ -441,7 +441,8 @@ def main():
            "scaling": "weak", "vs_baseline": None, "dtype": "u8", "data": "synthetic",
            "config": {"workload": case.name, "batch": args.batch, "input": list(case.input.shape),
                       "operators": len(case.nodes), "graph_replay": not args.no_graph, "passes_per_graph": inner,
-                      "tuned": bool(args.tune), "fused_residual_adds": len(ex.fused),
+                      "tuned": bool(args.tune), "fused_residual_adds": len(ex.fused), "whole_blocks": len(ex.blocks),
+                      "block_tails": len(ex.tails), "dual_shortcut_adds": len(ex.duals), "launches_per_step": len(ex.steps),
                       "conv_fc_gop_per_step": round(case.conv_ops() / 1e9, 2)},
            "conv_tops_whole_step": round(case.conv_ops() / (ms * 1e-3) / 1e12, 2),
            "roofline": roof, "kernel_families": families}
