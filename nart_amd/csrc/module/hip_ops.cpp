@@ -273,8 +273,22 @@ bool conv_continues_block(op_t *op, const op_t *r)
     if (in->pending == conv_launch_plain && reinterpret_cast<const conv_op_t *>(static_cast<op_t *>(in->pending_ctx))->blk_next == op)
         return true;
     const QSet &qi = add_inputs(a), &qo = add_output(a);
-    return hipq_bottleneck_tail_fusable(c2->plan, c3->plan, i == 1, qi.alpha[1 - i], qi.zp[1 - i], qo.alpha[0], qo.zp[0], qo.bits[0],
-                                        nullptr) != 0;
+    if (hipq_bottleneck_tail_fusable(c2->plan, c3->plan, i == 1, qi.alpha[1 - i], qi.zp[1 - i], qo.alpha[0], qo.zp[0], qo.bits[0], nullptr))
+        return true;
+    // a form that pays only when the 1x1 convolution that reads the sum rides along (add_defers will hand the launch on to it)
+    const reader_map &rm = readers_of(op);
+    const auto it = rm.find(a->output_tensors[0].mem);
+    if (it != rm.end())
+        for (const op_t *rn : it->second) {
+            if (rn->workspace != op->workspace || rn->entry->tp != &op_conv_2d_tp || rn->input_tensors[0]->mem != a->output_tensors[0].mem)
+                continue;
+            const conv_op_t *cn = reinterpret_cast<const conv_op_t *>(rn);
+            if (cn->plan != nullptr
+                && hipq_bottleneck_tail_fusable(c2->plan, c3->plan, i == 1, qi.alpha[1 - i], qi.zp[1 - i], qo.alpha[0], qo.zp[0], qo.bits[0],
+                                                cn->plan))
+                return true;
+        }
+    return false;
 }
 
 // 1: the only reader of the convolution's output is an add or a relu of this workspace that can take over the launch
