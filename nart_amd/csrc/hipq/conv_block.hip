@@ -418,7 +418,7 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? (NX ? 4 : 3) : G == 2 ? 3 : 2)) 
 #pragma unroll
             for (int t = 0; t < 2; t++) {
                 const v4i o = requant_add16(a3, acc[t], rc[t]);
-                if (valid[t])
+                if (!CHAIN && valid[t]) // 16 bytes of each of 32 pixels per instruction; the chained form stores whole rows below
                     *reinterpret_cast<v4i *>(a3.y + pix[t] * CW + ch + 16 * h) = o;
                 if (CHAIN) { // the sum tile: pixel row q, 16-byte piece c at piece c ^ (q & 15) of every 256 bytes
                     const int q = 32 * t + p, c16 = (ch >> 4) + h;
@@ -450,6 +450,19 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? (NX ? 4 : 3) : G == 2 ? 3 : 2)) 
         if (jx == 0) {
             __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0): this wave's part of the sum tile is written
             __builtin_amdgcn_s_barrier();
+            // The sum leaves from the tile as whole pixel rows: a wave instruction writes 1 KB of consecutive bytes, where a
+            // store per chunk writes 32 bytes of each of 32 rows.  Lines written in pieces cost the kernel that reads the sum
+            // dearly (the ResNet-50 pass: 0.724 -> 0.698 ms); the stores drain under the multiplies below.  (The same in the
+            // whole-block kernel and in the unchained form, where nothing follows to hide the drain, measured 1 % slower.)
+            constexpr int PPR = CW / 16; // 16-byte pieces per pixel row
+#pragma unroll
+            for (int k = 0; k < 64 * PPR / NT; k++) {
+                const int item = tid + k * NT, q = item / PPR, c16 = item % PPR;
+                const int py = q / PW, px = q - py * PW;
+                const v4i o = *reinterpret_cast<const v4i *>(lds + S_OFF + q * CW + (c16 & ~15) * 16 + (((c16 & 15) ^ (q & 15)) << 4));
+                if (q < NPIX)
+                    *reinterpret_cast<v4i *>(a3.y + (size_t)((n * geo.H + y0 + py) * geo.W + x0 + px) * CW + c16 * 16) = o;
+            }
         }
         reduce_all<4 * G, 2, DN>(accn, rr, (int)an.xmask, ldwn, ldbn);
 #pragma unroll
