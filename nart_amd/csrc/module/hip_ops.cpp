@@ -541,22 +541,29 @@ bool block_launch(op_t *op, op_t *cop, int i, void *y, op_t *nxt, int relu, void
     conv_op_t *c3 = reinterpret_cast<conv_op_t *>(cop), *c2 = reinterpret_cast<conv_op_t *>(cop2);
     const int o = 1 - i;
     hip_mem_t *m1 = as_hip(cop2->input_tensors[0]->mem);
-    if (nxt == nullptr && m1->pending == conv_launch_plain) {
+    const conv_op_t *cn = reinterpret_cast<const conv_op_t *>(nxt);
+    if (m1->pending == conv_launch_plain) {
         op_t *cop1 = static_cast<op_t *>(m1->pending_ctx);
         conv_op_t *c1 = reinterpret_cast<conv_op_t *>(cop1);
         if (cop1->entry->tp == &op_conv_2d_tp && c1->blk_next == cop2 && c1->blk_add == op
             && op->input_tensors[o]->mem == cop1->input_tensors[0]->mem && e->qi.alpha[o] == c1->desc.ialpha && e->qi.zp[o] == c1->desc.izp
-            && hipq_bottleneck_fusable(c1->plan, c2->plan, c3->plan, o == 0, e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0])) {
+            && (nxt ? hipq_bottleneck_conv_fusable(c1->plan, c2->plan, c3->plan, o == 0, e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0], cn->plan)
+                    : hipq_bottleneck_fusable(c1->plan, c2->plan, c3->plan, o == 0, e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0]))) {
             const void *x = in_ptr(cop1, 0);
-            if (x != y && hipq_bottleneck_run(c1->plan, c2->plan, c3->plan, x, o == 0, e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0], y,
-                                              op_stream(op)) == 0) {
+            if (x != y
+                && (nxt ? hipq_bottleneck_run_conv(c1->plan, c2->plan, c3->plan, x, o == 0, e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0], y,
+                                                   cn->plan, relu, y_next, op_stream(op))
+                        : hipq_bottleneck_run(c1->plan, c2->plan, c3->plan, x, o == 0, e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0], y,
+                                              op_stream(op)))
+                       == 0) {
                 ++g_fused_adds;
                 ++g_fused_blocks;
+                if (nxt)
+                    ++g_chained_convs;
                 return true; // the three convolutions' outputs stay unwritten; their hooks stay for whoever asks
             }
         }
     }
-    const conv_op_t *cn = reinterpret_cast<const conv_op_t *>(nxt);
     if (!hipq_bottleneck_tail_fusable(c2->plan, c3->plan, o == 0, e->qi.alpha[o], e->qi.zp[o], e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0],
                                       nxt ? cn->plan : nullptr))
         return false;
@@ -621,6 +628,22 @@ void add_launch_deferred(void *ctx)
         add_plain_into(op, y);
 }
 
+// the add `op` closes a whole block (head -> mid -> c -> add with the head's input) that hipq_bottleneck_run_conv computes
+// together with the 1x1 convolution rc that reads the sum
+static bool whole_block_chains(op_t *op, op_t *mid, const conv_op_t *c, int o, const conv_op_t *rc)
+{
+    ew_op_t *e = reinterpret_cast<ew_op_t *>(op);
+    hip_mem_t *m1 = as_hip(mid->input_tensors[0]->mem);
+    if (m1->pending != conv_launch_plain)
+        return false;
+    op_t *cop1 = static_cast<op_t *>(m1->pending_ctx);
+    const conv_op_t *c1 = reinterpret_cast<const conv_op_t *>(cop1);
+    return cop1->entry->tp == &op_conv_2d_tp && c1->blk_next == mid && c1->blk_add == op
+        && op->input_tensors[o]->mem == cop1->input_tensors[0]->mem && e->qi.alpha[o] == c1->desc.ialpha && e->qi.zp[o] == c1->desc.izp
+        && hipq_bottleneck_conv_fusable(c1->plan, reinterpret_cast<conv_op_t *>(mid)->plan, c->plan, o == 0, e->qo.alpha[0], e->qo.zp[0],
+                                        e->qo.bits[0], rc->plan);
+}
+
 // Does the add leave its launch to a reader?  Decided once per prepare: a convolution was deferred into this add, and a
 // 1x1 convolution of this workspace reads the sum and can run as the tail of the same kernel.
 bool add_defers(op_t *op)
@@ -646,8 +669,9 @@ bool add_defers(op_t *op)
                     && (hipq_conv2d_add_conv_fusable(c->plan, o == 0, e->qi.alpha[o], e->qi.zp[o], e->qo.alpha[0], e->qo.zp[0],
                                                      e->qo.bits[0], rc->plan)
                         || (mid != nullptr
-                            && hipq_bottleneck_tail_fusable(reinterpret_cast<conv_op_t *>(mid)->plan, c->plan, o == 0, e->qi.alpha[o],
-                                                            e->qi.zp[o], e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0], rc->plan)))) {
+                            && (hipq_bottleneck_tail_fusable(reinterpret_cast<conv_op_t *>(mid)->plan, c->plan, o == 0, e->qi.alpha[o],
+                                                             e->qi.zp[o], e->qo.alpha[0], e->qo.zp[0], e->qo.bits[0], rc->plan)
+                                || whole_block_chains(op, mid, c, o, rc))))) {
                     e->defer = 1;
                     break;
                 }

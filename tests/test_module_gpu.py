@@ -358,6 +358,58 @@ def test_whole_bottleneck_block_runs_as_one_kernel(own_rt):
     ws.delete()
 
 
+def test_whole_block_and_the_next_stage_first_layer_run_as_one_kernel(own_rt):
+    """The same block followed by conv_2d (1024 -> 512, 1x1) that reads the sum: the add leaves its launch to that
+    convolution, whose run() launches hipq_bottleneck_run_conv for all five operators; the sum is written as well.  A host
+    that reads the sum before that convolution has run gets the block's four operators as one launch and the
+    convolution as its own."""
+    import ctypes as C
+    from oracle import orc
+    blocks = own_rt.libs[1].hip_module_fused_blocks
+    blocks.restype = C.c_long
+    chained = own_rt.libs[1].hip_module_chained_convs
+    chained.restype = C.c_long
+    ws = own_rt.workspace("hip")
+    rng = np.random.default_rng(33)
+    x = rng.integers(0, 256, (2, 1024, 14, 14), dtype=np.uint8)
+    shapes = ((256, 1024, 1), (256, 256, 3), (1024, 256, 1))
+    ws_w = [rng.integers(1, 256, (K, Cc, k, k), dtype=np.uint8) for K, Cc, k in shapes]
+    bs = [rng.integers(-20000, 20000, K).astype(np.int32) for K, _, _ in shapes]
+    qs = [dict(ialpha=0.05, izp=9, walpha=0.0011, wzp=128, oalpha=0.06, ozp=0),
+          dict(ialpha=0.06, izp=0, walpha=0.0016, wzp=128, oalpha=0.055, ozp=0),
+          dict(ialpha=0.055, izp=0, walpha=0.0035, wzp=128, oalpha=0.07, ozp=121)]
+    wn, bn = rng.integers(1, 256, (512, 1024, 1, 1), dtype=np.uint8), rng.integers(-20000, 20000, 512).astype(np.int32)
+    qn = dict(ialpha=0.09, izp=0, walpha=0.0011, wzp=128, oalpha=0.08, ozp=0)
+    t = x
+    for w, b, q, (K, Cc, k) in zip(ws_w, bs, qs, shapes):
+        t = orc.conv2d_u8(t, w, b, k // 2, 1, 1, q["ialpha"], q["izp"], q["walpha"], 128, q["oalpha"], q["ozp"])
+    want = orc.add_u8(t, x, 0.07, 121, 0.05, 9, 0.09, 0)
+    wantn = orc.conv2d_u8(want, wn, bn, 0, 1, 1, 0.09, 0, 0.0011, 128, 0.08, 0)
+    assert len(np.unique(wantn)) > 32
+    for peek, expect_chain in ((False, 1), (True, 0)):
+        tx = ws.tensor(x)
+        convs, cur = [], tx
+        for w, b, q, (K, Cc, k) in zip(ws_w, bs, qs, shapes):
+            convs.append(ws.conv2d(cur, ws.tensor(w), ws.tensor(b), k // 2, 1, 1, q).prepare())
+            cur = convs[-1].output(0)
+        add = ws.add(cur, tx, dict(ialpha=[0.07, 0.05], izp=[121, 9], oalpha=0.09, ozp=0)).prepare()
+        nxt = ws.conv2d(add.output(0), ws.tensor(wn), ws.tensor(bn), 0, 1, 1, qn).prepare()
+        for rep in range(2):
+            b0, c0 = blocks(), chained()
+            for c in convs:
+                c.run()
+            add.run()
+            if peek:
+                assert same_bits(add.output(0).numpy(), want), (peek, rep)
+            nxt.run()
+            assert same_bits(nxt.output(0).numpy(), wantn), (peek, rep)
+            assert same_bits(add.output(0).numpy(), want), (peek, rep)
+            assert blocks() == b0 + 1 and chained() == c0 + expect_chain, (peek, rep, blocks() - b0, chained() - c0)
+        for o in [nxt, add] + convs[::-1]:
+            o.delete()
+    ws.delete()
+
+
 def test_block_tail_and_next_convolution_run_as_one_kernel(own_rt):
     """conv_2d (3x3, 128 -> 128) -> conv_2d (128 -> 512, 1x1) -> add with any residual -> conv_2d (512 -> 128, 1x1): the 3x3
     and the widening convolution leave their launches to the add, the add leaves its own to the convolution that reads
