@@ -91,29 +91,43 @@ __device__ static inline uint32_t add_one_generic(uint32_t x0, uint32_t x1, cons
     return (uint32_t)sat_hi((int32_t)(rshift_rn(t, p.sh) + p.oz), p.hi);
 }
 
-template <bool FAST>
-__device__ static inline uint32_t add_dword(uint32_t a, uint32_t b, const AddParams &p)
+// (v >> s) saturated to [0, 255] for four values, packed into one dword (v0 in the low byte); s is wave-uniform, 0..31.
+// gfx950's v_ashr_pk_u8_i32 shifts two values, saturates them and writes ONE half of its destination - op_sel[3] picks
+// the high half - leaving the other half as it was.  It issues at half rate (measured), so the pair costs four issue
+// slots against the nine of four shifts, two 16-bit packs, two saturating byte packs and a permute.
+__device__ static __forceinline__ uint32_t ashr_sat_u8x4(int32_t v0, int32_t v1, int32_t v2, int32_t v3, int32_t s)
 {
-    uint32_t o = 0;
-#pragma unroll
-    for (int e = 0; e < 4; e++) {
-        const uint32_t x0 = (a >> (8 * e)) & 255, x1 = (b >> (8 * e)) & 255;
-        uint32_t r;
-        if (FAST) {
-            // operands fit 24 bits: v_mad_i32_i24 is a full-rate instruction
-            const int32_t t0 = __mul24((int)x0, (int)p.m0) + p.c0, t1 = __mul24((int)x1, (int)p.m1) + p.c1;
-            const int32_t v = (((t0 >> p.s0) + (t1 >> p.s1)) + p.cadd) >> p.sh;
-            r = (uint32_t)(v > p.hi ? p.hi : (v < 0 ? 0 : v));
-        } else {
-            r = add_one_generic(x0, x1, p);
-        }
-        o |= r << (8 * e);
-    }
+    uint32_t o;
+    asm("v_ashr_pk_u8_i32 %0, %1, %2, %3" : "=v"(o) : "v"(v0), "v"(v1), "s"(s));
+    asm("v_ashr_pk_u8_i32 %0, %1, %2, %3 op_sel:[0,0,0,1]" : "+v"(o) : "v"(v2), "v"(v3), "s"(s));
     return o;
 }
 
 template <bool FAST>
-__device__ static inline u32x4 add_16(u32x4 a, u32x4 b, const AddParams &p)
+__device__ static __forceinline__ uint32_t add_dword(uint32_t a, uint32_t b, const AddParams &p)
+{
+    if (FAST) {
+        // operands fit 24 bits: v_mad_i32_i24 is a full-rate instruction.  The upper clamp moves in front of the last
+        // shift ((hi + 1) * 2^sh - 1 is the largest value that shifts to hi; sh <= 22), the lower one is the pack's.
+        const int32_t phi = ((p.hi + 1) << p.sh) - 1;
+        int32_t v[4];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const uint32_t x0 = (a >> (8 * e)) & 255, x1 = (b >> (8 * e)) & 255;
+            const int32_t t0 = __mul24((int)x0, (int)p.m0) + p.c0, t1 = __mul24((int)x1, (int)p.m1) + p.c1;
+            v[e] = min(((t0 >> p.s0) + (t1 >> p.s1)) + p.cadd, phi);
+        }
+        return ashr_sat_u8x4(v[0], v[1], v[2], v[3], p.sh);
+    }
+    uint32_t o = 0;
+#pragma unroll
+    for (int e = 0; e < 4; e++)
+        o |= add_one_generic((a >> (8 * e)) & 255, (b >> (8 * e)) & 255, p) << (8 * e);
+    return o;
+}
+
+template <bool FAST>
+__device__ static __forceinline__ u32x4 add_16(u32x4 a, u32x4 b, const AddParams &p)
 {
     u32x4 y;
 #pragma unroll

@@ -995,16 +995,7 @@ __device__ static inline void pointwise_strips(const ConvArgs &a, const uint8_t 
 #pragma unroll
             for (int g = 0; g < 4; g++) {
                 if (PLAIN_SAT) {
-                    int32_t r[4];
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        r[e] = (__mulhi(acc[g * 4 + e], (int)a.q.mult) + a.qadd) >> a.qt;
-                    uint32_t p01, p23, b01, b23;
-                    asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p01) : "v"(r[0]), "v"(r[1]));
-                    asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(r[2]), "v"(r[3]));
-                    asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
-                    asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
-                    cv[g] = __builtin_amdgcn_perm(b23, b01, 0x05040100u); // the low halves of both, one instruction
+                    cv[g] = conv_requant4<true>(a, acc[g * 4], acc[g * 4 + 1], acc[g * 4 + 2], acc[g * 4 + 3]);
                 } else {
                     int32_t rq[4];
 #pragma unroll
@@ -1385,16 +1376,7 @@ __device__ static inline void depthwise3x3_body(const ConvArgs &a, int idx, int 
             }
             uint32_t packed = 0;
             if (QMODE == 2) {
-                int32_t r[4];
-#pragma unroll
-                for (int c = 0; c < 4; c++)
-                    r[c] = (__mulhi(v[c], (int)a.q.mult) + a.qadd) >> a.qt;
-                uint32_t p01, p23, b01, b23;
-                asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p01) : "v"(r[0]), "v"(r[1]));
-                asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(r[2]), "v"(r[3]));
-                asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
-                asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
-                packed = __builtin_amdgcn_perm(b23, b01, 0x05040100u); // low halves of both
+                packed = conv_requant4<true>(a, v[0], v[1], v[2], v[3]);
             } else {
 #pragma unroll
                 for (int c = 0; c < 4; c++)

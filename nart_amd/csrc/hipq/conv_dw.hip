@@ -73,16 +73,7 @@ __device__ static inline void emit_row(const ConvArgs &a, const int32_t (&acc)[4
             *reinterpret_cast<v4i *>(a.acc_out + off) = v4i{acc[o][0], acc[o][1], acc[o][2], acc[o][3]};
         uint32_t packed = 0;
         if (QMODE == 2) {
-            int32_t r[4];
-#pragma unroll
-            for (int c = 0; c < 4; c++)
-                r[c] = (__mulhi(acc[o][c], (int)a.q.mult) + a.qadd) >> a.qt;
-            uint32_t p01, p23, b01, b23;
-            asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p01) : "v"(r[0]), "v"(r[1]));
-            asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(r[2]), "v"(r[3]));
-            asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
-            asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
-            packed = __builtin_amdgcn_perm(b23, b01, 0x05040100u); // the low halves of both
+            packed = conv_requant4<true>(a, acc[o][0], acc[o][1], acc[o][2], acc[o][3]);
         } else {
             int32_t r[4];
 #pragma unroll

@@ -54,16 +54,7 @@ __device__ inline void plain_to_staging(const ConvArgs &a, const v16i (&acc)[TN]
             uint32_t packed;
             if (PLAIN_SAT) {
                 // clamp range exactly [0, 255]: two saturating packs replace four clamps and the shifts
-                int32_t r[4];
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    r[e] = (__mulhi(acc[tn][g * 4 + e], (int)a.q.mult) + a.qadd) >> a.qt;
-                uint32_t p01, p23, b01, b23;
-                asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p01) : "v"(r[0]), "v"(r[1]));
-                asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(r[2]), "v"(r[3]));
-                asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
-                asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
-                packed = __builtin_amdgcn_perm(b23, b01, 0x05040100u); // the low halves of both, one instruction
+                packed = conv_requant4<true>(a, acc[tn][g * 4], acc[tn][g * 4 + 1], acc[tn][g * 4 + 2], acc[tn][g * 4 + 3]);
             } else {
                 int32_t rq[4];
 #pragma unroll
@@ -103,21 +94,16 @@ __device__ inline void fused_in_place(const ConvArgs &a, const v16i (&acc)[2], u
                 asm("v_med3_i32 %0, %1, %2, %3" : "=v"(d) : "v"(d), "s"(dlo), "v"(dhi));
                 const int32_t t0 = (__mul24(d, mc) + rc) >> sc;
                 const int32_t t1 = (__mul24((int)((rv >> (8 * e)) & 255), mr) + cr) >> sr;
-                y[e] = (t0 + t1 + q.cadd) >> q.sh;
+                y[e] = t0 + t1 + q.cadd;
             }
             uint32_t packed;
             if (ADD_SAT) {
-                uint32_t p01, p23, b01, b23;
-                asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p01) : "v"(y[0]), "v"(y[1]));
-                asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(y[2]), "v"(y[3]));
-                asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
-                asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
-                packed = __builtin_amdgcn_perm(b23, b01, 0x05040100u); // the low halves of both, one instruction
+                packed = ashr_sat_u8x4(y[0], y[1], y[2], y[3], q.sh); // the last shift, the clamp to [0, 255], the pack
             } else {
                 packed = 0;
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    int32_t v = y[e];
+                    int32_t v = y[e] >> q.sh;
                     asm("v_med3_i32 %0, %1, %2, %3" : "=v"(v) : "v"(v), "s"(0), "v"(q.hi));
                     packed |= (uint32_t)v << (8 * e);
                 }

@@ -21,20 +21,31 @@ __device__ static inline int swz(int row)
 __device__ static inline v4i requant16(const ConvArgs &a, const v16i &acc, uint32_t flip)
 {
     v4i o;
+    if (a.lo == 0 && a.q.hi == 255) {
 #pragma unroll
-    for (int g = 0; g < 4; g++) {
-        int32_t r[4];
+        for (int g = 0; g < 4; g++)
+            o[g] = (int)(conv_requant4<true>(a, acc[g * 4], acc[g * 4 + 1], acc[g * 4 + 2], acc[g * 4 + 3]) ^ flip);
+    } else if (a.lo >= 0) {
 #pragma unroll
-        for (int e = 0; e < 4; e++)
-            r[e] = conv_requant<true>(a, acc[g * 4 + e]);
-        o[g] = (int)(pack_low_bytes(r[0], r[1], r[2], r[3]) ^ flip);
+        for (int g = 0; g < 4; g++)
+            o[g] = (int)(conv_requant4<false>(a, acc[g * 4], acc[g * 4 + 1], acc[g * 4 + 2], acc[g * 4 + 3]) ^ flip);
+    } else { // two's complement outputs
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            int32_t r[4];
+#pragma unroll
+            for (int e = 0; e < 4; e++)
+                r[e] = conv_requant<true>(a, acc[g * 4 + e]);
+            o[g] = (int)(pack_low_bytes(r[0], r[1], r[2], r[3]) ^ flip);
+        }
     }
     return o;
 }
 
 // The same followed by the residual add (op_quant_add_run on the requantised bytes and the residual's 16 bytes `res`),
 // in the 32-bit form: per element the convolution's clamped result minus its zero point is clamp(q, lo - zp, hi - zp)
-// with q = (mulhi(acc, mult) + 2^(t-1)) >> t; the add's terms are (d * m + c) >> s; the sum saturates to [0, 255].
+// with q = (mulhi(acc, mult) + 2^(t-1)) >> t; the add's terms are (d * m + c) >> s; the sum's last shift and its
+// saturation to [0, 255] are the shifting, saturating pack.
 __device__ static inline v4i requant_add16(const ConvArgs &a, const v16i &acc, const v4i res)
 {
     const AddParams &q = a.addq;
@@ -54,14 +65,9 @@ __device__ static inline v4i requant_add16(const ConvArgs &a, const v16i &acc, c
             asm("v_med3_i32 %0, %1, %2, %3" : "=v"(d) : "v"(d), "s"(dlo), "v"(dhi));
             const int32_t t0 = (__mul24(d, mc) + rc) >> sc;
             const int32_t t1 = (__mul24((int)((rv >> (8 * e)) & 255), mr) + cr) >> sr;
-            y[e] = (t0 + t1 + q.cadd) >> q.sh;
+            y[e] = t0 + t1 + q.cadd;
         }
-        uint32_t p01, p23, b01, b23;
-        asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p01) : "v"(y[0]), "v"(y[1]));
-        asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(y[2]), "v"(y[3]));
-        asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
-        asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
-        o[g] = (int)__builtin_amdgcn_perm(b23, b01, 0x05040100u);
+        o[g] = (int)ashr_sat_u8x4(y[0], y[1], y[2], y[3], q.sh);
     }
     return o;
 }

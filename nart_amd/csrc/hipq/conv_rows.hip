@@ -161,16 +161,7 @@ __global__ __launch_bounds__(256, 2) void conv3x3_c64_rows_kernel(const ConvArgs
             for (int g = 0; g < 4; g++) {
                 uint32_t packed;
                 if (PLAIN_SAT) {
-                    int32_t r[4];
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        r[e] = (__mulhi(acc[tn][g * 4 + e], (int)a.q.mult) + a.qadd) >> a.qt;
-                    uint32_t p01, p23, b01, b23;
-                    asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p01) : "v"(r[0]), "v"(r[1]));
-                    asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(r[2]), "v"(r[3]));
-                    asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
-                    asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
-                    packed = __builtin_amdgcn_perm(b23, b01, 0x05040100u); // the low halves of both, one instruction
+                    packed = conv_requant4<true>(a, acc[tn][g * 4], acc[tn][g * 4 + 1], acc[tn][g * 4 + 2], acc[tn][g * 4 + 3]);
                 } else {
                     int32_t rq[4];
 #pragma unroll

@@ -104,8 +104,26 @@ __device__ static inline uint32_t pack_low_bytes(int32_t r0, int32_t r1, int32_t
     return __builtin_amdgcn_perm((uint32_t)r1, (uint32_t)r0, 0x0c0c0400u) | __builtin_amdgcn_perm((uint32_t)r3, (uint32_t)r2, 0x04000c0cu);
 }
 
+// One-multiply requantisation of four accumulators to the four bytes of a dword, for outputs whose clamp range lies in
+// [0, 255] (a.lo >= 0): mulhi and the rounding / zero-point constant as in conv_requant<true>, then the clamp IN FRONT of
+// the shift - lo << t and ((hi + 1) << t) - 1 are the smallest and largest values that shift to lo and hi - and the
+// shifting, saturating pack.  SAT: the range is exactly [0, 255], the pack's saturation is the clamp.
+template <bool SAT>
+__device__ static __forceinline__ uint32_t conv_requant4(const ConvArgs &a, int32_t v0, int32_t v1, int32_t v2, int32_t v3)
+{
+    int32_t r[4] = {v0, v1, v2, v3};
+    const int32_t plo = a.lo << a.qt, phi = ((a.q.hi + 1) << a.qt) - 1;
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        r[e] = __mulhi(r[e], (int)a.q.mult) + a.qadd;
+        if (!SAT)
+            asm("v_med3_i32 %0, %1, %2, %3" : "=v"(r[e]) : "v"(r[e]), "s"(plo), "v"(phi));
+    }
+    return ashr_sat_u8x4(r[0], r[1], r[2], r[3], a.qt);
+}
+
 template <int BM, int BN, int WM, int WN, bool HAS_WZP, bool FAST, bool PLAIN_SAT, int TM, int TN>
-__device__ static inline void conv_epilogue(const ConvArgs &a, v16i (&acc)[TN][TM], int (&colsum)[TM], uint8_t *lds,
+__device__ static __forceinline__ void conv_epilogue(const ConvArgs &a, v16i (&acc)[TN][TM], int (&colsum)[TM], uint8_t *lds,
                                             int bm, int bn, int wm, int wn)
 {
     constexpr int OSTR = BN + 16; // row stride of the output staging tile
@@ -160,19 +178,12 @@ __device__ static inline void conv_epilogue(const ConvArgs &a, v16i (&acc)[TN][T
             for (int g = 0; g < 4; g++) {
                 uint32_t packed = 0;
                 if (FAST && PLAIN_SAT) {
-                    // clamp range is exactly [0, 255]: two saturating packs replace four clamps and the shifts
-                    int32_t r[4];
+                    // clamp range is exactly [0, 255]: the shifting, saturating pack replaces four clamps and the shifts
+                    int32_t v[4];
 #pragma unroll
-                    for (int e = 0; e < 4; e++) {
-                        const int32_t v = (int32_t)((uint32_t)acc[tn][tm][g * 4 + e] + (HAS_WZP ? (uint32_t)colsum[tm] : 0u));
-                        r[e] = (__mulhi(v, (int)a.q.mult) + a.qadd) >> a.qt;
-                    }
-                    uint32_t p01, p23, b01, b23;
-                    asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p01) : "v"(r[0]), "v"(r[1]));
-                    asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(r[2]), "v"(r[3]));
-                    asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
-                    asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
-                    packed = __builtin_amdgcn_perm(b23, b01, 0x05040100u); // the low halves of both, one instruction
+                    for (int e = 0; e < 4; e++)
+                        v[e] = (int32_t)((uint32_t)acc[tn][tm][g * 4 + e] + (HAS_WZP ? (uint32_t)colsum[tm] : 0u));
+                    packed = conv_requant4<true>(a, v[0], v[1], v[2], v[3]);
                 } else {
                     int32_t rq[4];
 #pragma unroll
@@ -232,7 +243,7 @@ __device__ static inline void conv_epilogue(const ConvArgs &a, v16i (&acc)[TN][T
 // clamp(q, lo - zp, hi - zp) with q = (mulhi(acc, mult) + 2^(t-1)) >> t; the add's terms are (d * m + c) >> s; the sum
 // is clamped and packed.  Bit-identical to storing the convolution's bytes and running the add on them.
 template <int BM, int BN, int WM, int WN, int TM, int TN>
-__device__ static inline void conv_epilogue_fused_add(const ConvArgs &a, v16i (&acc)[TN][TM], uint8_t *lds_out,
+__device__ static __forceinline__ void conv_epilogue_fused_add(const ConvArgs &a, v16i (&acc)[TN][TM], uint8_t *lds_out,
                                                       const uint8_t *lds_res, int bm, int bn, int wm, int wn)
 {
     constexpr int OSTR = BN + 16, CMASK = BN / 16 - 1;
@@ -244,6 +255,7 @@ __device__ static inline void conv_epilogue_fused_add(const ConvArgs &a, v16i (&
     const int rc = 1 << (sc - 1);                    // rounding of the convolution's term (its zero point cancels)
     const int qround = 1 << (a.qt - 1);
     const int dlo = a.lo - a.q.zp, dhi = a.q.hi - a.q.zp; // clamp range of (conv byte - conv zero point)
+    const int yhi = ((q.hi + 1) << q.sh) - 1;             // the largest value that the last shift takes to q.hi
 #pragma unroll
     for (int tm = 0; tm < TM; tm++) {
         const int pl = wm * (TM * 32) + tm * 32 + (lane & 31);
@@ -254,18 +266,16 @@ __device__ static inline void conv_epilogue_fused_add(const ConvArgs &a, v16i (&
             for (int g = 0; g < 4; g++) {
                 const int chl = wn * (TN * 32) + tn * 32 + g * 8 + half * 4;
                 const uint32_t rv = *reinterpret_cast<const uint32_t *>(lds_res + pl * BN + (((chl >> 4) ^ rsw) << 4) + (chl & 15));
-                uint32_t packed = 0;
+                int32_t y[4];
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     int32_t d = (__mulhi(acc[tn][tm][g * 4 + e], (int)a.q.mult) + qround) >> a.qt;
                     asm("v_med3_i32 %0, %1, %2, %3" : "=v"(d) : "v"(d), "s"(dlo), "v"(dhi));
                     const int32_t t0 = (__mul24(d, mc) + rc) >> sc;
                     const int32_t t1 = (__mul24((int)((rv >> (8 * e)) & 255), mr) + cr) >> sr;
-                    int32_t y = (t0 + t1 + q.cadd) >> q.sh;
-                    asm("v_med3_i32 %0, %1, %2, %3" : "=v"(y) : "v"(y), "s"(0), "v"(q.hi));
-                    packed |= (uint32_t)y << (8 * e);
+                    y[e] = min(t0 + t1 + q.cadd, yhi); // the upper clamp in front of the last shift, the lower one is the pack's
                 }
-                *reinterpret_cast<uint32_t *>(lds_out + pl * OSTR + chl) = packed;
+                *reinterpret_cast<uint32_t *>(lds_out + pl * OSTR + chl) = ashr_sat_u8x4(y[0], y[1], y[2], y[3], q.sh);
             }
     }
     __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)

@@ -114,6 +114,7 @@ __global__ __launch_bounds__(256, 2) void conv_stem_maxpool_kernel(const ConvArg
     const int owc = min(px, a.OW - 1);                        // lanes beyond the row compute a copy that is never stored
     const uint8_t *bbase = lds + 16 + (owc * 2 - a.pad_w + 4 * half) * 4; // + patch row * PITCH
     constexpr int32_t kNone = -2147483647 - 1;                // a row outside the image takes no part in the maximum
+    const bool sat = a.lo == 0 && a.q.hi == 255;              // the clamp is the saturation of the pack
 
     // convolution row i of this work-group: 32 pixels x 64 channels per wave, accumulators start from the bias
     auto conv_row = [&](int i, v16i(&acc)[2]) {
@@ -161,11 +162,19 @@ __global__ __launch_bounds__(256, 2) void conv_stem_maxpool_kernel(const ConvArg
                     int32_t rq[4];
 #pragma unroll
                     for (int e = 0; e < 4; e++)
-                        rq[e] = conv_requant<FAST>(a, max(vm[tn][g * 4 + e], acc[tn][g * 4 + e]));
+                        rq[e] = max(vm[tn][g * 4 + e], acc[tn][g * 4 + e]);
+                    uint32_t packed;
+                    if (FAST && sat) {
+                        packed = conv_requant4<true>(a, rq[0], rq[1], rq[2], rq[3]);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            rq[e] = conv_requant<FAST>(a, rq[e]);
+                        packed = pack_low_bytes(rq[0], rq[1], rq[2], rq[3]);
+                    }
                     const int ch = tn * 32 + g * 8 + half * 4;
                     // 16-byte piece c of pixel px sits at piece c ^ (px & 3): spreads a wave's dword stores over the banks
-                    *reinterpret_cast<uint32_t *>(rowbuf + px * 64 + (((ch >> 4) ^ (px & 3)) << 4) + (ch & 15))
-                        = pack_low_bytes(rq[0], rq[1], rq[2], rq[3]);
+                    *reinterpret_cast<uint32_t *>(rowbuf + px * 64 + (((ch >> 4) ^ (px & 3)) << 4) + (ch & 15)) = packed;
                 }
         }
 #pragma unroll
@@ -380,16 +389,7 @@ __global__ __launch_bounds__(256) void conv_stem3x3_kernel(const ConvArgs a, con
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             if (SAT) { // clamp range exactly [0, 255]: saturating packs instead of clamps
-                int32_t r[4];
-#pragma unroll
-                for (int e = 0; e < 4; e++)
-                    r[e] = (__mulhi(acc[g * 4 + e], (int)a.q.mult) + a.qadd) >> a.qt;
-                uint32_t p01, p23, b01, b23;
-                asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p01) : "v"(r[0]), "v"(r[1]));
-                asm("v_cvt_pk_i16_i32 %0, %1, %2" : "=v"(p23) : "v"(r[2]), "v"(r[3]));
-                asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b01) : "v"(p01));
-                asm("v_sat_pk_u8_i16 %0, %1" : "=v"(b23) : "v"(p23));
-                out[g] = __builtin_amdgcn_perm(b23, b01, 0x05040100u);
+                out[g] = conv_requant4<true>(a, acc[g * 4], acc[g * 4 + 1], acc[g * 4 + 2], acc[g * 4 + 3]);
             } else {
                 out[g] = pack_low_bytes(conv_requant<FAST>(a, acc[g * 4]), conv_requant<FAST>(a, acc[g * 4 + 1]),
                                         conv_requant<FAST>(a, acc[g * 4 + 2]), conv_requant<FAST>(a, acc[g * 4 + 3]));
