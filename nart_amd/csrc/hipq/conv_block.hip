@@ -46,6 +46,15 @@ constexpr int kPatch = 7;          // a work-group's output pixels: kPatch x kPa
 constexpr int kGridW = kPatch + 2; // the patch with its border: kGridW x kGridW pixel rows in LDS
 constexpr int kGridRows = 96;      // rows held for that grid (81 positions; the row-padded output index reaches row 83)
 
+// LDS tiles whose rows are the CM bytes of a pixel (the grid, layer 2's bytes): rows of 128 bytes or more lie 16 bytes
+// further apart than their length, so that the lanes of a wave, which read the same 16-byte chunk of consecutive rows,
+// fall on different bank groups, and a tap's shift on the grid is a constant added to the address (no swizzle to redo
+// per tap); 64-byte rows read without conflicts as they are.
+template <int CM>
+constexpr int kRowStride = CM >= 128 ? CM + 16 : CM;
+template <int CM>
+__device__ static inline int row_off(int row, int chunk) { return row * kRowStride<CM> + (chunk << 4); }
+
 struct BlockGeom {
     int H, W, PY, PX, npatch;
     int IH, IW; // the tail kernel's input image where its 3x3 layer has stride 2 (H, W: the output image)
@@ -63,7 +72,7 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
 {
     constexpr int NW = 2 * G, NT = 128 * G, CM = 64 * G, CW = 256 * G;
     constexpr int X_BYTES = 32 * MT1 * CW;                  // the region's pixel rows, CW bytes each
-    constexpr int G_OFF = X_BYTES, G_BYTES = kGridRows * CM; // layer 1's bytes on the 9 x 9 grid, CM bytes a row; later layer 2's
+    constexpr int G_OFF = X_BYTES, G_BYTES = kGridRows * kRowStride<CM>; // layer 1's bytes on the 9 x 9 grid, CM bytes a row; later layer 2's
     constexpr int D1 = MT1 == 2 ? 10 : 8, D2 = 10;          // slabs of weights a wave holds ahead, layers 1 and 2
     __shared__ __attribute__((aligned(1024))) uint8_t lds[G_OFF + G_BYTES];
 
@@ -125,8 +134,8 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
     // layer 2, slab s: channels 64 cb .. + 63 of tap (tap / 3, tap % 3), read at the tap's shift on the grid
     auto ldb2 = [&](int s, int kk, int t) {
         const int tap = s / G, cb = s % G, tr = (tap * 11) >> 5, off = tr * kGridW + (tap - 3 * tr);
-        const int gr = 32 * t + p + off, hs = h ^ swz<CM>(gr);
-        return *reinterpret_cast<const v4i *>(lds + G_OFF + gr * CM + (((4 * cb + 2 * kk) ^ hs) << 4));
+        const int gr = 32 * t + p + off;
+        return *reinterpret_cast<const v4i *>(lds + G_OFF + row_off<CM>(gr, 4 * cb + 2 * kk + h));
     };
 
     // ================= layer 1: CW -> CM on the region's pixels =================
@@ -156,7 +165,7 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
             const int jy = (j * rwinv) >> 16, jx = j - jy * RW;
             const int g = (ry0 + jy - y0 + 1) * kGridW + (rx0 + jx - x0 + 1);
             const v4i o = requant16(a1, acc1[t], a2.xmask);
-            *reinterpret_cast<v4i *>(lds + G_OFF + g * CM + ((((ct0 >> 4) + h) ^ swz<CM>(g)) << 4)) = o;
+            *reinterpret_cast<v4i *>(lds + G_OFF + row_off<CM>(g, (ct0 >> 4) + h)) = o;
         }
     }
     __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
@@ -185,7 +194,7 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
     for (int t = 0; t < 2; t++) {
         const int m = 32 * t + p;
         const v4i o = o2[t];
-        *reinterpret_cast<v4i *>(lds + G_OFF + m * CM + ((((ct0 >> 4) + h) ^ swz<CM>(m)) << 4)) = o;
+        *reinterpret_cast<v4i *>(lds + G_OFF + row_off<CM>(m, (ct0 >> 4) + h)) = o;
     }
     __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
@@ -202,7 +211,7 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
             const int m = 32 * t + p;
 #pragma unroll
             for (int ks = 0; ks < 2 * G; ks++)
-                bf[t][ks] = *reinterpret_cast<const v4i *>(lds + G_OFF + m * CM + (((2 * ks + h) ^ swz<CM>(m)) << 4));
+                bf[t][ks] = *reinterpret_cast<const v4i *>(lds + G_OFF + row_off<CM>(m, 2 * ks + h));
             const int py = (m * 57) >> 9, px = m - py * kGridW; // m / 9 for m < 64
             valid[t] = py < kPatch && px < kPatch;
             jres[t] = valid[t] ? (y0 + py - ry0) * RW + (x0 + px - rx0) : 0;
@@ -295,8 +304,8 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? (NX ? 4 : 3) : G == 2 ? 3 : 2)) 
     constexpr int NW = 2 * G, NT = 128 * G, CM = 64 * G, CW = 256 * G;
     constexpr bool CHAIN = NX != 0; // the next layer has NX * CM output channels
     constexpr int GW = ST * (PW - 1) + 3, GH = ST * (PH - 1) + 3, NPIX = PH * PW, GROWS = (GH * GW + 7) / 8 * 8;
-    constexpr int G_OFF = 0, G_BYTES = GROWS * CM;            // layer 2's input on the bordered grid
-    constexpr int M_OFF = G_OFF + G_BYTES, M_BYTES = 64 * CM; // layer 2's bytes, row = pixel
+    constexpr int G_OFF = 0, G_BYTES = GROWS * kRowStride<CM>;            // layer 2's input on the bordered grid
+    constexpr int M_OFF = G_OFF + G_BYTES, M_BYTES = 64 * kRowStride<CM>; // layer 2's bytes, row = pixel
     // the sum tile takes the place of the grid and of layer 2's bytes once every wave holds its operands of layer 3
     constexpr int S_OFF = 0, S_BYTES = CHAIN ? 64 * CW : 0;
     constexpr int D2 = G == 1 ? 4 : G == 2 ? 6 : 10, DN = D2; // slabs of weights a wave holds ahead (four or three waves per SIMD: fewer registers)
@@ -325,7 +334,7 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? (NX ? 4 : 3) : G == 2 ? 3 : 2)) 
                 const int ih = ST == 1 ? geo.H : geo.IH, iw = ST == 1 ? geo.W : geo.IW;
                 const bool in = g < GH * GW && (unsigned)iy < (unsigned)ih && (unsigned)ix < (unsigned)iw;
                 const uint8_t *src = in ? a2.x + (size_t)((n * ih + iy) * iw + ix) * CM + c * 16 : a2.padbuf;
-                *reinterpret_cast<v4i *>(lds + G_OFF + g * CM + ((c ^ swz<CM>(g)) << 4)) = ldg128(src) ^ (int)a2.xmask;
+                *reinterpret_cast<v4i *>(lds + G_OFF + row_off<CM>(g, c)) = ldg128(src) ^ (int)a2.xmask;
             }
         }
     }
@@ -346,8 +355,8 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? (NX ? 4 : 3) : G == 2 ? 3 : 2)) 
     }
     auto ldb2 = [&](int s, int kk, int t) {
         const int tap = s / G, cb = s % G, tr = (tap * 11) >> 5;
-        const int gr = grow[t] + (tr - 1) * GW + (tap - 3 * tr - 1), hs = h ^ swz<CM>(gr);
-        return *reinterpret_cast<const v4i *>(lds + G_OFF + gr * CM + (((4 * cb + 2 * kk) ^ hs) << 4));
+        const int gr = grow[t] + (tr - 1) * GW + (tap - 3 * tr - 1);
+        return *reinterpret_cast<const v4i *>(lds + G_OFF + row_off<CM>(gr, 4 * cb + 2 * kk + h));
     };
 
     // ================= layer 2: 3x3, CM -> CM =================
@@ -379,7 +388,7 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? (NX ? 4 : 3) : G == 2 ? 3 : 2)) 
     for (int t = 0; t < 2; t++) {
         const int q = 32 * t + p;
         const v4i o = requant16(a2, acc2[t], a3.xmask);
-        *reinterpret_cast<v4i *>(lds + M_OFF + q * CM + ((((ct0 >> 4) + h) ^ swz<CM>(q)) << 4)) = o;
+        *reinterpret_cast<v4i *>(lds + M_OFF + row_off<CM>(q, (ct0 >> 4) + h)) = o;
     }
     __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
     __builtin_amdgcn_s_barrier();
@@ -392,7 +401,7 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? (NX ? 4 : 3) : G == 2 ? 3 : 2)) 
             const int q = 32 * t + p;
 #pragma unroll
             for (int ks = 0; ks < 2 * G; ks++)
-                bf[t][ks] = *reinterpret_cast<const v4i *>(lds + M_OFF + q * CM + (((2 * ks + h) ^ swz<CM>(q)) << 4));
+                bf[t][ks] = *reinterpret_cast<const v4i *>(lds + M_OFF + row_off<CM>(q, 2 * ks + h));
         }
         if (CHAIN) { // the sum tile lies over what the waves have just read
             __builtin_amdgcn_s_waitcnt(0xC07F); // lgkmcnt(0)
