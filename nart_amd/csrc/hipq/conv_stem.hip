@@ -155,27 +155,34 @@ __global__ __launch_bounds__(256, 2) void conv_stem_maxpool_kernel(const ConvArg
         // the vertical maxima of pooled row j, requantised, into the row buffer; the last row starts the next maximum
         uint8_t *rowbuf = lds + R_OFF + (j & 1) * kStemRowBuf;
         if (px < a.OW) {
+            // sat_c: the clamp range is exactly [0, 255] and the pack's saturation is the clamp (one test per row, not per dword)
+            auto emit = [&](auto sat_c) {
 #pragma unroll
-            for (int tn = 0; tn < 2; tn++)
+                for (int tn = 0; tn < 2; tn++)
 #pragma unroll
-                for (int g = 0; g < 4; g++) {
-                    int32_t rq[4];
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        rq[e] = max(vm[tn][g * 4 + e], acc[tn][g * 4 + e]);
-                    uint32_t packed;
-                    if (FAST && sat) {
-                        packed = conv_requant4<true>(a, rq[0], rq[1], rq[2], rq[3]);
-                    } else {
+                    for (int g = 0; g < 4; g++) {
+                        int32_t rq[4];
 #pragma unroll
                         for (int e = 0; e < 4; e++)
-                            rq[e] = conv_requant<FAST>(a, rq[e]);
-                        packed = pack_low_bytes(rq[0], rq[1], rq[2], rq[3]);
+                            rq[e] = max(vm[tn][g * 4 + e], acc[tn][g * 4 + e]);
+                        uint32_t packed;
+                        if (FAST && decltype(sat_c)::value) {
+                            packed = conv_requant4<true>(a, rq[0], rq[1], rq[2], rq[3]);
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; e++)
+                                rq[e] = conv_requant<FAST>(a, rq[e]);
+                            packed = pack_low_bytes(rq[0], rq[1], rq[2], rq[3]);
+                        }
+                        const int ch = tn * 32 + g * 8 + half * 4;
+                        // 16-byte piece c of pixel px sits at piece c ^ (px & 3): spreads a wave's dword stores over the banks
+                        *reinterpret_cast<uint32_t *>(rowbuf + px * 64 + (((ch >> 4) ^ (px & 3)) << 4) + (ch & 15)) = packed;
                     }
-                    const int ch = tn * 32 + g * 8 + half * 4;
-                    // 16-byte piece c of pixel px sits at piece c ^ (px & 3): spreads a wave's dword stores over the banks
-                    *reinterpret_cast<uint32_t *>(rowbuf + px * 64 + (((ch >> 4) ^ (px & 3)) << 4) + (ch & 15)) = packed;
-                }
+            };
+            if (sat)
+                emit(std::true_type{});
+            else
+                emit(std::false_type{});
         }
 #pragma unroll
         for (int tn = 0; tn < 2; tn++)
