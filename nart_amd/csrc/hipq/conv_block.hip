@@ -501,7 +501,7 @@ bool conv_block_tail_applies(const ConvArgs &a2, const ConvArgs &a3, const ConvA
 {
     const int cm = a2.in_cs, cw = a3.out_cs;
     auto plain = [](const ConvArgs &a) {
-        return a.group == 1 && a.bwz == 0 && a.xmask != 0 && a.fastq && a.qmult == nullptr && a.acc_out == nullptr && a.deq_out == nullptr && a.wfrag != nullptr;
+        return a.group == 1 && a.bwz == 0 && a.xmask != 0 && a.lo >= 0 && a.fastq && a.qmult == nullptr && a.acc_out == nullptr && a.deq_out == nullptr && a.wfrag != nullptr;
     };
     auto one = [](const ConvArgs &a) {
         return a.R == 1 && a.S == 1 && a.pad_h == 0 && a.pad_w == 0 && a.stride_h == 1 && a.stride_w == 1;
@@ -577,7 +577,7 @@ bool conv_block_applies(const ConvArgs &a1, const ConvArgs &a2, const ConvArgs &
 {
     const int cm = a1.out_cs, cw = a1.in_cs;
     auto plain = [](const ConvArgs &a) {
-        return a.group == 1 && a.bwz == 0 && a.xmask != 0 && a.fastq && a.qmult == nullptr && a.acc_out == nullptr && a.deq_out == nullptr && a.wfrag != nullptr;
+        return a.group == 1 && a.bwz == 0 && a.xmask != 0 && a.lo >= 0 && a.fastq && a.qmult == nullptr && a.acc_out == nullptr && a.deq_out == nullptr && a.wfrag != nullptr;
     };
     auto one = [](const ConvArgs &a) {
         return a.R == 1 && a.S == 1 && a.pad_h == 0 && a.pad_w == 0 && a.stride_h == 1 && a.stride_w == 1;

@@ -17,7 +17,8 @@ __device__ static inline int swz(int row)
     return ROWBYTES >= 256 ? (row & 15) : ROWBYTES == 128 ? ((row >> 1) & 7) : ((row >> 2) & 3);
 }
 
-// 16 accumulators (16 consecutive channels of one pixel) -> 16 requantised bytes, each XORed with the low byte of flip
+// 16 accumulators (16 consecutive channels of one pixel) -> 16 requantised bytes, each XORed with the low byte of flip.
+// For clamp ranges within [0, 255] (a.lo >= 0: the callers' hosts check it).
 __device__ static inline v4i requant16(const ConvArgs &a, const v16i &acc, uint32_t flip)
 {
     v4i o;
@@ -25,19 +26,10 @@ __device__ static inline v4i requant16(const ConvArgs &a, const v16i &acc, uint3
 #pragma unroll
         for (int g = 0; g < 4; g++)
             o[g] = (int)(conv_requant4<true>(a, acc[g * 4], acc[g * 4 + 1], acc[g * 4 + 2], acc[g * 4 + 3]) ^ flip);
-    } else if (a.lo >= 0) {
+    } else {
 #pragma unroll
         for (int g = 0; g < 4; g++)
             o[g] = (int)(conv_requant4<false>(a, acc[g * 4], acc[g * 4 + 1], acc[g * 4 + 2], acc[g * 4 + 3]) ^ flip);
-    } else { // two's complement outputs
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-            int32_t r[4];
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-                r[e] = conv_requant<true>(a, acc[g * 4 + e]);
-            o[g] = (int)(pack_low_bytes(r[0], r[1], r[2], r[3]) ^ flip);
-        }
     }
     return o;
 }

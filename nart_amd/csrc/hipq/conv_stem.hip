@@ -307,7 +307,7 @@ bool conv_stem_next_applies(const ConvArgs &a, int POH, int POW, const ConvArgs 
     auto ok = [&](const ConvArgs &l) {
         return l.R == 1 && l.S == 1 && l.pad_h == 0 && l.pad_w == 0 && l.stride_h == 1 && l.stride_w == 1 && l.group == 1 && l.C == 64
             && l.in_cs == 64 && l.K >= 64 && l.K % 64 == 0 && l.out_cs == l.K && l.nslab == 1 && l.kout_pad >= l.K && l.N == a.N
-            && l.H == POH && l.W == POW && l.OH == POH && l.OW == POW && l.bwz == 0 && l.xmask == an.xmask && l.xmask != 0 && l.fastq
+            && l.H == POH && l.W == POW && l.OH == POH && l.OW == POW && l.bwz == 0 && l.xmask == an.xmask && l.xmask != 0 && l.lo >= 0 && l.fastq
             && l.qmult == nullptr && l.acc_out == nullptr && l.deq_out == nullptr && l.res == nullptr && l.wfrag != nullptr;
     };
     return a.fastq && POW <= 64 && ok(an) && (!an2 || ok(*an2)) && an.K + (an2 ? an2->K : 0) <= kStemNextCh;

@@ -272,7 +272,7 @@ __global__ __launch_bounds__(256, (4096 * (CPT + CPT2) + 16384 <= 81920 ? 2 : 1)
 bool conv_wreg_dual_applies(const ConvArgs &a, const ConvArgs &b)
 {
     auto plain1x1 = [](const ConvArgs &c) {
-        return c.group == 1 && c.bwz == 0 && c.xmask != 0 && c.fastq && c.qmult == nullptr && c.acc_out == nullptr && c.deq_out == nullptr
+        return c.group == 1 && c.bwz == 0 && c.xmask != 0 && c.lo >= 0 && c.fastq && c.qmult == nullptr && c.acc_out == nullptr && c.deq_out == nullptr
             && c.wfrag != nullptr && c.C == c.in_cs && c.in_cs % 64 == 0 && c.K == c.out_cs && c.out_cs % 128 == 0 && c.R == 1 && c.S == 1
             && c.pad_h == 0 && c.pad_w == 0 && c.stride_h == c.stride_w && c.nslab == c.in_cs / 64;
     };
@@ -310,7 +310,7 @@ void launch_conv_wreg_dual(const ConvArgs &a, const ConvArgs &b, hipStream_t st)
 
 bool conv_wreg_applies(const ConvArgs &a)
 {
-    if (!(a.group == 1 && a.bwz == 0 && a.xmask != 0 && a.fastq && a.qmult == nullptr && a.acc_out == nullptr && a.deq_out == nullptr
+    if (!(a.group == 1 && a.bwz == 0 && a.xmask != 0 && a.lo >= 0 && a.fastq && a.qmult == nullptr && a.acc_out == nullptr && a.deq_out == nullptr
           && a.wfrag != nullptr && a.C == a.in_cs && a.in_cs % 64 == 0 && a.K == a.out_cs && a.out_cs % 128 == 0
           && a.stride_h == a.stride_w && (a.stride_h == 1 || a.stride_h == 2) && a.nslab == a.R * a.S * a.in_cs / 64
           && (a.res == nullptr || (a.addq.fast && a.addq.hi == 255))))
