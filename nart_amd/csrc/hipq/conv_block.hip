@@ -298,7 +298,7 @@ __global__ __launch_bounds__(128 * G, 2) void conv_bottleneck_kernel(const ConvA
 //   * CHAIN: the next layer (CW -> CM, or CW -> 2 CM where the next stage begins) reads that tile as its pixel operand.
 // ST: the 3x3 layer's stride (1, or 2 - the first block of a stage: the grid then holds (2 PH + 1) x (2 PW + 1) input pixels).
 template <int G, int PH, int PW, int NX, int ST>
-__global__ __launch_bounds__(128 * G, (G == 1 ? (NX ? 4 : 3) : G == 2 ? 3 : 2)) void conv_bottleneck_tail_kernel(const ConvArgs a2, const ConvArgs a3, const ConvArgs an,
+__global__ __launch_bounds__(128 * G, (G == 1 ? (NX ? 4 : 3) : G == 2 ? (NX && ST == 1 && (NX == 1 || PH == 4) ? 4 : 3) : 2)) void conv_bottleneck_tail_kernel(const ConvArgs a2, const ConvArgs a3, const ConvArgs an,
                                                                          const BlockGeom geo)
 {
     constexpr int NW = 2 * G, NT = 128 * G, CM = 64 * G, CW = 256 * G;
@@ -308,9 +308,14 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? (NX ? 4 : 3) : G == 2 ? 3 : 2)) 
     constexpr int M_OFF = G_OFF + G_BYTES, M_BYTES = 64 * kRowStride<CM>; // layer 2's bytes, row = pixel
     // the sum tile takes the place of the grid and of layer 2's bytes once every wave holds its operands of layer 3
     constexpr int S_OFF = 0, S_BYTES = CHAIN ? 64 * CW : 0;
+    // LDSB: layer 3's folded biases wait in LDS instead of in registers a chunk ahead - 16 registers less at the add's
+    // arithmetic, which is what lets the 128-channel chained form keep four waves per SIMD (896 work-groups at 28x28 and
+    // batch 64: one round of 1024 slots instead of 768 and a nearly empty second round)
+    constexpr bool LDSB = G == 2 && CHAIN && ST == 1;
+    constexpr int B3_OFF = (M_OFF + M_BYTES > S_BYTES ? M_OFF + M_BYTES : S_BYTES), B3_BYTES = LDSB ? 4 * CW : 0;
     constexpr int D2 = G == 1 ? 4 : G == 2 ? 6 : 10, DN = D2; // slabs of weights a wave holds ahead (four or three waves per SIMD: fewer registers)
     static_assert(NPIX <= 64, "pixel slots");
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[M_OFF + M_BYTES > S_BYTES ? M_OFF + M_BYTES : S_BYTES];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[B3_OFF + B3_BYTES];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int p = lane & 31, h = lane >> 5;
@@ -337,6 +342,10 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? (NX ? 4 : 3) : G == 2 ? 3 : 2)) 
                 *reinterpret_cast<v4i *>(lds + G_OFF + row_off<CM>(g, c)) = ldg128(src) ^ (int)a2.xmask;
             }
         }
+    }
+    if (LDSB) {
+        for (int i = tid * 4; i < CW; i += NT * 4)
+            *reinterpret_cast<v4i *>(lds + B3_OFF + i * 4) = *reinterpret_cast<const v4i *>(a3.bias2 + i);
     }
     const int ct0 = 32 * wave; // layers 2 and next: a wave owns 32 of the CM channels and the whole reduction
     const size_t wslab2 = (size_t)a2.kout_pad * 64, wslab3 = (size_t)a3.kout_pad * 64, wslabn = (size_t)an.kout_pad * 64;
@@ -376,9 +385,11 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? (NX ? 4 : 3) : G == 2 ? 3 : 2)) 
 #pragma unroll
         for (int ks = 0; ks < 2 * G; ks++)
             wf[ks] = ldg128(w3 + (size_t)(ks >> 1) * wslab3 + (size_t)cc * 2048 + (ks & 1) * 1024);
+        if (!LDSB) {
 #pragma unroll
-        for (int g = 0; g < 4; g++)
-            b3[g] = *reinterpret_cast<const v4i *>(a3.bias2 + 128 * wave + 32 * cc + 16 * h + 4 * g);
+            for (int g = 0; g < 4; g++)
+                b3[g] = *reinterpret_cast<const v4i *>(a3.bias2 + 128 * wave + 32 * cc + 16 * h + 4 * g);
+        }
 #pragma unroll
         for (int t = 0; t < 2; t++)
             rn[t] = ldg128(a3.res + pix[t] * CW + 128 * wave + 32 * cc + 16 * h);
@@ -411,10 +422,12 @@ __global__ __launch_bounds__(128 * G, (G == 1 ? (NX ? 4 : 3) : G == 2 ? 3 : 2)) 
             const int ch = 128 * wave + 32 * cc;
             v16i acc[2];
 #pragma unroll
-            for (int g = 0; g < 4; g++)
+            for (int g = 0; g < 4; g++) {
+                const v4i bv = LDSB ? *reinterpret_cast<const v4i *>(lds + B3_OFF + (ch + 16 * h + 4 * g) * 4) : b3[g];
 #pragma unroll
                 for (int e = 0; e < 4; e++)
-                    acc[0][4 * g + e] = b3[g][e];
+                    acc[0][4 * g + e] = bv[e];
+            }
             acc[1] = acc[0];
 #pragma unroll
             for (int ks = 0; ks < 2 * G; ks++)
