@@ -11,12 +11,13 @@
 //     other pixel of every other row), for a 3x3 layer the 7x7 output patch's input region with its border (9x9 pixel rows,
 //     15x15 at stride 2; out-of-image positions read the pad bytes), tap (r, s) of output pixel (y, x) being grid row
 //     (S y + r) * GW + S x + s;
-//   * the four waves are two pairs, 64 channels each; a pair's waves split the reduction (every other 64-byte slab)
-//     and load their MFMA weight operands straight from memory in fragment order (ConvArgs::wfrag), six slabs ahead of
-//     the multiplies - no two waves want the same weight bytes, so LDS bandwidth is left to the pixel operands and the
-//     loop has no barrier;
-//   * the halves meet once in LDS (frag::pair_reduce); each wave requantises 32 channels of the 64 pixels - a lane holds
-//     16 consecutive channels of a pixel - adds the residual where there is one, and stores 16 bytes per lane.
+//   * each of the four waves owns 32 of the 128 channels for all 64 pixels and the whole reduction, and loads its MFMA
+//     weight operands straight from memory in fragment order (ConvArgs::wfrag), eight slabs ahead of the multiplies - no
+//     two waves want the same weight bytes, so LDS bandwidth is left to the pixel operands, the loop has no barrier and
+//     the waves exchange nothing (splitting the reduction between two waves read every pixel operand once instead of
+//     twice, but the exchange of partial sums through LDS cost more: 0.644 -> 0.639 ms per ResNet-50 pass);
+//   * a lane holds 16 consecutive channels of a pixel: it requantises them, adds the residual where there is one, and
+//     stores 16 bytes.
 // Requirements (checked by the host): uint8 tensors, weight zero point 128, per-tensor scale, one-multiply
 // requantisation, dense channel strides, input channels a multiple of 64 (1x1: 256, 512, 1024 or 2048; 3x3: 128, 256 or
 // 512), output channels a multiple of 128; 3x3: pad 1, output height and width multiples of 7.
@@ -50,13 +51,12 @@ __global__ __launch_bounds__(256, 2) void conv_wreg_kernel(const ConvArgs a, con
     constexpr int GW = TAPS == 9 ? S * (kWregPatch - 1) + 3 : 0;  // 3x3: the input region of a patch is GW x GW pixels
     constexpr int ROWS0 = TAPS == 9 ? GW * GW : 64;
     constexpr int X_BYTES = (ROWS0 * RB + 4095) / 4096 * 4096;    // whole instructions of the four waves
-    constexpr int S_OFF = X_BYTES, STOT = TAPS * CPT, D = 6;
+    constexpr int STOT = TAPS * CPT, D = 8;
     static_assert(TAPS == 9 || CPT >= 4, "1x1 layers: pixel rows of at least 256 bytes");
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[S_OFF + 4 * 4096];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[X_BYTES];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int p = lane & 31, h = lane >> 5;
-    const int ng = wave & 1, kh = wave >> 1, partner = wave ^ 2;
     // work-groups go to the 8 XCDs in turn: XCD x takes the x-th contiguous eighth of the list, in which the channel
     // blocks of one pixel group are neighbours (they read the same pixels)
     const int gid = (int)(blockIdx.x % 8) * (int)(gridDim.x / 8) + (int)(blockIdx.x / 8);
@@ -94,11 +94,11 @@ __global__ __launch_bounds__(256, 2) void conv_wreg_kernel(const ConvArgs a, con
         }
     }
 
-    // the wave's two channel tiles: tile 0 (kept after the pair's exchange) and tile 1 (sent)
-    const int ct0 = 128 * nb + 64 * ng + 32 * kh, ct1 = 128 * nb + 64 * ng + 32 * (1 - kh);
+    // the wave's channel tile: 32 of the block's 128 channels, for all 64 pixels and the whole reduction
+    const int ct0 = 128 * nb + 32 * wave;
     const size_t wslab = (size_t)a.kout_pad * 64;
-    const uint8_t *w0 = a.wfrag + (size_t)ct0 * 64 + lane * 16, *w1 = a.wfrag + (size_t)ct1 * 64 + lane * 16;
-    auto ldw = [&](int s, int kk, int nt) { return ldg128((nt ? w1 : w0) + (size_t)s * wslab + kk * 1024); };
+    const uint8_t *w0 = a.wfrag + (size_t)ct0 * 64 + lane * 16;
+    auto ldw = [&](int s, int kk) { return ldg128(w0 + (size_t)s * wslab + kk * 1024); };
     // the lane's output pixels q = 32 t + p
     int prow[2];    // 1x1: the pixel's row in LDS; 3x3: the grid row of its first tap
     size_t pix[2];  // the output pixel's index in y
@@ -127,14 +127,12 @@ __global__ __launch_bounds__(256, 2) void conv_wreg_kernel(const ConvArgs a, con
         return *reinterpret_cast<const v4i *>(lds + j * RB + (s >> 2) * 256 + (((4 * (s & 3) + 2 * kk) ^ hs) << 4));
     };
 
-    v16i acc[2][2];
+    v16i acc[2];
 #pragma unroll
-    for (int t = 0; t < 2; t++) {
-        init_acc(acc[t][0], a.bias2 + ct0 + 16 * h, kh != 0);
-        init_acc(acc[t][1], a.bias2 + ct1 + 16 * h, kh != 0);
-    }
-    WeightRing<D> ring;
-    ring_fill<STOT, D>(ring, kh, ldw);
+    for (int t = 0; t < 2; t++)
+        init_acc(acc[t], a.bias2 + ct0 + 16 * h, false);
+    WeightRing1<D> ring;
+    ring_fill1<STOT, D>(ring, ldw);
     v4i res[2];
     if (ADD) {
 #pragma unroll
@@ -144,11 +142,10 @@ __global__ __launch_bounds__(256, 2) void conv_wreg_kernel(const ConvArgs a, con
     // every wave's share of the pixel operand has landed before anyone reads it
     wait_vmcnt<0>();
     __builtin_amdgcn_s_barrier();
-    reduce_half<STOT, 2, D>(acc, ring, kh, (int)a.xmask, ldw, ldb);
-    pair_reduce<2, false>(acc, lds + S_OFF, wave, partner, lane);
+    reduce_all<STOT, 2, D>(acc, ring, (int)a.xmask, ldw, ldb);
 #pragma unroll
     for (int t = 0; t < 2; t++) {
-        const v4i o = ADD ? requant_add16(a, acc[t][0], res[t]) : requant16(a, acc[t][0], 0);
+        const v4i o = ADD ? requant_add16(a, acc[t], res[t]) : requant16(a, acc[t], 0);
         if (valid[t])
             *reinterpret_cast<v4i *>(a.y + pix[t] * a.out_cs + ct0 + 16 * h) = o;
     }
