@@ -158,16 +158,15 @@ __global__ __launch_bounds__(256, 2) void conv_wreg_kernel(const ConvArgs a, con
 // operands go to LDS at the start; b is reduced first and its 16 bytes per lane and pixel tile wait in registers while a is
 // reduced into the same accumulators.
 template <int CPT, int CPT2, int S2>
-__global__ __launch_bounds__(256, (4096 * (CPT + CPT2) + 16384 <= 81920 ? 2 : 1)) void conv_wreg_dual_kernel(const ConvArgs a, const ConvArgs b, const WregGeom geo)
+__global__ __launch_bounds__(256, (4096 * (CPT + CPT2) <= 53248 ? 3 : 4096 * (CPT + CPT2) <= 81920 ? 2 : 1)) void conv_wreg_dual_kernel(const ConvArgs a, const ConvArgs b, const WregGeom geo)
 {
     constexpr int RB = 64 * CPT, RB2 = 64 * CPT2, X_BYTES = 64 * RB, X2_BYTES = 64 * RB2;
-    constexpr int S_OFF = X_BYTES + X2_BYTES, D = 6;
+    constexpr int D = 6;
     static_assert(CPT >= 4 && CPT2 >= 4, "pixel rows of at least 256 bytes");
-    __shared__ __attribute__((aligned(1024))) uint8_t lds[S_OFF + 4 * 4096];
+    __shared__ __attribute__((aligned(1024))) uint8_t lds[X_BYTES + X2_BYTES];
 
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int p = lane & 31, h = lane >> 5;
-    const int ng = wave & 1, kh = wave >> 1, partner = wave ^ 2;
     const int gid = (int)(blockIdx.x % 8) * (int)(gridDim.x / 8) + (int)(blockIdx.x / 8); // XCD x: the x-th eighth of the list
     if (gid >= geo.npg * geo.nnb)
         return;
@@ -193,13 +192,13 @@ __global__ __launch_bounds__(256, (4096 * (CPT + CPT2) + 16384 <= 81920 ? 2 : 1)
         __builtin_amdgcn_global_load_lds((gptr_t)src, (lptr_t)(lds + (k * 4 + wave) * 1024), 16, 0, 0);
     }
 
-    // The work-group walks geo.nbpw blocks of 128 output channels with the pixel operands it has loaded once.  Per block
-    // the wave's two channel tiles: tile 0 (kept after the pair's exchange) and tile 1 (sent).
+    // The work-group walks geo.nbpw blocks of 128 output channels with the pixel operands it has loaded once; per block a
+    // wave owns 32 channels for all 64 pixels and both reductions.
     const size_t wslab = (size_t)a.kout_pad * 64, wslab2 = (size_t)b.kout_pad * 64;
-    int ct0 = 128 * nb * geo.nbpw + 64 * ng + 32 * kh, ct1 = 128 * nb * geo.nbpw + 64 * ng + 32 * (1 - kh);
-    const uint8_t *w0, *w1, *v0, *v1;
-    auto ldw = [&](int s, int kk, int nt) { return ldg128((nt ? w1 : w0) + (size_t)s * wslab + kk * 1024); };
-    auto ldw2 = [&](int s, int kk, int nt) { return ldg128((nt ? v1 : v0) + (size_t)s * wslab2 + kk * 1024); };
+    int ct0 = 128 * nb * geo.nbpw + 32 * wave;
+    const uint8_t *w0, *v0;
+    auto ldw = [&](int s, int kk) { return ldg128(w0 + (size_t)s * wslab + kk * 1024); };
+    auto ldw2 = [&](int s, int kk) { return ldg128(v0 + (size_t)s * wslab2 + kk * 1024); };
     auto ldb = [&](int s, int kk, int t) {
         const int j = 32 * t + p, hs = h ^ (j & 15);
         return *reinterpret_cast<const v4i *>(lds + j * RB + (s >> 2) * 256 + (((4 * (s & 3) + 2 * kk) ^ hs) << 4));
@@ -215,50 +214,38 @@ __global__ __launch_bounds__(256, (4096 * (CPT + CPT2) + 16384 <= 81920 ? 2 : 1)
         valid[t] = pg * 64 + 32 * t + p < a.P;
         pix[t] = (size_t)min(pg * 64 + 32 * t + p, a.P - 1);
     }
-    WeightRing<D> ring, ringa;
-    v0 = b.wfrag + (size_t)ct0 * 64 + lane * 16, v1 = b.wfrag + (size_t)ct1 * 64 + lane * 16;
-    ring_fill<CPT2, D>(ring, kh, ldw2);
+    WeightRing1<D> ring, ringa;
+    v0 = b.wfrag + (size_t)ct0 * 64 + lane * 16;
+    ring_fill1<CPT2, D>(ring, ldw2);
     wait_vmcnt<0>(); // every wave's share of both pixel operands has landed before anyone reads them
     __builtin_amdgcn_s_barrier();
     for (int bi = 0; bi < geo.nbpw; bi++) {
         // ---- the shortcut b: its bytes for this wave's 32 channels of the 64 pixels stay in registers ----
-        v16i acc[2][2];
+        v16i acc[2];
 #pragma unroll
-        for (int t = 0; t < 2; t++) {
-            init_acc(acc[t][0], b.bias2 + ct0 + 16 * h, kh != 0);
-            init_acc(acc[t][1], b.bias2 + ct1 + 16 * h, kh != 0);
-        }
-        reduce_half<CPT2, 2, D>(acc, ring, kh, (int)b.xmask, ldw2, ldb2);
-        w0 = a.wfrag + (size_t)ct0 * 64 + lane * 16, w1 = a.wfrag + (size_t)ct1 * 64 + lane * 16;
-        ring_fill<CPT, D>(ringa, kh, ldw); // a's first weights travel while b's halves meet
-        if (bi > 0) {
-            __builtin_amdgcn_s_waitcnt(0xC07F);
-            __builtin_amdgcn_s_barrier(); // every wave has read the exchange slots of the previous block
-        }
-        pair_reduce<2, false>(acc, lds + S_OFF, wave, partner, lane);
+        for (int t = 0; t < 2; t++)
+            init_acc(acc[t], b.bias2 + ct0 + 16 * h, false);
+        w0 = a.wfrag + (size_t)ct0 * 64 + lane * 16;
+        ring_fill1<CPT, D>(ringa, ldw); // a's first weights travel while b is reduced
+        reduce_all<CPT2, 2, D>(acc, ring, (int)b.xmask, ldw2, ldb2);
         v4i res[2];
 #pragma unroll
         for (int t = 0; t < 2; t++)
-            res[t] = requant16(b, acc[t][0], 0);
+            res[t] = requant16(b, acc[t], 0);
         // ---- a, then the add ----
 #pragma unroll
-        for (int t = 0; t < 2; t++) {
-            init_acc(acc[t][0], a.bias2 + ct0 + 16 * h, kh != 0);
-            init_acc(acc[t][1], a.bias2 + ct1 + 16 * h, kh != 0);
-        }
-        reduce_half<CPT, 2, D>(acc, ringa, kh, (int)a.xmask, ldw, ldb);
-        const int st0 = ct0; // this block's channels; the next block's shortcut weights travel during the exchange and the add
-        ct0 += 128, ct1 += 128;
+        for (int t = 0; t < 2; t++)
+            init_acc(acc[t], a.bias2 + ct0 + 16 * h, false);
+        const int st0 = ct0; // this block's channels; the next block's shortcut weights travel during a's reduction and the add
+        ct0 += 128;
         if (bi + 1 < geo.nbpw) {
-            v0 = b.wfrag + (size_t)ct0 * 64 + lane * 16, v1 = b.wfrag + (size_t)ct1 * 64 + lane * 16;
-            ring_fill<CPT2, D>(ring, kh, ldw2);
+            v0 = b.wfrag + (size_t)ct0 * 64 + lane * 16;
+            ring_fill1<CPT2, D>(ring, ldw2);
         }
-        __builtin_amdgcn_s_waitcnt(0xC07F);
-        __builtin_amdgcn_s_barrier(); // every wave has read the exchange slots of b
-        pair_reduce<2, false>(acc, lds + S_OFF, wave, partner, lane);
+        reduce_all<CPT, 2, D>(acc, ringa, (int)a.xmask, ldw, ldb);
 #pragma unroll
         for (int t = 0; t < 2; t++) {
-            const v4i o = requant_add16(a, acc[t][0], res[t]);
+            const v4i o = requant_add16(a, acc[t], res[t]);
             if (valid[t])
                 *reinterpret_cast<v4i *>(a.y + pix[t] * a.out_cs + st0 + 16 * h) = o;
         }
