@@ -2429,11 +2429,11 @@ extern "C" int hipq_conv2d_add2_fusable(const hipq_conv2d_plan *p, const hipq_co
     ConvArgs a;
     if (!add_args(p, shortcut_is_input0, sc->d.oalpha, sc->d.ozp, oalpha, ozp, obits, &a) || !conv_wreg_dual_applies(a, sc->args))
         return 0;
-    // built-in rule: where it measured faster than the two launches - 256 -> 1024 with a 512-channel shortcut on 14x14
-    // images at batch 64 (28.1 us against 15.8 + 14.1 and a launch gap; 512 -> 2048 on 7x7 images loses, 28.9 against
-    // 12.6 + 10.7: its pixel operands leave LDS room for one work-group of four waves per CU);
+    // built-in rule: where it measured at least as fast as the two launches at batch 64 - 256 -> 1024 with a 512-channel
+    // shortcut on 14x14 images, and 512 -> 2048 with a 1024-channel shortcut on 7x7 images (one work-group of four waves
+    // per CU: level with the two launches inside a ResNet-50 pass, 0.6543 against 0.6555 ms, one launch fewer);
     // hipq_conv2d_plan_special(plan, 2): wherever it applies
-    return p->special == 2 || (a.P <= 16384 && a.in_cs == 256) ? 1 : 0;
+    return p->special == 2 || (a.P <= 16384 && (a.in_cs == 256 || a.in_cs == 512)) ? 1 : 0;
 }
 
 extern "C" int hipq_conv2d_run_add2(const hipq_conv2d_plan *p, const void *x, const hipq_conv2d_plan *sc, const void *x_shortcut,
