@@ -136,6 +136,9 @@ struct conv_op_t {
     // A convolution that heads a bottleneck block (1x1, then 3x3, then 1x1 and the add with the block's input) which
     // hipq_bottleneck_run computes in one launch: the block's 3x3 convolution and its add (else null).
     const op_t *blk_next, *blk_add;
+    // this pass's output has already been written by the kernel of the pooling operator whose output this convolution
+    // reads (hipq_conv2d_run_maxpool_conv): run() has nothing left to do
+    bool computed_ahead;
 };
 
 void conv_config(op_t *op)
@@ -321,6 +324,10 @@ bool sole_reader_fuses(op_t *op)
 void conv_run(op_t *op)
 {
     conv_op_t *c = reinterpret_cast<conv_op_t *>(op);
+    if (c->computed_ahead) {
+        c->computed_ahead = false;
+        return;
+    }
     if (c->defer == 0)
         c->defer = sole_reader_fuses(op) ? 1 : -1;
     if (c->defer == 1) {
@@ -1028,6 +1035,35 @@ bool pool_run_fused(op_t *op)
         return false;
     const hip_mem_t *y = as_hip(op->output_tensors[0].mem);
     const void *xin = in_ptr(cop, 0);
+    // The 1x1 convolutions that read the pooled tensor - a residual network's first layer and its projection shortcut -
+    // are computed by the same kernel while a pooled row is in LDS, when they are its only readers (one or two): their
+    // run() then finds its work done.
+    static const bool no_chain = getenv("NART_HIP_NO_FUSION") != nullptr;
+    const reader_map &rm = readers_of(op);
+    const auto it = rm.find(op->output_tensors[0].mem);
+    if (!no_chain && it != rm.end() && (it->second.size() == 1 || it->second.size() == 2)) {
+        conv_op_t *nx[2] = {nullptr, nullptr};
+        int n = 0;
+        bool ok = true;
+        for (const op_t *r : it->second) {
+            conv_op_t *cn = reinterpret_cast<conv_op_t *>(const_cast<op_t *>(r));
+            ok = ok && r->workspace == op->workspace && r->entry->tp == &op_conv_2d_tp
+                && r->input_tensors[0]->mem == op->output_tensors[0].mem && cn->plan != nullptr;
+            nx[n++] = cn;
+        }
+        if (ok && hipq_conv2d_maxpool_conv_fusable(c->plan, y->H, y->W, nx[0]->plan, nx[1] ? nx[1]->plan : nullptr)) {
+            void *y0 = out_ptr(&nx[0]->o), *y1 = nx[1] ? out_ptr(&nx[1]->o) : nullptr;
+            if (hipq_conv2d_run_maxpool_conv(c->plan, xin, out_ptr(op), y->H, y->W, relu, nx[0]->plan, 0, y0,
+                                             nx[1] ? nx[1]->plan : nullptr, 0, y1, op_stream(op)) == 0) {
+                nx[0]->computed_ahead = true;
+                if (nx[1])
+                    nx[1]->computed_ahead = true;
+                ++g_fused_pools;
+                g_chained_convs += n;
+                return true;
+            }
+        }
+    }
     if (hipq_conv2d_run_maxpool(c->plan, xin, out_ptr(op), y->H, y->W, relu, op_stream(op)) != 0)
         return false;
     ++g_fused_pools;

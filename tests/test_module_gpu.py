@@ -566,6 +566,53 @@ def test_stem_convolution_relu_and_max_pooling_run_as_one_kernel(own_rt):
     ws.delete()
 
 
+def test_stem_pooling_and_the_convolutions_that_read_it_run_as_one_kernel(own_rt):
+    """conv_2d (7x7, stride 2) -> max pooling 3x3 / 2 / 1 -> two 1x1 conv_2d operators on the pooled tensor (64 -> 64 and
+    64 -> 256, a residual network's first layer and its projection shortcut): the pooling's run() launches the stem's
+    kernel for all four operators and the two convolutions' run() find their work done.  A third reader of the pooled
+    tensor, or a reader the kernel does not take (3x3), gets the stem with its pooling and the readers one by one."""
+    import ctypes as C
+    from oracle import orc
+    pools = own_rt.libs[1].hip_module_fused_pools
+    pools.restype = C.c_long
+    chained = own_rt.libs[1].hip_module_chained_convs
+    chained.restype = C.c_long
+    ws = own_rt.workspace("hip")
+    rng = np.random.default_rng(29)
+    x = rng.integers(0, 256, (2, 3, 64, 96), dtype=np.uint8)
+    w = rng.integers(0, 256, (64, 3, 7, 7), dtype=np.uint8)
+    b = rng.integers(-5000, 5000, 64).astype(np.int32)
+    q = dict(ialpha=0.031, izp=77, walpha=0.0042, wzp=128, oalpha=0.09, ozp=0)
+    qp = dict(ialpha=0.09, izp=0, oalpha=0.09, ozp=0)
+    want_c = orc.conv2d_u8(x, w, b, 3, 2, 1, 0.031, 77, 0.0042, 128, 0.09, 0)
+    want_p = orc.pool_u8(want_c, 3, 1, 2, 0, False, 0.09, 0, 0.09, 0)
+    readers = []
+    for K, k, oa, oz in ((64, 1, 0.07, 0), (256, 1, 0.11, 113), (64, 3, 0.2, 0)):
+        wr = rng.integers(1, 256, (K, 64, k, k), dtype=np.uint8)
+        br = rng.integers(-9000, 9000, K).astype(np.int32)
+        qr = dict(ialpha=0.09, izp=0, walpha=0.004, wzp=128, oalpha=oa, ozp=oz)
+        readers.append((wr, br, qr, k, orc.conv2d_u8(want_p, wr, br, k // 2, 1, 1, 0.09, 0, 0.004, 128, oa, oz)))
+    assert all(len(np.unique(r[4])) > 32 for r in readers)
+    for pick, expect_chain in (((0, 1), 2), ((0,), 1), ((0, 1, 2), 0), ((2,), 0)):
+        conv = ws.conv2d(ws.tensor(x), ws.tensor(w), ws.tensor(b), 3, 2, 1, q).prepare()
+        pool = ws.pool(conv.output(0), 3, 1, 2, 0, False, qp).prepare()
+        ops = [ws.conv2d(pool.output(0), ws.tensor(readers[i][0]), ws.tensor(readers[i][1]), readers[i][3] // 2, 1, 1,
+                         readers[i][2]).prepare() for i in pick]
+        for rep in range(2):
+            n0, c0 = pools(), chained()
+            conv.run()
+            pool.run()
+            for o in ops:
+                o.run()
+            for i, o in zip(pick, ops):
+                assert same_bits(o.output(0).numpy(), readers[i][4]), (pick, i, rep)
+            assert same_bits(pool.output(0).numpy(), want_p), (pick, rep)
+            assert pools() == n0 + 1 and chained() == c0 + expect_chain, (pick, rep, pools() - n0, chained() - c0)
+        for o in ops[::-1] + [pool, conv]:
+            o.delete()
+    ws.delete()
+
+
 def test_concat_softmax_through_the_op_api(own_rt):
     import refrun
     from oracle import orc
