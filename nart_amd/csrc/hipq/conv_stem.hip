@@ -210,20 +210,20 @@ __global__ __launch_bounds__(256, 2) void conv_stem_maxpool_kernel(const ConvArg
         if (NEXT) {
             // every thread passes the next row's barrier only after its reads below: one buffer is enough
             __syncthreads();
-            // wave w: pixel tile w & 1, the 32-channel tiles (w >> 1), (w >> 1) + 2, ... of each layer
+            // wave w: pixel tile w & 1, pairs of neighbouring 32-channel tiles of each layer in turn with wave w ^ 2
             const int q = 32 * (wave & 1) + p;
             v4i b[2];
 #pragma unroll
             for (int kk = 0; kk < 2; kk++) // both layers read the pooled bytes with the same zero point (the host checks)
                 b[kk] = *reinterpret_cast<const v4i *>(lds + P_OFF + q * 64 + (((2 * kk + half) ^ (q & 3)) << 4)) ^ (int)an.xmask;
             const size_t pixn = (size_t)(n * POH + ph0 + j) * POW + q;
-            // ch0: the layer's first channel among all chained channels; U tiles at a time, so that one tile's LDS reads
-            // and multiplies run under another's requantisation
+            // ch0: the layer's first channel among all chained channels; U neighbouring tiles at a time, so that one tile's
+            // LDS reads and multiplies run under another's requantisation and a lane's two stores are 64 consecutive bytes
             auto tiles = [&](const ConvArgs &al, const int ch0, const int nt0, auto U) {
                 v16i accn[U.value];
 #pragma unroll
                 for (int u = 0; u < U.value; u++) {
-                    const int c = ch0 + 32 * (nt0 + 2 * u);
+                    const int c = ch0 + 32 * (nt0 + u);
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
                         const v4i bv = *reinterpret_cast<const v4i *>(lds + B_OFF + (c + 16 * half + 4 * g) * 4);
@@ -236,23 +236,24 @@ __global__ __launch_bounds__(256, 2) void conv_stem_maxpool_kernel(const ConvArg
                 for (int kk = 0; kk < 2; kk++)
 #pragma unroll
                     for (int u = 0; u < U.value; u++) {
-                        const uint8_t *wp = lds + W_OFF + (ch0 + 32 * (nt0 + 2 * u)) * 64 + lane * 16;
+                        const uint8_t *wp = lds + W_OFF + (ch0 + 32 * (nt0 + u)) * 64 + lane * 16;
                         accn[u] = __builtin_amdgcn_mfma_i32_32x32x32_i8(*reinterpret_cast<const v4i *>(wp + kk * 1024), b[kk], accn[u], 0, 0, 0);
                     }
 #pragma unroll
                 for (int u = 0; u < U.value; u++) {
                     const v4i o = frag::requant16(al, accn[u], 0);
                     if (q < POW)
-                        *reinterpret_cast<v4i *>(al.y + pixn * al.K + 32 * (nt0 + 2 * u) + 16 * half) = o;
+                        *reinterpret_cast<v4i *>(al.y + pixn * al.K + 32 * (nt0 + u) + 16 * half) = o;
                 }
             };
             auto layer = [&](const ConvArgs &al, const int ch0) {
-                const int ntl = al.K / 32; // a multiple of 2: the wave's tiles are (wave >> 1) + 2 i, i < ntl / 2
-                int nt = wave >> 1;
-                for (; nt + 2 < ntl; nt += 4)
+                const int ntl = al.K / 32; // a multiple of 2; the waves of a pixel tile (wave >> 1 = 0, 1) take pairs of tiles in turn
+                if (ntl == 2) {
+                    tiles(al, ch0, wave >> 1, std::integral_constant<int, 1>());
+                    return;
+                }
+                for (int nt = 2 * (wave >> 1); nt < ntl; nt += 4)
                     tiles(al, ch0, nt, std::integral_constant<int, 2>());
-                if (nt < ntl)
-                    tiles(al, ch0, nt, std::integral_constant<int, 1>());
             };
             layer(an, 0);
             if (NEXT == 2)
