@@ -40,7 +40,7 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s (published)
 # (traffic is null, with the reason, once a kernel has changed and the profile has not been taken again).
 TRAFFIC_FROM_PROFILE = {"workload": "resnet50", "batch": 64, "bytes_per_launch": 52.38e6,
                         "source": "profiles/conv_mfma_i8_resnet50_n64.md",
-                        "sources_sha256": "ff05c3101d319545"}
+                        "sources_sha256": "6d68c9770807851a"}
 
 
 def kernel_sources_digest():
