@@ -136,15 +136,15 @@ __device__ static __forceinline__ u32x4 add_16(u32x4 a, u32x4 b, const AddParams
     return y;
 }
 
-// byte-wise unsigned maximum of two packed dwords
+// byte-wise unsigned maximum of two packed dwords: bytes 0 and 2 are compared as the 16-bit halves of x & 0x00ff00ff,
+// bytes 1 and 3 in place as the halves of x & 0xff00ff00 (their low bytes are zero on both sides), two v_pk_max_u16
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
 __device__ static inline uint32_t max_u8x4(uint32_t a, uint32_t b)
 {
-    // per byte: a >= b ? a : b, from the borrow of (a | 0x80) - (b & 0x7f) combined with the top bits
-    const uint32_t H = 0x80808080u;
-    const uint32_t d = (a | H) - (b & ~H);       // no borrow across bytes
-    const uint32_t ge = ((a & ~b) | (~(a ^ b) & d)) & H; // top bit set where a >= b
-    const uint32_t m = (ge >> 7) * 0xffu;        // 0xff in those bytes
-    return (a & m) | (b & ~m);
+    const uint32_t E = 0x00ff00ffu;
+    const u16x2 lo = __builtin_elementwise_max(__builtin_bit_cast(u16x2, a & E), __builtin_bit_cast(u16x2, b & E));
+    const u16x2 hi = __builtin_elementwise_max(__builtin_bit_cast(u16x2, a & ~E), __builtin_bit_cast(u16x2, b & ~E));
+    return __builtin_bit_cast(uint32_t, lo) | __builtin_bit_cast(uint32_t, hi);
 }
 
 // Fills *p from the operator's settings; returns false if a scale is outside the fixed-point range.
