@@ -251,6 +251,8 @@ __global__ __launch_bounds__(256) void pool_max16_u8_kernel(const PoolArgs p, do
     const int c16n = p.cs >> 4;
     const int total = p.N * p.OH * p.OW * c16n; // the host guarantees 31 bits
     const int radd = (1 << (p.shift - 1)) + (p.oz << p.shift);
+    const int phi = ((p.hi + 1) << p.shift) - 1; // the largest value that the shift takes to hi
+    const bool same = p.mult == (1u << p.shift) && p.iz == p.oz && p.hi == 255;
     // work-groups go to the 8 XCDs in turn: renumbered so that each XCD works on a contiguous eighth of the (image-major)
     // index space, the eighth whose pixels its convolution tiles read (the grid is a multiple of 8)
     const int L = (int)(blockIdx.x & 7) * (int)(gridDim.x >> 3) + (int)(blockIdx.x >> 3);
@@ -273,17 +275,20 @@ __global__ __launch_bounds__(256) void pool_max16_u8_kernel(const PoolArgs p, do
                 for (int d = 0; d < 4; d++)
                     mx[d] = max_u8x4(mx[d], v[d]);
             }
-        u32x4 o;
+        u32x4 o = mx;
+        if (!same) { // else equal scales (a multiplier of exactly 2^shift), equal zero points, 8 bits: the maximum is the result
 #pragma unroll
-        for (int d = 0; d < 4; d++) {
-            uint32_t w = 0;
+            for (int d = 0; d < 4; d++) {
+                int32_t v[4];
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                // mult < 2^16, |max - zp| <= 255: the product fits 24 bits, shift <= 30 (host): 32-bit arithmetic is exact
-                const int32_t pr = __mul24((int)p.mult, (int)((mx[d] >> (8 * e)) & 255) - p.iz);
-                w |= (uint32_t)sat_hi((pr + radd) >> p.shift, p.hi) << (8 * e);
+                for (int e = 0; e < 4; e++) {
+                    // mult < 2^16, |max - zp| <= 255: the product fits 24 bits, shift <= 22 (host): 32-bit arithmetic is
+                    // exact; the upper clamp in front of the shift, the lower one is the pack's saturation
+                    const int32_t pr = __mul24((int)p.mult, (int)((mx[d] >> (8 * e)) & 255) - p.iz);
+                    v[e] = min(pr + radd, phi);
+                }
+                o[d] = ashr_sat_u8x4(v[0], v[1], v[2], v[3], p.shift);
             }
-            o[d] = w;
         }
         *reinterpret_cast<u32x4 *>(p.y + (size_t)mm * p.cs + c0) = o;
     }
