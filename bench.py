@@ -38,9 +38,9 @@ PEAK_HBM_GBS = 8000.0     # MI355X HBM3E, GB/s (published)
 # file that holds the counter readings and a digest of the kernel sources it was taken with: the line reports it only
 # for the default workload with default flags and only while the sources under nart_amd/csrc/hipq still have that digest
 # (traffic is null, with the reason, once a kernel has changed and the profile has not been taken again).
-TRAFFIC_FROM_PROFILE = {"workload": "resnet50", "batch": 64, "bytes_per_launch": 52.38e6,
+TRAFFIC_FROM_PROFILE = {"workload": "resnet50", "batch": 64, "bytes_per_launch": 52.40e6,
                         "source": "profiles/conv_mfma_i8_resnet50_n64.md",
-                        "sources_sha256": "6d68c9770807851a"}
+                        "sources_sha256": "7b2ea2a739053335"}
 
 
 def kernel_sources_digest():
